@@ -1,0 +1,124 @@
+"""Builds the native pieces of the HIP backend for gfx950, in-tree.
+
+Outputs, next to this file (the reference keeps its runtime libraries in the
+package directory as well and finds them there,
+reference: numba_mlir/numba_mlir/mlir/utils.py:17-42):
+
+  libnumba-mlir-gpu-runtime-hip.so    the 13 gpux* entry points
+  libnumba-mlir-math-hip-runtime.so   mkl_gemm_<dtype>_device
+  libnumba-mlir-hip-offload.so        lowered host code, dispatcher and the
+                                      embedded code objects of the kernels
+
+The HIP runtime is built by its own hipcc step, separate from everything
+else, as the reference builds its SYCL runtime with its own compiler
+(reference: numba_mlir/setup_helper.py:34-81).
+
+Run:  python -m numba_mlir_amd.build   (or call build_all()).
+"""
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+BUILD = os.path.join(CSRC, "build")
+INCLUDE = os.path.join(ROOT, "include")
+
+ARCH = "gfx950"
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+HIPCC = os.environ.get("HIPCC", os.path.join(ROCM, "bin", "hipcc"))
+CXX = os.environ.get("CXX", "g++")
+
+# Packed-FP32 instructions are kept out of all device code.
+DEVICE_FLAGS = [
+    f"--offload-arch={ARCH}",
+    "-O3",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+HOST_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-fvisibility=hidden", f"-I{INCLUDE}",
+              "-Wall"]
+# Host-only libraries are plain C++ that call the HIP runtime API.
+HIP_HOST_FLAGS = ["-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(ROCM, "include")]
+HIP_LINK_FLAGS = ["-L" + os.path.join(ROCM, "lib"), "-lamdhip64",
+                  "-Wl,-rpath," + os.path.join(ROCM, "lib")]
+
+KERNEL_FAMILIES = ["maps", "reduce", "twins"]
+
+RUNTIME_LIB = "libnumba-mlir-gpu-runtime-hip.so"
+MATH_LIB = "libnumba-mlir-math-hip-runtime.so"
+OFFLOAD_LIB = "libnumba-mlir-hip-offload.so"
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                          text=True)
+    out = "\n".join(
+        line for line in proc.stdout.splitlines()
+        if "packed-fp32-ops" not in line and line.strip()
+    )
+    if proc.returncode != 0:
+        raise RuntimeError("build step failed:\n  " + " ".join(cmd) + "\n" + out)
+    if out:
+        print(out, file=sys.stderr)
+
+
+def build_code_object(family):
+    """One gfx950 ELF code object per kernel family.
+
+    -ffp-contract=off keeps a*b+c as two roundings, matching the reference's
+    CPU lowering (no fma without fastmath).
+    """
+    src = os.path.join(CSRC, "kernels", family + ".hip")
+    out = os.path.join(BUILD, family + ".hsaco")
+    _run([HIPCC, "--genco", "--no-gpu-bundle-output", *DEVICE_FLAGS,
+          "-ffp-contract=off", "-o", out, src])
+    return out
+
+
+def build_runtime():
+    srcs = [os.path.join(CSRC, "runtime", f)
+            for f in ("GpuRuntime.cpp", "HipApiReal.cpp")]
+    _run([CXX, *HOST_FLAGS, *HIP_HOST_FLAGS, "-shared", *srcs,
+          "-Wl,--version-script=" + os.path.join(CSRC, "runtime", "export.map"),
+          "-o", os.path.join(HERE, RUNTIME_LIB), *HIP_LINK_FLAGS, "-lpthread"])
+
+
+def build_math():
+    _run([HIPCC, *HOST_FLAGS, "-Wno-unused-command-line-argument",
+          *DEVICE_FLAGS, "-shared",
+          os.path.join(CSRC, "math", "Gemm.hip"),
+          "-Wl,--version-script=" + os.path.join(CSRC, "math", "export.map"),
+          "-o", os.path.join(HERE, MATH_LIB)])
+
+
+def build_offload():
+    _run([CXX, *HOST_FLAGS, *HIP_HOST_FLAGS, "-shared",
+          os.path.join(CSRC, "offload", "Offload.cpp"),
+          os.path.join(CSRC, "offload", "Blobs.S"),
+          "-Wa,-I" + BUILD,
+          "-Wl,--version-script=" + os.path.join(CSRC, "offload", "export.map"),
+          "-o", os.path.join(HERE, OFFLOAD_LIB), *HIP_LINK_FLAGS, "-lpthread"])
+
+
+def build_all(jobs=4):
+    os.makedirs(BUILD, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        futures = [pool.submit(build_code_object, f) for f in KERNEL_FAMILIES]
+        futures.append(pool.submit(build_runtime))
+        futures.append(pool.submit(build_math))
+        for f in futures:
+            f.result()
+    build_offload()  # embeds the code objects built above
+
+
+def libraries_present():
+    return all(os.path.exists(os.path.join(HERE, n))
+               for n in (RUNTIME_LIB, MATH_LIB, OFFLOAD_LIB))
+
+
+if __name__ == "__main__":
+    build_all()
+    print("built:", RUNTIME_LIB, MATH_LIB, OFFLOAD_LIB)

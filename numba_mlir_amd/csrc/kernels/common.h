@@ -1,0 +1,75 @@
+// Shared device helpers for the gfx950 kernel families.
+//
+// All kernels are built for wave64 CDNA4 only, with -ffp-contract=off so a
+// separate multiply and add stay two IEEE roundings, as on the reference's
+// CPU path (fma contraction there needs fastmath=True; reference:
+// numba_mlir/numba_mlir/mlir/tests/test_gpu.py:980-1008).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define NMK_WAVE 64
+
+#define NMK_KERNEL(threads)                                                    \
+  extern "C" __global__ __launch_bounds__(threads) void
+
+namespace nmk {
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef double double2_t __attribute__((ext_vector_type(2)));
+typedef int int4_t __attribute__((ext_vector_type(4)));
+
+// Butterfly reduction over the 64 lanes of a wave; every lane ends up with
+// the total.  The combination tree is fixed, so the result is deterministic.
+template <typename T, typename Op>
+__device__ __forceinline__ T waveAllReduce(T v, Op op) {
+#pragma unroll
+  for (int off = NMK_WAVE / 2; off > 0; off >>= 1)
+    v = op(v, __shfl_xor(v, off, NMK_WAVE));
+  return v;
+}
+
+struct AddOp {
+  template <typename T> __device__ __forceinline__ T operator()(T a, T b) const {
+    return a + b;
+  }
+};
+struct MulOp {
+  template <typename T> __device__ __forceinline__ T operator()(T a, T b) const {
+    return a * b;
+  }
+};
+struct MinOp {
+  template <typename T> __device__ __forceinline__ T operator()(T a, T b) const {
+    return b < a ? b : a;
+  }
+};
+struct MaxOp {
+  template <typename T> __device__ __forceinline__ T operator()(T a, T b) const {
+    return a < b ? b : a;
+  }
+};
+
+// Block-wide reduction for blocks of THREADS (multiple of 64): wave butterfly,
+// one LDS slot per wave, then every thread folds the slots in wave order.
+template <int THREADS, typename T, typename Op>
+__device__ __forceinline__ T blockAllReduce(T v, Op op, T *slots) {
+  constexpr int WAVES = THREADS / NMK_WAVE;
+  v = waveAllReduce(v, op);
+  if (WAVES == 1)
+    return v;
+  const int wave = threadIdx.x / NMK_WAVE;
+  const int lane = threadIdx.x % NMK_WAVE;
+  __syncthreads(); // slots may still be read from a previous call
+  if (lane == 0)
+    slots[wave] = v;
+  __syncthreads();
+  T total = slots[0];
+#pragma unroll
+  for (int w = 1; w < WAVES; ++w)
+    total = op(total, slots[w]);
+  return total;
+}
+
+} // namespace nmk

@@ -1,0 +1,291 @@
+// Reductions for gfx950: axis sums, full sum-of-squares norm, and a generic
+// strided fallback for sum/prod/min/max.
+//
+// They replace what the reference generates from a linalg.generic with
+// `reduction` iterators (reference: numba_mlir/numba_mlir/mlir/numpy/funcs.py:163-229).
+// There an axis reduction makes ONE work-item walk a whole row or column
+// (mlir_compiler/lib/pipelines/LowerToGpu.cpp:228-245) and a full reduction
+// stores per-workgroup partials to host-shared memory and finishes on the
+// host (mlir/lib/Conversion/GpuToGpuRuntime.cpp:2161-2277).  Here a wave owns
+// a row (axis=1), a block owns a column strip (axis=0), and full reductions
+// finish on the device in the last block to arrive: a single launch, no
+// arithmetic atomics, a fixed combination order.
+//
+// Integer reductions accumulate in, and produce, int64 (promote_int,
+// numpy/funcs.py:120-123, 176, 210); min/max start from the accumulator
+// type's extreme or +-inf (numpy/funcs.py:275-300).
+#include "common.h"
+
+#include <limits>
+
+using namespace nmk;
+
+// ---------------------------------------------------------------------------
+// out[r] = sum_c x[r * ld + c], float32.  One wave per row, four rows per
+// block.  When ld and cols are multiples of 4 and x is 16-byte aligned
+// (vec != 0) lanes read float4, four loads in flight; lane partials are
+// folded pairwise, then a wave butterfly.
+NMK_KERNEL(256)
+nmk_sum_axis1_f32(const float *__restrict__ x, float *__restrict__ out,
+                  int64_t rows, int64_t cols, int64_t ld, int32_t vec) {
+  const int lane = threadIdx.x % NMK_WAVE;
+  const int64_t row =
+      int64_t(blockIdx.x) * (blockDim.x / NMK_WAVE) + threadIdx.x / NMK_WAVE;
+  if (row >= rows)
+    return;
+  const float *p = x + row * ld;
+  float total;
+  if (vec) {
+    const float4_t *pv = reinterpret_cast<const float4_t *>(p);
+    const int64_t nvec = cols / 4;
+    float4_t a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0, a3 = a0;
+    int64_t i = lane;
+    for (; i + 3 * NMK_WAVE < nvec; i += 4 * NMK_WAVE) {
+      float4_t v0 = __builtin_nontemporal_load(pv + i);
+      float4_t v1 = __builtin_nontemporal_load(pv + i + NMK_WAVE);
+      float4_t v2 = __builtin_nontemporal_load(pv + i + 2 * NMK_WAVE);
+      float4_t v3 = __builtin_nontemporal_load(pv + i + 3 * NMK_WAVE);
+      a0 += v0;
+      a1 += v1;
+      a2 += v2;
+      a3 += v3;
+    }
+    for (; i < nvec; i += NMK_WAVE)
+      a0 += pv[i];
+    float4_t a = (a0 + a1) + (a2 + a3);
+    total = (a[0] + a[1]) + (a[2] + a[3]);
+  } else {
+    total = 0.f;
+    for (int64_t i = lane; i < cols; i += NMK_WAVE)
+      total += p[i];
+  }
+  total = waveAllReduce(total, AddOp());
+  if (lane == 0)
+    out[row] = total;
+}
+
+// ---------------------------------------------------------------------------
+// out[c] = sum_r int64(x[r * ld + c]), int32 input.  Requires cols % 4 == 0,
+// ld % 4 == 0 and a 16-byte aligned base (dispatcher falls back to the
+// generic kernel otherwise).
+//
+// grid.x = column strips of 256 columns (64 lanes x int4), grid.y = row
+// chunks of rowsPerBlock.  The four waves of a block take interleaved rows of
+// the chunk, fold through LDS, and store one int64 partial per column to
+// partial[chunk][col].  The last block of a strip to finish (ordered by a
+// ticket counter, used for ordering only) adds the chunks in index order and
+// writes out[]; it also resets the ticket, so the counters are zero again
+// when the kernel ends.
+NMK_KERNEL(256)
+nmk_sum_axis0_i32_i64(const int32_t *__restrict__ x, int64_t *__restrict__ out,
+                      int64_t rows, int64_t cols, int64_t ld,
+                      int64_t rowsPerBlock, int64_t *__restrict__ partial,
+                      uint32_t *__restrict__ tickets) {
+  __shared__ int64_t fold[4][256];
+  __shared__ uint32_t isLast;
+  const int lane = threadIdx.x % NMK_WAVE;
+  const int wave = threadIdx.x / NMK_WAVE;
+  const int64_t strip = blockIdx.x;
+  const int64_t chunk = blockIdx.y;
+  const int64_t col = strip * 256 + lane * 4;
+  int64_t acc[4] = {0, 0, 0, 0};
+  if (col < cols) {
+    int64_t r = chunk * rowsPerBlock + wave;
+    int64_t rEnd = (chunk + 1) * rowsPerBlock;
+    if (rEnd > rows)
+      rEnd = rows;
+    const int32_t *p = x + r * ld + col;
+    const int64_t step = 4 * ld;
+    for (; r + 12 < rEnd; r += 16) {
+      int4_t v0 = __builtin_nontemporal_load(reinterpret_cast<const int4_t *>(p));
+      int4_t v1 =
+          __builtin_nontemporal_load(reinterpret_cast<const int4_t *>(p + step));
+      int4_t v2 = __builtin_nontemporal_load(
+          reinterpret_cast<const int4_t *>(p + 2 * step));
+      int4_t v3 = __builtin_nontemporal_load(
+          reinterpret_cast<const int4_t *>(p + 3 * step));
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        acc[k] += (int64_t(v0[k]) + int64_t(v1[k])) +
+                  (int64_t(v2[k]) + int64_t(v3[k]));
+      p += 4 * step;
+    }
+    for (; r < rEnd; r += 4) {
+      int4_t v0 = *reinterpret_cast<const int4_t *>(p);
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        acc[k] += int64_t(v0[k]);
+      p += step;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+    fold[wave][lane * 4 + k] = acc[k];
+  __syncthreads();
+  const int64_t myCol = strip * 256 + threadIdx.x;
+  if (myCol < cols) {
+    int64_t s = (fold[0][threadIdx.x] + fold[1][threadIdx.x]) +
+                (fold[2][threadIdx.x] + fold[3][threadIdx.x]);
+    partial[chunk * cols + myCol] = s;
+  }
+  // Publish the partials, then take a ticket.
+  __threadfence();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t ticket = atomicAdd(&tickets[strip], 1u);
+    isLast = (ticket == gridDim.y - 1) ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!isLast)
+    return;
+  __threadfence();
+  if (myCol < cols) {
+    int64_t s = 0;
+    for (int64_t c = 0; c < int64_t(gridDim.y); ++c)
+      s += __builtin_nontemporal_load(partial + c * cols + myCol);
+    out[myCol] = s;
+  }
+  if (threadIdx.x == 0)
+    tickets[strip] = 0;
+}
+
+// ---------------------------------------------------------------------------
+// out[0] = sqrt(sum_i x[i] * x[i]), float32, n elements contiguous
+// (np.sqrt(np.sum(x * x)): the square is fused into the reduction as the
+// reference's elementwise fusion does, mlir_compiler/lib/pipelines/PlierToLinalg.cpp:3149-3199;
+// the sqrt of the 0-d result is the scalar path, numpy/funcs.py:364-368).
+//
+// Grid-stride float4 loads (vec != 0 needs a 16-byte aligned base), float32
+// lane partials, block tree, one partial per block; the last block to take a
+// ticket folds the partials in block order and applies sqrtf.
+template <bool SQUARE_ROOT_OF_SQUARES>
+__device__ __forceinline__ void
+fullSumF32(const float *__restrict__ x, float *__restrict__ out, int64_t n,
+           int32_t vec, float *__restrict__ partial,
+           uint32_t *__restrict__ ticket) {
+  __shared__ float slots[4];
+  __shared__ uint32_t isLast;
+  const int64_t tid = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t stride = int64_t(gridDim.x) * blockDim.x;
+  float total = 0.f;
+  int64_t done = 0;
+  if (vec) {
+    const float4_t *pv = reinterpret_cast<const float4_t *>(x);
+    const int64_t nvec = n / 4;
+    float4_t a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0, a3 = a0;
+    int64_t i = tid;
+    for (; i + 3 * stride < nvec; i += 4 * stride) {
+      float4_t v0 = __builtin_nontemporal_load(pv + i);
+      float4_t v1 = __builtin_nontemporal_load(pv + i + stride);
+      float4_t v2 = __builtin_nontemporal_load(pv + i + 2 * stride);
+      float4_t v3 = __builtin_nontemporal_load(pv + i + 3 * stride);
+      if (SQUARE_ROOT_OF_SQUARES) {
+        v0 *= v0;
+        v1 *= v1;
+        v2 *= v2;
+        v3 *= v3;
+      }
+      a0 += v0;
+      a1 += v1;
+      a2 += v2;
+      a3 += v3;
+    }
+    for (; i < nvec; i += stride) {
+      float4_t v0 = pv[i];
+      if (SQUARE_ROOT_OF_SQUARES)
+        v0 *= v0;
+      a0 += v0;
+    }
+    float4_t a = (a0 + a1) + (a2 + a3);
+    total = (a[0] + a[1]) + (a[2] + a[3]);
+    done = nvec * 4;
+  }
+  for (int64_t i = done + tid; i < n; i += stride) {
+    float v = x[i];
+    total += SQUARE_ROOT_OF_SQUARES ? v * v : v;
+  }
+  total = blockAllReduce<256>(total, AddOp(), slots);
+  if (threadIdx.x == 0) {
+    partial[blockIdx.x] = total;
+    __threadfence();
+    uint32_t t = atomicAdd(ticket, 1u);
+    isLast = (t == gridDim.x - 1) ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!isLast)
+    return;
+  __threadfence();
+  float s = 0.f;
+  for (int64_t b = threadIdx.x; b < int64_t(gridDim.x); b += blockDim.x)
+    s += __builtin_nontemporal_load(partial + b);
+  s = blockAllReduce<256>(s, AddOp(), slots);
+  if (threadIdx.x == 0) {
+    out[0] = SQUARE_ROOT_OF_SQUARES ? sqrtf(s) : s;
+    *ticket = 0;
+  }
+}
+
+NMK_KERNEL(256)
+nmk_norm2_f32(const float *x, float *out, int64_t n, int32_t vec,
+              float *partial, uint32_t *ticket) {
+  fullSumF32<true>(x, out, n, vec, partial, ticket);
+}
+
+NMK_KERNEL(256)
+nmk_sum_all_f32(const float *x, float *out, int64_t n, int32_t vec,
+                float *partial, uint32_t *ticket) {
+  fullSumF32<false>(x, out, n, vec, partial, ticket);
+}
+
+// ---------------------------------------------------------------------------
+// Generic strided reduction: out[k * so] = fold_r op(x[k * sk + r * sr]) for
+// k < nKeep, r < nRed, accumulating in ACC starting from `init`.  One wave per
+// kept index; lanes stride over the reduced axis, then a wave butterfly.
+// Covers every (op, dtype, axis) combination at modest speed; a full
+// reduction is nKeep == 1.
+template <typename IN, typename ACC, typename Op>
+__device__ __forceinline__ void
+reduceStrided(const IN *x, ACC *out, int64_t nKeep, int64_t nRed, int64_t sk,
+              int64_t sr, int64_t so, ACC init, Op op) {
+  const int lane = threadIdx.x % NMK_WAVE;
+  const int64_t k =
+      int64_t(blockIdx.x) * (blockDim.x / NMK_WAVE) + threadIdx.x / NMK_WAVE;
+  if (k >= nKeep)
+    return;
+  ACC acc = init;
+  const IN *p = x + k * sk;
+  for (int64_t r = lane; r < nRed; r += NMK_WAVE)
+    acc = op(acc, ACC(p[r * sr]));
+  acc = waveAllReduce(acc, op);
+  if (lane == 0)
+    out[k * so] = acc;
+}
+
+#define NMK_DEFINE_REDUCE(OPNAME, OP, INIT, TNAME, IN, ACC)                    \
+  NMK_KERNEL(256)                                                              \
+  nmk_reduce_##OPNAME##_##TNAME(const IN *x, ACC *out, int64_t nKeep,          \
+                                int64_t nRed, int64_t sk, int64_t sr,          \
+                                int64_t so) {                                  \
+    reduceStrided<IN, ACC>(x, out, nKeep, nRed, sk, sr, so, ACC(INIT), OP());  \
+  }
+
+NMK_DEFINE_REDUCE(sum, AddOp, 0, i32, int32_t, int64_t)
+NMK_DEFINE_REDUCE(sum, AddOp, 0, i64, int64_t, int64_t)
+NMK_DEFINE_REDUCE(sum, AddOp, 0, f32, float, float)
+NMK_DEFINE_REDUCE(sum, AddOp, 0, f64, double, double)
+NMK_DEFINE_REDUCE(prod, MulOp, 1, i32, int32_t, int64_t)
+NMK_DEFINE_REDUCE(prod, MulOp, 1, i64, int64_t, int64_t)
+NMK_DEFINE_REDUCE(prod, MulOp, 1, f32, float, float)
+NMK_DEFINE_REDUCE(prod, MulOp, 1, f64, double, double)
+NMK_DEFINE_REDUCE(min, MinOp, std::numeric_limits<int64_t>::max(), i32,
+                  int32_t, int64_t)
+NMK_DEFINE_REDUCE(min, MinOp, std::numeric_limits<int64_t>::max(), i64,
+                  int64_t, int64_t)
+NMK_DEFINE_REDUCE(min, MinOp, __builtin_inff(), f32, float, float)
+NMK_DEFINE_REDUCE(min, MinOp, __builtin_inf(), f64, double, double)
+NMK_DEFINE_REDUCE(max, MaxOp, std::numeric_limits<int64_t>::min(), i32,
+                  int32_t, int64_t)
+NMK_DEFINE_REDUCE(max, MaxOp, std::numeric_limits<int64_t>::min(), i64,
+                  int64_t, int64_t)
+NMK_DEFINE_REDUCE(max, MaxOp, -__builtin_inff(), f32, float, float)
+NMK_DEFINE_REDUCE(max, MaxOp, -__builtin_inf(), f64, double, double)

@@ -1,0 +1,330 @@
+// HIP math runtime: device gemm behind mkl_gemm_<dtype>_device
+// (include/numba_mlir_hip/MathRuntime.h).
+//
+// Entry points, argument meaning and layout rules follow the oneMKL-backed
+// runtime they replace (reference:
+// numba_mlir/numba_mlir/math_runtime/sycl/lib/NumpyLinalg.cpp:67-183); the
+// arithmetic is a hand-written LDS-tiled fp32 MFMA kernel for gfx950 plus a
+// strided fallback.
+#include "numba_mlir_hip/GpuQueueInterface.hpp"
+#include "numba_mlir_hip/MathRuntime.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// fatal_failure of the reference prints to stderr and aborts
+// (math_runtime/include/Common.hpp:10-15).
+[[noreturn]] void fatal(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  std::vfprintf(stderr, fmt, ap);
+  va_end(ap);
+  std::fflush(stderr);
+  std::abort();
+}
+
+void checkHip(hipError_t err, const char *what) {
+  if (err != hipSuccess)
+    fatal("%s failed: %s (%d)\n", what, hipGetErrorString(err),
+          static_cast<int>(err));
+}
+
+thread_local const char *lastKernel = "";
+
+// ---------------------------------------------------------------------------
+// C[M,N] = alpha * A[M,K] * B[K,N] + beta * C, all row-major with leading
+// dimensions lda/ldb/ldc, fp32 in, fp32 accumulate on the matrix cores.
+//
+// Block tile 128 x 128, K step 16, 256 threads = 4 waves in a 2 x 2 grid,
+// each wave owns 64 x 64 = 2 x 2 tiles of v_mfma_f32_32x32x2_f32.
+//
+// LDS holds both operands K-major ([k][m] and [k][n], rows padded by 4 floats)
+// so that the MFMA operand fetch -- lane l needs element (l % 32) of row
+// (k + l / 32) -- is a conflict-free ds_read_b32.  Two LDS stages: the next
+// K slab is fetched from global memory into registers before the MFMAs of the
+// current slab are issued and written to the other stage after them, one
+// barrier per slab.
+//
+// MFMA 32x32x2 operand layout (64 lanes):
+//   A (32 x 2): lane l holds A[l % 32][l / 32]
+//   B (2 x 32): lane l holds B[l / 32][l % 32]
+//   D (32 x 32): lane l, register r holds D[8*(r/4) + 4*(l/32) + r%4][l % 32]
+//
+// Requirements (checked by the host): M % 128 == 0, N % 128 == 0,
+// K % 16 == 0, lda/ldb % 4 == 0, A and B 16-byte aligned.
+constexpr int BM = 128, BN = 128, BK = 16, PAD = 4;
+
+__global__ __launch_bounds__(256) void
+sgemm_mfma_128x128(const float *__restrict__ A, const float *__restrict__ B,
+                   float *__restrict__ C, int M, int N, int K, int64_t lda,
+                   int64_t ldb, int64_t ldc, float alpha, float beta) {
+  __shared__ float As[2][BK][BM + PAD];
+  __shared__ float Bs[2][BK][BN + PAD];
+
+  const int tid = threadIdx.x;
+  const int lane = tid % 64;
+  const int wave = tid / 64;
+  const int wm = wave / 2, wn = wave % 2;
+  const int bm = blockIdx.y * BM;
+  const int bn = blockIdx.x * BN;
+
+  // Global fetch mapping: A slab 128 x 16 -> 2 float4 per thread (k
+  // contiguous); B slab 16 x 128 -> 2 float4 per thread (n contiguous).
+  const int aRow = tid / 4, aK = (tid % 4) * 4;
+  const int bK = tid / 32, bN = (tid % 32) * 4;
+  const float *aPtr = A + int64_t(bm + aRow) * lda + aK;
+  const float *bPtr = B + int64_t(bK) * ldb + bn + bN;
+
+  floatx4 aReg[2], bReg[2];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      aReg[i] = *reinterpret_cast<const floatx4 *>(aPtr + int64_t(64 * i) * lda +
+                                                   k0);
+      bReg[i] = *reinterpret_cast<const floatx4 *>(bPtr +
+                                                   int64_t(k0 + 8 * i) * ldb);
+    }
+  };
+  auto stash = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        As[stage][aK + q][aRow + 64 * i] = aReg[i][q];
+      *reinterpret_cast<floatx4 *>(&Bs[stage][bK + 8 * i][bN]) = bReg[i];
+    }
+  };
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        acc[i][j][r] = 0.f;
+
+  fetch(0);
+  stash(0);
+  __syncthreads();
+
+  const int nSlabs = K / BK;
+  const int kLane = lane / 32, xLane = lane % 32;
+  for (int s = 0; s < nSlabs; ++s) {
+    const int cur = s & 1;
+    if (s + 1 < nSlabs)
+      fetch((s + 1) * BK);
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 2) {
+      float a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        a[i] = As[cur][kk + kLane][wm * 64 + i * 32 + xLane];
+        b[i] = Bs[cur][kk + kLane][wn * 64 + i * 32 + xLane];
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j],
+                                                           acc[i][j], 0, 0, 0);
+    }
+    if (s + 1 < nSlabs)
+      stash(cur ^ 1);
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = bn + wn * 64 + j * 32 + xLane;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = bm + wm * 64 + i * 32 + 8 * (r / 4) + 4 * kLane + r % 4;
+        float *dst = C + int64_t(row) * ldc + col;
+        float v = alpha * acc[i][j][r];
+        if (beta != 0.f)
+          v += beta * *dst;
+        *dst = v;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Any shape, any strides (element strides per dimension), float or double:
+// classic 32 x 32 LDS tiling, one output per thread x 4 rows, bounds checked.
+// Used for the transposed / column-major / ragged cases the MFMA kernel does
+// not take.
+template <typename T>
+__global__ __launch_bounds__(256) void
+gemm_generic(const T *A, const T *B, T *C, int64_t M, int64_t N, int64_t K,
+             int64_t as0, int64_t as1, int64_t bs0, int64_t bs1, int64_t cs0,
+             int64_t cs1, T alpha, T beta) {
+  constexpr int TILE = 32;
+  __shared__ T As[TILE][TILE + 1];
+  __shared__ T Bs[TILE][TILE + 1];
+  const int tx = threadIdx.x % TILE; // column within the tile
+  const int ty = threadIdx.x / TILE; // 0..7, rows ty, ty+8, ty+16, ty+24
+  const int64_t row0 = int64_t(blockIdx.y) * TILE;
+  const int64_t col = int64_t(blockIdx.x) * TILE + tx;
+  T acc[4] = {T(0), T(0), T(0), T(0)};
+  for (int64_t k0 = 0; k0 < K; k0 += TILE) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = ty + 8 * i;
+      const int64_t ar = row0 + r, ak = k0 + tx;
+      As[r][tx] = (ar < M && ak < K) ? A[ar * as0 + ak * as1] : T(0);
+      const int64_t bk = k0 + r;
+      Bs[r][tx] = (bk < K && col < N) ? B[bk * bs0 + col * bs1] : T(0);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < TILE; ++k) {
+      const T b = Bs[k][tx];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        acc[i] += As[ty + 8 * i][k] * b;
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t row = row0 + ty + 8 * i;
+    if (row < M && col < N) {
+      T *dst = C + row * cs0 + col * cs1;
+      T v = alpha * acc[i];
+      if (beta != T(0))
+        v += beta * *dst;
+      *dst = v;
+    }
+  }
+}
+
+template <typename T> struct MemrefOf;
+template <> struct MemrefOf<float> {
+  typedef NmhipMemref2F32 type;
+};
+template <> struct MemrefOf<double> {
+  typedef NmhipMemref2F64 type;
+};
+
+template <typename T>
+void requireUnitStride(const typename MemrefOf<T>::type *arr, char name) {
+  if (arr->strides[0] != 1 && arr->strides[1] != 1)
+    fatal("mkl gemm suports only arrays contiguous on inner dimension.\n"
+          "stride for at least one dimension should be equal to 1.\n"
+          "'%c' parameter is not contiguous. '%c' strides are %d and %d.\n",
+          name, name, int(arr->strides[0]), int(arr->strides[1]));
+}
+
+bool aligned16(const void *p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+template <typename T>
+void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
+                const typename MemrefOf<T>::type *b,
+                typename MemrefOf<T>::type *c, T alpha, T beta) {
+  if (!queueObj || !a || !b || !c)
+    fatal("mkl_gemm_device: null argument\n");
+  auto *base = static_cast<numba::GPUQueueInterface *>(queueObj);
+  auto *queue = static_cast<numba::HipQueueInterface *>(base);
+  if (queue->hipMagic() != numba::HipQueueInterface::kMagic)
+    fatal("mkl_gemm_device: queue '%.*s' was not created by the HIP GPU "
+          "runtime\n",
+          int(base->getDeviceName().size()), base->getDeviceName().data());
+
+  requireUnitStride<T>(a, 'a');
+  requireUnitStride<T>(b, 'b');
+  requireUnitStride<T>(c, 'c');
+
+  const int64_t M = int64_t(a->dims[0]);
+  const int64_t N = int64_t(b->dims[1]);
+  const int64_t K = int64_t(a->dims[1]);
+  if (int64_t(b->dims[0]) != K || int64_t(c->dims[0]) != M ||
+      int64_t(c->dims[1]) != N)
+    fatal("mkl_gemm_device: shape mismatch: a [%lld,%lld] b [%lld,%lld] c "
+          "[%lld,%lld]\n",
+          (long long)a->dims[0], (long long)a->dims[1], (long long)b->dims[0],
+          (long long)b->dims[1], (long long)c->dims[0], (long long)c->dims[1]);
+
+  const T *aData = a->data + a->offset;
+  const T *bData = b->data + b->offset;
+  T *cData = c->data + c->offset;
+
+  checkHip(hipSetDevice(queue->hipDevice()), "hipSetDevice");
+  auto stream = static_cast<hipStream_t>(queue->hipStream());
+
+  if (M > 0 && N > 0) {
+    bool launched = false;
+    if constexpr (sizeof(T) == 4) {
+      const bool rowMajor = a->strides[1] == 1 && b->strides[1] == 1 &&
+                            c->strides[1] == 1;
+      if (rowMajor && K > 0 && M % BM == 0 && N % BN == 0 && K % BK == 0 &&
+          a->strides[0] % 4 == 0 && b->strides[0] % 4 == 0 &&
+          aligned16(aData) && aligned16(bData) && M <= 0x7fffffff &&
+          N <= 0x7fffffff && K <= 0x7fffffff && M / BM <= 65535) {
+        dim3 grid(unsigned(N / BN), unsigned(M / BM), 1);
+        hipLaunchKernelGGL(sgemm_mfma_128x128, grid, dim3(256), 0, stream,
+                           aData, bData, cData, int(M), int(N), int(K),
+                           int64_t(a->strides[0]), int64_t(b->strides[0]),
+                           int64_t(c->strides[0]), alpha, beta);
+        lastKernel = "sgemm_mfma_128x128";
+        launched = true;
+      }
+    }
+    if (!launched) {
+      const int64_t gx = (N + 31) / 32, gy = (M + 31) / 32;
+      if (gy > 65535)
+        fatal("mkl_gemm_device: M = %lld is too large for the strided "
+              "kernel\n",
+              (long long)M);
+      dim3 grid{unsigned(gx), unsigned(gy), 1};
+      hipLaunchKernelGGL(gemm_generic<T>, grid, dim3(256), 0, stream, aData,
+                         bData, cData, M, N, K, int64_t(a->strides[0]),
+                         int64_t(a->strides[1]), int64_t(b->strides[0]),
+                         int64_t(b->strides[1]), int64_t(c->strides[0]),
+                         int64_t(c->strides[1]), alpha, beta);
+      lastKernel = sizeof(T) == 4 ? "sgemm_generic" : "dgemm_generic";
+    }
+    checkHip(hipGetLastError(), "gemm launch");
+  }
+  // The reference call returns only when C is complete (.wait(), 127/145).
+  checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
+}
+
+} // namespace
+
+#define NMHIP_MATH_EXPORT extern "C" __attribute__((visibility("default")))
+
+NMHIP_MATH_EXPORT void mkl_gemm_float32_device(void *queue,
+                                               const NmhipMemref2F32 *a,
+                                               const NmhipMemref2F32 *b,
+                                               float alpha, float beta,
+                                               NmhipMemref2F32 *c) {
+  deviceGemm<float>(queue, a, b, c, alpha, beta);
+}
+
+NMHIP_MATH_EXPORT void mkl_gemm_float64_device(void *queue,
+                                               const NmhipMemref2F64 *a,
+                                               const NmhipMemref2F64 *b,
+                                               double alpha, double beta,
+                                               NmhipMemref2F64 *c) {
+  deviceGemm<double>(queue, a, b, c, alpha, beta);
+}
+
+NMHIP_MATH_EXPORT void nmrtMathRuntimeInit(void) {}
+NMHIP_MATH_EXPORT void nmrtMathRuntimeFinalize(void) {}
+
+NMHIP_MATH_EXPORT const char *nmhipMathLastKernel(void) { return lastKernel; }

@@ -1,0 +1,891 @@
+// Lowered host code + kernel dispatcher (include/numba_mlir_hip/Offload.h).
+//
+// Every device action goes through the registered gpux* pointers in the order
+// the reference's generated host code uses (reference:
+// mlir/lib/Conversion/GpuRuntimeToLlvm.cpp:228-857; handle caching
+// mlir_compiler/lib/pipelines/LowerToGpu.cpp:742-940 and
+// numba_mlir_runtime/lib/Context.cpp:25-60).
+#include "numba_mlir_hip/Offload.h"
+
+#include "numba_mlir_hip/GpuQueueInterface.hpp"
+#include "numba_mlir_hip/MathRuntime.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <initializer_list>
+#include <mutex>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+// Code objects, embedded by Blobs.S.
+extern "C" const unsigned char nmhip_blob_maps[], nmhip_blob_maps_end[];
+extern "C" const unsigned char nmhip_blob_reduce[], nmhip_blob_reduce_end[];
+extern "C" const unsigned char nmhip_blob_twins[], nmhip_blob_twins_end[];
+
+namespace {
+
+[[noreturn]] void fail(const char *fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  std::vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  throw std::runtime_error(buf);
+}
+
+template <typename F> auto guarded(F &&body) noexcept {
+  try {
+    return body();
+  } catch (const std::exception &e) {
+    std::fprintf(stdout, "An exception was thrown: %s\n", e.what());
+    std::fflush(stdout);
+    std::abort();
+  } catch (...) {
+    std::fprintf(stdout, "An unknown exception was thrown\n");
+    std::fflush(stdout);
+    std::abort();
+  }
+}
+
+void checkHip(hipError_t err, const char *what) {
+  if (err != hipSuccess)
+    fail("%s failed: %s (%d)", what, hipGetErrorString(err),
+         static_cast<int>(err));
+}
+
+// ---- the symbol table the lowered code calls through ----------------------
+
+struct Symbols {
+  void *(*QueueCreate)(const char *) = nullptr;
+  void (*QueueDestroy)(void *) = nullptr;
+  void *(*ModuleLoad)(void *, const void *, size_t) = nullptr;
+  void (*ModuleDestroy)(void *) = nullptr;
+  void *(*KernelGet)(void *, const char *) = nullptr;
+  void (*KernelDestroy)(void *) = nullptr;
+  void *(*LaunchKernel)(void *, void *, size_t, size_t, size_t, size_t, size_t,
+                        size_t, void *, void *) = nullptr;
+  void (*Wait)(void *, void *) = nullptr;
+  void (*DestroyEvent)(void *, void *) = nullptr;
+  void (*Alloc)(void *, size_t, size_t, int, void *, GpuxAllocResult *) =
+      nullptr;
+  void (*DeAlloc)(void *, void *) = nullptr;
+  void (*SuggestBlockSize)(void *, void *, const uint32_t *, uint32_t *,
+                           size_t) = nullptr;
+  void *(*DuplicateQueue)(void *) = nullptr;
+  void (*GemmF32)(void *, const NmhipMemref2F32 *, const NmhipMemref2F32 *,
+                  float, float, NmhipMemref2F32 *) = nullptr;
+  void (*GemmF64)(void *, const NmhipMemref2F64 *, const NmhipMemref2F64 *,
+                  double, double, NmhipMemref2F64 *) = nullptr;
+};
+
+Symbols &symbols() {
+  static Symbols s;
+  return s;
+}
+
+template <typename T> T need(T fn, const char *name) {
+  if (!fn)
+    fail("Runtime symbol '%s' is not registered (load the HIP GPU runtime "
+         "first)",
+         name);
+  return fn;
+}
+#define SYM(field, cname) need(symbols().field, cname)
+
+// ---- tuning knobs ----------------------------------------------------------
+
+struct Tuning {
+  int64_t rowbcastRows = 0;
+  int64_t mapBlocks = 0;
+  int64_t reduceBlocks = 0;
+  int64_t axis0Rows = 0;
+  int64_t pairwiseRows = 0;
+  int64_t bsBlocks = 0;
+};
+
+Tuning &tuning() {
+  static Tuning t;
+  return t;
+}
+
+int64_t ceilDiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+bool aligned16(const void *p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+// ---- kernel argument packing ----------------------------------------------
+
+struct Arg {
+  union {
+    int64_t i64;
+    int32_t i32;
+    double f64;
+    float f32;
+    const void *ptr;
+  } v;
+  int32_t size;
+  int32_t type;
+
+  static Arg I64(int64_t x) {
+    Arg a;
+    a.v.i64 = x;
+    a.size = 8;
+    a.type = GPUX_PARAM_INT64;
+    return a;
+  }
+  static Arg I32(int32_t x) {
+    Arg a;
+    a.v.i64 = 0;
+    a.v.i32 = x;
+    a.size = 4;
+    a.type = GPUX_PARAM_INT32;
+    return a;
+  }
+  static Arg F32(float x) {
+    Arg a;
+    a.v.i64 = 0;
+    a.v.f32 = x;
+    a.size = 4;
+    a.type = GPUX_PARAM_FLOAT32;
+    return a;
+  }
+  static Arg F64(double x) {
+    Arg a;
+    a.v.f64 = x;
+    a.size = 8;
+    a.type = GPUX_PARAM_FLOAT64;
+    return a;
+  }
+  static Arg Ptr(const void *p) {
+    Arg a;
+    a.v.ptr = p;
+    a.size = 8;
+    a.type = GPUX_PARAM_PTR;
+    return a;
+  }
+};
+
+struct Blob {
+  const char *family;
+  const unsigned char *begin;
+  const unsigned char *end;
+};
+
+const Blob *findBlob(const char *family) {
+  static const Blob blobs[] = {
+      {"maps", nmhip_blob_maps, nmhip_blob_maps_end},
+      {"reduce", nmhip_blob_reduce, nmhip_blob_reduce_end},
+      {"twins", nmhip_blob_twins, nmhip_blob_twins_end},
+  };
+  for (const Blob &b : blobs)
+    if (std::strcmp(b.family, family) == 0)
+      return &b;
+  return nullptr;
+}
+
+// Kernel name -> family.  Names are prefixed by family:
+//   nmk_map2_*, nmk_black_scholes_*, nmk_fill_* : maps
+//   nmk_sum_*, nmk_norm2_*, nmk_reduce_*        : reduce
+//   nmk_twin_*                                  : twins
+const char *familyOf(const std::string &kernel) {
+  auto starts = [&](const char *p) { return kernel.rfind(p, 0) == 0; };
+  if (starts("nmk_map2_") || starts("nmk_black_scholes_") ||
+      starts("nmk_fill_"))
+    return "maps";
+  if (starts("nmk_sum_") || starts("nmk_norm2_") || starts("nmk_reduce_"))
+    return "reduce";
+  if (starts("nmk_twin_"))
+    return "twins";
+  fail("Kernel '%s' does not belong to a built-in code object", kernel.c_str());
+}
+
+constexpr size_t kMaxTickets = 4096;
+
+class Context {
+public:
+  explicit Context(const char *device) {
+    queue = SYM(QueueCreate, "gpuxQueueCreate")(device);
+  }
+
+  ~Context() {
+    // Outlined deinit: kernels, modules, then the queue
+    // (LowerToGpu.cpp:698-715, 832-858).
+    if (lastEvent)
+      retireEvent(lastEvent, true);
+    if (scratch)
+      symbols().DeAlloc(queue, scratch);
+    if (tickets)
+      symbols().DeAlloc(queue, tickets);
+    for (auto &kv : kernels)
+      symbols().KernelDestroy(kv.second);
+    for (auto &kv : modules)
+      symbols().ModuleDestroy(kv.second);
+    symbols().QueueDestroy(queue);
+  }
+
+  void *queue = nullptr;
+  bool async = false;
+  std::string lastKernel;
+  std::mutex mutex;
+
+  void *kernel(const std::string &name) {
+    auto it = kernels.find(name);
+    if (it != kernels.end())
+      return it->second;
+    const char *family = familyOf(name);
+    void *&mod = modules[family];
+    if (!mod) {
+      const Blob *blob = findBlob(family);
+      mod = SYM(ModuleLoad, "gpuxModuleLoad")(
+          queue, blob->begin, static_cast<size_t>(blob->end - blob->begin));
+    }
+    void *k = SYM(KernelGet, "gpuxKernelGet")(mod, name.c_str());
+    kernels.emplace(name, k);
+    return k;
+  }
+
+  void launchDesc(const std::string &name, const size_t grid[3],
+                  const size_t block[3], GpuxParamDesc *params) {
+    void *k = kernel(name);
+    lastKernel = name;
+    void *deps[1] = {nullptr};
+    void *ev = SYM(LaunchKernel, "gpuxLaunchKernel")(
+        queue, k, grid[0], grid[1], grid[2], block[0], block[1], block[2], deps,
+        params);
+    if (async) {
+      if (lastEvent)
+        retireEvent(lastEvent, false);
+      lastEvent = ev;
+    } else {
+      retireEvent(ev, true);
+    }
+  }
+
+  void launch(const std::string &name, size_t gx, size_t gy, size_t gz,
+              size_t bx, size_t by, size_t bz, std::initializer_list<Arg> args) {
+    std::vector<Arg> slots(args);
+    std::vector<GpuxParamDesc> descs(slots.size() + 1);
+    for (size_t i = 0; i < slots.size(); ++i) {
+      descs[i].data = &slots[i].v;
+      descs[i].size = slots[i].size;
+      descs[i].type = slots[i].type;
+    }
+    descs[slots.size()] = GpuxParamDesc{nullptr, 0, GPUX_PARAM_NULL};
+    const size_t grid[3] = {gx, gy, gz};
+    const size_t block[3] = {bx, by, bz};
+    launchDesc(name, grid, block, descs.data());
+  }
+
+  void synchronize() {
+    if (lastEvent) {
+      retireEvent(lastEvent, true);
+      lastEvent = nullptr;
+    }
+  }
+
+  void *alloc(size_t bytes, int type) {
+    void *deps[1] = {nullptr};
+    GpuxAllocResult res = {nullptr, nullptr};
+    // 64-byte alignment request, then wait + destroy of the alloc event
+    // (GpuRuntimeToLlvm.cpp:670, 741-744).
+    SYM(Alloc, "gpuxAlloc")(queue, bytes, 64, type, deps, &res);
+    retireEvent(res.event, true);
+    return res.ptr;
+  }
+
+  void free(void *ptr) { SYM(DeAlloc, "gpuxDeAlloc")(queue, ptr); }
+
+  // Device scratch for single-launch reductions: `bytes` of partials plus
+  // kMaxTickets zeroed ticket counters.  Kernels leave the tickets at zero.
+  void *scratchFor(size_t bytes) {
+    if (!tickets) {
+      tickets = static_cast<uint32_t *>(
+          alloc(kMaxTickets * sizeof(uint32_t), GPUX_ALLOC_DEVICE));
+      launch("nmk_fill_u32", 16, 1, 1, 256, 1, 1,
+             {Arg::Ptr(tickets), Arg::I32(0), Arg::I64(kMaxTickets)});
+    }
+    if (bytes > scratchBytes) {
+      if (scratch) {
+        synchronize();
+        free(scratch);
+      }
+      scratchBytes = bytes < (size_t(1) << 20) ? (size_t(1) << 20) : bytes;
+      scratch = alloc(scratchBytes, GPUX_ALLOC_DEVICE);
+    }
+    return scratch;
+  }
+
+  uint32_t *tickets = nullptr;
+
+  hipStream_t stream() {
+    auto *iface = static_cast<numba::HipQueueInterface *>(queue);
+    if (iface->hipMagic() != numba::HipQueueInterface::kMagic)
+      fail("Queue was not created by the HIP GPU runtime");
+    checkHip(hipSetDevice(iface->hipDevice()), "hipSetDevice");
+    return static_cast<hipStream_t>(iface->hipStream());
+  }
+
+private:
+  std::unordered_map<std::string, void *> modules;
+  std::unordered_map<std::string, void *> kernels;
+  void *lastEvent = nullptr;
+  void *scratch = nullptr;
+  size_t scratchBytes = 0;
+
+  void retireEvent(void *ev, bool wait) {
+    if (wait)
+      SYM(Wait, "gpuxWait")(queue, ev);
+    SYM(DestroyEvent, "gpuxDestroyEvent")(queue, ev);
+  }
+};
+
+Context *toCtx(void *ctx) {
+  if (!ctx)
+    fail("Invalid context");
+  return static_cast<Context *>(ctx);
+}
+
+const char *dtypeName(int dtype) {
+  switch (dtype) {
+  case NMHIP_I32:
+    return "i32";
+  case NMHIP_I64:
+    return "i64";
+  case NMHIP_F32:
+    return "f32";
+  case NMHIP_F64:
+    return "f64";
+  }
+  fail("Unsupported dtype %d", dtype);
+}
+
+size_t dtypeSize(int dtype) {
+  return (dtype == NMHIP_I32 || dtype == NMHIP_F32) ? 4 : 8;
+}
+
+struct Timer {
+  Context *ctx;
+  hipEvent_t start;
+  hipEvent_t stop;
+};
+
+} // namespace
+
+#define NMHIP_EXPORT extern "C" __attribute__((visibility("default")))
+
+NMHIP_EXPORT int nmhipRegisterSymbol(const char *name, void *address) {
+  return guarded([&]() -> int {
+    if (!name)
+      fail("nmhipRegisterSymbol: null name");
+    Symbols &s = symbols();
+    struct Entry {
+      const char *name;
+      void **slot;
+    };
+    const Entry table[] = {
+        {"gpuxQueueCreate", reinterpret_cast<void **>(&s.QueueCreate)},
+        {"gpuxQueueDestroy", reinterpret_cast<void **>(&s.QueueDestroy)},
+        {"gpuxModuleLoad", reinterpret_cast<void **>(&s.ModuleLoad)},
+        {"gpuxModuleDestroy", reinterpret_cast<void **>(&s.ModuleDestroy)},
+        {"gpuxKernelGet", reinterpret_cast<void **>(&s.KernelGet)},
+        {"gpuxKernelDestroy", reinterpret_cast<void **>(&s.KernelDestroy)},
+        {"gpuxLaunchKernel", reinterpret_cast<void **>(&s.LaunchKernel)},
+        {"gpuxWait", reinterpret_cast<void **>(&s.Wait)},
+        {"gpuxDestroyEvent", reinterpret_cast<void **>(&s.DestroyEvent)},
+        {"gpuxAlloc", reinterpret_cast<void **>(&s.Alloc)},
+        {"gpuxDeAlloc", reinterpret_cast<void **>(&s.DeAlloc)},
+        {"gpuxSuggestBlockSize",
+         reinterpret_cast<void **>(&s.SuggestBlockSize)},
+        {"gpuxDuplicateQueue", reinterpret_cast<void **>(&s.DuplicateQueue)},
+        {"mkl_gemm_float32_device", reinterpret_cast<void **>(&s.GemmF32)},
+        {"mkl_gemm_float64_device", reinterpret_cast<void **>(&s.GemmF64)},
+    };
+    // The JIT sees the gemm entry points under the _mlir_ciface_ prefix
+    // (math_runtime.py:21-40).
+    static const char prefix[] = "_mlir_ciface_";
+    if (std::strncmp(name, prefix, sizeof(prefix) - 1) == 0)
+      name += sizeof(prefix) - 1;
+    for (const Entry &e : table) {
+      if (std::strcmp(e.name, name) == 0) {
+        *e.slot = address;
+        return 0;
+      }
+    }
+    return -1;
+  });
+}
+
+NMHIP_EXPORT void *nmhipContextCreate(const char *deviceName) {
+  return guarded([&]() -> void * { return new Context(deviceName); });
+}
+
+NMHIP_EXPORT void nmhipContextDestroy(void *ctx) {
+  guarded([&]() { delete toCtx(ctx); });
+}
+
+NMHIP_EXPORT void nmhipContextSetAsync(void *ctx, int async) {
+  guarded([&]() {
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    if (!async)
+      c->synchronize();
+    c->async = async != 0;
+  });
+}
+
+NMHIP_EXPORT void nmhipContextSynchronize(void *ctx) {
+  guarded([&]() {
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    c->synchronize();
+  });
+}
+
+NMHIP_EXPORT void *nmhipContextQueue(void *ctx) {
+  return guarded([&]() -> void * { return toCtx(ctx)->queue; });
+}
+
+NMHIP_EXPORT const char *nmhipLastKernelName(void *ctx) {
+  return guarded([&]() -> const char * { return toCtx(ctx)->lastKernel.c_str(); });
+}
+
+NMHIP_EXPORT void *nmhipAlloc(void *ctx, size_t bytes, int type) {
+  return guarded([&]() -> void * { return toCtx(ctx)->alloc(bytes, type); });
+}
+
+NMHIP_EXPORT void nmhipFree(void *ctx, void *dev) {
+  guarded([&]() {
+    Context *c = toCtx(ctx);
+    {
+      std::lock_guard<std::mutex> lock(c->mutex);
+      c->synchronize();
+    }
+    c->free(dev);
+  });
+}
+
+NMHIP_EXPORT void nmhipMemcpyHtoD(void *ctx, void *dev, const void *host,
+                                  size_t bytes) {
+  guarded([&]() {
+    if (bytes == 0)
+      return;
+    hipStream_t s = toCtx(ctx)->stream();
+    checkHip(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, s),
+             "hipMemcpyAsync(HtoD)");
+    checkHip(hipStreamSynchronize(s), "hipStreamSynchronize");
+  });
+}
+
+NMHIP_EXPORT void nmhipMemcpyDtoH(void *ctx, void *host, const void *dev,
+                                  size_t bytes) {
+  guarded([&]() {
+    if (bytes == 0)
+      return;
+    hipStream_t s = toCtx(ctx)->stream();
+    checkHip(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, s),
+             "hipMemcpyAsync(DtoH)");
+    checkHip(hipStreamSynchronize(s), "hipStreamSynchronize");
+  });
+}
+
+NMHIP_EXPORT void nmhipMapBinary(void *ctx, int op, int dtype, const void *a,
+                                 const int64_t aS[2], const void *b,
+                                 const int64_t bS[2], void *out,
+                                 const int64_t oS[2], int64_t n0, int64_t n1) {
+  guarded([&]() {
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    if (n0 < 0 || n1 < 0)
+      fail("nmhipMapBinary: negative extent");
+    if (n0 == 0 || n1 == 0)
+      return;
+    static const char *const opNames[] = {"add", "sub", "mul"};
+    if (op < 0 || op > NMHIP_MUL)
+      fail("Unsupported binary op %d", op);
+    const std::string suffix =
+        std::string(opNames[op]) + "_" + dtypeName(dtype);
+    const bool isFloat = dtype == NMHIP_F32 || dtype == NMHIP_F64;
+    const int64_t lanesElems = 16 / static_cast<int64_t>(dtypeSize(dtype));
+    auto dense = [&](const int64_t s[2]) {
+      return s[1] == 1 && (n0 == 1 || s[0] == n1);
+    };
+    auto rowBroadcast = [&](const int64_t s[2]) {
+      return s[1] == 1 && s[0] == 0 && n0 > 1;
+    };
+    const bool alignedAll = aligned16(a) && aligned16(b) && aligned16(out);
+
+    if (isFloat && alignedAll && dense(oS) && dense(aS) && dense(bS) &&
+        (n0 * n1) % lanesElems == 0) {
+      const int64_t nvec = n0 * n1 / lanesElems;
+      int64_t blocks = tuning().mapBlocks ? tuning().mapBlocks : 256 * 16;
+      const int64_t need = ceilDiv(nvec, 2 * 256);
+      if (blocks > need)
+        blocks = need;
+      c->launch("nmk_map2_contig_" + suffix, size_t(blocks), 1, 1, 256, 1, 1,
+                {Arg::Ptr(a), Arg::Ptr(b), Arg::Ptr(out), Arg::I64(n0 * n1)});
+      return;
+    }
+    // Row-broadcast operand on either side (commutative ops may swap).
+    const void *full = a;
+    const void *row = b;
+    bool rowCase = dense(aS) && rowBroadcast(bS);
+    if (!rowCase && op != NMHIP_SUB && dense(bS) && rowBroadcast(aS)) {
+      full = b;
+      row = a;
+      rowCase = true;
+    }
+    if (isFloat && alignedAll && rowCase && dense(oS) && n1 % lanesElems == 0) {
+      const int64_t gx = ceilDiv(n1, 256 * lanesElems);
+      int64_t rowsPerBlock = tuning().rowbcastRows;
+      if (!rowsPerBlock) {
+        // Aim at ~4096 blocks (16 per CU) with at least 4 rows each.
+        rowsPerBlock = ceilDiv(n0 * gx, 4096);
+        if (rowsPerBlock < 4)
+          rowsPerBlock = 4;
+      }
+      const int64_t gy = ceilDiv(n0, rowsPerBlock);
+      if (gy <= 65535) {
+        c->launch("nmk_map2_rowbcast_" + suffix, size_t(gx), size_t(gy), 1, 256,
+                  1, 1,
+                  {Arg::Ptr(full), Arg::Ptr(row), Arg::Ptr(out), Arg::I64(n0),
+                   Arg::I64(n1), Arg::I64(rowsPerBlock)});
+        return;
+      }
+    }
+    // General case: one element per work-item, x <-> last dimension, block
+    // from the runtime's suggestion, tail guarded in the kernel
+    // (GpuToGpuRuntime.cpp:1395-1584).
+    const std::string name = "nmk_map2_strided_" + suffix;
+    if (n0 > 0xffffffffll || n1 > 0xffffffffll)
+      fail("nmhipMapBinary: extent above 2^32");
+    const uint32_t global[2] = {static_cast<uint32_t>(n1),
+                                static_cast<uint32_t>(n0)};
+    uint32_t block[2] = {1, 1};
+    SYM(SuggestBlockSize, "gpuxSuggestBlockSize")(c->queue, c->kernel(name),
+                                                  global, block, 2);
+    c->launch(name, size_t(ceilDiv(n1, block[0])), size_t(ceilDiv(n0, block[1])),
+              1, block[0], block[1], 1,
+              {Arg::Ptr(a), Arg::I64(aS[0]), Arg::I64(aS[1]), Arg::Ptr(b),
+               Arg::I64(bS[0]), Arg::I64(bS[1]), Arg::Ptr(out), Arg::I64(oS[0]),
+               Arg::I64(oS[1]), Arg::I64(n0), Arg::I64(n1)});
+  });
+}
+
+NMHIP_EXPORT void nmhipBlackScholesF32(void *ctx, const float *price,
+                                       const float *strike, const float *t,
+                                       float rate, float volatility,
+                                       float *call, float *put, int64_t n,
+                                       int wide) {
+  guarded([&]() {
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    if (n <= 0)
+      return;
+    if (!(aligned16(price) && aligned16(strike) && aligned16(t) &&
+          aligned16(call) && aligned16(put)))
+      fail("nmhipBlackScholesF32: arrays must be 16-byte aligned");
+    int64_t blocks = tuning().bsBlocks ? tuning().bsBlocks : 256 * 8;
+    const int64_t need = ceilDiv(ceilDiv(n, 4), 256);
+    if (blocks > need)
+      blocks = need;
+    c->launch(wide ? "nmk_black_scholes_f32_w64" : "nmk_black_scholes_f32_w32",
+              size_t(blocks), 1, 1, 256, 1, 1,
+              {Arg::Ptr(price), Arg::Ptr(strike), Arg::Ptr(t), Arg::F32(rate),
+               Arg::F32(volatility), Arg::Ptr(call), Arg::Ptr(put),
+               Arg::I64(n)});
+  });
+}
+
+NMHIP_EXPORT void nmhipReduce(void *ctx, int op, int dtype, const void *x,
+                              int64_t n0, int64_t n1, int64_t s0, int64_t s1,
+                              int axis, void *out) {
+  guarded([&]() {
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    if (n0 < 0 || n1 < 0)
+      fail("nmhipReduce: negative extent");
+    if (axis < -1 || axis > 1)
+      fail("nmhipReduce: axis must be -1, 0 or 1");
+    static const char *const opNames[] = {"sum", "prod", "min", "max"};
+    if (op < 0 || op > NMHIP_MAX)
+      fail("Unsupported reduce op %d", op);
+    const bool rowMajor = s1 == 1 && (n0 <= 1 || s0 >= n1);
+    const bool contiguous = s1 == 1 && (n0 <= 1 || s0 == n1);
+
+    // float32 row sums: a wave per row.
+    if (op == NMHIP_SUM && dtype == NMHIP_F32 && axis == 1 && rowMajor &&
+        n0 > 0 && n1 > 0) {
+      const int vec = (aligned16(x) && s0 % 4 == 0 && n1 % 4 == 0) ? 1 : 0;
+      c->launch("nmk_sum_axis1_f32", size_t(ceilDiv(n0, 4)), 1, 1, 256, 1, 1,
+                {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(n0), Arg::I64(n1),
+                 Arg::I64(s0), Arg::I32(vec)});
+      return;
+    }
+    // int32 column sums into int64: column strips x row chunks, device finish.
+    if (op == NMHIP_SUM && dtype == NMHIP_I32 && axis == 0 && rowMajor &&
+        aligned16(x) && s0 % 4 == 0 && n1 % 4 == 0 && n0 >= 64 && n1 > 0) {
+      const int64_t strips = ceilDiv(n1, 256);
+      int64_t rowsPerBlock = tuning().axis0Rows;
+      if (!rowsPerBlock) {
+        // ~2048 blocks, at least 16 rows (4 per wave) each.
+        rowsPerBlock = ceilDiv(n0 * strips, 2048);
+        if (rowsPerBlock < 16)
+          rowsPerBlock = 16;
+        rowsPerBlock = ceilDiv(rowsPerBlock, 16) * 16;
+      }
+      const int64_t chunks = ceilDiv(n0, rowsPerBlock);
+      if (strips <= int64_t(kMaxTickets) && chunks <= 65535) {
+        void *partial = c->scratchFor(size_t(chunks) * size_t(n1) * 8);
+        c->launch("nmk_sum_axis0_i32_i64", size_t(strips), size_t(chunks), 1,
+                  256, 1, 1,
+                  {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(n0), Arg::I64(n1),
+                   Arg::I64(s0), Arg::I64(rowsPerBlock), Arg::Ptr(partial),
+                   Arg::Ptr(c->tickets)});
+        return;
+      }
+    }
+    // float32 full sum: grid-stride, device finish.
+    if (op == NMHIP_SUM && dtype == NMHIP_F32 && axis == -1 && contiguous &&
+        n0 * n1 >= 4096) {
+      const int64_t n = n0 * n1;
+      int64_t blocks = tuning().reduceBlocks ? tuning().reduceBlocks : 2048;
+      const int64_t need = ceilDiv(n, 256 * 16);
+      if (blocks > need)
+        blocks = need;
+      void *partial = c->scratchFor(size_t(blocks) * 4);
+      c->launch("nmk_sum_all_f32", size_t(blocks), 1, 1, 256, 1, 1,
+                {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(n),
+                 Arg::I32(aligned16(x) ? 1 : 0), Arg::Ptr(partial),
+                 Arg::Ptr(c->tickets)});
+      return;
+    }
+    // Generic strided fallback: a wave per kept index.
+    int64_t nKeep, nRed, sk, sr;
+    if (axis == 1) {
+      nKeep = n0;
+      nRed = n1;
+      sk = s0;
+      sr = s1;
+    } else if (axis == 0) {
+      nKeep = n1;
+      nRed = n0;
+      sk = s1;
+      sr = s0;
+    } else {
+      if (!contiguous)
+        fail("nmhipReduce: a full reduction needs a C-contiguous array");
+      nKeep = 1;
+      nRed = n0 * n1;
+      sk = 0;
+      sr = 1;
+    }
+    if (nKeep == 0)
+      return;
+    c->launch(std::string("nmk_reduce_") + opNames[op] + "_" + dtypeName(dtype),
+              size_t(ceilDiv(nKeep, 4)), 1, 1, 256, 1, 1,
+              {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(nKeep), Arg::I64(nRed),
+               Arg::I64(sk), Arg::I64(sr), Arg::I64(1)});
+  });
+}
+
+NMHIP_EXPORT void nmhipNorm2F32(void *ctx, const float *x, int64_t n,
+                                float *out) {
+  guarded([&]() {
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    if (n < 0)
+      fail("nmhipNorm2F32: negative extent");
+    int64_t blocks = tuning().reduceBlocks ? tuning().reduceBlocks : 2048;
+    int64_t need = ceilDiv(n, 256 * 16);
+    if (need < 1)
+      need = 1;
+    if (blocks > need)
+      blocks = need;
+    void *partial = c->scratchFor(size_t(blocks) * 4);
+    c->launch("nmk_norm2_f32", size_t(blocks), 1, 1, 256, 1, 1,
+              {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(n),
+               Arg::I32(aligned16(x) ? 1 : 0), Arg::Ptr(partial),
+               Arg::Ptr(c->tickets)});
+  });
+}
+
+NMHIP_EXPORT void nmhipGemm(void *ctx, int dtype, const void *a,
+                            const int64_t aS[2], const void *b,
+                            const int64_t bS[2], void *cPtr,
+                            const int64_t cS[2], int64_t m, int64_t n,
+                            int64_t k, double alpha, double beta) {
+  guarded([&]() {
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    if (m < 0 || n < 0 || k < 0)
+      fail("nmhipGemm: negative extent");
+    // The gemm entry point blocks on the queue's stream; drain our own
+    // pending event first so async mode keeps its ordering guarantees.
+    c->synchronize();
+    c->lastKernel = "mkl_gemm";
+    auto fill = [&](auto &ref, const void *data, const int64_t s[2], int64_t d0,
+                    int64_t d1) {
+      ref.userData = nullptr;
+      ref.data = static_cast<decltype(ref.data)>(const_cast<void *>(data));
+      ref.offset = 0;
+      ref.dims[0] = size_t(d0);
+      ref.dims[1] = size_t(d1);
+      ref.strides[0] = size_t(s[0]);
+      ref.strides[1] = size_t(s[1]);
+    };
+    if (dtype == NMHIP_F32) {
+      NmhipMemref2F32 ra, rb, rc;
+      fill(ra, a, aS, m, k);
+      fill(rb, b, bS, k, n);
+      fill(rc, cPtr, cS, m, n);
+      SYM(GemmF32, "mkl_gemm_float32_device")(c->queue, &ra, &rb, float(alpha),
+                                              float(beta), &rc);
+    } else if (dtype == NMHIP_F64) {
+      NmhipMemref2F64 ra, rb, rc;
+      fill(ra, a, aS, m, k);
+      fill(rb, b, bS, k, n);
+      fill(rc, cPtr, cS, m, n);
+      SYM(GemmF64, "mkl_gemm_float64_device")(c->queue, &ra, &rb, alpha, beta,
+                                              &rc);
+    } else {
+      fail("nmhipGemm: dtype must be float32 or float64");
+    }
+  });
+}
+
+NMHIP_EXPORT void nmhipSuggestBlockSize(void *ctx, const char *kernelName,
+                                        const uint32_t *globalSize,
+                                        uint32_t *blockSize, size_t numDims) {
+  guarded([&]() {
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    SYM(SuggestBlockSize, "gpuxSuggestBlockSize")(
+        c->queue, c->kernel(kernelName), globalSize, blockSize, numDims);
+  });
+}
+
+NMHIP_EXPORT void nmhipLaunch(void *ctx, const char *kernelName,
+                              const size_t grid[3], const size_t block[3],
+                              GpuxParamDesc *params) {
+  guarded([&]() {
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    if (!kernelName || !grid || !block || !params)
+      fail("nmhipLaunch: null argument");
+    c->launchDesc(kernelName, grid, block, params);
+  });
+}
+
+NMHIP_EXPORT void nmhipPairwiseF64(void *ctx, const double *X1,
+                                   const double *X2, double *D, int64_t n1,
+                                   int64_t n2) {
+  guarded([&]() {
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    if (n1 <= 0 || n2 <= 0)
+      return;
+    if (n2 % 2 != 0 || !aligned16(D))
+      fail("nmhipPairwiseF64: needs an even n2 and a 16-byte aligned D");
+    const int64_t gx = ceilDiv(n2, 512);
+    int64_t rows = tuning().pairwiseRows;
+    if (!rows) {
+      rows = ceilDiv(n1 * gx, 4096);
+      if (rows < 4)
+        rows = 4;
+    }
+    const int64_t gy = ceilDiv(n1, rows);
+    if (gy > 65535)
+      fail("nmhipPairwiseF64: too many row chunks");
+    c->launch("nmk_twin_pairwise_f64_rows", size_t(gx), size_t(gy), 1, 256, 1, 1,
+              {Arg::Ptr(X1), Arg::Ptr(X2), Arg::Ptr(D), Arg::I64(n1),
+               Arg::I64(n2), Arg::I64(rows)});
+  });
+}
+
+NMHIP_EXPORT const void *nmhipKernelBlob(const char *family, size_t *size) {
+  return guarded([&]() -> const void * {
+    const Blob *b = family ? findBlob(family) : nullptr;
+    if (!b)
+      fail("Unknown kernel family '%s'", family ? family : "(null)");
+    if (size)
+      *size = static_cast<size_t>(b->end - b->begin);
+    return b->begin;
+  });
+}
+
+NMHIP_EXPORT void nmhipSetTuning(const char *knob, int64_t value) {
+  guarded([&]() {
+    if (!knob)
+      fail("nmhipSetTuning: null knob");
+    Tuning &t = tuning();
+    const std::string k(knob);
+    if (k == "rowbcast_rows")
+      t.rowbcastRows = value;
+    else if (k == "map_blocks")
+      t.mapBlocks = value;
+    else if (k == "reduce_blocks")
+      t.reduceBlocks = value;
+    else if (k == "axis0_rows")
+      t.axis0Rows = value;
+    else if (k == "pairwise_rows")
+      t.pairwiseRows = value;
+    else if (k == "bs_blocks")
+      t.bsBlocks = value;
+    else
+      fail("Unknown tuning knob '%s'", knob);
+  });
+}
+
+NMHIP_EXPORT void *nmhipTimerCreate(void *ctx) {
+  return guarded([&]() -> void * {
+    Context *c = toCtx(ctx);
+    (void)c->stream(); // selects the device
+    auto *t = new Timer{c, nullptr, nullptr};
+    checkHip(hipEventCreate(&t->start), "hipEventCreate");
+    checkHip(hipEventCreate(&t->stop), "hipEventCreate");
+    return t;
+  });
+}
+
+NMHIP_EXPORT void nmhipTimerStart(void *timer) {
+  guarded([&]() {
+    auto *t = static_cast<Timer *>(timer);
+    checkHip(hipEventRecord(t->start, t->ctx->stream()), "hipEventRecord");
+  });
+}
+
+NMHIP_EXPORT void nmhipTimerStop(void *timer) {
+  guarded([&]() {
+    auto *t = static_cast<Timer *>(timer);
+    checkHip(hipEventRecord(t->stop, t->ctx->stream()), "hipEventRecord");
+  });
+}
+
+NMHIP_EXPORT double nmhipTimerElapsedMs(void *timer) {
+  return guarded([&]() -> double {
+    auto *t = static_cast<Timer *>(timer);
+    checkHip(hipEventSynchronize(t->stop), "hipEventSynchronize");
+    float ms = 0.f;
+    checkHip(hipEventElapsedTime(&ms, t->start, t->stop),
+             "hipEventElapsedTime");
+    return ms;
+  });
+}
+
+NMHIP_EXPORT void nmhipTimerDestroy(void *timer) {
+  guarded([&]() {
+    auto *t = static_cast<Timer *>(timer);
+    if (!t)
+      return;
+    (void)hipEventDestroy(t->start);
+    (void)hipEventDestroy(t->stop);
+    delete t;
+  });
+}

@@ -1,0 +1,14 @@
+"""Kernel API surface (reference: numba_mlir/numba_mlir/kernel.py:5-23)."""
+
+from .mlir.kernel_impl import (
+    DEFAULT_LOCAL_SIZE,
+    GLOBAL_MEM_FENCE,
+    LOCAL_MEM_FENCE,
+    Kernel,
+    get_global_id,
+    get_global_size,
+    get_group_id,
+    get_local_id,
+    get_local_size,
+    kernel,
+)

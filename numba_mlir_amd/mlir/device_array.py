@@ -1,0 +1,262 @@
+"""Device arrays for the HIP backend.
+
+The reference takes its device arrays from dpctl (``usm_ndarray``; typing and
+unboxing in reference: numba_mlir/numba_mlir/mlir/dpctl_interop.py:77-262,
+numba_mlir/numba_mlir/python_runtime/lib/Boxing.cpp:45-136).  ``HipNdArray`` is
+the analogue for HIP: a strided view over memory obtained from ``gpuxAlloc``,
+carrying the queue it belongs to, exposing ``__hip_array_interface__`` with the
+fields of ``__sycl_usm_array_interface__`` (data, shape, strides, typestr,
+version, syclobj -> queue), and released through ``gpuxDeAlloc`` when the last
+view dies, as the reference's NRT MemInfo destructor does
+(reference: mlir/lib/Conversion/GpuRuntimeToLlvm.cpp:717-720).
+"""
+
+import ctypes
+import weakref
+
+import numpy as np
+
+from . import lowered
+from .lowered import lib
+from .utils import readenv
+
+DEFAULT_DEVICE = readenv("NUMBA_MLIR_DEFAULT_DEVICE", str, "hip:gpu:0")
+
+_USM_TYPES = {
+    "device": lowered.ALLOC_DEVICE,
+    "shared": lowered.ALLOC_SHARED,
+    "host": lowered.ALLOC_HOST,
+}
+
+
+class Context:
+    """Queue plus cached module/kernel handles of one device string.
+
+    Counterpart of the per-function context the reference's compiled code
+    obtains from ``nmrtTakeContext`` (reference:
+    numba_mlir_runtime/lib/Context.cpp:25-60): created on first use, reused by
+    every later call, purged at interpreter exit.
+    """
+
+    def __init__(self, device):
+        self.device = device
+        self.handle = lib.nmhipContextCreate(device.encode() if device else None)
+        self._finalizer = weakref.finalize(self, lib.nmhipContextDestroy,
+                                           self.handle)
+
+    @property
+    def queue(self):
+        return lib.nmhipContextQueue(self.handle)
+
+    def set_async(self, flag):
+        lib.nmhipContextSetAsync(self.handle, 1 if flag else 0)
+
+    def synchronize(self):
+        lib.nmhipContextSynchronize(self.handle)
+
+    def last_kernel(self):
+        return lib.nmhipLastKernelName(self.handle).decode()
+
+
+_contexts = {}
+
+
+def get_context(device=None):
+    device = DEFAULT_DEVICE if device is None else device
+    ctx = _contexts.get(device)
+    if ctx is None:
+        ctx = _contexts[device] = Context(device)
+    return ctx
+
+
+class DeviceCaps:
+    """Capabilities the compiler asks of a device (reference:
+    dpctl_interop.py:148-209, 293-306): MI355X has native fp64 and fp16."""
+
+    def __init__(self, filter_string):
+        self.filter_string = filter_string
+        self.arch = "gfx950"
+        self.has_fp64 = True
+        self.has_fp16 = True
+        self.subgroup_size = 64
+
+
+def get_default_device():
+    return DeviceCaps(DEFAULT_DEVICE)
+
+
+class _Buffer:
+    """Owner of one gpuxAlloc allocation."""
+
+    def __init__(self, ctx, nbytes, usm_type):
+        self.ctx = ctx
+        self.nbytes = nbytes
+        self.usm_type = usm_type
+        self.ptr = lib.nmhipAlloc(ctx.handle, max(nbytes, 1), _USM_TYPES[usm_type])
+        self._finalizer = weakref.finalize(self, lib.nmhipFree, ctx.handle,
+                                           self.ptr)
+
+
+class HipNdArray:
+    def __init__(self, buffer, shape, dtype, strides, offset):
+        self._buffer = buffer
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+        self.strides = tuple(int(s) for s in strides)  # bytes, as NumPy
+        self._offset = int(offset)                      # bytes
+
+    # -- construction --------------------------------------------------------
+    @classmethod
+    def empty(cls, shape, dtype, usm_type="device", device=None, order="C"):
+        if isinstance(shape, int):
+            shape = (shape,)
+        dtype = np.dtype(dtype)
+        ctx = get_context(device)
+        count = int(np.prod(shape, dtype=np.int64)) if len(shape) else 1
+        buf = _Buffer(ctx, count * dtype.itemsize, usm_type)
+        strides = np.empty(shape, dtype, order=order).strides if count else \
+            np.empty(shape, dtype).strides
+        return cls(buf, shape, dtype, strides, 0)
+
+    @classmethod
+    def from_numpy(cls, arr, usm_type="device", device=None):
+        arr = np.asarray(arr)
+        order = "F" if (arr.flags["F_CONTIGUOUS"] and not
+                        arr.flags["C_CONTIGUOUS"]) else "C"
+        host = np.asarray(arr, order=order)
+        if not (host.flags["C_CONTIGUOUS"] or host.flags["F_CONTIGUOUS"]):
+            host = np.ascontiguousarray(host)
+            order = "C"
+        res = cls.empty(host.shape, host.dtype, usm_type, device, order)
+        if host.nbytes:
+            lib.nmhipMemcpyHtoD(res.ctx.handle, res.ptr,
+                                host.ctypes.data_as(ctypes.c_void_p), host.nbytes)
+        return res
+
+    # -- properties ----------------------------------------------------------
+    @property
+    def ctx(self):
+        return self._buffer.ctx
+
+    @property
+    def usm_type(self):
+        return self._buffer.usm_type
+
+    @property
+    def ptr(self):
+        return self._buffer.ptr + self._offset
+
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    @property
+    def size(self):
+        return int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
+
+    @property
+    def nbytes(self):
+        return self.size * self.dtype.itemsize
+
+    @property
+    def elem_strides(self):
+        return tuple(s // self.dtype.itemsize for s in self.strides)
+
+    @property
+    def T(self):
+        return HipNdArray(self._buffer, self.shape[::-1], self.dtype,
+                          self.strides[::-1], self._offset)
+
+    @property
+    def __hip_array_interface__(self):
+        return {
+            "data": (self.ptr, False),
+            "shape": self.shape,
+            "strides": self.strides,
+            "typestr": self.dtype.str,
+            "version": 1,
+            "queue": self.ctx.queue,
+            "usm_type": self.usm_type,
+        }
+
+    def is_c_contiguous(self):
+        expect = self.dtype.itemsize
+        for n, s in zip(reversed(self.shape), reversed(self.strides)):
+            if n != 1 and s != expect:
+                return False
+            expect *= n
+        return True
+
+    def is_f_contiguous(self):
+        return self.T.is_c_contiguous()
+
+    def reshape(self, *shape):
+        if len(shape) == 1 and isinstance(shape[0], (tuple, list)):
+            shape = tuple(shape[0])
+        if not self.is_c_contiguous():
+            raise ValueError("reshape needs a C-contiguous device array")
+        strides = np.empty(shape, self.dtype).strides
+        if int(np.prod(shape, dtype=np.int64)) != self.size:
+            raise ValueError("cannot reshape: size mismatch")
+        return HipNdArray(self._buffer, shape, self.dtype, strides, self._offset)
+
+    # -- host transfer -------------------------------------------------------
+    def asnumpy(self):
+        """Copies the viewed elements back into a new NumPy array."""
+        self.ctx.synchronize()
+        if self.size == 0:
+            return np.empty(self.shape, self.dtype)
+        if self.is_c_contiguous() or self.is_f_contiguous():
+            order = "C" if self.is_c_contiguous() else "F"
+            out = np.empty(self.shape, self.dtype, order=order)
+            lib.nmhipMemcpyDtoH(self.ctx.handle,
+                                out.ctypes.data_as(ctypes.c_void_p), self.ptr,
+                                out.nbytes)
+            return out
+        # Strided view: fetch the whole allocation and view it on the host.
+        raw = np.empty(self._buffer.nbytes, np.uint8)
+        lib.nmhipMemcpyDtoH(self.ctx.handle, raw.ctypes.data_as(ctypes.c_void_p),
+                            self._buffer.ptr, raw.nbytes)
+        view = np.ndarray(self.shape, self.dtype, raw.data, self._offset,
+                          self.strides)
+        return view.copy()
+
+    def copy_from_host(self, arr):
+        arr = np.ascontiguousarray(arr, dtype=self.dtype)
+        if arr.shape != self.shape or not self.is_c_contiguous():
+            raise ValueError("copy_from_host needs a C-contiguous array of the "
+                             "same shape")
+        if arr.nbytes:
+            lib.nmhipMemcpyHtoD(self.ctx.handle, self.ptr,
+                                arr.ctypes.data_as(ctypes.c_void_p), arr.nbytes)
+
+    def as_host_view(self):
+        """NumPy view of a shared/host allocation (host-dereferenceable, as the
+        reference's results over shared USM are, dpctl_interop.py:113-115)."""
+        if self.usm_type == "device":
+            raise ValueError("device allocations are not host-dereferenceable")
+        self.ctx.synchronize()
+        buf = (ctypes.c_uint8 * max(self._buffer.nbytes, 1)).from_address(
+            self._buffer.ptr)
+        view = np.ndarray(self.shape, self.dtype, buf, self._offset, self.strides)
+        view.flags.writeable = True
+        self._host_keepalive = buf
+        return view
+
+    def __repr__(self):
+        return (f"HipNdArray(shape={self.shape}, dtype={self.dtype}, "
+                f"usm_type={self.usm_type!r})")
+
+
+def asarray(arr, usm_type="device", device=None):
+    if isinstance(arr, HipNdArray):
+        return arr
+    return HipNdArray.from_numpy(arr, usm_type, device)
+
+
+def asnumpy(arr):
+    return arr.asnumpy() if isinstance(arr, HipNdArray) else np.asarray(arr)
+
+
+def empty(shape, dtype, usm_type="device", device=None):
+    return HipNdArray.empty(shape, dtype, usm_type, device)
