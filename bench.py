@@ -1,0 +1,269 @@
+#!/usr/bin/env python3
+"""Benchmark of the offloaded hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME[,NAME]]
+
+Prints ONE JSON line.  The headline metric is Black-Scholes options/s on
+2^24 float32 options (the configuration the metric is quoted on); every other
+configuration is measured in the same run and reported under "per_config".
+
+A step is one pass of a kernel over its full-size input, resident in HBM
+before the timed region.  Steps are enqueued back to back through the gpux*
+C-ABI (gpuxLaunchKernel returns an event; the wait happens after the last
+step) and the region is bracketed by queue synchronisation.  The per-kernel
+duration used for the roofline comes from HIP events recorded on the queue's
+own stream around the same region.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--only", type=str, default="",
+                    help="comma-separated subset of: add,bs,bs32,sum1,norm2,"
+                         "sum0,pairwise,matmul")
+    ap.add_argument("--no-cpu", action="store_true",
+                    help="skip the CPU baseline leg")
+    return ap.parse_args()
+
+
+class Bench:
+    def __init__(self, steps, warmup):
+        from numba_mlir_amd import build as native_build
+
+        if not native_build.libraries_present():
+            native_build.build_all()
+        from numba_mlir_amd.mlir import device_array as da
+        from numba_mlir_amd.mlir import ops
+
+        self.da, self.ops = da, ops
+        self.lib = da.lib
+        self.ctx = da.get_context()
+        self.steps, self.warmup = steps, warmup
+
+    def measure(self, launch, blocking=False):
+        """Returns (wall ms/step, HIP-event ms/step, kernel name)."""
+        ctx, lib = self.ctx, self.lib
+        ctx.set_async(not blocking)
+        for _ in range(self.warmup):
+            launch()
+        ctx.synchronize()
+        timer = lib.nmhipTimerCreate(ctx.handle)
+        lib.nmhipTimerStart(timer)
+        t0 = time.perf_counter()
+        for _ in range(self.steps):
+            launch()
+        lib.nmhipTimerStop(timer)
+        ctx.synchronize()
+        ev_ms = lib.nmhipTimerElapsedMs(timer)
+        t1 = time.perf_counter()
+        lib.nmhipTimerDestroy(timer)
+        ctx.set_async(False)
+        return ((t1 - t0) * 1e3 / self.steps, ev_ms / self.steps,
+                ctx.last_kernel())
+
+
+def hbm_entry(name, workload, alg_bytes, wall_ms, ev_ms, kernel, extra=None):
+    achieved = alg_bytes / (ev_ms * 1e-3) / 1e9
+    e = {
+        "name": name, "workload": workload, "kernel": kernel,
+        "ms_per_step": round(wall_ms, 5), "kernel_ms": round(ev_ms, 5),
+        "algorithmic_bytes": alg_bytes,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None},
+    }
+    if extra:
+        e.update(extra)
+    return e
+
+
+def run(args):
+    import numpy as np
+
+    from numba_mlir_amd import workloads
+    from numba_mlir_amd.mlir import math_runtime
+
+    b = Bench(args.steps, args.warmup)
+    da, ops = b.da, b.ops
+    only = set(x for x in args.only.split(",") if x)
+    want = lambda n: not only or n in only
+    per_config = []
+    headline = None
+
+    # -- config 2: Black-Scholes (headline) ---------------------------------
+    if want("bs") or want("bs32"):
+        nopt = 2 ** 24
+        price, strike, t, rate, vol, call, put = workloads.black_scholes(nopt)
+        d = [da.asarray(x) for x in (price, strike, t, call, put)]
+        alg = 20 * nopt
+        for key, wide in (("bs", True), ("bs32", False)):
+            if not want(key):
+                continue
+            launch = lambda: ops.black_scholes(d[0], d[1], d[2], rate, vol, d[3],
+                                               d[4], float64_literals=wide)
+            wall, ev, kern = b.measure(launch)
+            e = hbm_entry(
+                key, f"Black-Scholes, 2^24 float32 options, literals typed "
+                     f"{'float64 (reference typing)' if wide else 'float32'}",
+                alg, wall, ev, kern,
+                {"options_per_s": nopt / (wall * 1e-3)})
+            per_config.append(e)
+            if wide:
+                headline = (e, nopt, (price, strike, t, rate, vol))
+        del d
+
+    # -- config 1: broadcast add --------------------------------------------
+    if want("add"):
+        a, bb = workloads.broadcast_add()
+        d_a, d_b = da.asarray(a), da.asarray(bb)
+        d_o = da.empty(a.shape, a.dtype)
+        wall, ev, kern = b.measure(lambda: ops.add(d_a, d_b, out=d_o))
+        per_config.append(hbm_entry(
+            "add", "a[4096,4096] + b[1,4096], float64",
+            2 * a.nbytes + bb.nbytes, wall, ev, kern))
+        del d_a, d_b, d_o, a, bb
+
+    # -- config 3: reductions ------------------------------------------------
+    if want("sum1") or want("norm2"):
+        x = workloads.reduce_f32()
+        d_x = da.asarray(x)
+        if want("sum1"):
+            d_o = da.empty((x.shape[0],), np.float32)
+            launch = lambda: b.lib.nmhipReduce(
+                b.ctx.handle, 0, 2, d_x.ptr, x.shape[0], x.shape[1], x.shape[1],
+                1, 1, d_o.ptr)
+            wall, ev, kern = b.measure(launch)
+            per_config.append(hbm_entry(
+                "sum1", "np.sum(x, axis=1), float32 [16384,8192]",
+                x.nbytes + 4 * x.shape[0], wall, ev, kern))
+        if want("norm2"):
+            d_o = da.empty((1,), np.float32)
+            wall, ev, kern = b.measure(
+                lambda: ops.sqrt_sum_squares(d_x, out=d_o))
+            per_config.append(hbm_entry(
+                "norm2", "np.sqrt(np.sum(x*x)), float32 [16384,8192]",
+                x.nbytes + 4, wall, ev, kern))
+        del d_x, x
+    if want("sum0"):
+        xi = workloads.reduce_i32()
+        d_x = da.asarray(xi)
+        d_o = da.empty((xi.shape[1],), np.int64)
+        launch = lambda: b.lib.nmhipReduce(
+            b.ctx.handle, 0, 0, d_x.ptr, xi.shape[0], xi.shape[1], xi.shape[1],
+            1, 0, d_o.ptr)
+        wall, ev, kern = b.measure(launch)
+        per_config.append(hbm_entry(
+            "sum0", "np.sum(x, axis=0), int32 [16384,8192] -> int64",
+            xi.nbytes + 8 * xi.shape[1], wall, ev, kern))
+        del d_x, xi
+
+    # -- config 4: pairwise distance @kernel ---------------------------------
+    if want("pairwise"):
+        X, Y = workloads.pairwise()
+        d_X, d_Y = da.asarray(X), da.asarray(Y)
+        d_D = da.empty((X.shape[0], Y.shape[0]), np.float64)
+        wall, ev, kern = b.measure(lambda: ops.pairwise_distance(d_X, d_Y, d_D))
+        per_config.append(hbm_entry(
+            "pairwise", "pairwise distance @kernel, float64 [8192,3]^2",
+            X.nbytes + Y.nbytes + 8 * X.shape[0] * Y.shape[0], wall, ev, kern))
+        del d_X, d_Y, d_D
+
+    # -- config 5: matmul ----------------------------------------------------
+    if want("matmul"):
+        n = 4096
+        A, B = workloads.matmul(n)
+        d_A, d_B = da.asarray(A), da.asarray(B)
+        d_C = da.empty((n, n), np.float32)
+        saved = b.steps
+        b.steps = max(5, min(saved, 20))
+        wall, ev, _ = b.measure(lambda: ops.dot(d_A, d_B, out=d_C),
+                                blocking=True)
+        b.steps = saved
+        flops = 2.0 * n ** 3
+        tf = flops / (ev * 1e-3) / 1e12
+        per_config.append({
+            "name": "matmul", "workload": "np.dot float32 [4096,4096]^2",
+            "kernel": math_runtime.last_kernel(),
+            "ms_per_step": round(wall, 5), "kernel_ms": round(ev, 5),
+            "algorithmic_flops": flops,
+            "roofline": {"bound": "mfma", "achieved": round(tf, 2),
+                         "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4),
+                         "traffic": None},
+        })
+        del d_A, d_B, d_C
+
+    # -- CPU baseline for the headline (oracle, all host cores) --------------
+    cpu = None
+    if headline is not None and not args.no_cpu:
+        from oracle import oracle as orc
+
+        price, strike, t, rate, vol = headline[2]
+        threads = min(orc.max_threads(), os.cpu_count() or 1)
+        orc.black_scholes(price[:1 << 16], strike[:1 << 16], t[:1 << 16], rate,
+                          vol, True, threads)
+        reps = 3
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            orc.black_scholes(price, strike, t, rate, vol, True, threads)
+        dt = (time.perf_counter() - t0) / reps
+        cpu = {"value": headline[1] / dt, "unit": "options/s", "cores": threads,
+               "kind": "port",
+               "sample": f"all 2^24 options, {reps} passes, C restatement of "
+                         "the reference CPU path with OpenMP threads"}
+
+    if headline is None:
+        e = per_config[0]
+        line = {"metric": e["name"], "value": None, "unit": "",
+                "per_config": per_config}
+    else:
+        e, nopt, _ = headline
+        line = {
+            "metric": "black_scholes_options_per_sec",
+            "value": nopt / (e["ms_per_step"] * 1e-3),
+            "unit": "options/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": e["ms_per_step"],
+            "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None,
+            "dtype": "f32 (literal-bearing intermediates f64)",
+            "data": "synthetic",
+            "config": {"workload": "Black-Scholes, 2^24 float32 options, "
+                                   "price/strike~U(10,50), t~U(1,2), rate=0.1, "
+                                   "vol=0.2, seed 777777"},
+            "roofline": e["roofline"],
+            "cpu_baseline": cpu,
+            "per_config": per_config,
+        }
+    print(json.dumps(line))
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every box of this build has a single "
+              "MI355X and the hot path uses no collectives; run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    run(args)
+
+
+if __name__ == "__main__":
+    main()

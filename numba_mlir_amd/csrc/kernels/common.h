@@ -72,4 +72,33 @@ __device__ __forceinline__ T blockAllReduce(T v, Op op, T *slots) {
   return total;
 }
 
+// ---------------------------------------------------------------------------
+// Hand-off of per-block partial results to the last block of a launch.
+//
+// A device-wide fence (__threadfence) writes back and invalidates the whole
+// L2 of the XCD; issued once per block it costs more than the reduction
+// itself.  Instead every value that crosses blocks moves through agent-scope
+// accesses, which the hardware keeps coherent across the XCDs' L2s on their
+// own: partials are published with agent-scope stores (written through), the
+// publishing wave waits until the stores are acknowledged, then takes a
+// ticket with an agent-scope add; the block that draws the last ticket reads
+// the partials back with agent-scope loads.  The ticket only orders blocks;
+// no value is ever accumulated with an atomic.
+template <typename T> __device__ __forceinline__ void publish(T *p, T v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <typename T> __device__ __forceinline__ T collect(const T *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Blocks until every store this wave issued has been acknowledged
+// (s_waitcnt vmcnt(0) expcnt(0) lgkmcnt(0)).
+__device__ __forceinline__ void awaitStores() { __builtin_amdgcn_s_waitcnt(0); }
+
+__device__ __forceinline__ uint32_t takeTicket(uint32_t *ticket) {
+  return __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED,
+                                __HIP_MEMORY_SCOPE_AGENT);
+}
+
 } // namespace nmk

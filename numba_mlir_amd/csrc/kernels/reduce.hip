@@ -66,21 +66,21 @@ nmk_sum_axis1_f32(const float *__restrict__ x, float *__restrict__ out,
 
 // ---------------------------------------------------------------------------
 // out[c] = sum_r int64(x[r * ld + c]), int32 input.  Requires cols % 4 == 0,
-// ld % 4 == 0 and a 16-byte aligned base (dispatcher falls back to the
+// ld % 4 == 0 and a 16-byte aligned base (the dispatcher falls back to the
 // generic kernel otherwise).
 //
-// grid.x = column strips of 256 columns (64 lanes x int4), grid.y = row
-// chunks of rowsPerBlock.  The four waves of a block take interleaved rows of
-// the chunk, fold through LDS, and store one int64 partial per column to
-// partial[chunk][col].  The last block of a strip to finish (ordered by a
-// ticket counter, used for ordering only) adds the chunks in index order and
-// writes out[]; it also resets the ticket, so the counters are zero again
-// when the kernel ends.
+// grid.x = column strips of 256 columns (64 lanes x int4 = 1 KiB of a row),
+// grid.y = row chunks of rowsPerBlock.  The four waves of a block take
+// interleaved rows of the chunk, eight row loads in flight per lane, fold
+// through LDS, and publish one int64 partial per column to
+// partial[chunk][col].  The block that draws the last ticket of its strip
+// adds the chunks in index order and writes out[]; it also resets the ticket,
+// so the counters are zero again when the kernel ends.
 NMK_KERNEL(256)
 nmk_sum_axis0_i32_i64(const int32_t *__restrict__ x, int64_t *__restrict__ out,
                       int64_t rows, int64_t cols, int64_t ld,
-                      int64_t rowsPerBlock, int64_t *__restrict__ partial,
-                      uint32_t *__restrict__ tickets) {
+                      int64_t rowsPerBlock, int64_t *partial,
+                      uint32_t *tickets) {
   __shared__ int64_t fold[4][256];
   __shared__ uint32_t isLast;
   const int lane = threadIdx.x % NMK_WAVE;
@@ -95,20 +95,20 @@ nmk_sum_axis0_i32_i64(const int32_t *__restrict__ x, int64_t *__restrict__ out,
     if (rEnd > rows)
       rEnd = rows;
     const int32_t *p = x + r * ld + col;
-    const int64_t step = 4 * ld;
-    for (; r + 12 < rEnd; r += 16) {
-      int4_t v0 = __builtin_nontemporal_load(reinterpret_cast<const int4_t *>(p));
-      int4_t v1 =
-          __builtin_nontemporal_load(reinterpret_cast<const int4_t *>(p + step));
-      int4_t v2 = __builtin_nontemporal_load(
-          reinterpret_cast<const int4_t *>(p + 2 * step));
-      int4_t v3 = __builtin_nontemporal_load(
-          reinterpret_cast<const int4_t *>(p + 3 * step));
+    const int64_t step = 4 * ld; // the block's waves interleave rows
+    for (; r + 28 < rEnd; r += 32) {
+      int4_t v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        v[u] = __builtin_nontemporal_load(
+            reinterpret_cast<const int4_t *>(p + u * step));
 #pragma unroll
       for (int k = 0; k < 4; ++k)
-        acc[k] += (int64_t(v0[k]) + int64_t(v1[k])) +
-                  (int64_t(v2[k]) + int64_t(v3[k]));
-      p += 4 * step;
+        acc[k] += ((int64_t(v[0][k]) + int64_t(v[1][k])) +
+                   (int64_t(v[2][k]) + int64_t(v[3][k]))) +
+                  ((int64_t(v[4][k]) + int64_t(v[5][k])) +
+                   (int64_t(v[6][k]) + int64_t(v[7][k])));
+      p += 8 * step;
     }
     for (; r < rEnd; r += 4) {
       int4_t v0 = *reinterpret_cast<const int4_t *>(p);
@@ -126,59 +126,68 @@ nmk_sum_axis0_i32_i64(const int32_t *__restrict__ x, int64_t *__restrict__ out,
   if (myCol < cols) {
     int64_t s = (fold[0][threadIdx.x] + fold[1][threadIdx.x]) +
                 (fold[2][threadIdx.x] + fold[3][threadIdx.x]);
-    partial[chunk * cols + myCol] = s;
+    publish(partial + chunk * cols + myCol, s);
   }
-  // Publish the partials, then take a ticket.
-  __threadfence();
+  awaitStores();
   __syncthreads();
-  if (threadIdx.x == 0) {
-    uint32_t ticket = atomicAdd(&tickets[strip], 1u);
-    isLast = (ticket == gridDim.y - 1) ? 1u : 0u;
-  }
+  if (threadIdx.x == 0)
+    isLast = (takeTicket(&tickets[strip]) == gridDim.y - 1) ? 1u : 0u;
   __syncthreads();
   if (!isLast)
     return;
-  __threadfence();
   if (myCol < cols) {
+    const int64_t nChunks = gridDim.y;
+    const int64_t *p = partial + myCol;
     int64_t s = 0;
-    for (int64_t c = 0; c < int64_t(gridDim.y); ++c)
-      s += __builtin_nontemporal_load(partial + c * cols + myCol);
+    int64_t c = 0;
+    for (; c + 8 <= nChunks; c += 8) {
+      int64_t v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        v[u] = collect(p + (c + u) * cols);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        s += v[u];
+    }
+    for (; c < nChunks; ++c)
+      s += collect(p + c * cols);
     out[myCol] = s;
   }
   if (threadIdx.x == 0)
-    tickets[strip] = 0;
+    publish(&tickets[strip], 0u);
 }
 
 // ---------------------------------------------------------------------------
-// out[0] = sqrt(sum_i x[i] * x[i]), float32, n elements contiguous
-// (np.sqrt(np.sum(x * x)): the square is fused into the reduction as the
-// reference's elementwise fusion does, mlir_compiler/lib/pipelines/PlierToLinalg.cpp:3149-3199;
-// the sqrt of the 0-d result is the scalar path, numpy/funcs.py:364-368).
+// out[0] = sqrt(sum_i x[i] * x[i]) or sum_i x[i], float32, n contiguous
+// elements (np.sqrt(np.sum(x * x)): the square is fused into the reduction as
+// the reference's elementwise fusion does,
+// mlir_compiler/lib/pipelines/PlierToLinalg.cpp:3149-3199; the sqrt of the 0-d
+// result is the scalar path, numpy/funcs.py:364-368).
 //
-// Grid-stride float4 loads (vec != 0 needs a 16-byte aligned base), float32
-// lane partials, block tree, one partial per block; the last block to take a
-// ticket folds the partials in block order and applies sqrtf.
+// Each block streams 16 KiB pieces (256 lanes x 4 float4, vec != 0 needs a
+// 16-byte aligned base), piece index strided by the grid, float32 lane
+// partials folded pairwise, block tree, one published partial per block; the
+// block that draws the last ticket folds the partials in block order and
+// applies sqrtf.  The result depends on the grid size only.
 template <bool SQUARE_ROOT_OF_SQUARES>
 __device__ __forceinline__ void
 fullSumF32(const float *__restrict__ x, float *__restrict__ out, int64_t n,
-           int32_t vec, float *__restrict__ partial,
-           uint32_t *__restrict__ ticket) {
+           int32_t vec, float *partial, uint32_t *ticket) {
   __shared__ float slots[4];
   __shared__ uint32_t isLast;
-  const int64_t tid = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-  const int64_t stride = int64_t(gridDim.x) * blockDim.x;
   float total = 0.f;
   int64_t done = 0;
   if (vec) {
     const float4_t *pv = reinterpret_cast<const float4_t *>(x);
     const int64_t nvec = n / 4;
+    const int64_t nPieces = nvec / 1024;
     float4_t a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0, a3 = a0;
-    int64_t i = tid;
-    for (; i + 3 * stride < nvec; i += 4 * stride) {
-      float4_t v0 = __builtin_nontemporal_load(pv + i);
-      float4_t v1 = __builtin_nontemporal_load(pv + i + stride);
-      float4_t v2 = __builtin_nontemporal_load(pv + i + 2 * stride);
-      float4_t v3 = __builtin_nontemporal_load(pv + i + 3 * stride);
+    for (int64_t piece = blockIdx.x; piece < nPieces; piece += gridDim.x) {
+      const float4_t *q = pv + piece * 1024 + threadIdx.x;
+      float4_t v0 = __builtin_nontemporal_load(q);
+      float4_t v1 = __builtin_nontemporal_load(q + 256);
+      float4_t v2 = __builtin_nontemporal_load(q + 512);
+      float4_t v3 = __builtin_nontemporal_load(q + 768);
       if (SQUARE_ROOT_OF_SQUARES) {
         v0 *= v0;
         v1 *= v1;
@@ -190,7 +199,10 @@ fullSumF32(const float *__restrict__ x, float *__restrict__ out, int64_t n,
       a2 += v2;
       a3 += v3;
     }
-    for (; i < nvec; i += stride) {
+    // Vectors past the last whole piece: grid-strided, one per lane.
+    for (int64_t i = nPieces * 1024 + int64_t(blockIdx.x) * blockDim.x +
+                     threadIdx.x;
+         i < nvec; i += int64_t(gridDim.x) * blockDim.x) {
       float4_t v0 = pv[i];
       if (SQUARE_ROOT_OF_SQUARES)
         v0 *= v0;
@@ -200,28 +212,27 @@ fullSumF32(const float *__restrict__ x, float *__restrict__ out, int64_t n,
     total = (a[0] + a[1]) + (a[2] + a[3]);
     done = nvec * 4;
   }
-  for (int64_t i = done + tid; i < n; i += stride) {
+  for (int64_t i = done + int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += int64_t(gridDim.x) * blockDim.x) {
     float v = x[i];
     total += SQUARE_ROOT_OF_SQUARES ? v * v : v;
   }
   total = blockAllReduce<256>(total, AddOp(), slots);
   if (threadIdx.x == 0) {
-    partial[blockIdx.x] = total;
-    __threadfence();
-    uint32_t t = atomicAdd(ticket, 1u);
-    isLast = (t == gridDim.x - 1) ? 1u : 0u;
+    publish(partial + blockIdx.x, total);
+    awaitStores();
+    isLast = (takeTicket(ticket) == gridDim.x - 1) ? 1u : 0u;
   }
   __syncthreads();
   if (!isLast)
     return;
-  __threadfence();
   float s = 0.f;
   for (int64_t b = threadIdx.x; b < int64_t(gridDim.x); b += blockDim.x)
-    s += __builtin_nontemporal_load(partial + b);
+    s += collect(partial + b);
   s = blockAllReduce<256>(s, AddOp(), slots);
   if (threadIdx.x == 0) {
     out[0] = SQUARE_ROOT_OF_SQUARES ? sqrtf(s) : s;
-    *ticket = 0;
+    publish(ticket, 0u);
   }
 }
 

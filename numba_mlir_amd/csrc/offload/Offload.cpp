@@ -634,11 +634,9 @@ NMHIP_EXPORT void nmhipReduce(void *ctx, int op, int dtype, const void *x,
       const int64_t strips = ceilDiv(n1, 256);
       int64_t rowsPerBlock = tuning().axis0Rows;
       if (!rowsPerBlock) {
-        // ~2048 blocks, at least 16 rows (4 per wave) each.
-        rowsPerBlock = ceilDiv(n0 * strips, 2048);
-        if (rowsPerBlock < 16)
-          rowsPerBlock = 16;
-        rowsPerBlock = ceilDiv(rowsPerBlock, 16) * 16;
+        // ~1024 blocks; whole 32-row groups (8 loads x 4 waves) per block.
+        rowsPerBlock = ceilDiv(n0 * strips, 1024);
+        rowsPerBlock = ceilDiv(rowsPerBlock, 32) * 32;
       }
       const int64_t chunks = ceilDiv(n0, rowsPerBlock);
       if (strips <= int64_t(kMaxTickets) && chunks <= 65535) {
@@ -655,7 +653,7 @@ NMHIP_EXPORT void nmhipReduce(void *ctx, int op, int dtype, const void *x,
     if (op == NMHIP_SUM && dtype == NMHIP_F32 && axis == -1 && contiguous &&
         n0 * n1 >= 4096) {
       const int64_t n = n0 * n1;
-      int64_t blocks = tuning().reduceBlocks ? tuning().reduceBlocks : 2048;
+      int64_t blocks = tuning().reduceBlocks ? tuning().reduceBlocks : 1024;
       const int64_t need = ceilDiv(n, 256 * 16);
       if (blocks > need)
         blocks = need;
@@ -702,7 +700,7 @@ NMHIP_EXPORT void nmhipNorm2F32(void *ctx, const float *x, int64_t n,
     std::lock_guard<std::mutex> lock(c->mutex);
     if (n < 0)
       fail("nmhipNorm2F32: negative extent");
-    int64_t blocks = tuning().reduceBlocks ? tuning().reduceBlocks : 2048;
+    int64_t blocks = tuning().reduceBlocks ? tuning().reduceBlocks : 1024;
     int64_t need = ceilDiv(n, 256 * 16);
     if (need < 1)
       need = 1;

@@ -85,6 +85,17 @@ def get_default_device():
     return DeviceCaps(DEFAULT_DEVICE)
 
 
+def _dense_strides(shape, itemsize, order="C"):
+    """Byte strides of a dense array (NumPy reports zeros for empty arrays)."""
+    strides = [0] * len(shape)
+    step = itemsize
+    dims = range(len(shape) - 1, -1, -1) if order == "C" else range(len(shape))
+    for i in dims:
+        strides[i] = step
+        step *= max(int(shape[i]), 1)
+    return tuple(strides)
+
+
 class _Buffer:
     """Owner of one gpuxAlloc allocation."""
 
@@ -114,9 +125,8 @@ class HipNdArray:
         ctx = get_context(device)
         count = int(np.prod(shape, dtype=np.int64)) if len(shape) else 1
         buf = _Buffer(ctx, count * dtype.itemsize, usm_type)
-        strides = np.empty(shape, dtype, order=order).strides if count else \
-            np.empty(shape, dtype).strides
-        return cls(buf, shape, dtype, strides, 0)
+        return cls(buf, shape, dtype, _dense_strides(shape, dtype.itemsize, order),
+                   0)
 
     @classmethod
     def from_numpy(cls, arr, usm_type="device", device=None):
@@ -180,6 +190,8 @@ class HipNdArray:
         }
 
     def is_c_contiguous(self):
+        if self.size == 0:
+            return True
         expect = self.dtype.itemsize
         for n, s in zip(reversed(self.shape), reversed(self.strides)):
             if n != 1 and s != expect:
@@ -195,7 +207,7 @@ class HipNdArray:
             shape = tuple(shape[0])
         if not self.is_c_contiguous():
             raise ValueError("reshape needs a C-contiguous device array")
-        strides = np.empty(shape, self.dtype).strides
+        strides = _dense_strides(shape, self.dtype.itemsize)
         if int(np.prod(shape, dtype=np.int64)) != self.size:
             raise ValueError("cannot reshape: size mismatch")
         return HipNdArray(self._buffer, shape, self.dtype, strides, self._offset)

@@ -1,0 +1,176 @@
+"""GPU parity: elementwise/broadcast maps and the fused Black-Scholes map,
+through the gpux* C-ABI, against the CPU oracle."""
+
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "reference_vectors.json")) as f:
+    GOLD = json.load(f)
+
+
+@pytest.fixture(scope="module")
+def env(hip):
+    from numba_mlir_amd.mlir import ops
+    from oracle import oracle as orc
+    return hip, ops, orc
+
+
+def _bits(a):
+    return np.ascontiguousarray(a).tobytes()
+
+
+@pytest.mark.parametrize("i", range(6))
+@pytest.mark.parametrize("j", range(6))
+def test_broadcast_fixtures_bit_exact(env, i, j):
+    """The reference's own broadcast cases (tests/test_numpy.py:483-514)."""
+    hip, ops, orc = env
+    arrs = [np.array(a, np.int64) for a in GOLD["broadcast_arrays"]["arrays"]]
+    a, b = arrs[i], arrs[j]
+    got = ops.add(hip.asarray(a), hip.asarray(b)).asnumpy()
+    expect = orc.add(a, b)
+    assert got.shape == expect.shape and got.dtype == expect.dtype
+    assert np.array_equal(got, expect)
+    assert np.array_equal(got, np.add(a, b))
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32, np.int32, np.int64])
+def test_golden_linalg_addf(env, dtype):
+    hip, ops, _ = env
+    g = GOLD["linalg_addf"]
+    a, b = np.array(g["a"], dtype), np.array(g["b"], dtype)
+    got = ops.add(hip.asarray(a), hip.asarray(b)).asnumpy()
+    assert np.array_equal(got, np.array(g["out"], dtype))
+
+
+@pytest.mark.parametrize("shape,expect_kernel", [
+    ((4096, 4096), "nmk_map2_rowbcast_add_f64"),     # benchmark configuration
+    ((1000, 4098), "nmk_map2_rowbcast_add_f64"),     # ragged rows / column tail
+    ((3, 2), "nmk_map2_rowbcast_add_f64"),
+    ((7, 4097), "nmk_map2_strided_add_f64"),         # odd column count
+    ((5, 1), "nmk_map2_strided_add_f64"),
+])
+def test_row_broadcast_add_f64_bit_exact(env, shape, expect_kernel):
+    hip, ops, orc = env
+    rng = np.random.Generator(np.random.PCG64(1001))
+    a = rng.uniform(-1, 1, shape)
+    b = rng.uniform(-1, 1, (1, shape[1]))
+    d_a, d_b = hip.asarray(a), hip.asarray(b)
+    got = ops.add(d_a, d_b).asnumpy()
+    assert hip.get_context().last_kernel() == expect_kernel
+    assert _bits(got) == _bits(orc.add(a, b))
+    # broadcast operand on the left (add commutes bit-exactly)
+    got = ops.add(d_b, d_a).asnumpy()
+    assert _bits(got) == _bits(orc.add(a, b))
+    # rank-1 row operand
+    got = ops.add(d_a, hip.asarray(b[0])).asnumpy()
+    assert _bits(got) == _bits(a + b[0])
+
+
+def test_config1_workload_matches_oracle(env):
+    hip, ops, orc = env
+    from numba_mlir_amd import workloads
+    a, b = workloads.broadcast_add()
+    assert a.shape == (4096, 4096) and b.shape == (1, 4096) and a.dtype == np.float64
+    got = ops.add(hip.asarray(a), hip.asarray(b)).asnumpy()
+    assert _bits(got) == _bits(orc.add(a, b))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n", [4, 1024, 1 << 20, (1 << 20) + 4, 1027])
+def test_contiguous_maps(env, dtype, n):
+    hip, ops, _ = env
+    rng = np.random.default_rng(n)
+    a = rng.standard_normal(n).astype(dtype)
+    b = rng.standard_normal(n).astype(dtype)
+    d_a, d_b = hip.asarray(a), hip.asarray(b)
+    for fn, ref in ((ops.add, np.add), (ops.subtract, np.subtract),
+                    (ops.multiply, np.multiply)):
+        got = fn(d_a, d_b).asnumpy()
+        assert _bits(got) == _bits(ref(a, b))
+    kern = hip.get_context().last_kernel()
+    vec = 16 // np.dtype(dtype).itemsize
+    assert ("contig" in kern) == (n % vec == 0)
+
+
+def test_column_broadcast_and_transposed_operands(env):
+    hip, ops, _ = env
+    rng = np.random.default_rng(2)
+    a = rng.standard_normal((37, 53))
+    col = rng.standard_normal((37, 1))
+    d_a = hip.asarray(a)
+    assert _bits(ops.add(d_a, hip.asarray(col)).asnumpy()) == _bits(a + col)
+    assert _bits(ops.subtract(hip.asarray(col), d_a).asnumpy()) == _bits(col - a)
+    at = hip.asarray(np.ascontiguousarray(a.T)).T      # strided view of a
+    assert at.shape == a.shape and not at.is_c_contiguous()
+    assert _bits(ops.multiply(at, d_a).asnumpy()) == _bits(a * a)
+
+
+def test_empty_inputs(env):
+    hip, ops, _ = env
+    a = np.zeros((0, 8)); b = np.zeros((1, 8))
+    assert ops.add(hip.asarray(a), hip.asarray(b)).asnumpy().shape == (0, 8)
+    assert ops.add(hip.asarray(np.zeros(0)), hip.asarray(np.zeros(0))).asnumpy().shape == (0,)
+
+
+# -- Black-Scholes -------------------------------------------------------------
+# Tolerance: |gpu - oracle| <= 1e-4 * |oracle| + 1e-7 for the reference typing
+# (float64 literals).  The absolute term covers float32 denormal-range outputs;
+# prices are O(1..40).
+BS_RTOL, BS_ATOL = 1e-4, 1e-7
+
+
+def _run_bs(hip, ops, n, wide):
+    from numba_mlir_amd import workloads
+    price, strike, t, rate, vol, call, put = workloads.black_scholes(n)
+    d = [hip.asarray(x) for x in (price, strike, t, call, put)]
+    ops.black_scholes(d[0], d[1], d[2], rate, vol, d[3], d[4],
+                      float64_literals=wide)
+    return (price, strike, t, rate, vol), d[3].asnumpy(), d[4].asnumpy()
+
+
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 1023, 524288, 524291])
+def test_black_scholes_reference_typing(env, n):
+    hip, ops, orc = env
+    inp, call, put = _run_bs(hip, ops, n, True)
+    assert hip.get_context().last_kernel() == "nmk_black_scholes_f32_w64"
+    rc, rp = orc.black_scholes(*inp, wide=True)
+    np.testing.assert_allclose(call, rc, rtol=BS_RTOL, atol=BS_ATOL)
+    np.testing.assert_allclose(put, rp, rtol=BS_RTOL, atol=BS_ATOL)
+
+
+def test_black_scholes_float32_typing(env):
+    hip, ops, orc = env
+    inp, call, put = _run_bs(hip, ops, 524288, False)
+    assert hip.get_context().last_kernel() == "nmk_black_scholes_f32_w32"
+    rc, rp = orc.black_scholes(*inp, wide=False)
+    # float32 throughout: the tails cancel catastrophically on both sides, so
+    # only an absolute bound is meaningful (prices up to ~40, eps 6e-8).
+    np.testing.assert_allclose(call, rc, rtol=1e-4, atol=2e-5)
+    np.testing.assert_allclose(put, rp, rtol=1e-4, atol=2e-5)
+    # and the reference's own bar against the other typing
+    wc, wp = orc.black_scholes(*inp, wide=True)
+    np.testing.assert_allclose(call, wc, atol=GOLD["black_scholes"]["atol"])
+    np.testing.assert_allclose(put, wp, atol=GOLD["black_scholes"]["atol"])
+
+
+def test_black_scholes_full_size(env):
+    """2^24 options: oracle parity plus put-call parity and the closed form."""
+    hip, ops, orc = env
+    inp, call, put = _run_bs(hip, ops, 2 ** 24, True)
+    rc, rp = orc.black_scholes(*inp, wide=True)
+    np.testing.assert_allclose(call, rc, rtol=BS_RTOL, atol=BS_ATOL)
+    np.testing.assert_allclose(put, rp, rtol=BS_RTOL, atol=BS_ATOL)
+    price, strike, t, rate, vol = inp
+    disc = strike.astype(np.float64) * np.exp(-float(rate) * t.astype(np.float64))
+    np.testing.assert_allclose(call.astype(np.float64) - put, price - disc,
+                               rtol=0, atol=2e-5)
+    tc, tp = orc.black_scholes_truth(*inp)
+    np.testing.assert_allclose(call, tc, rtol=5e-5, atol=1e-12)
+    np.testing.assert_allclose(put, tp, rtol=5e-5, atol=1e-12)
+    assert (call >= 0).all() and (put >= -1e-6).all()   # r - P + Se cancels

@@ -1,0 +1,146 @@
+"""GPU parity: axis and full reductions through the gpux* C-ABI."""
+
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "reference_vectors.json")) as f:
+    GOLD = json.load(f)
+
+DIMS = GOLD["reduce_shapes"]["dims_2d"]
+
+
+@pytest.fixture(scope="module")
+def env(hip):
+    from numba_mlir_amd.mlir import ops
+    from oracle import oracle as orc
+    return hip, ops, orc
+
+
+def test_small_golden(env):
+    hip, ops, _ = env
+    g = GOLD["reduce_axis_small"]
+    for dtype in (np.int32, np.float32):
+        d = hip.asarray(np.array(g["arr"], dtype))
+        assert ops.sum(d, axis=0).asnumpy().tolist() == g["sum_axis0"]
+        assert ops.sum(d, axis=1).asnumpy().tolist() == g["sum_axis1"]
+        assert ops.sum(d, axis=-1).asnumpy().tolist() == g["sum_axis1"]
+        assert ops.sum(d) == g["sum_all"]
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64, np.float32])
+@pytest.mark.parametrize("n0", DIMS)
+@pytest.mark.parametrize("n1", DIMS)
+def test_reference_reduce_shapes(env, dtype, n0, n1):
+    """test_cfd_reduce2 of the reference (tests/test_gpu.py:2068-2098):
+    arange(1..count) reshaped, sum/prod/amin/amax, rtol 1e-5."""
+    hip, ops, _ = env
+    count = n0 * n1
+    a = np.arange(1, count + 1, dtype=dtype).reshape(n0, n1).copy()
+    d = hip.asarray(a)
+    rtol = GOLD["reduce_shapes"]["rtol"]
+    np.testing.assert_allclose(ops.sum(d), a.sum(), rtol=rtol)
+    np.testing.assert_allclose(ops.sum(d, axis=0).asnumpy(), a.sum(axis=0), rtol=rtol)
+    np.testing.assert_allclose(ops.sum(d, axis=1).asnumpy(), a.sum(axis=1), rtol=rtol)
+    assert ops.amin(d) == a.min() and ops.amax(d) == a.max()
+    np.testing.assert_array_equal(ops.amin(d, axis=0).asnumpy(), a.min(axis=0))
+    np.testing.assert_array_equal(ops.amax(d, axis=1).asnumpy(), a.max(axis=1))
+    if count <= 30:          # the reference skips larger products (overflow)
+        np.testing.assert_allclose(ops.prod(d), np.prod(a), rtol=rtol)
+        np.testing.assert_allclose(ops.prod(d, axis=0).asnumpy(),
+                                   np.prod(a, axis=0), rtol=rtol)
+
+
+@pytest.mark.parametrize("size", GOLD["reduce_shapes"]["sizes_1d"])
+def test_reference_reduce_1d(env, size):
+    """test_cfd_reduce1 (tests/test_gpu.py:2045-2062): arange float32, rtol 1e-5."""
+    hip, ops, _ = env
+    a = np.arange(size, dtype=np.float32)
+    got = ops.sum(hip.asarray(a))
+    np.testing.assert_allclose(got, a.astype(np.float64).sum(), rtol=1e-5)
+
+
+def test_int_dtype_promotion(env):
+    hip, ops, _ = env
+    a = np.full((70000, 8), 2 ** 31 - 1, np.int32)
+    out = ops.sum(hip.asarray(a), axis=0).asnumpy()
+    assert out.dtype == np.int64 and out.tolist() == [70000 * (2 ** 31 - 1)] * 8
+    assert hip.get_context().last_kernel() == "nmk_sum_axis0_i32_i64"
+
+
+@pytest.mark.parametrize("shape", [(64, 256), (100, 260), (16384, 8192),
+                                   (1000, 1028), (4097, 512), (65, 4)])
+def test_sum_axis0_i32_bit_exact(env, shape):
+    hip, ops, orc = env
+    rng = np.random.Generator(np.random.PCG64(1013))
+    x = rng.integers(-1000, 1000, shape, dtype=np.int32, endpoint=True)
+    d = hip.asarray(x)
+    for _ in range(2):       # second call reuses scratch and self-reset tickets
+        got = ops.sum(d, axis=0).asnumpy()
+        assert got.dtype == np.int64
+        assert np.array_equal(got, orc.sum_axis0_i32(x))
+    assert hip.get_context().last_kernel() == "nmk_sum_axis0_i32_i64"
+
+
+# Tolerance for float32 sums: |gpu - truth| <= 1e-4 * sum|x| (float64 truth).
+# The reference states rel 1e-4/1e-5 on positive data; for zero-mean data the
+# sum itself can be arbitrarily close to 0, so the bound is relative to the
+# sum of magnitudes.
+@pytest.mark.parametrize("shape", [(4, 8192), (333, 1000), (16384, 8192),
+                                   (7, 5), (1024, 4100)])
+def test_sum_axis1_f32(env, shape):
+    hip, ops, orc = env
+    rng = np.random.Generator(np.random.PCG64(1003))
+    x = rng.standard_normal(shape, dtype=np.float32)
+    got = ops.sum(hip.asarray(x), axis=1).asnumpy()
+    assert hip.get_context().last_kernel() == "nmk_sum_axis1_f32"
+    x64 = x.astype(np.float64)
+    truth, mag = x64.sum(axis=1), np.abs(x64).sum(axis=1)
+    assert (np.abs(got - truth) <= 1e-4 * mag).all()
+    if shape[0] * shape[1] <= 1 << 22:
+        # the oracle (sequential float32 rows) obeys the same bound
+        assert (np.abs(orc.sum_axis1_f32(x) - truth) <= 1e-4 * mag).all()
+    # positive data: plain relative tolerance, as the reference states it
+    y = np.abs(x)
+    got = ops.sum(hip.asarray(y), axis=1).asnumpy()
+    np.testing.assert_allclose(got, y.astype(np.float64).sum(axis=1), rtol=1e-5)
+
+
+@pytest.mark.parametrize("n", [0, 1, 5, 4096, 4099, 1 << 20, 16384 * 8192])
+def test_sqrt_sum_squares(env, n):
+    hip, ops, orc = env
+    rng = np.random.Generator(np.random.PCG64(1003))
+    x = rng.standard_normal(n, dtype=np.float32)
+    d = hip.asarray(x)
+    got = [float(ops.sqrt_sum_squares(d).asnumpy()[0]) for _ in range(2)]
+    assert got[0] == got[1]          # fixed combination order
+    truth = float(np.sqrt((x.astype(np.float64) ** 2).sum()))
+    assert abs(got[0] - truth) <= 1e-5 * truth + 0.0
+    if 0 < n <= 1 << 20:
+        assert abs(float(orc.norm2_f32(x)) - truth) <= 1e-4 * truth
+
+
+def test_sqrt_sum_squares_exact(env):
+    hip, ops, _ = env
+    assert ops.sqrt_sum_squares(hip.asarray(np.array([3, 4], np.float32))).asnumpy()[0] == 5
+    x = np.zeros(1 << 16, np.float32)
+    x[::1024] = 2
+    assert ops.sqrt_sum_squares(hip.asarray(x)).asnumpy()[0] == 16
+
+
+def test_strided_and_transposed_inputs(env):
+    hip, ops, _ = env
+    rng = np.random.default_rng(8)
+    a = rng.integers(-50, 50, (45, 67)).astype(np.int64)
+    dt = hip.asarray(np.ascontiguousarray(a.T)).T
+    np.testing.assert_array_equal(ops.sum(dt, axis=0).asnumpy(), a.sum(axis=0))
+    np.testing.assert_array_equal(ops.sum(dt, axis=1).asnumpy(), a.sum(axis=1))
+    f = rng.standard_normal((45, 67))
+    np.testing.assert_allclose(ops.amax(hip.asarray(f), axis=1).asnumpy(), f.max(axis=1))
+    np.testing.assert_allclose(ops.sum(hip.asarray(f), axis=0).asnumpy(), f.sum(axis=0),
+                               rtol=1e-12)
