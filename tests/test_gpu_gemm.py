@@ -1,0 +1,171 @@
+"""GPU parity: np.dot / __internal_gemm through mkl_gemm_<dtype>_device."""
+
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "reference_vectors.json")) as f:
+    GOLD = json.load(f)
+
+
+@pytest.fixture(scope="module")
+def env(hip):
+    from numba_mlir_amd.mlir import math_runtime, ops
+    from oracle import oracle as orc
+    return hip, ops, orc, math_runtime
+
+
+def _printed(x):
+    return np.array([float("%.6g" % v) for v in np.ravel(x)]).reshape(np.shape(x))
+
+
+def _to_dev(hip, a):
+    """Device copy that keeps the host array's layout (C, F or a transposed view)."""
+    if a.flags["C_CONTIGUOUS"]:
+        return hip.asarray(a)
+    assert a.T.flags["C_CONTIGUOUS"]
+    return hip.asarray(np.ascontiguousarray(a.T)).T
+
+
+def test_dot_golden(env):
+    hip, ops, _, _ = env
+    g = GOLD["dot_2d"]
+    a, b = np.array(g["a"], np.float32), np.array(g["b"], np.float32)
+    got = ops.dot(hip.asarray(a), hip.asarray(b)).asnumpy()
+    assert np.array_equal(got, np.array(g["out"], np.float32))
+    # test_dot's flipped variants are copies made by the compiler before the
+    # call; here: their materialised equivalents
+    for aa, bb in ((a[::-1].copy(), b), (a, b[:, ::-1].copy())):
+        got = ops.dot(hip.asarray(aa), hip.asarray(bb)).asnumpy()
+        assert np.array_equal(got, np.dot(aa, bb))
+
+
+def test_linalg_gemmf_golden(env):
+    hip, ops, _, _ = env
+    g = GOLD["linalg_gemmf"]
+    c = hip.asarray(np.array(g["c0"], np.float32))
+    ops.gemm(hip.asarray(np.array(g["a"], np.float32)),
+             hip.asarray(np.array(g["b"], np.float32)), c, 1.0, 1.0)
+    assert np.array_equal(_printed(c.asnumpy()), np.array(g["printed"]))
+
+
+def _fixture_cases():
+    sq = [np.zeros((4, 4), np.float32), np.ones((4, 4), np.float32),
+          np.arange(16).reshape(4, 4).astype(np.float32)]
+    rect = [np.zeros((4, 6), np.float32), np.ones((4, 6), np.float32),
+            np.arange(24).reshape(4, 6).astype(np.float32)]
+    rect_t = [a.T for a in rect]
+    ab = GOLD["internal_gemm"]["alpha_beta"]
+    return list(itertools.product(sq, sq, sq, ab, ab)) + \
+        list(itertools.product(rect, rect_t, sq, ab, ab))
+
+
+def test_internal_gemm_fixture_grid(env):
+    """test_internal_gemm (tests/test_gpu.py:2141-2193): assert_equal."""
+    hip, ops, orc, _ = env
+    for a, b, c, alpha, beta in _fixture_cases():
+        expect = (beta * c + alpha * np.dot(a, b)).astype(np.float32)
+        d_c = hip.asarray(c.copy())
+        ops.gemm(_to_dev(hip, a), _to_dev(hip, b), d_c, alpha, beta)
+        got = d_c.asnumpy()
+        assert np.array_equal(got, expect)
+        assert np.array_equal(got, orc.gemm_f32(a, b, c.copy(), alpha, beta))
+
+
+@pytest.mark.parametrize("ta,tb,tc", list(itertools.product([False, True], repeat=3)))
+@pytest.mark.parametrize("m,n,k", [(33, 29, 47), (128, 128, 16), (1, 1, 1), (64, 1, 300)])
+def test_layouts_against_float64(env, ta, tb, tc, m, n, k):
+    """Every stride pattern the entry point accepts (row/column major A, B, C)."""
+    hip, ops, orc, mrt = env
+    rng = np.random.default_rng(m * 1000 + n * 10 + k)
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    b = rng.standard_normal((k, n), dtype=np.float32)
+    c0 = rng.standard_normal((m, n), dtype=np.float32)
+    lay = lambda x, t: np.asfortranarray(x) if t else x
+    d_c = _to_dev(hip, lay(c0, tc))
+    ops.gemm(_to_dev(hip, lay(a, ta)), _to_dev(hip, lay(b, tb)), d_c, 0.5, 2.0)
+    got = d_c.asnumpy()
+    truth = 2.0 * c0 + 0.5 * (a.astype(np.float64) @ b.astype(np.float64))
+    bound = 1e-5 * (2.0 * np.abs(c0) + 0.5 * (np.abs(a).astype(np.float64) @ np.abs(b))) + 1e-30
+    assert (np.abs(got - truth) <= bound).all()
+
+
+# Tolerance for float32 matmul: |gpu - truth| <= 1e-4 * (|a| @ |b|) elementwise
+# against a float64 ground truth, and relative 1e-4 in the Frobenius norm.
+def _check(got, a, b):
+    truth = a.astype(np.float64) @ b.astype(np.float64)
+    bound = 1e-4 * (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64))
+    assert (np.abs(got - truth) <= bound).all()
+    assert np.linalg.norm(got - truth) <= 1e-4 * np.linalg.norm(truth)
+
+
+@pytest.mark.parametrize("m,n,k", [(128, 128, 16), (256, 384, 512), (128, 256, 4096),
+                                   (1024, 1024, 1024), (384, 128, 48)])
+def test_mfma_kernel(env, m, n, k):
+    hip, ops, orc, mrt = env
+    rng = np.random.Generator(np.random.PCG64(1005))
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    b = rng.standard_normal((k, n), dtype=np.float32)
+    got = ops.dot(hip.asarray(a), hip.asarray(b)).asnumpy()
+    assert mrt.last_kernel().startswith("sgemm_mfma")
+    _check(got, a, b)
+    if m * n * k <= 1 << 27:
+        # against the oracle's float32 contraction (k innermost)
+        ref = orc.gemm_f32(a, b)
+        bound = 2e-4 * (np.abs(a).astype(np.float64) @ np.abs(b))
+        assert (np.abs(got - ref) <= bound).all()
+    # alpha/beta epilogue on the MFMA path
+    c0 = rng.standard_normal((m, n), dtype=np.float32)
+    d_c = hip.asarray(c0.copy())
+    ops.gemm(hip.asarray(a), hip.asarray(b), d_c, 0.5, -1.5)
+    truth = -1.5 * c0 + 0.5 * (a.astype(np.float64) @ b.astype(np.float64))
+    bound = 1e-4 * (1.5 * np.abs(c0) + 0.5 * (np.abs(a).astype(np.float64) @ np.abs(b)))
+    assert (np.abs(d_c.asnumpy() - truth) <= bound).all()
+
+
+def test_beta_zero_ignores_c(env):
+    hip, ops, _, _ = env
+    a = np.ones((128, 16), np.float32); b = np.ones((16, 128), np.float32)
+    c = hip.asarray(np.full((128, 128), np.nan, np.float32))
+    ops.gemm(hip.asarray(a), hip.asarray(b), c, 1.0, 0.0)
+    assert (c.asnumpy() == 16).all()
+
+
+def test_identity_and_linearity_full_size(env):
+    """Configuration 5 (4096^3): rows checked against float64, plus
+    size-independent properties: A @ I == A exactly, and linearity."""
+    hip, ops, _, mrt = env
+    from numba_mlir_amd import workloads
+    A, B = workloads.matmul()
+    d_A, d_B = hip.asarray(A), hip.asarray(B)
+    C = ops.dot(d_A, d_B).asnumpy()
+    assert mrt.last_kernel().startswith("sgemm_mfma")
+    rows = np.array([0, 1, 63, 64, 127, 128, 2047, 2048, 4032, 4095])
+    truth = A[rows].astype(np.float64) @ B.astype(np.float64)
+    bound = 1e-4 * (np.abs(A[rows]).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert (np.abs(C[rows] - truth) <= bound).all()
+    assert np.linalg.norm(C[rows] - truth) <= 1e-4 * np.linalg.norm(truth)
+    # column checks too (catches a transposed tile)
+    cols = np.array([0, 31, 32, 100, 4095])
+    truth_c = A.astype(np.float64) @ B[:, cols].astype(np.float64)
+    assert np.linalg.norm(C[:, cols] - truth_c) <= 1e-4 * np.linalg.norm(truth_c)
+    eye = hip.asarray(np.eye(4096, dtype=np.float32))
+    assert np.array_equal(ops.dot(d_A, eye).asnumpy(), A)
+    assert np.array_equal(ops.dot(eye, d_B).asnumpy(), B)
+    # numpy's own float32 sgemm as a second reference
+    np.testing.assert_allclose(C[::97, ::89], np.dot(A, B)[::97, ::89], rtol=0,
+                               atol=1e-4 * 64 * 3)
+
+
+def test_float64_gemm(env):
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(4)
+    a, b = rng.standard_normal((70, 90)), rng.standard_normal((90, 50))
+    got = ops.dot(hip.asarray(a), hip.asarray(b)).asnumpy()
+    np.testing.assert_allclose(got, a @ b, rtol=1e-12, atol=1e-12)
