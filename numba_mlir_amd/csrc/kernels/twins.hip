@@ -208,3 +208,27 @@ nmk_twin_pairwise_f64_rows(const double *__restrict__ X1,
     __builtin_nontemporal_store(r, reinterpret_cast<double2_t *>(D + i * n2 + j));
   }
 }
+
+// ---------------------------------------------------------------------------
+// Workgroup-memory kernel: every work-group reverses its slice of `a` through
+// a local array and a barrier,
+//   tmp = local.array(group_size); tmp[lid] = a[gid]; barrier();
+//   b[gid] = tmp[group_size - 1 - lid]
+// (local arrays and barriers: reference
+// mlir_compiler/lib/pipelines/LowerToGpu.cpp:1296-1386, 1515-1553).
+// The local array arrives the way the runtime passes workgroup memory: a
+// uint64 byte offset into the launch's dynamic LDS block.  Requires the
+// global size to be a multiple of the local size (uniform barrier).
+NMK_KERNEL(256)
+nmk_twin_group_reverse_i32(const int32_t *a, int64_t an, int64_t as, int32_t *b,
+                           int64_t bn, int64_t bs, uint64_t tmpOffset,
+                           int64_t gs0, int64_t gs1, int64_t gs2) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char ldsBase[];
+  int32_t *tmp = reinterpret_cast<int32_t *>(ldsBase + tmpOffset);
+  Ids t = ids(gs0, gs1, gs2);
+  if (t.inside)
+    tmp[t.l[0]] = a[t.g[0] * as];
+  __syncthreads();
+  if (t.inside)
+    b[t.g[0] * bs] = tmp[t.ls[0] - 1 - t.l[0]];
+}
