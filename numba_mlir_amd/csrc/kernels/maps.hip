@@ -7,7 +7,7 @@
 // per work-item with scalar loads.  Here the contiguous cases move 128 bits
 // per lane per access and keep a row-broadcast operand in registers.
 //
-// Kernel signatures are owned by the dispatcher (csrc/offload/Dispatch.cpp);
+// Kernel signatures are owned by the dispatcher (csrc/offload/Offload.cpp);
 // sizes and strides are int64 element counts, as the reference's flattened
 // memref ABI passes them (mlir/lib/Conversion/DecomposeMemrefs.cpp:85-206).
 #include "common.h"
@@ -45,8 +45,8 @@ template <> struct Vec128<float> {
 //
 // grid.x tiles the columns (256 lanes x 128 bit), grid.y tiles the rows in
 // chunks of rowsPerBlock.  A lane loads its slice of b once and reuses it for
-// every row of the chunk; row loads are issued four at a time so each lane
-// has 4 x 16 B reads in flight.
+// every row of the chunk; rows are taken two at a time.  Short chunks (1-2
+// rows, thousands of blocks each streaming a few KiB) measured fastest.
 template <typename T, typename Op>
 __device__ __forceinline__ void
 mapRowBroadcast(const T *__restrict__ a, const T *__restrict__ b,
@@ -64,37 +64,27 @@ mapRowBroadcast(const T *__restrict__ a, const T *__restrict__ b,
     rEnd = rows;
   const T *ap = a + r * cols + col;
   T *op = out + r * cols + col;
-  for (; r + 4 <= rEnd; r += 4) {
-    V v0 = __builtin_nontemporal_load(reinterpret_cast<const V *>(ap));
-    V v1 = __builtin_nontemporal_load(reinterpret_cast<const V *>(ap + cols));
-    V v2 =
-        __builtin_nontemporal_load(reinterpret_cast<const V *>(ap + 2 * cols));
-    V v3 =
-        __builtin_nontemporal_load(reinterpret_cast<const V *>(ap + 3 * cols));
-    V o0, o1, o2, o3;
+  for (; r + 2 <= rEnd; r += 2) {
+    V v0 = streamLoad(reinterpret_cast<const V *>(ap));
+    V v1 = streamLoad(reinterpret_cast<const V *>(ap + cols));
+    V o0, o1;
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       o0[i] = Op::apply(v0[i], bv[i]);
       o1[i] = Op::apply(v1[i], bv[i]);
-      o2[i] = Op::apply(v2[i], bv[i]);
-      o3[i] = Op::apply(v3[i], bv[i]);
     }
-    __builtin_nontemporal_store(o0, reinterpret_cast<V *>(op));
-    __builtin_nontemporal_store(o1, reinterpret_cast<V *>(op + cols));
-    __builtin_nontemporal_store(o2, reinterpret_cast<V *>(op + 2 * cols));
-    __builtin_nontemporal_store(o3, reinterpret_cast<V *>(op + 3 * cols));
-    ap += 4 * cols;
-    op += 4 * cols;
+    streamStore(o0, reinterpret_cast<V *>(op));
+    streamStore(o1, reinterpret_cast<V *>(op + cols));
+    ap += 2 * cols;
+    op += 2 * cols;
   }
-  for (; r < rEnd; ++r) {
-    V v0 = *reinterpret_cast<const V *>(ap);
+  if (r < rEnd) {
+    V v0 = streamLoad(reinterpret_cast<const V *>(ap));
     V o0;
 #pragma unroll
     for (int i = 0; i < N; ++i)
       o0[i] = Op::apply(v0[i], bv[i]);
-    *reinterpret_cast<V *>(op) = o0;
-    ap += cols;
-    op += cols;
+    streamStore(o0, reinterpret_cast<V *>(op));
   }
 }
 
@@ -113,18 +103,18 @@ mapContiguous(const T *__restrict__ a, const T *__restrict__ b,
   V *ov = reinterpret_cast<V *>(out);
   int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   for (; i + stride < nvec; i += 2 * stride) {
-    V a0 = __builtin_nontemporal_load(av + i);
-    V a1 = __builtin_nontemporal_load(av + i + stride);
-    V b0 = __builtin_nontemporal_load(bv + i);
-    V b1 = __builtin_nontemporal_load(bv + i + stride);
+    V a0 = streamLoad(av + i);
+    V a1 = streamLoad(av + i + stride);
+    V b0 = streamLoad(bv + i);
+    V b1 = streamLoad(bv + i + stride);
     V o0, o1;
 #pragma unroll
     for (int k = 0; k < N; ++k) {
       o0[k] = Op::apply(a0[k], b0[k]);
       o1[k] = Op::apply(a1[k], b1[k]);
     }
-    __builtin_nontemporal_store(o0, ov + i);
-    __builtin_nontemporal_store(o1, ov + i + stride);
+    streamStore(o0, ov + i);
+    streamStore(o1, ov + i + stride);
   }
   if (i < nvec) {
     V a0 = av[i], b0 = bv[i], o0;
@@ -200,89 +190,148 @@ NMK_DEFINE_MAP2_ALL_T(mul, OpMul)
 // W = float evaluates the same expression tree entirely in float32 (what
 // NumPy computes for the same source, and what the reference computes when
 // the literals are written as np.float32).
+//
+// Transcendentals.  log(P/S) and exp(b) are the float32 library routines.
+// The two float64 erf calls and 1.0 / sqrt(z) dominate the instruction count
+// (the kernel is ALU-bound, not HBM-bound), so the float64 path evaluates
+//   erf  by a piecewise degree-9 polynomial on 24 intervals of [0, 6)
+//        (erf_table.inc, absolute error < 1e-14; erf(|x| >= 6) = 1 in
+//        double), coefficients staged in LDS;
+//   1/sqrt(z)  by v_rsq_f64 refined with two Newton steps (relative error a
+//        few 1e-16), falling back to 1.0 / sqrt(z) outside [1e-290, 1e290].
+// Both stay within a few ulp of the library results, far inside the
+// tolerance the path is checked at.
+#include "erf_table.inc"
+
 template <typename W> struct BsMath;
 template <> struct BsMath<double> {
-  __device__ static double sqrt_(double x) { return sqrt(x); }
-  __device__ static double erf_(double x) { return erf(x); }
+  __device__ static __forceinline__ double rsqrt_(double z) {
+    if (!(z > 1e-290 && z < 1e290))
+      return 1.0 / sqrt(z);
+    double y = __builtin_amdgcn_rsq(z);
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const double r = __builtin_fma(-z, y * y, 1.0); // 1 - z y^2
+      y = __builtin_fma(0.5 * y, r, y);
+    }
+    return y;
+  }
+  __device__ static __forceinline__ double erf_(double x, const double *tab) {
+    double ax = __builtin_fabs(x);
+    ax = ax < 6.0 ? ax : 0x1.7ffffffffffffp+2; // largest double below 6
+    int idx = int(ax * 4.0);
+    const double u = __builtin_fma(ax, 8.0, -double(2 * idx + 1));
+    const double *c = tab + idx * NMK_ERF_COEFFS;
+    double p = c[NMK_ERF_COEFFS - 1];
+#pragma unroll
+    for (int k = NMK_ERF_COEFFS - 2; k >= 0; --k)
+      p = __builtin_fma(p, u, c[k]);
+    return __builtin_copysign(p, x);
+  }
 };
 template <> struct BsMath<float> {
-  __device__ static float sqrt_(float x) { return sqrtf(x); }
-  __device__ static float erf_(float x) { return erff(x); }
+  __device__ static __forceinline__ float rsqrt_(float z) {
+    return 1.0f / sqrtf(z);
+  }
+  __device__ static __forceinline__ float erf_(float x, const double *) {
+    return erff(x);
+  }
 };
 
 template <typename W>
-__device__ __forceinline__ void blackScholesOne(float P, float S, float T,
-                                                float mr, W sigSigTwo,
-                                                float &call, float &put) {
+__device__ __forceinline__ void
+blackScholesOne(float P, float S, float T, float mr, W sigSigTwo,
+                const double *erfTab, float &call, float &put) {
   const float a = logf(P / S);
   const float b = T * mr;
   const W z = W(T) * sigSigTwo;
   const W c = W(0.25) * z;
-  const W y = W(1.0) / BsMath<W>::sqrt_(z);
+  const W y = BsMath<W>::rsqrt_(z);
   const float amb = a - b;
   const W w1 = (W(amb) + c) * y;
   const W w2 = (W(amb) - c) * y;
-  const W d1 = W(0.5) + W(0.5) * BsMath<W>::erf_(w1);
-  const W d2 = W(0.5) + W(0.5) * BsMath<W>::erf_(w2);
+  const W d1 = W(0.5) + W(0.5) * BsMath<W>::erf_(w1, erfTab);
+  const W d2 = W(0.5) + W(0.5) * BsMath<W>::erf_(w2, erfTab);
   const float Se = expf(b) * S;
   const W r = W(P) * d1 - W(Se) * d2;
   call = float(r);
   put = float(r - W(P) + W(Se));
 }
 
-template <typename W>
+// VEC options per lane per iteration (float4 or float2 accesses).  The
+// float64 variant is ALU-bound and register-hungry: two options per lane at
+// six waves per SIMD measured fastest; the float32 variant takes four.
+template <int VEC> struct BsVec;
+template <> struct BsVec<4> {
+  typedef float4_t type;
+};
+template <> struct BsVec<2> {
+  typedef float type __attribute__((ext_vector_type(2)));
+};
+
+template <typename W, int VEC>
 __device__ __forceinline__ void
 blackScholes(const float *__restrict__ price, const float *__restrict__ strike,
              const float *__restrict__ t, float rate, float volatility,
              float *__restrict__ call, float *__restrict__ put, int64_t n) {
+  typedef typename BsVec<VEC>::type V;
+  __shared__ double erfTab[sizeof(W) == 8 ? NMK_ERF_INTERVALS * NMK_ERF_COEFFS
+                                          : 1];
+  if (sizeof(W) == 8) {
+    for (int i = threadIdx.x; i < NMK_ERF_INTERVALS * NMK_ERF_COEFFS;
+         i += blockDim.x)
+      erfTab[i] = kErfTable[i];
+    __syncthreads();
+  }
   const float mr = -rate;
   const W sigSigTwo = W(volatility * volatility) * W(2);
-  const int64_t nvec = n / 4;
+  const int64_t nvec = n / VEC;
   const int64_t stride = int64_t(gridDim.x) * blockDim.x;
-  const float4_t *pv = reinterpret_cast<const float4_t *>(price);
-  const float4_t *sv = reinterpret_cast<const float4_t *>(strike);
-  const float4_t *tv = reinterpret_cast<const float4_t *>(t);
-  float4_t *cv = reinterpret_cast<float4_t *>(call);
-  float4_t *uv = reinterpret_cast<float4_t *>(put);
+  const V *pv = reinterpret_cast<const V *>(price);
+  const V *sv = reinterpret_cast<const V *>(strike);
+  const V *tv = reinterpret_cast<const V *>(t);
+  V *cv = reinterpret_cast<V *>(call);
+  V *uv = reinterpret_cast<V *>(put);
   for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec;
        i += stride) {
-    const float4_t P = __builtin_nontemporal_load(pv + i);
-    const float4_t S = __builtin_nontemporal_load(sv + i);
-    const float4_t T = __builtin_nontemporal_load(tv + i);
-    float4_t c, u;
+    const V P = streamLoad(pv + i);
+    const V S = streamLoad(sv + i);
+    const V T = streamLoad(tv + i);
+    V c, u;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < VEC; ++k) {
       float ck, uk;
-      blackScholesOne<W>(P[k], S[k], T[k], mr, sigSigTwo, ck, uk);
+      blackScholesOne<W>(P[k], S[k], T[k], mr, sigSigTwo, erfTab, ck, uk);
       c[k] = ck;
       u[k] = uk;
     }
-    __builtin_nontemporal_store(c, cv + i);
-    __builtin_nontemporal_store(u, uv + i);
+    streamStore(c, cv + i);
+    streamStore(u, uv + i);
   }
-  // n % 4 trailing options, one per lane of the first block.
-  const int64_t tail = nvec * 4 + threadIdx.x;
+  // n % VEC trailing options, one per lane of the first block.
+  const int64_t tail = nvec * VEC + threadIdx.x;
   if (blockIdx.x == 0 && tail < n) {
     float ck, uk;
-    blackScholesOne<W>(price[tail], strike[tail], t[tail], mr, sigSigTwo, ck,
-                       uk);
+    blackScholesOne<W>(price[tail], strike[tail], t[tail], mr, sigSigTwo,
+                       erfTab, ck, uk);
     call[tail] = ck;
     put[tail] = uk;
   }
 }
 
-NMK_KERNEL(256)
+extern "C" __global__ __launch_bounds__(256)
+__attribute__((amdgpu_waves_per_eu(6, 6))) void
 nmk_black_scholes_f32_w64(const float *price, const float *strike,
                           const float *t, float rate, float volatility,
                           float *call, float *put, int64_t n) {
-  blackScholes<double>(price, strike, t, rate, volatility, call, put, n);
+  blackScholes<double, 2>(price, strike, t, rate, volatility, call, put, n);
 }
 
 NMK_KERNEL(256)
 nmk_black_scholes_f32_w32(const float *price, const float *strike,
                           const float *t, float rate, float volatility,
                           float *call, float *put, int64_t n) {
-  blackScholes<float>(price, strike, t, rate, volatility, call, put, n);
+  blackScholes<float, 4>(price, strike, t, rate, volatility, call, put, n);
 }
 
 // Fills n 32-bit words with a value (used to zero ticket counters: a

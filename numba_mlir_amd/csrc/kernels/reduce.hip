@@ -41,10 +41,10 @@ nmk_sum_axis1_f32(const float *__restrict__ x, float *__restrict__ out,
     float4_t a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0, a3 = a0;
     int64_t i = lane;
     for (; i + 3 * NMK_WAVE < nvec; i += 4 * NMK_WAVE) {
-      float4_t v0 = __builtin_nontemporal_load(pv + i);
-      float4_t v1 = __builtin_nontemporal_load(pv + i + NMK_WAVE);
-      float4_t v2 = __builtin_nontemporal_load(pv + i + 2 * NMK_WAVE);
-      float4_t v3 = __builtin_nontemporal_load(pv + i + 3 * NMK_WAVE);
+      float4_t v0 = streamLoad(pv + i);
+      float4_t v1 = streamLoad(pv + i + NMK_WAVE);
+      float4_t v2 = streamLoad(pv + i + 2 * NMK_WAVE);
+      float4_t v3 = streamLoad(pv + i + 3 * NMK_WAVE);
       a0 += v0;
       a1 += v1;
       a2 += v2;
@@ -71,11 +71,15 @@ nmk_sum_axis1_f32(const float *__restrict__ x, float *__restrict__ out,
 //
 // grid.x = column strips of 256 columns (64 lanes x int4 = 1 KiB of a row),
 // grid.y = row chunks of rowsPerBlock.  The four waves of a block take
-// interleaved rows of the chunk, eight row loads in flight per lane, fold
+// interleaved rows of the chunk, NMK_AX0_UNROLL row loads in flight per lane, fold
 // through LDS, and publish one int64 partial per column to
 // partial[chunk][col].  The block that draws the last ticket of its strip
 // adds the chunks in index order and writes out[]; it also resets the ticket,
 // so the counters are zero again when the kernel ends.
+#ifndef NMK_AX0_UNROLL
+#define NMK_AX0_UNROLL 16 // row loads in flight per lane
+#endif
+
 NMK_KERNEL(256)
 nmk_sum_axis0_i32_i64(const int32_t *__restrict__ x, int64_t *__restrict__ out,
                       int64_t rows, int64_t cols, int64_t ld,
@@ -96,19 +100,20 @@ nmk_sum_axis0_i32_i64(const int32_t *__restrict__ x, int64_t *__restrict__ out,
       rEnd = rows;
     const int32_t *p = x + r * ld + col;
     const int64_t step = 4 * ld; // the block's waves interleave rows
-    for (; r + 28 < rEnd; r += 32) {
-      int4_t v[8];
+    for (; r + 4 * (NMK_AX0_UNROLL - 1) < rEnd; r += 4 * NMK_AX0_UNROLL) {
+      int4_t v[NMK_AX0_UNROLL];
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        v[u] = __builtin_nontemporal_load(
-            reinterpret_cast<const int4_t *>(p + u * step));
+      for (int u = 0; u < NMK_AX0_UNROLL; ++u)
+        v[u] = streamLoad(reinterpret_cast<const int4_t *>(p + u * step));
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
-        acc[k] += ((int64_t(v[0][k]) + int64_t(v[1][k])) +
-                   (int64_t(v[2][k]) + int64_t(v[3][k]))) +
-                  ((int64_t(v[4][k]) + int64_t(v[5][k])) +
-                   (int64_t(v[6][k]) + int64_t(v[7][k])));
-      p += 8 * step;
+      for (int k = 0; k < 4; ++k) {
+        int64_t s = 0;
+#pragma unroll
+        for (int u = 0; u < NMK_AX0_UNROLL; ++u)
+          s += int64_t(v[u][k]);
+        acc[k] += s;
+      }
+      p += NMK_AX0_UNROLL * step;
     }
     for (; r < rEnd; r += 4) {
       int4_t v0 = *reinterpret_cast<const int4_t *>(p);
@@ -184,10 +189,10 @@ fullSumF32(const float *__restrict__ x, float *__restrict__ out, int64_t n,
     float4_t a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0, a3 = a0;
     for (int64_t piece = blockIdx.x; piece < nPieces; piece += gridDim.x) {
       const float4_t *q = pv + piece * 1024 + threadIdx.x;
-      float4_t v0 = __builtin_nontemporal_load(q);
-      float4_t v1 = __builtin_nontemporal_load(q + 256);
-      float4_t v2 = __builtin_nontemporal_load(q + 512);
-      float4_t v3 = __builtin_nontemporal_load(q + 768);
+      float4_t v0 = streamLoad(q);
+      float4_t v1 = streamLoad(q + 256);
+      float4_t v2 = streamLoad(q + 512);
+      float4_t v3 = streamLoad(q + 768);
       if (SQUARE_ROOT_OF_SQUARES) {
         v0 *= v0;
         v1 *= v1;

@@ -144,7 +144,7 @@ pairwiseFaithful(const T *X1, int64_t x1r, int64_t x1c, int64_t x1s0,
     T tmp = X1[i * x1s0 + k * x1s1] - X2[j * x2s0 + k * x2s1];
     d += double(tmp * tmp);
   }
-  D[i * ds0 + j * ds1] = T(sqrt(d));
+  D[i * ds0 + j * ds1] = T(sqrtF64(d));
 }
 
 NMK_KERNEL(256)
@@ -204,8 +204,8 @@ nmk_twin_pairwise_f64_rows(const double *__restrict__ X1,
     d1 += t * t;
     t = x2 - y12;
     d1 += t * t;
-    double2_t r = {sqrt(d0), sqrt(d1)};
-    __builtin_nontemporal_store(r, reinterpret_cast<double2_t *>(D + i * n2 + j));
+    double2_t r = {sqrtF64(d0), sqrtF64(d1)};
+    streamStore(r, reinterpret_cast<double2_t *>(D + i * n2 + j));
   }
 }
 

@@ -545,10 +545,11 @@ NMHIP_EXPORT void nmhipMapBinary(void *ctx, int op, int dtype, const void *a,
       const int64_t gx = ceilDiv(n1, 256 * lanesElems);
       int64_t rowsPerBlock = tuning().rowbcastRows;
       if (!rowsPerBlock) {
-        // Aim at ~4096 blocks (16 per CU) with at least 4 rows each.
-        rowsPerBlock = ceilDiv(n0 * gx, 4096);
-        if (rowsPerBlock < 4)
-          rowsPerBlock = 4;
+        // Two rows per block: many short-lived blocks stream best; more
+        // only when grid.y would overflow.
+        rowsPerBlock = 2;
+        if (ceilDiv(n0, rowsPerBlock) > 65535)
+          rowsPerBlock = ceilDiv(n0, 65535);
       }
       const int64_t gy = ceilDiv(n0, rowsPerBlock);
       if (gy <= 65535) {
@@ -591,8 +592,12 @@ NMHIP_EXPORT void nmhipBlackScholesF32(void *ctx, const float *price,
     if (!(aligned16(price) && aligned16(strike) && aligned16(t) &&
           aligned16(call) && aligned16(put)))
       fail("nmhipBlackScholesF32: arrays must be 16-byte aligned");
-    int64_t blocks = tuning().bsBlocks ? tuning().bsBlocks : 256 * 8;
-    const int64_t need = ceilDiv(ceilDiv(n, 4), 256);
+    if (n < 0)
+      fail("nmhipBlackScholesF32: negative extent");
+    int64_t blocks = tuning().bsBlocks ? tuning().bsBlocks : 256 * 16;
+    // The float64-literal kernel takes two options per lane, the float32 one
+    // four.
+    const int64_t need = ceilDiv(ceilDiv(n, wide ? 2 : 4), 256);
     if (blocks > need)
       blocks = need;
     c->launch(wide ? "nmk_black_scholes_f32_w64" : "nmk_black_scholes_f32_w32",
@@ -634,9 +639,10 @@ NMHIP_EXPORT void nmhipReduce(void *ctx, int op, int dtype, const void *x,
       const int64_t strips = ceilDiv(n1, 256);
       int64_t rowsPerBlock = tuning().axis0Rows;
       if (!rowsPerBlock) {
-        // ~1024 blocks; whole 32-row groups (8 loads x 4 waves) per block.
-        rowsPerBlock = ceilDiv(n0 * strips, 1024);
-        rowsPerBlock = ceilDiv(rowsPerBlock, 32) * 32;
+        // One block per CU (256) measured fastest: few, long-lived blocks
+        // keep the finish short.  Whole 64-row groups (16 loads x 4 waves).
+        rowsPerBlock = ceilDiv(n0 * strips, 256);
+        rowsPerBlock = ceilDiv(rowsPerBlock, 64) * 64;
       }
       const int64_t chunks = ceilDiv(n0, rowsPerBlock);
       if (strips <= int64_t(kMaxTickets) && chunks <= 65535) {
@@ -653,7 +659,7 @@ NMHIP_EXPORT void nmhipReduce(void *ctx, int op, int dtype, const void *x,
     if (op == NMHIP_SUM && dtype == NMHIP_F32 && axis == -1 && contiguous &&
         n0 * n1 >= 4096) {
       const int64_t n = n0 * n1;
-      int64_t blocks = tuning().reduceBlocks ? tuning().reduceBlocks : 1024;
+      int64_t blocks = tuning().reduceBlocks ? tuning().reduceBlocks : 512;
       const int64_t need = ceilDiv(n, 256 * 16);
       if (blocks > need)
         blocks = need;
@@ -700,7 +706,7 @@ NMHIP_EXPORT void nmhipNorm2F32(void *ctx, const float *x, int64_t n,
     std::lock_guard<std::mutex> lock(c->mutex);
     if (n < 0)
       fail("nmhipNorm2F32: negative extent");
-    int64_t blocks = tuning().reduceBlocks ? tuning().reduceBlocks : 1024;
+    int64_t blocks = tuning().reduceBlocks ? tuning().reduceBlocks : 512;
     int64_t need = ceilDiv(n, 256 * 16);
     if (need < 1)
       need = 1;
@@ -794,9 +800,9 @@ NMHIP_EXPORT void nmhipPairwiseF64(void *ctx, const double *X1,
     const int64_t gx = ceilDiv(n2, 512);
     int64_t rows = tuning().pairwiseRows;
     if (!rows) {
-      rows = ceilDiv(n1 * gx, 4096);
-      if (rows < 4)
-        rows = 4;
+      rows = 4;
+      if (ceilDiv(n1, rows) > 65535)
+        rows = ceilDiv(n1, 65535);
     }
     const int64_t gy = ceilDiv(n1, rows);
     if (gy > 65535)
