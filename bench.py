@@ -37,7 +37,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", type=str, default="",
                     help="comma-separated subset of: add,bs,bs32,sum1,norm2,"
-                         "sum0,pairwise,matmul")
+                         "sum0,pairwise,matmul (plus copy, only on request)")
     ap.add_argument("--no-cpu", action="store_true",
                     help="skip the CPU baseline leg")
     return ap.parse_args()
@@ -136,6 +136,16 @@ def run(args):
             if wide:
                 headline = (e, nopt, (price, strike, t, rate, vol))
         del d
+
+    # -- yardstick: plain copy of known size (scales the HBM counters) -------
+    if "copy" in only:
+        nbytes = 1 << 28
+        src, dst = da.empty((nbytes,), np.uint8), da.empty((nbytes,), np.uint8)
+        wall, ev, kern = b.measure(c_call(b.lib.nmhipCopy, b.ctx.handle, dst.ptr,
+                                          src.ptr, nbytes))
+        per_config.append(hbm_entry("copy", "device copy of 256 MiB",
+                                    2 * nbytes, wall, ev, kern))
+        del src, dst
 
     # -- config 1: broadcast add --------------------------------------------
     if want("add"):

@@ -97,6 +97,11 @@ void nmhipFree(void *ctx, void *dev);
 void nmhipMemcpyHtoD(void *ctx, void *dev, const void *host, size_t bytes);
 void nmhipMemcpyDtoH(void *ctx, void *host, const void *dev, size_t bytes);
 
+/* Device-to-device copy of a contiguous buffer on the context's queue (what
+ * the compiler's force_copy of a contiguous operand lowers to,
+ * numpy/funcs.py:759-764); bytes and pointers must be multiples of 16. */
+void nmhipCopy(void *ctx, void *dst, const void *src, size_t bytes);
+
 /* ---- elementwise / broadcast maps -------------------------------------- */
 
 /*
@@ -177,7 +182,7 @@ void nmhipPairwiseF64(void *ctx, const double *X1, const double *X2, double *D,
 /* The embedded gfx950 code object of a family: "maps", "reduce", "twins". */
 const void *nmhipKernelBlob(const char *family, size_t *size);
 
-/* Overrides a launch-shape knob ("rowbcast_rows", "map_blocks",
+/* Overrides a launch-shape knob ("rowbcast_rows", "map_blocks", "bs_blocks",
  * "reduce_blocks", "axis0_rows", "pairwise_rows"); 0 restores the default. */
 void nmhipSetTuning(const char *knob, int64_t value);
 

@@ -334,6 +334,18 @@ nmk_black_scholes_f32_w32(const float *price, const float *strike,
   blackScholes<float, 4>(price, strike, t, rate, volatility, call, put, n);
 }
 
+// Plain copy of nvec 128-bit words (force_copy of a contiguous operand; also
+// the known-size yardstick the HBM counters are scaled against).  One 4 KiB
+// piece per block iteration.
+NMK_KERNEL(256)
+nmk_copy_b128(const int4_t *__restrict__ src, int4_t *__restrict__ dst,
+              int64_t nvec) {
+  const int64_t stride = int64_t(gridDim.x) * blockDim.x;
+  for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec;
+       i += stride)
+    streamStore(streamLoad(src + i), dst + i);
+}
+
 // Fills n 32-bit words with a value (used to zero ticket counters: a
 // hipMemset node would not be safe inside a captured graph).
 NMK_KERNEL(256) nmk_fill_u32(uint32_t *dst, uint32_t value, int64_t n) {

@@ -44,7 +44,7 @@ thread_local const char *lastKernel = "";
 // C[M,N] = alpha * A[M,K] * B[K,N] + beta * C, all row-major with leading
 // dimensions lda/ldb/ldc, fp32 in, fp32 accumulate on the matrix cores.
 //
-// Block tile 128 x 128, K step 16, 256 threads = 4 waves in a 2 x 2 grid,
+// Block tile 128 x 128, K step BK = 16, 256 threads = 4 waves in a 2 x 2 grid,
 // each wave owns 64 x 64 = 2 x 2 tiles of v_mfma_f32_32x32x2_f32.
 //
 // LDS holds both operands K-major ([k][m] and [k][n], rows padded by 4 floats)
@@ -61,8 +61,9 @@ thread_local const char *lastKernel = "";
 //
 // Requirements (checked by the host): M % 128 == 0, N % 128 == 0,
 // K % 16 == 0, lda/ldb % 4 == 0, A and B 16-byte aligned.
-constexpr int BM = 128, BN = 128, BK = 16, PAD = 4;
+constexpr int BM = 128, BN = 128, PAD = 4;
 
+template <int BK>
 __global__ __launch_bounds__(256) void
 sgemm_mfma_128x128(const float *__restrict__ A, const float *__restrict__ B,
                    float *__restrict__ C, int M, int N, int K, int64_t lda,
@@ -77,29 +78,32 @@ sgemm_mfma_128x128(const float *__restrict__ A, const float *__restrict__ B,
   const int bm = blockIdx.y * BM;
   const int bn = blockIdx.x * BN;
 
-  // Global fetch mapping: A slab 128 x 16 -> 2 float4 per thread (k
-  // contiguous); B slab 16 x 128 -> 2 float4 per thread (n contiguous).
-  const int aRow = tid / 4, aK = (tid % 4) * 4;
+  // Global fetch mapping, NV = BK / 8 float4 per thread and operand:
+  // A slab 128 x BK, k contiguous: a pass of the block covers 1024 / BK rows;
+  // B slab BK x 128, n contiguous: a pass covers 8 k-rows.
+  constexpr int NV = BK / 8;
+  constexpr int A_ROWS = 1024 / BK;
+  const int aRow = tid / (BK / 4), aK = (tid % (BK / 4)) * 4;
   const int bK = tid / 32, bN = (tid % 32) * 4;
   const float *aPtr = A + int64_t(bm + aRow) * lda + aK;
   const float *bPtr = B + int64_t(bK) * ldb + bn + bN;
 
-  floatx4 aReg[2], bReg[2];
+  floatx4 aReg[NV], bReg[NV];
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      aReg[i] = *reinterpret_cast<const floatx4 *>(aPtr + int64_t(64 * i) * lda +
-                                                   k0);
+    for (int i = 0; i < NV; ++i) {
+      aReg[i] = *reinterpret_cast<const floatx4 *>(
+          aPtr + int64_t(A_ROWS * i) * lda + k0);
       bReg[i] = *reinterpret_cast<const floatx4 *>(bPtr +
                                                    int64_t(k0 + 8 * i) * ldb);
     }
   };
   auto stash = [&](int stage) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NV; ++i) {
 #pragma unroll
       for (int q = 0; q < 4; ++q)
-        As[stage][aK + q][aRow + 64 * i] = aReg[i][q];
+        As[stage][aK + q][aRow + A_ROWS * i] = aReg[i][q];
       *reinterpret_cast<floatx4 *>(&Bs[stage][bK + 8 * i][bN]) = bReg[i];
     }
   };
@@ -211,6 +215,10 @@ gemm_generic(const T *A, const T *B, T *C, int64_t M, int64_t N, int64_t K,
   }
 }
 
+// K-slab depth of the MFMA kernel (32 measured 6 % slower: half the blocks
+// per CU for the same MFMA work).
+constexpr int SGEMM_BK = 16;
+
 template <typename T> struct MemrefOf;
 template <> struct MemrefOf<float> {
   typedef NmhipMemref2F32 type;
@@ -271,13 +279,14 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
     if constexpr (sizeof(T) == 4) {
       const bool rowMajor = a->strides[1] == 1 && b->strides[1] == 1 &&
                             c->strides[1] == 1;
-      if (rowMajor && K > 0 && M % BM == 0 && N % BN == 0 && K % BK == 0 &&
+      if (rowMajor && K > 0 && M % BM == 0 && N % BN == 0 &&
+          K % SGEMM_BK == 0 &&
           a->strides[0] % 4 == 0 && b->strides[0] % 4 == 0 &&
           aligned16(aData) && aligned16(bData) && M <= 0x7fffffff &&
           N <= 0x7fffffff && K <= 0x7fffffff && M / BM <= 65535) {
         dim3 grid(unsigned(N / BN), unsigned(M / BM), 1);
-        hipLaunchKernelGGL(sgemm_mfma_128x128, grid, dim3(256), 0, stream,
-                           aData, bData, cData, int(M), int(N), int(K),
+        hipLaunchKernelGGL(sgemm_mfma_128x128<SGEMM_BK>, grid, dim3(256), 0,
+                           stream, aData, bData, cData, int(M), int(N), int(K),
                            int64_t(a->strides[0]), int64_t(b->strides[0]),
                            int64_t(c->strides[0]), alpha, beta);
         lastKernel = "sgemm_mfma_128x128";

@@ -197,7 +197,7 @@ const Blob *findBlob(const char *family) {
 const char *familyOf(const std::string &kernel) {
   auto starts = [&](const char *p) { return kernel.rfind(p, 0) == 0; };
   if (starts("nmk_map2_") || starts("nmk_black_scholes_") ||
-      starts("nmk_fill_"))
+      starts("nmk_fill_") || starts("nmk_copy_"))
     return "maps";
   if (starts("nmk_sum_") || starts("nmk_norm2_") || starts("nmk_reduce_"))
     return "reduce";
@@ -492,6 +492,24 @@ NMHIP_EXPORT void nmhipMemcpyDtoH(void *ctx, void *host, const void *dev,
     checkHip(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, s),
              "hipMemcpyAsync(DtoH)");
     checkHip(hipStreamSynchronize(s), "hipStreamSynchronize");
+  });
+}
+
+NMHIP_EXPORT void nmhipCopy(void *ctx, void *dst, const void *src,
+                            size_t bytes) {
+  guarded([&]() {
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    if (bytes == 0)
+      return;
+    if (bytes % 16 != 0 || !aligned16(dst) || !aligned16(src))
+      fail("nmhipCopy: needs 16-byte aligned pointers and size");
+    const int64_t nvec = int64_t(bytes / 16);
+    int64_t blocks = ceilDiv(nvec, 256);
+    if (blocks > (int64_t(1) << 20))
+      blocks = int64_t(1) << 20;
+    c->launch("nmk_copy_b128", size_t(blocks), 1, 1, 256, 1, 1,
+              {Arg::Ptr(src), Arg::Ptr(dst), Arg::I64(nvec)});
   });
 }
 

@@ -31,6 +31,7 @@ _SIGNATURES = {
     "nmhipFree": (None, [_vp, _vp]),
     "nmhipMemcpyHtoD": (None, [_vp, _vp, _vp, _sz]),
     "nmhipMemcpyDtoH": (None, [_vp, _vp, _vp, _sz]),
+    "nmhipCopy": (None, [_vp, _vp, _vp, _sz]),
     "nmhipMapBinary": (None, [_vp, ctypes.c_int, ctypes.c_int, _vp, _i64x2, _vp,
                               _i64x2, _vp, _i64x2, _i64, _i64]),
     "nmhipBlackScholesF32": (None, [_vp, _vp, _vp, _vp, ctypes.c_float,
