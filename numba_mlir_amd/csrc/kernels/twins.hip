@@ -232,3 +232,358 @@ nmk_twin_group_reverse_i32(const int32_t *a, int64_t an, int64_t as, int32_t *b,
   if (t.inside)
     b[t.g[0] * bs] = tmp[t.ls[0] - 1 - t.l[0]];
 }
+
+// ===========================================================================
+// Kernel builtins beyond ids: atomics, barriers / fences, local and private
+// arrays, group reductions.  Each twin is the body of a reference test
+// (numba_mlir/numba_mlir/mlir/tests/test_gpu.py, cited per kernel); together
+// they are the HIP device-side forms of what the reference lowers in
+// mlir_compiler/lib/pipelines/LowerToGpu.cpp:1296-1780.
+//
+//  * atomic.add / atomic.sub (1404-1465): agent-scope atomicAdd; sub adds the
+//    negated value, as the reference does (kernel_impl.py:263-322).
+//  * barrier(flags) (1515-1553): __syncthreads(), preceded by a device-scope
+//    fence for GLOBAL_MEM_FENCE; mem_fence(flags) is the fence alone.
+//    Barriers sit outside the bounds guard so every lane reaches them (the
+//    reference's MakeBarriersUniform transform does the same hoisting).
+//  * local.array (1296-1386): workgroup memory passed by the runtime as a
+//    byte offset into dynamic LDS.
+//  * private.array: a per-lane array (registers / scratch).
+//  * group.reduce_* (1564-1780): an LDS tree over the work-group (any local
+//    size up to 256; the reference reduces subgroups of a hard-coded 8 lanes
+//    first, 1683-1688); lanes past the global size contribute the neutral
+//    element.
+// ===========================================================================
+
+namespace {
+
+__device__ __forceinline__ int linearLocalId() {
+  return threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z);
+}
+
+__device__ __forceinline__ int localCount() {
+  return blockDim.x * blockDim.y * blockDim.z;
+}
+
+// Workgroup-wide reduction for any block shape up to 256 lanes (full and
+// partial waves alike): an LDS tree.  Lanes outside the global size pass the
+// neutral element.  Every lane of the block must call it.
+template <typename T, typename Op>
+__device__ __forceinline__ T groupReduce(T v, T neutral, bool active, Op op) {
+  __shared__ T scratch[256];
+  const int tid = linearLocalId();
+  const int n = localCount();
+  __syncthreads(); // scratch may still be read by a previous call
+  scratch[tid] = active ? v : neutral;
+  __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) {
+    if (tid < s && tid + s < n)
+      scratch[tid] = op(scratch[tid], scratch[tid + s]);
+    __syncthreads();
+  }
+  return scratch[0];
+}
+
+template <typename T> __device__ __forceinline__ void atomicAddT(T *p, T v) {
+  atomicAdd(p, v);
+}
+template <>
+__device__ __forceinline__ void atomicAddT<int64_t>(int64_t *p, int64_t v) {
+  atomicAdd(reinterpret_cast<unsigned long long *>(p),
+            static_cast<unsigned long long>(v));
+}
+
+} // namespace
+
+// c[i, j, k] = a[i, j, k] + b[i, j, k]   (test_simple1/2, test_gpu.py:178-232)
+NMK_KERNEL(256)
+nmk_twin_add3_f32(const float *a, int64_t a0, int64_t a1, int64_t a2,
+                  int64_t as0, int64_t as1, int64_t as2, const float *b,
+                  int64_t b0, int64_t b1, int64_t b2, int64_t bs0, int64_t bs1,
+                  int64_t bs2, float *c, int64_t c0, int64_t c1, int64_t c2,
+                  int64_t cs0, int64_t cs1, int64_t cs2, int64_t gs0,
+                  int64_t gs1, int64_t gs2) {
+  Ids t = ids(gs0, gs1, gs2);
+  if (t.inside)
+    c[t.g[0] * cs0 + t.g[1] * cs1 + t.g[2] * cs2] =
+        a[t.g[0] * as0 + t.g[1] * as1 + t.g[2] * as2] +
+        b[t.g[0] * bs0 + t.g[1] * bs1 + t.g[2] * bs2];
+}
+
+// b[i, 0] = a[i, 0]; b[i, 1] = a[i, 1]   (test_simple3, 235-259)
+NMK_KERNEL(256)
+nmk_twin_copy_cols2_f32(const float *a, int64_t a0, int64_t a1, int64_t as0,
+                        int64_t as1, float *b, int64_t b0, int64_t b1,
+                        int64_t bs0, int64_t bs1, int64_t gs0, int64_t gs1,
+                        int64_t gs2) {
+  Ids t = ids(gs0, gs1, gs2);
+  if (t.inside) {
+    b[t.g[0] * bs0] = a[t.g[0] * as0];
+    b[t.g[0] * bs0 + bs1] = a[t.g[0] * as0 + as1];
+  }
+}
+
+// res[i] = a[i] * b[i] + c[i] with two roundings (test_fastmath, 981-1008:
+// no fma unless fastmath=True; this file is built with -ffp-contract=off).
+NMK_KERNEL(256)
+nmk_twin_mul_add_f32(const float *a, int64_t an, int64_t as, const float *b,
+                     int64_t bn, int64_t bs, const float *c, int64_t cn,
+                     int64_t cs, float *res, int64_t rn, int64_t rs,
+                     int64_t gs0, int64_t gs1, int64_t gs2) {
+  Ids t = ids(gs0, gs1, gs2);
+  if (t.inside)
+    res[t.g[0] * rs] = a[t.g[0] * as] * b[t.g[0] * bs] + c[t.g[0] * cs];
+}
+
+// Atomics (test_atomics*, 806-955).  MODE selects the body:
+//   0: op(b, 0, a[i])          1: op(b, i % 2, a[i])
+//   2: op(b, 0, a[i] + 1)      3: op(b, 0, 1)
+// SIGN is +1 for atomic.add, -1 for atomic.sub.
+template <typename T, int MODE, int SIGN>
+__device__ __forceinline__ void atomicBody(const T *a, int64_t as, T *b,
+                                           int64_t bs, int64_t gs0,
+                                           int64_t gs1, int64_t gs2) {
+  Ids t = ids(gs0, gs1, gs2);
+  if (!t.inside)
+    return;
+  const int64_t i = t.g[0];
+  T v = MODE == 3 ? T(1) : (MODE == 2 ? T(a[i * as] + T(1)) : a[i * as]);
+  if (SIGN < 0)
+    v = -v;
+  atomicAddT(b + (MODE == 1 ? (i % 2) * bs : 0), v);
+}
+
+#define NMK_TWIN_ATOMIC(OPNAME, SIGN, TNAME, T, MODE)                          \
+  NMK_KERNEL(256)                                                              \
+  nmk_twin_atomic_##OPNAME##_m##MODE##_##TNAME(                                \
+      const T *a, int64_t an, int64_t as, T *b, int64_t bn, int64_t bs,        \
+      int64_t gs0, int64_t gs1, int64_t gs2) {                                 \
+    atomicBody<T, MODE, SIGN>(a, as, b, bs, gs0, gs1, gs2);                    \
+  }
+#define NMK_TWIN_ATOMIC_ALL(TNAME, T)                                          \
+  NMK_TWIN_ATOMIC(add, 1, TNAME, T, 0)                                         \
+  NMK_TWIN_ATOMIC(sub, -1, TNAME, T, 0)                                        \
+  NMK_TWIN_ATOMIC(add, 1, TNAME, T, 1)                                         \
+  NMK_TWIN_ATOMIC(sub, -1, TNAME, T, 1)
+NMK_TWIN_ATOMIC_ALL(i32, int32_t)
+NMK_TWIN_ATOMIC_ALL(i64, int64_t)
+NMK_TWIN_ATOMIC_ALL(f32, float)
+NMK_TWIN_ATOMIC(add, 1, i32, int32_t, 2)
+NMK_TWIN_ATOMIC(sub, -1, i32, int32_t, 2)
+NMK_TWIN_ATOMIC(add, 1, i32, int32_t, 3)
+NMK_TWIN_ATOMIC(sub, -1, i32, int32_t, 3)
+
+// atomic.add(b, (i % 2, 0), a[i, j]) / (i % 2, j % 2)   (test_atomics_multidim)
+template <int FUNC>
+__device__ __forceinline__ void
+atomicMultidim(const int32_t *a, int64_t as0, int64_t as1, int32_t *b,
+               int64_t bs0, int64_t bs1, int64_t gs0, int64_t gs1,
+               int64_t gs2) {
+  Ids t = ids(gs0, gs1, gs2);
+  if (!t.inside)
+    return;
+  const int64_t i = t.g[0], j = t.g[1];
+  atomicAdd(b + (i % 2) * bs0 + (FUNC == 2 ? (j % 2) * bs1 : 0),
+            a[i * as0 + j * as1]);
+}
+NMK_KERNEL(256)
+nmk_twin_atomic_multidim1_i32(const int32_t *a, int64_t a0, int64_t a1,
+                              int64_t as0, int64_t as1, int32_t *b, int64_t b0,
+                              int64_t b1, int64_t bs0, int64_t bs1,
+                              int64_t gs0, int64_t gs1, int64_t gs2) {
+  atomicMultidim<1>(a, as0, as1, b, bs0, bs1, gs0, gs1, gs2);
+}
+NMK_KERNEL(256)
+nmk_twin_atomic_multidim2_i32(const int32_t *a, int64_t a0, int64_t a1,
+                              int64_t as0, int64_t as1, int32_t *b, int64_t b0,
+                              int64_t b1, int64_t bs0, int64_t bs1,
+                              int64_t gs0, int64_t gs1, int64_t gs2) {
+  atomicMultidim<2>(a, as0, as1, b, bs0, bs1, gs0, gs1, gs2);
+}
+
+// atomic.add(a, (i, j), c[i, j]); atomic.add(b, (i), c[i, j])
+// (test_atomics_different_dims, 928-955)
+NMK_KERNEL(256)
+nmk_twin_atomic_dims_i32(int32_t *a, int64_t a0, int64_t a1, int64_t as0,
+                         int64_t as1, int32_t *b, int64_t b0, int64_t bs0,
+                         const int32_t *c, int64_t c0, int64_t c1, int64_t cs0,
+                         int64_t cs1, int64_t gs0, int64_t gs1, int64_t gs2) {
+  Ids t = ids(gs0, gs1, gs2);
+  if (!t.inside)
+    return;
+  const int64_t i = t.g[0], j = t.g[1];
+  const int32_t v = c[i * cs0 + j * cs1];
+  atomicAdd(a + i * as0 + j * as1, v);
+  atomicAdd(b + i * bs0, v);
+}
+
+// v = a[i]; op(flags); b[i] = a[i]   (test_barrier_ops, 1074-1102)
+// isBarrier: barrier(flags) or mem_fence(flags); flags: 1 local, 2 global.
+NMK_KERNEL(256)
+nmk_twin_barrier_ops_i64(const int64_t *a, int64_t an, int64_t as, int64_t *b,
+                         int64_t bn, int64_t bs, int64_t isBarrier,
+                         int64_t flags, int64_t gs0, int64_t gs1, int64_t gs2) {
+  Ids t = ids(gs0, gs1, gs2);
+  int64_t v = 0;
+  if (t.inside)
+    v = a[t.g[0] * as];
+  if (flags & 2)
+    __threadfence();
+  else
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+  if (isBarrier)
+    __syncthreads();
+  if (t.inside)
+    b[t.g[0] * bs] = v;
+}
+
+// off = i // local_size; atomic.add(a, off, i); barrier(GLOBAL_MEM_FENCE);
+// b[i] = a[off]   (test_barrier1, 1105-1133)
+NMK_KERNEL(256)
+nmk_twin_barrier1_i64(int64_t *a, int64_t an, int64_t as, int64_t *b,
+                      int64_t bn, int64_t bs, int64_t localSize, int64_t gs0,
+                      int64_t gs1, int64_t gs2) {
+  Ids t = ids(gs0, gs1, gs2);
+  const int64_t i = t.g[0];
+  const int64_t off = i / localSize;
+  if (t.inside)
+    atomicAddT(a + off * as, i);
+  __threadfence();
+  __syncthreads();
+  if (t.inside)
+    b[i * bs] = __hip_atomic_load(a + off * as, __ATOMIC_RELAXED,
+                                  __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// lm = local.array(blocksize, float32); lm[i] = A[i]; barrier(LOCAL);
+// A[i] += lm[blocksize - 1 - i]   (test_local_memory1/2, 1136-1198; one
+// work-group).  lmOffset: byte offset of lm in dynamic LDS.
+NMK_KERNEL(256)
+nmk_twin_local_memory_f32(float *A, int64_t an, int64_t as, int64_t blocksize,
+                          uint64_t lmOffset, int64_t gs0, int64_t gs1,
+                          int64_t gs2) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char ldsBase[];
+  float *lm = reinterpret_cast<float *>(ldsBase + lmOffset);
+  Ids t = ids(gs0, gs1, gs2);
+  const int64_t i = t.g[0];
+  if (t.inside)
+    lm[i] = A[i * as];
+  __syncthreads();
+  if (t.inside)
+    A[i * as] += lm[blocksize - 1 - i];
+}
+
+// Private arrays (test_private_memory1-4, 1202-1326).  VARIANT:
+//   1/2: p[0] = i; barrier; A[i] = p[0] * 2
+//   3  : p[j] = j + i for j < n; res = sum_j p[(j + i) % n]; A[i] = res
+//   4  : p[j][k] = i (10 x 10); barrier; A[i] = p[i % 10][i % 10] * 2
+NMK_KERNEL(256)
+nmk_twin_private_memory_f32(float *A, int64_t an, int64_t as, int64_t variant,
+                            int64_t privSize, int64_t gs0, int64_t gs1,
+                            int64_t gs2) {
+  Ids t = ids(gs0, gs1, gs2);
+  const int64_t i = t.g[0];
+  float p[100];
+  float res = 0.f;
+  if (variant == 3) {
+    for (int64_t j = 0; j < privSize; ++j)
+      p[j] = float(j + i);
+    // `res` starts as the integer 0 and becomes float32 on the first add
+    for (int64_t j = 0; j < privSize; ++j)
+      res += p[(j + i) % privSize];
+  } else if (variant == 4) {
+    for (int j = 0; j < 100; ++j)
+      p[j] = float(i);
+    __syncthreads();
+    res = p[(i % 10) * 10 + (i % 10)] * 2.f;
+  } else {
+    p[0] = float(i);
+    __syncthreads();
+    res = p[0] * 2.f;
+  }
+  if (t.inside)
+    A[i * as] = res;
+}
+
+// v = group.reduce_<op>(a[i]); b[i] = v   (test_group_func, 1360-1393)
+#define NMK_TWIN_GROUP(OPNAME, OP, TNAME, T, NEUTRAL)                          \
+  NMK_KERNEL(256)                                                              \
+  nmk_twin_group_reduce_##OPNAME##_##TNAME(const T *a, int64_t an, int64_t as, \
+                                           T *b, int64_t bn, int64_t bs,       \
+                                           int64_t gs0, int64_t gs1,           \
+                                           int64_t gs2) {                      \
+    Ids t = ids(gs0, gs1, gs2);                                                \
+    T v = t.inside ? a[t.g[0] * as] : T(NEUTRAL);                              \
+    v = groupReduce<T>(v, T(NEUTRAL), t.inside, OP());                         \
+    if (t.inside)                                                              \
+      b[t.g[0] * bs] = v;                                                      \
+  }
+#define NMK_TWIN_GROUP_ALL(TNAME, T, TMIN, TMAX)                               \
+  NMK_TWIN_GROUP(add, AddOp, TNAME, T, 0)                                      \
+  NMK_TWIN_GROUP(mul, MulOp, TNAME, T, 1)                                      \
+  NMK_TWIN_GROUP(min, MinOp, TNAME, T, TMAX)                                   \
+  NMK_TWIN_GROUP(max, MaxOp, TNAME, T, TMIN)
+NMK_TWIN_GROUP_ALL(i32, int32_t, INT32_MIN, INT32_MAX)
+NMK_TWIN_GROUP_ALL(i64, int64_t, INT64_MIN, INT64_MAX)
+NMK_TWIN_GROUP_ALL(f32, float, -__builtin_inff(), __builtin_inff())
+
+// c[i] = a[i] <op> b[i] with Python semantics (test_gpu_ops_binary, 551-566):
+// `/` is true division (the result is converted back to the array dtype),
+// `//` floors, `%` takes the sign of the divisor, `**` is pow.
+namespace {
+template <typename T> struct PyOps {
+  __device__ static T floordiv(T a, T b) { return T(floor(double(a) / double(b))); }
+  __device__ static T mod(T a, T b) {
+    T r = T(fmod(double(a), double(b)));
+    return (r != T(0) && ((r < T(0)) != (b < T(0)))) ? r + b : r;
+  }
+  __device__ static T truediv(T a, T b) { return a / b; }
+  __device__ static T power(T a, T b) { return T(pow(double(a), double(b))); }
+};
+template <> struct PyOps<int32_t> {
+  __device__ static int32_t floordiv(int32_t a, int32_t b) {
+    int32_t q = a / b;
+    return ((a % b != 0) && ((a < 0) != (b < 0))) ? q - 1 : q;
+  }
+  __device__ static int32_t mod(int32_t a, int32_t b) {
+    int32_t r = a % b;
+    return (r != 0 && ((r < 0) != (b < 0))) ? r + b : r;
+  }
+  __device__ static int32_t truediv(int32_t a, int32_t b) {
+    return int32_t(double(a) / double(b));
+  }
+  __device__ static int32_t power(int32_t a, int32_t b) {
+    int64_t r = 1, base = a;
+    for (int32_t e = b; e > 0; e >>= 1) {
+      if (e & 1)
+        r *= base;
+      base *= base;
+    }
+    return int32_t(r);
+  }
+};
+} // namespace
+
+#define NMK_TWIN_BINARY(OPNAME, TNAME, T, EXPR)                                \
+  NMK_KERNEL(256)                                                              \
+  nmk_twin_binary_##OPNAME##_##TNAME(const T *a, int64_t an, int64_t as,       \
+                                     const T *b, int64_t bn, int64_t bs, T *c, \
+                                     int64_t cn, int64_t cs, int64_t gs0,      \
+                                     int64_t gs1, int64_t gs2) {               \
+    Ids t = ids(gs0, gs1, gs2);                                                \
+    if (t.inside) {                                                            \
+      const T x = a[t.g[0] * as], y = b[t.g[0] * bs];                          \
+      c[t.g[0] * cs] = EXPR;                                                   \
+    }                                                                          \
+  }
+#define NMK_TWIN_BINARY_ALL(TNAME, T)                                          \
+  NMK_TWIN_BINARY(add, TNAME, T, x + y)                                        \
+  NMK_TWIN_BINARY(sub, TNAME, T, x - y)                                        \
+  NMK_TWIN_BINARY(mul, TNAME, T, x *y)                                         \
+  NMK_TWIN_BINARY(truediv, TNAME, T, PyOps<T>::truediv(x, y))                  \
+  NMK_TWIN_BINARY(floordiv, TNAME, T, PyOps<T>::floordiv(x, y))                \
+  NMK_TWIN_BINARY(mod, TNAME, T, PyOps<T>::mod(x, y))                          \
+  NMK_TWIN_BINARY(pow, TNAME, T, PyOps<T>::power(x, y))
+NMK_TWIN_BINARY_ALL(i32, int32_t)
+NMK_TWIN_BINARY_ALL(f32, float)
+NMK_TWIN_BINARY_ALL(f64, double)

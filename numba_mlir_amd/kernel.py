@@ -5,10 +5,17 @@ from .mlir.kernel_impl import (
     GLOBAL_MEM_FENCE,
     LOCAL_MEM_FENCE,
     Kernel,
+    atomic,
+    barrier,
     get_global_id,
     get_global_size,
     get_group_id,
     get_local_id,
     get_local_size,
+    group,
     kernel,
+    kernel_func,
+    local,
+    mem_fence,
+    private,
 )

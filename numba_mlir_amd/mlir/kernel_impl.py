@@ -62,6 +62,66 @@ def get_local_size(axis):
     _stub_error()
 
 
+class Stub(object):
+    """Namespace of kernel-only functions; not instantiable (reference:
+    numba_mlir/numba_mlir/mlir/kernel_impl.py:252-260)."""
+
+    __slots__ = ()
+
+    def __new__(cls):
+        raise NotImplementedError("%s is not instantiable" % cls)
+
+
+def _stub(name, params):
+    exec(f"def {name}({params}): _stub_error()", globals())
+    return globals()[name]
+
+
+class atomic(Stub):
+    """``atomic.add(arr, idx, val)`` / ``atomic.sub`` (kernel_impl.py:263-322)."""
+
+    add = staticmethod(_stub("atomic_add", "arr, idx, val"))
+    sub = staticmethod(_stub("atomic_sub", "arr, idx, val"))
+
+
+def barrier(flags=None):
+    """Work-group barrier with LOCAL_MEM_FENCE / GLOBAL_MEM_FENCE
+    (kernel_impl.py:330-345)."""
+    _stub_error()
+
+
+def mem_fence(flags=None):
+    _stub_error()
+
+
+class local(Stub):
+    """``local.array(shape, dtype)``: work-group memory (kernel_impl.py:366-400)."""
+
+    array = staticmethod(_stub("local_array", "shape, dtype"))
+
+
+class private(Stub):
+    """``private.array(shape, dtype)``: per-work-item memory."""
+
+    array = staticmethod(_stub("private_array", "shape, dtype"))
+
+
+class group(Stub):
+    """Work-group reductions (kernel_impl.py:440-482)."""
+
+    reduce_add = staticmethod(_stub("group_reduce_add", "value"))
+    reduce_mul = staticmethod(_stub("group_reduce_mul", "value"))
+    reduce_min = staticmethod(_stub("group_reduce_min", "value"))
+    reduce_max = staticmethod(_stub("group_reduce_max", "value"))
+
+
+def kernel_func(func):
+    """Device function callable from kernels (``mlir_njit(mlir_force_inline=
+    True)`` in the reference, kernel_impl.py:209); a plain function here, the
+    twin inlines it by construction."""
+    return func
+
+
 def check_device_args(args):
     """All device arrays of a launch must share a queue."""
     ctx = None
@@ -95,6 +155,9 @@ class _ParamList:
         for s in arr.elem_strides:
             self._add(ctypes.c_int64(s), lowered.PARAM_INT64)
 
+    def add_local(self, nbytes):
+        self._slots.append((None, nbytes))
+
     def add_scalar(self, value):
         if isinstance(value, (bool, np.bool_)):
             self._add(ctypes.c_bool(bool(value)), lowered.PARAM_BOOL)
@@ -113,6 +176,11 @@ class _ParamList:
     def build(self):
         descs = (GPUParamDesc * (len(self._slots) + 1))()
         for i, (cvalue, ptype) in enumerate(self._slots):
+            if cvalue is None:     # workgroup memory: data == NULL, size = bytes
+                descs[i].data = None
+                descs[i].size = ptype
+                descs[i].type = lowered.PARAM_PTR
+                continue
             descs[i].data = ctypes.cast(ctypes.pointer(cvalue), ctypes.c_void_p)
             descs[i].size = ctypes.sizeof(cvalue)
             descs[i].type = ptype
@@ -126,6 +194,10 @@ class Kernel(KernelBase):
     def __init__(self, func, kwargs):
         super().__init__(func)
         self.twin = kwargs.get("twin")
+        # local.array sizes of the body in bytes: a list, or a callable
+        # (global_size, local_size) -> list.  Each becomes a workgroup-memory
+        # parameter after the user arguments (GpuRuntimeToLlvm.cpp:507-536).
+        self.local_bytes = kwargs.get("local_bytes", ())
         self.last_launch = None
 
     def _twin_name(self, args):
@@ -165,6 +237,11 @@ class Kernel(KernelBase):
                 params.add_array(a)
             else:
                 params.add_scalar(a)
+        local_bytes = self.local_bytes
+        if callable(local_bytes):
+            local_bytes = local_bytes(tuple(gsize3[:ndim]), tuple(block[:ndim]))
+        for nbytes in local_bytes:
+            params.add_local(int(nbytes))
         for g in gsize3:
             params.add_scalar(int(g))
         descs = params.build()

@@ -337,3 +337,101 @@ def test_kernel_sim_visits_every_item_once_in_group_order():
     # first group is ids {0,1} x {0,1} in row-major order
     assert order[:4] == [(0, 0), (0, 1), (1, 0), (1, 1)]
     assert len(order) == 15
+
+
+# -- kernel simulator: barriers, local/private arrays, group ops, atomics ------
+from numba_mlir_amd import kernel as _K  # stubs only; nothing here runs a GPU
+
+_STUBS = {
+    "get_global_id": _K.get_global_id, "get_local_id": _K.get_local_id,
+    "get_group_id": _K.get_group_id, "get_global_size": _K.get_global_size,
+    "get_local_size": _K.get_local_size, "barrier": _K.barrier,
+    "mem_fence": _K.mem_fence, "atomic_add": _K.atomic.add,
+    "atomic_sub": _K.atomic.sub, "local_array": _K.local.array,
+    "private_array": _K.private.array,
+    "group_reduce_add": _K.group.reduce_add, "group_reduce_mul": _K.group.reduce_mul,
+    "group_reduce_min": _K.group.reduce_min, "group_reduce_max": _K.group.reduce_max,
+}
+
+
+@pytest.mark.parametrize("blocksize", [1, 10, 17, 64])
+def test_kernel_sim_local_memory_and_barrier(blocksize):
+    local_array, barrier, gid = _K.local.array, _K.barrier, _K.get_global_id
+
+    def func(A):
+        lm = local_array(shape=blocksize, dtype=np.float32)
+        i = gid(0)
+        lm[i] = A[i]
+        barrier(_K.LOCAL_MEM_FENCE)
+        A[i] += lm[blocksize - 1 - i]
+
+    arr = np.arange(blocksize).astype(np.float32)
+    res = arr.copy()
+    kernel_sim(func, _STUBS)[blocksize, blocksize](res)
+    # closed form: i + (blocksize - 1 - i)
+    assert np.array_equal(res, np.full(blocksize, blocksize - 1, np.float32))
+
+
+@pytest.mark.parametrize("global_size,local_size", [(1, 1), (4, 2), (27, 7), (101, 33)])
+def test_kernel_sim_group_reduce_closed_form(global_size, local_size):
+    gid = _K.get_global_id
+    for name, fold in (("add", sum), ("max", max), ("min", min)):
+        op = getattr(_K.group, "reduce_" + name)
+
+        def func(a, b):
+            i = gid(0)
+            b[i] = op(a[i])
+
+        a = np.arange(global_size, dtype=np.int64)
+        b = np.zeros(global_size, np.int64)
+        kernel_sim(func, _STUBS)[(global_size,), (local_size,)](a, b)
+        expect = np.empty_like(b)
+        for start in range(0, global_size, local_size):
+            stop = min(start + local_size, global_size)
+            expect[start:stop] = fold(range(start, stop))
+        assert np.array_equal(b, expect)
+
+
+def test_kernel_sim_atomics_and_barrier_order():
+    atomic_add, atomic_sub, barrier, gid = _K.atomic.add, _K.atomic.sub, _K.barrier, _K.get_global_id
+
+    def func(a, b):
+        i = gid(0)
+        off = i // 7
+        atomic_add(a, off, i)
+        barrier(_K.GLOBAL_MEM_FENCE)
+        b[i] = a[off]
+
+    n = 27
+    a = np.zeros(4, np.int64)
+    b = np.zeros(n, np.int64)
+    kernel_sim(func, _STUBS)[n, 7](a, b)
+    groups = [sum(range(s, min(s + 7, n))) for s in range(0, n, 7)]
+    assert a.tolist() == groups
+    assert b.tolist() == [groups[i // 7] for i in range(n)]   # all adds land before reads
+
+    def func2(a, b):
+        i = gid(0)
+        atomic_sub(b, i % 2, a[i])
+
+    a = np.arange(1, 10, dtype=np.int32)
+    b = np.zeros(2, np.int32)
+    kernel_sim(func2, _STUBS)[a.shape, ()](a, b)
+    assert b.tolist() == [-(1 + 3 + 5 + 7 + 9), -(2 + 4 + 6 + 8)]
+
+
+def test_kernel_sim_private_arrays_are_per_item():
+    private_array, barrier, gid = _K.private.array, _K.barrier, _K.get_global_id
+
+    def func(A):
+        i = gid(0)
+        p = private_array(shape=(10, 10), dtype=np.float32)
+        for j in range(10):
+            for k in range(10):
+                p[j, k] = i
+        barrier(_K.LOCAL_MEM_FENCE)
+        A[i] = p[i % 10, i % 10] * 2
+
+    res = np.zeros(17, np.float32)
+    kernel_sim(func, _STUBS)[17, 17](res)
+    assert np.array_equal(res, 2 * np.arange(17, dtype=np.float32))
