@@ -106,14 +106,18 @@ def _check(got, a, b):
 
 
 @pytest.mark.parametrize("m,n,k", [(128, 128, 16), (256, 384, 512), (128, 256, 4096),
-                                   (1024, 1024, 1024), (384, 128, 48)])
+                                   (1024, 1024, 1024), (384, 128, 48),
+                                   (4096, 3072, 64), (3584, 3584, 16)])
 def test_mfma_kernel(env, m, n, k):
     hip, ops, orc, mrt = env
     rng = np.random.Generator(np.random.PCG64(1005))
     a = rng.standard_normal((m, k), dtype=np.float32)
     b = rng.standard_normal((k, n), dtype=np.float32)
     got = ops.dot(hip.asarray(a), hip.asarray(b)).asnumpy()
-    assert mrt.last_kernel().startswith("sgemm_mfma")
+    expect_kernel = "sgemm_mfma_256x256" if (m % 256 == 0 and n % 256 == 0 and
+                                             (m // 256) * (n // 256) >= 192) \
+        else "sgemm_mfma_128x128"
+    assert mrt.last_kernel() == expect_kernel
     _check(got, a, b)
     if m * n * k <= 1 << 27:
         # against the oracle's float32 contraction (k innermost)
