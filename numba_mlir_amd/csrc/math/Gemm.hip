@@ -41,8 +41,13 @@ void checkHip(hipError_t err, const char *what) {
 thread_local const char *lastKernel = "";
 
 // ---------------------------------------------------------------------------
-// C[M,N] = alpha * A[M,K] * B[K,N] + beta * C, all row-major with leading
-// dimensions lda/ldb/ldc, fp32 in, fp32 accumulate on the matrix cores.
+// C[M,N] = alpha * A[M,K] * B[K,N] + beta * C with C row-major (ldc), fp32 in,
+// fp32 accumulate on the matrix cores.  Each input operand may be stored with
+// either of its two dimensions contiguous:
+//   A_KC: A(m,k) = A[m * lda + k]   (row-major A)   else A[k * lda + m]
+//   B_NC: B(k,n) = B[k * ldb + n]   (row-major B)   else B[n * ldb + k]
+// which covers the four transpose cases of a BLAS gemm; a column-major C is
+// handled by the host as C^T = B^T A^T.
 //
 // 256 threads = 4 waves in a 2 x 2 grid; each wave owns TM x TN tiles of
 // v_mfma_f32_32x32x2_f32, so the block tile is (64 TM) x (64 TN) and a wave
@@ -50,10 +55,12 @@ thread_local const char *lastKernel = "";
 //
 // LDS holds both operands K-major ([k][m] and [k][n], rows padded by 4 floats)
 // so that the MFMA operand fetch -- lane l needs element (l % 32) of row
-// (k + l / 32) -- is a conflict-free ds_read_b32.  Two LDS stages: the next
-// K slab is fetched from global memory into registers before the MFMAs of the
-// current slab are issued and written to the other stage after them, one
-// barrier per slab.
+// (k + l / 32) -- is a conflict-free ds_read_b32.  Global fetches are float4
+// along the operand's contiguous dimension: an operand contiguous in m / n
+// is written to LDS as float4, one contiguous in k is scattered over four LDS
+// rows.  Two LDS stages: the next K slab is fetched from global memory into
+// registers before the MFMAs of the current slab are issued and written to
+// the other stage after them, one barrier per slab.
 //
 // MFMA 32x32x2 operand layout (64 lanes):
 //   A (32 x 2): lane l holds A[l % 32][l / 32]
@@ -64,7 +71,53 @@ thread_local const char *lastKernel = "";
 // K % 16 == 0, lda/ldb % 4 == 0, A and B 16-byte aligned.
 constexpr int BK = 16, PAD = 4;
 
-template <int TM, int TN>
+// One operand's slab of X x 16 (X = BM or BN) on its way from global memory
+// to LDS[stage][k][x].  T float4 per thread.
+template <int X, bool K_CONTIG> struct SlabFetch {
+  static constexpr int T = X / 64;
+  // K_CONTIG: thread -> (x = tid / 4 + 64 i, k = 4 (tid % 4) .. +3)
+  // else    : thread -> (k = tid / (X / 4) + (1024 / X) i, x = 4 (tid % (X/4)) .. +3)
+  static constexpr int K_ROWS = 1024 / X;
+  int x, k;
+  const float *base;
+  int64_t ld;
+  floatx4 reg[T];
+
+  __device__ __forceinline__ void init(const float *p, int64_t ld_, int origin,
+                                       int tid) {
+    ld = ld_;
+    if (K_CONTIG) {
+      x = tid / 4;
+      k = (tid % 4) * 4;
+      base = p + int64_t(origin + x) * ld + k;
+    } else {
+      k = tid / (X / 4);
+      x = (tid % (X / 4)) * 4;
+      base = p + int64_t(k) * ld + origin + x;
+    }
+  }
+  __device__ __forceinline__ void fetch(int k0) {
+#pragma unroll
+    for (int i = 0; i < T; ++i)
+      reg[i] = *reinterpret_cast<const floatx4 *>(
+          K_CONTIG ? base + int64_t(64 * i) * ld + k0
+                   : base + int64_t(k0 + K_ROWS * i) * ld);
+  }
+  __device__ __forceinline__ void stash(float (*lds)[X + PAD]) const {
+#pragma unroll
+    for (int i = 0; i < T; ++i) {
+      if (K_CONTIG) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          lds[k + q][x + 64 * i] = reg[i][q];
+      } else {
+        *reinterpret_cast<floatx4 *>(&lds[k + K_ROWS * i][x]) = reg[i];
+      }
+    }
+  }
+};
+
+template <int TM, int TN, bool A_KC, bool B_NC>
 __global__ __launch_bounds__(256) void
 sgemm_mfma(const float *__restrict__ A, const float *__restrict__ B,
            float *__restrict__ C, int M, int N, int K, int64_t lda, int64_t ldb,
@@ -80,36 +133,10 @@ sgemm_mfma(const float *__restrict__ A, const float *__restrict__ B,
   const int bm = blockIdx.y * BM;
   const int bn = blockIdx.x * BN;
 
-  // Global fetch mapping (float4 = 4 consecutive k of A / 4 consecutive n of
-  // B): A slab BM x 16: a pass of the block covers 64 rows, TM passes;
-  // B slab 16 x BN: a pass covers 1024 / BN k-rows, BN / 64 = TN passes.
-  constexpr int B_ROWS = 1024 / BN;
-  const int aRow = tid / 4, aK = (tid % 4) * 4;
-  const int bK = tid / (BN / 4), bN = (tid % (BN / 4)) * 4;
-  const float *aPtr = A + int64_t(bm + aRow) * lda + aK;
-  const float *bPtr = B + int64_t(bK) * ldb + bn + bN;
-
-  floatx4 aReg[TM], bReg[TN];
-  auto fetch = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-      aReg[i] =
-          *reinterpret_cast<const floatx4 *>(aPtr + int64_t(64 * i) * lda + k0);
-#pragma unroll
-    for (int i = 0; i < TN; ++i)
-      bReg[i] = *reinterpret_cast<const floatx4 *>(
-          bPtr + int64_t(k0 + B_ROWS * i) * ldb);
-  };
-  auto stash = [&](int stage) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        As[stage][aK + q][aRow + 64 * i] = aReg[i][q];
-#pragma unroll
-    for (int i = 0; i < TN; ++i)
-      *reinterpret_cast<floatx4 *>(&Bs[stage][bK + B_ROWS * i][bN]) = bReg[i];
-  };
+  SlabFetch<BM, A_KC> fa;
+  SlabFetch<BN, !B_NC> fb;
+  fa.init(A, lda, bm, tid);
+  fb.init(B, ldb, bn, tid);
 
   floatx16 acc[TM][TN];
 #pragma unroll
@@ -120,16 +147,20 @@ sgemm_mfma(const float *__restrict__ A, const float *__restrict__ B,
       for (int r = 0; r < 16; ++r)
         acc[i][j][r] = 0.f;
 
-  fetch(0);
-  stash(0);
+  fa.fetch(0);
+  fb.fetch(0);
+  fa.stash(As[0]);
+  fb.stash(Bs[0]);
   __syncthreads();
 
   const int nSlabs = K / BK;
   const int kLane = lane / 32, xLane = lane % 32;
   for (int s = 0; s < nSlabs; ++s) {
     const int cur = s & 1;
-    if (s + 1 < nSlabs)
-      fetch((s + 1) * BK);
+    if (s + 1 < nSlabs) {
+      fa.fetch((s + 1) * BK);
+      fb.fetch((s + 1) * BK);
+    }
 #pragma unroll
     for (int kk = 0; kk < BK; kk += 2) {
       float a[TM], b[TN];
@@ -146,8 +177,10 @@ sgemm_mfma(const float *__restrict__ A, const float *__restrict__ B,
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j],
                                                            acc[i][j], 0, 0, 0);
     }
-    if (s + 1 < nSlabs)
-      stash(cur ^ 1);
+    if (s + 1 < nSlabs) {
+      fa.stash(As[cur ^ 1]);
+      fb.stash(Bs[cur ^ 1]);
+    }
     __syncthreads();
   }
 
@@ -278,32 +311,58 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
   if (M > 0 && N > 0) {
     bool launched = false;
     if constexpr (sizeof(T) == 4) {
-      const bool rowMajor = a->strides[1] == 1 && b->strides[1] == 1 &&
-                            c->strides[1] == 1;
+      // Operands as the kernel sees them: X(m,k), Y(k,n), Z row-major.  A
+      // column-major C is computed as C^T = B^T A^T (swap and transpose the
+      // inputs); which dimension of each input is contiguous follows from
+      // its unit stride (NumpyLinalg.cpp:87-102).
+      const bool cRow = c->strides[1] == 1;
+      const float *X = cRow ? aData : bData;
+      const float *Y = cRow ? bData : aData;
+      // strides of X over (m, k) and Y over (k, n)
+      const int64_t xm = cRow ? a->strides[0] : b->strides[1];
+      const int64_t xk = cRow ? a->strides[1] : b->strides[0];
+      const int64_t yk = cRow ? b->strides[0] : a->strides[1];
+      const int64_t yn = cRow ? b->strides[1] : a->strides[0];
+      const int64_t Mz = cRow ? M : N, Nz = cRow ? N : M;
+      const int64_t ldz = cRow ? c->strides[0] : c->strides[1];
+      const bool xKc = xk == 1, yNc = yn == 1;
+      const int64_t ldx = xKc ? xm : xk, ldy = yNc ? yk : yn;
       // 256 x 256 block tiles (one block per CU on a 4096^2 problem) when the
       // shape allows and there are enough tiles to fill the 256 CUs; 128 x
       // 128 otherwise.  Measured within 3 % of each other; the larger tile
       // halves the operand traffic.
-      const bool big = M % 256 == 0 && N % 256 == 0 &&
-                       (M / 256) * (N / 256) >= 192;
+      const bool big = Mz % 256 == 0 && Nz % 256 == 0 &&
+                       (Mz / 256) * (Nz / 256) >= 192;
       const int BM = big ? 256 : 128, BN = BM;
-      if (rowMajor && K > 0 && M % BM == 0 && N % BN == 0 && K % BK == 0 &&
-          a->strides[0] % 4 == 0 && b->strides[0] % 4 == 0 &&
-          aligned16(aData) && aligned16(bData) && M <= 0x7fffffff &&
-          N <= 0x7fffffff && K <= 0x7fffffff && M / BM <= 65535) {
-        dim3 grid(unsigned(N / BN), unsigned(M / BM), 1);
-#define NMHIP_SGEMM_LAUNCH(TM, TN)                                             \
-  hipLaunchKernelGGL((sgemm_mfma<TM, TN>), grid, dim3(256), 0, stream, aData,  \
-                     bData, cData, int(M), int(N), int(K),                     \
-                     int64_t(a->strides[0]), int64_t(b->strides[0]),           \
-                     int64_t(c->strides[0]), alpha, beta)
+      const bool unitOk = (xk == 1 || xm == 1) && (yk == 1 || yn == 1);
+      if (unitOk && K > 0 && Mz % BM == 0 && Nz % BN == 0 && K % BK == 0 &&
+          ldx % 4 == 0 && ldy % 4 == 0 && ldx > 0 && ldy > 0 && aligned16(X) &&
+          aligned16(Y) && M <= 0x7fffffff && N <= 0x7fffffff &&
+          K <= 0x7fffffff && Mz / BM <= 65535) {
+        dim3 grid(unsigned(Nz / BN), unsigned(Mz / BM), 1);
+#define NMHIP_SGEMM_LAUNCH(TM, TN, XKC, YNC)                                   \
+  hipLaunchKernelGGL((sgemm_mfma<TM, TN, XKC, YNC>), grid, dim3(256), 0,       \
+                     stream, X, Y, cData, int(Mz), int(Nz), int(K), ldx, ldy,  \
+                     ldz, alpha, beta)
+#define NMHIP_SGEMM_LAYOUTS(TM, TN)                                            \
+  do {                                                                         \
+    if (xKc && yNc)                                                            \
+      NMHIP_SGEMM_LAUNCH(TM, TN, true, true);                                  \
+    else if (xKc)                                                              \
+      NMHIP_SGEMM_LAUNCH(TM, TN, true, false);                                 \
+    else if (yNc)                                                              \
+      NMHIP_SGEMM_LAUNCH(TM, TN, false, true);                                 \
+    else                                                                       \
+      NMHIP_SGEMM_LAUNCH(TM, TN, false, false);                                \
+  } while (0)
         if (big) {
-          NMHIP_SGEMM_LAUNCH(4, 4);
+          NMHIP_SGEMM_LAYOUTS(4, 4);
           lastKernel = "sgemm_mfma_256x256";
         } else {
-          NMHIP_SGEMM_LAUNCH(2, 2);
+          NMHIP_SGEMM_LAYOUTS(2, 2);
           lastKernel = "sgemm_mfma_128x128";
         }
+#undef NMHIP_SGEMM_LAYOUTS
 #undef NMHIP_SGEMM_LAUNCH
         launched = true;
       }

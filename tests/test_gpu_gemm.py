@@ -79,7 +79,8 @@ def test_internal_gemm_fixture_grid(env):
 
 
 @pytest.mark.parametrize("ta,tb,tc", list(itertools.product([False, True], repeat=3)))
-@pytest.mark.parametrize("m,n,k", [(33, 29, 47), (128, 128, 16), (1, 1, 1), (64, 1, 300)])
+@pytest.mark.parametrize("m,n,k", [(33, 29, 47), (128, 128, 16), (1, 1, 1), (64, 1, 300),
+                                   (256, 384, 64), (4096, 3072, 32)])
 def test_layouts_against_float64(env, ta, tb, tc, m, n, k):
     """Every stride pattern the entry point accepts (row/column major A, B, C)."""
     hip, ops, orc, mrt = env
@@ -91,6 +92,11 @@ def test_layouts_against_float64(env, ta, tb, tc, m, n, k):
     d_c = _to_dev(hip, lay(c0, tc))
     ops.gemm(_to_dev(hip, lay(a, ta)), _to_dev(hip, lay(b, tb)), d_c, 0.5, 2.0)
     got = d_c.asnumpy()
+    if m % 128 == 0 and n % 128 == 0 and k % 16 == 0:
+        # every layout of a tile-aligned problem runs on the matrix cores
+        assert mrt.last_kernel().startswith("sgemm_mfma")
+    else:
+        assert mrt.last_kernel() == "sgemm_generic"
     truth = 2.0 * c0 + 0.5 * (a.astype(np.float64) @ b.astype(np.float64))
     bound = 1e-5 * (2.0 * np.abs(c0) + 0.5 * (np.abs(a).astype(np.float64) @ np.abs(b))) + 1e-30
     assert (np.abs(got - truth) <= bound).all()
