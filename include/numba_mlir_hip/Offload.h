@@ -135,6 +135,11 @@ void nmhipBlackScholesF32(void *ctx, const float *price, const float *strike,
 void nmhipReduce(void *ctx, int op, int dtype, const void *x, int64_t n0,
                  int64_t n1, int64_t s0, int64_t s1, int axis, void *out);
 
+/* out[r] = sqrt(sum_c x[r, c]^2) for a row-major float32 [n0, n1] array with
+ * row stride s0: np.sqrt(np.square(a).sum(axis=1)) fused into one kernel. */
+void nmhipNorm2RowsF32(void *ctx, const float *x, int64_t n0, int64_t n1,
+                       int64_t s0, float *out);
+
 /* out[0] = sqrt(sum(x * x)) over n contiguous float32. */
 void nmhipNorm2F32(void *ctx, const float *x, int64_t n, float *out);
 

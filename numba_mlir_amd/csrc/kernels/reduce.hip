@@ -21,13 +21,16 @@
 using namespace nmk;
 
 // ---------------------------------------------------------------------------
-// out[r] = sum_c x[r * ld + c], float32.  One wave per row, four rows per
-// block.  When ld and cols are multiples of 4 and x is 16-byte aligned
-// (vec != 0) lanes read float4, four loads in flight; lane partials are
-// folded pairwise, then a wave butterfly.
-NMK_KERNEL(256)
-nmk_sum_axis1_f32(const float *__restrict__ x, float *__restrict__ out,
-                  int64_t rows, int64_t cols, int64_t ld, int32_t vec) {
+// out[r] = sum_c x[r * ld + c], float32 (NORM == false), or the fused row
+// norm out[r] = sqrt(sum_c x[r,c]^2) (NORM == true: np.sqrt(np.square(a).sum(
+// axis=1)), the reference's test_l2_norm, tests/test_gpu.py:2198-2223).
+// One wave per row, four rows per block.  When ld and cols are multiples of 4
+// and x is 16-byte aligned (vec != 0) lanes read float4, four loads in
+// flight; lane partials are folded pairwise, then a wave butterfly.
+template <bool NORM>
+__device__ __forceinline__ void
+rowSumF32(const float *__restrict__ x, float *__restrict__ out, int64_t rows,
+          int64_t cols, int64_t ld, int32_t vec) {
   const int lane = threadIdx.x % NMK_WAVE;
   const int64_t row =
       int64_t(blockIdx.x) * (blockDim.x / NMK_WAVE) + threadIdx.x / NMK_WAVE;
@@ -45,23 +48,47 @@ nmk_sum_axis1_f32(const float *__restrict__ x, float *__restrict__ out,
       float4_t v1 = streamLoad(pv + i + NMK_WAVE);
       float4_t v2 = streamLoad(pv + i + 2 * NMK_WAVE);
       float4_t v3 = streamLoad(pv + i + 3 * NMK_WAVE);
+      if (NORM) {
+        v0 *= v0;
+        v1 *= v1;
+        v2 *= v2;
+        v3 *= v3;
+      }
       a0 += v0;
       a1 += v1;
       a2 += v2;
       a3 += v3;
     }
-    for (; i < nvec; i += NMK_WAVE)
-      a0 += pv[i];
+    for (; i < nvec; i += NMK_WAVE) {
+      float4_t v0 = pv[i];
+      if (NORM)
+        v0 *= v0;
+      a0 += v0;
+    }
     float4_t a = (a0 + a1) + (a2 + a3);
     total = (a[0] + a[1]) + (a[2] + a[3]);
   } else {
     total = 0.f;
-    for (int64_t i = lane; i < cols; i += NMK_WAVE)
-      total += p[i];
+    for (int64_t i = lane; i < cols; i += NMK_WAVE) {
+      const float v = p[i];
+      total += NORM ? v * v : v;
+    }
   }
   total = waveAllReduce(total, AddOp());
   if (lane == 0)
-    out[row] = total;
+    out[row] = NORM ? sqrtf(total) : total;
+}
+
+NMK_KERNEL(256)
+nmk_sum_axis1_f32(const float *x, float *out, int64_t rows, int64_t cols,
+                  int64_t ld, int32_t vec) {
+  rowSumF32<false>(x, out, rows, cols, ld, vec);
+}
+
+NMK_KERNEL(256)
+nmk_norm2_axis1_f32(const float *x, float *out, int64_t rows, int64_t cols,
+                    int64_t ld, int32_t vec) {
+  rowSumF32<true>(x, out, rows, cols, ld, vec);
 }
 
 // ---------------------------------------------------------------------------

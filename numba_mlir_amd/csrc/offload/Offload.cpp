@@ -717,6 +717,22 @@ NMHIP_EXPORT void nmhipReduce(void *ctx, int op, int dtype, const void *x,
   });
 }
 
+NMHIP_EXPORT void nmhipNorm2RowsF32(void *ctx, const float *x, int64_t n0,
+                                    int64_t n1, int64_t s0, float *out) {
+  guarded([&]() {
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    if (n0 < 0 || n1 < 0 || (n0 > 1 && s0 < n1))
+      fail("nmhipNorm2RowsF32: needs a row-major array");
+    if (n0 == 0)
+      return;
+    const int vec = (aligned16(x) && s0 % 4 == 0 && n1 % 4 == 0) ? 1 : 0;
+    c->launch("nmk_norm2_axis1_f32", size_t(ceilDiv(n0, 4)), 1, 1, 256, 1, 1,
+              {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(n0), Arg::I64(n1),
+               Arg::I64(s0), Arg::I32(vec)});
+  });
+}
+
 NMHIP_EXPORT void nmhipNorm2F32(void *ctx, const float *x, int64_t n,
                                 float *out) {
   guarded([&]() {

@@ -40,6 +40,7 @@ _SIGNATURES = {
     "nmhipReduce": (None, [_vp, ctypes.c_int, ctypes.c_int, _vp, _i64, _i64, _i64,
                            _i64, ctypes.c_int, _vp]),
     "nmhipNorm2F32": (None, [_vp, _vp, _i64, _vp]),
+    "nmhipNorm2RowsF32": (None, [_vp, _vp, _i64, _i64, _i64, _vp]),
     "nmhipGemm": (None, [_vp, ctypes.c_int, _vp, _i64x2, _vp, _i64x2, _vp, _i64x2,
                          _i64, _i64, _i64, ctypes.c_double, ctypes.c_double]),
     "nmhipSuggestBlockSize": (None, [_vp, ctypes.c_char_p,

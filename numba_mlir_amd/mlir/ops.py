@@ -175,6 +175,22 @@ def sqrt_sum_squares(x, out=None):
     return out
 
 
+def l2_norm_rows(a, out=None):
+    """``np.sqrt(np.square(a).sum(axis=1))`` of a row-major float32 matrix,
+    fused (the body of the reference's ``test_l2_norm``,
+    numba_mlir/numba_mlir/mlir/tests/test_gpu.py:2198-2223)."""
+    a = asarray(a)
+    if a.dtype != np.float32 or a.ndim != 2 or (a.shape[1] > 1 and
+                                                a.elem_strides[1] != 1):
+        raise ValueError("l2_norm_rows needs a row-major float32 matrix")
+    if out is None:
+        out = empty((a.shape[0],), np.float32, usm_type=a.usm_type,
+                    device=a.ctx.device)
+    lib.nmhipNorm2RowsF32(a.ctx.handle, a.ptr, a.shape[0], a.shape[1],
+                          a.elem_strides[0], out.ptr)
+    return out
+
+
 def gemm(a, b, c, alpha, beta):
     """``c[:] = beta * c + alpha * np.dot(a, b)`` through
     ``mkl_gemm_<dtype>_device`` (reference: numpy/funcs.py:866-876)."""
