@@ -175,8 +175,20 @@ int parseDeviceOrdinal(const std::string &name) {
   return ordinal;
 }
 
+class Queue;
+
+// What gpuxLaunchKernel / gpuxAlloc hand out.  A queue is one in-order
+// stream, so an event is just a position in that stream: the ticket of the
+// launch it follows.  Nothing is recorded on the device for it -- a marker
+// packet after every kernel costs several microseconds of idle GPU between
+// back-to-back launches -- until another queue has to wait for it, which
+// records a real hipEvent_t at the stream's current tail (a later, hence
+// sufficient, position).
 struct Event {
-  hipEvent_t event = nullptr;
+  Queue *owner = nullptr;
+  uint64_t ticket = 0;          // launches enqueued on owner up to this one
+  hipEvent_t event = nullptr;   // created on first cross-queue use, then kept
+  bool recorded = false;        // event holds a record covering `ticket`
   Event *next = nullptr;
 };
 
@@ -240,7 +252,8 @@ public:
     while (freeList) {
       Event *ev = freeList;
       freeList = ev->next;
-      (void)hipApi().eventDestroy(ev->event);
+      if (ev->event)
+        (void)hipApi().eventDestroy(ev->event);
       delete ev;
     }
     if (stream)
@@ -374,15 +387,32 @@ public:
                 stream, args.data(), nullptr),
             "hipModuleLaunchKernel");
     }
-    check(hipApi().eventRecord(ev->event, stream), "hipEventRecord");
+    ev->ticket = enqueued.fetch_add(1, std::memory_order_acq_rel) + 1;
     return ev;
   }
 
-  void wait(Event *ev) {
+  // Host wait.  Events of this queue are stream positions: if the position
+  // is not known to be complete yet, drain the stream (which also completes
+  // everything enqueued before the call) and remember how far that got.
+  void waitHost(Event *ev) {
     if (!ev)
       fail("Invalid event");
-    check(hipApi().eventSynchronize(ev->event), "hipEventSynchronize");
+    if (ev->owner != this) {
+      ev->owner->waitHost(ev);
+      return;
+    }
+    if (completed.load(std::memory_order_acquire) >= ev->ticket)
+      return;
+    const uint64_t upTo = enqueued.load(std::memory_order_acquire);
+    makeCurrent();
+    check(hipApi().streamSynchronize(stream), "hipStreamSynchronize");
+    uint64_t seen = completed.load(std::memory_order_relaxed);
+    while (seen < upTo && !completed.compare_exchange_weak(
+                              seen, upTo, std::memory_order_release)) {
+    }
   }
+
+  void wait(Event *ev) { waitHost(ev); }
 
   void destroyEvent(Event *ev) {
     if (!ev)
@@ -402,7 +432,7 @@ public:
     // Allocation is synchronous: wait for the dependencies on the host
     // (GpuRuntime.cpp:218-224).
     for (Event **d = deps; *d; ++d)
-      check(hipApi().eventSynchronize((*d)->event), "hipEventSynchronize");
+      waitHost(*d);
     if (alignment > 256 && type != GPUX_ALLOC_LOCAL)
       fail("gpuxAlloc: alignment %zu above the 256 bytes HIP guarantees",
            alignment);
@@ -435,9 +465,11 @@ public:
     if (ptr)
       allocRegistry().add(ptr, type);
 
+    // The allocation is synchronous, so its event is complete already
+    // (position 0), as the reference's default-constructed event is
+    // (GpuRuntime.cpp:226, 251).
     Event *ev = getEvent();
-    // Complete as soon as prior work of the (otherwise idle) stream is.
-    check(hipApi().eventRecord(ev->event, stream), "hipEventRecord");
+    ev->ticket = 0;
     retain(); // until gpuxDeAlloc (GpuRuntime.cpp:248-251)
     return {ptr, ev};
   }
@@ -489,11 +521,33 @@ private:
   hipStream_t stream = nullptr;
   std::mutex poolMutex;
   Event *freeList = nullptr;
+  std::atomic<uint64_t> enqueued{0};  // launches put on the stream so far
+  std::atomic<uint64_t> completed{0}; // launches known to have finished
 
+  // Makes this queue's stream wait for the dependencies.  Events of this
+  // queue are earlier positions of the same in-order stream: nothing to do.
   void waitOnStream(Event **deps) {
-    for (Event **d = deps; *d; ++d)
-      check(hipApi().streamWaitEvent(stream, (*d)->event, 0),
+    for (Event **d = deps; *d; ++d) {
+      Event *dep = *d;
+      if (dep->owner == this)
+        continue;
+      dep->owner->recordForOthers(dep);
+      check(hipApi().streamWaitEvent(stream, dep->event, 0),
             "hipStreamWaitEvent");
+    }
+  }
+
+  // Gives `ev` a real device event other streams can wait on.
+  void recordForOthers(Event *ev) {
+    std::lock_guard<std::mutex> lock(poolMutex);
+    if (ev->recorded)
+      return;
+    check(hipApi().setDevice(device), "hipSetDevice");
+    if (!ev->event)
+      check(hipApi().eventCreateWithFlags(&ev->event, hipEventDisableTiming),
+            "hipEventCreateWithFlags");
+    check(hipApi().eventRecord(ev->event, stream), "hipEventRecord");
+    ev->recorded = true;
   }
 
   Event *getEvent() {
@@ -506,15 +560,10 @@ private:
         ev->next = nullptr;
       }
     }
-    if (!ev) {
+    if (!ev)
       ev = new Event;
-      hipError_t err =
-          hipApi().eventCreateWithFlags(&ev->event, hipEventDisableTiming);
-      if (err != hipSuccess) {
-        delete ev;
-        check(err, "hipEventCreateWithFlags");
-      }
-    }
+    ev->owner = this;
+    ev->recorded = false;
     retain(); // until gpuxDestroyEvent (GpuRuntime.cpp:287-299)
     return ev;
   }

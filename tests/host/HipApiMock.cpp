@@ -29,7 +29,7 @@ struct State {
   int currentDevice = -1;
   long streamsCreated = 0, streamsDestroyed = 0;
   long eventsCreated = 0, eventsDestroyed = 0;
-  long eventRecords = 0, eventSyncs = 0, streamWaits = 0;
+  long eventRecords = 0, eventSyncs = 0, streamWaits = 0, streamSyncs = 0;
   long launches = 0;
   long modulesLoaded = 0, modulesUnloaded = 0;
   int expectParams = 0;
@@ -77,7 +77,11 @@ hipError_t mStreamWaitEvent(hipStream_t, hipEvent_t, unsigned) {
   ++st().streamWaits;
   return hipSuccess;
 }
-hipError_t mStreamSync(hipStream_t) { return hipSuccess; }
+hipError_t mStreamSync(hipStream_t) {
+  std::lock_guard<std::mutex> l(st().mutex);
+  ++st().streamSyncs;
+  return hipSuccess;
+}
 hipError_t mEventCreate(hipEvent_t *e, unsigned) {
   std::lock_guard<std::mutex> l(st().mutex);
   ++st().eventsCreated;
@@ -207,6 +211,7 @@ MOCK_EXPORT long mockCounter(const char *name) {
   if (n == "event_records") return s.eventRecords;
   if (n == "event_syncs") return s.eventSyncs;
   if (n == "stream_waits") return s.streamWaits;
+  if (n == "stream_syncs") return s.streamSyncs;
   if (n == "launches") return s.launches;
   if (n == "allocs_live") return long(s.allocs.size());
   if (n == "frees_device") return s.freesDevice;

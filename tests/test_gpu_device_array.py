@@ -47,7 +47,7 @@ def test_default_device_caps(env):
 def test_buffers_are_released(env):
     hip, _ = env
     import gc
-    for _ in range(400):                 # 400 x 256 MiB = 100 GiB: only fits if freed
+    for _ in range(1500):                # 1500 x 256 MiB = 375 GiB > HBM: only fits if freed
         x = hip.empty((1 << 28,), np.uint8)   # released through gpuxDeAlloc
         del x
     gc.collect()

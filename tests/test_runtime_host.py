@@ -155,34 +155,90 @@ def test_workgroup_memory_params_become_offsets(rt, qk):
 
 @pytest.mark.parametrize("ndeps", [0, 1, 5])
 def test_dependency_arrays_are_null_terminated(rt, qk, ndeps):
+    """Dependencies from another queue become stream waits on recorded events;
+    the array is scanned up to its NULL terminator."""
+    q, _, k = qk
+    q2 = rt.gpuxQueueCreate(b"gpu:1")
+    m2 = rt.gpuxModuleLoad(q2, ELF, len(ELF))
+    k2 = rt.gpuxKernelGet(m2, b"kern")
+    descs, _ = make_params([])
+    rt.mockExpectParams(0)
+    evs = [rt.gpuxLaunchKernel(q2, k2, 1, 1, 1, 1, 1, 1, NO_DEPS, descs)
+           for _ in range(ndeps)]
+    deps = (ctypes.c_void_p * (ndeps + 1))(*evs, None)
+    before = counter(rt, "stream_waits"), counter(rt, "event_records")
+    ev = rt.gpuxLaunchKernel(q, k, 1, 1, 1, 1, 1, 1, deps, descs)
+    assert counter(rt, "stream_waits") - before[0] == ndeps
+    assert counter(rt, "event_records") - before[1] == ndeps
+    # using the same dependencies again re-uses their records
+    ev2 = rt.gpuxLaunchKernel(q, k, 1, 1, 1, 1, 1, 1, deps, descs)
+    assert counter(rt, "event_records") - before[1] == ndeps
+    # allocation waits for its dependencies on the host: one drain of the
+    # other queue's stream covers them all
+    before = counter(rt, "stream_syncs")
+    res = AllocResult()
+    rt.gpuxAlloc(q, 64, 64, 0, deps, ctypes.byref(res))
+    assert counter(rt, "stream_syncs") - before == (1 if ndeps else 0)
+    rt.gpuxDeAlloc(q, res.ptr)
+    for e in [ev, ev2, res.event]:
+        rt.gpuxDestroyEvent(q, e)
+    for e in evs:
+        rt.gpuxDestroyEvent(q2, e)
+    rt.gpuxKernelDestroy(k2)
+    rt.gpuxModuleDestroy(m2)
+    rt.gpuxQueueDestroy(q2)
+
+
+def test_same_queue_events_are_stream_positions(rt, qk):
+    """A queue is one in-order stream: its own events need no device marker,
+    no stream wait, and one drain completes every earlier position."""
     q, _, k = qk
     descs, _ = make_params([])
     rt.mockExpectParams(0)
-    evs = [rt.gpuxLaunchKernel(q, k, 1, 1, 1, 1, 1, 1, NO_DEPS, descs)
-           for _ in range(ndeps)]
-    deps = (ctypes.c_void_p * (ndeps + 1))(*evs, None)
-    before = counter(rt, "stream_waits")
-    ev = rt.gpuxLaunchKernel(q, k, 1, 1, 1, 1, 1, 1, deps, descs)
-    assert counter(rt, "stream_waits") - before == ndeps
-    # allocation waits for its dependencies on the host
-    before = counter(rt, "event_syncs")
-    res = AllocResult()
-    rt.gpuxAlloc(q, 64, 64, 0, deps, ctypes.byref(res))
-    assert counter(rt, "event_syncs") - before == ndeps
-    rt.gpuxDeAlloc(q, res.ptr)
-    for e in evs + [ev, res.event]:
+    base = {n: counter(rt, n) for n in ("event_records", "stream_waits",
+                                        "stream_syncs", "events_created")}
+    evs = []
+    for _ in range(4):
+        deps = (ctypes.c_void_p * 2)(evs[-1], None) if evs else NO_DEPS
+        evs.append(rt.gpuxLaunchKernel(q, k, 1, 1, 1, 1, 1, 1, deps, descs))
+    assert counter(rt, "event_records") == base["event_records"]
+    assert counter(rt, "stream_waits") == base["stream_waits"]
+    assert counter(rt, "events_created") == base["events_created"]
+    rt.gpuxWait(q, evs[-1])                       # drains the stream once
+    assert counter(rt, "stream_syncs") == base["stream_syncs"] + 1
+    for e in evs[:-1]:                            # earlier positions: known done
+        rt.gpuxWait(q, e)
+    assert counter(rt, "stream_syncs") == base["stream_syncs"] + 1
+    ev = rt.gpuxLaunchKernel(q, k, 1, 1, 1, 1, 1, 1, NO_DEPS, descs)
+    rt.gpuxWait(q, ev)                            # a new position: drains again
+    assert counter(rt, "stream_syncs") == base["stream_syncs"] + 2
+    for e in evs + [ev]:
         rt.gpuxDestroyEvent(q, e)
 
 
-def test_empty_launch_records_an_event_but_launches_nothing(rt, qk):
+def test_empty_launch_returns_a_waitable_event_but_launches_nothing(rt, qk):
     q, _, k = qk
     descs, _ = make_params([])
-    before = counter(rt, "launches"), counter(rt, "event_records")
+    before = counter(rt, "launches")
     ev = rt.gpuxLaunchKernel(q, k, 0, 1, 1, 64, 1, 1, NO_DEPS, descs)
-    assert counter(rt, "launches") == before[0]
-    assert counter(rt, "event_records") == before[1] + 1
+    assert counter(rt, "launches") == before and ev
     rt.gpuxWait(q, ev)
     rt.gpuxDestroyEvent(q, ev)
+
+
+def test_allocation_event_is_already_complete(rt, qk):
+    q, _, k = qk
+    descs, _ = make_params([])
+    rt.mockExpectParams(0)
+    pending = rt.gpuxLaunchKernel(q, k, 1, 1, 1, 1, 1, 1, NO_DEPS, descs)
+    res = AllocResult()
+    rt.gpuxAlloc(q, 64, 64, 0, NO_DEPS, ctypes.byref(res))
+    before = counter(rt, "stream_syncs")
+    rt.gpuxWait(q, res.event)                     # no drain needed
+    assert counter(rt, "stream_syncs") == before
+    rt.gpuxDestroyEvent(q, res.event)
+    rt.gpuxDestroyEvent(q, pending)
+    rt.gpuxDeAlloc(q, res.ptr)
 
 
 def test_queue_lives_until_last_event_and_allocation(rt):
@@ -240,15 +296,25 @@ def test_allocation_kinds(rt, qk):
 
 
 def test_event_pool_reuses_events(rt, qk):
+    """Cross-queue use creates a device event once per pooled slot."""
     q, _, k = qk
+    q2 = rt.gpuxQueueCreate(None)
+    m2 = rt.gpuxModuleLoad(q2, ELF, len(ELF))
+    k2 = rt.gpuxKernelGet(m2, b"kern")
     descs, _ = make_params([])
     rt.mockExpectParams(0)
     created = counter(rt, "events_created")
     for _ in range(200):
         ev = rt.gpuxLaunchKernel(q, k, 1, 1, 1, 1, 1, 1, NO_DEPS, descs)
-        rt.gpuxWait(q, ev)
+        deps = (ctypes.c_void_p * 2)(ev, None)
+        ev2 = rt.gpuxLaunchKernel(q2, k2, 1, 1, 1, 1, 1, 1, deps, descs)
+        rt.gpuxWait(q2, ev2)
+        rt.gpuxDestroyEvent(q2, ev2)
         rt.gpuxDestroyEvent(q, ev)
     assert counter(rt, "events_created") - created <= 1
+    rt.gpuxKernelDestroy(k2)
+    rt.gpuxModuleDestroy(m2)
+    rt.gpuxQueueDestroy(q2)
 
 
 def test_event_pool_is_thread_safe(rt, qk):
