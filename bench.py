@@ -29,6 +29,22 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 
+# HBM bytes per launch at the benchmark shapes, from two rocprofv3 --pmc runs
+# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch) scaled by what the same
+# counters read for a 256 MiB device copy (FETCH x2.000, WRITE x1.000); the
+# runs and the table are in profiles/bench_all_configs_hbm_counters.txt.
+MEASURED_TRAFFIC = {
+    "nmk_black_scholes_f32_w64": 335603175,
+    "nmk_black_scholes_f32_w32": 335607569,
+    "nmk_map2_rowbcast_add_f64": 268483579,
+    "nmk_sum_axis1_f32": 536996441,
+    "nmk_norm2_f32": 536896400,
+    "nmk_sum_axis0_i32_i64": 538012349,
+    "nmk_twin_pairwise_f64_rows": 540323459,
+    "nmk_copy_b128": 536870912,
+    "sgemm_mfma_256x256": 709036864,
+}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -94,7 +110,7 @@ def hbm_entry(name, workload, alg_bytes, wall_ms, ev_ms, kernel, extra=None):
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": None},
+                     "traffic": MEASURED_TRAFFIC.get(kernel)},
     }
     if extra:
         e.update(extra)
@@ -228,7 +244,8 @@ def run(args):
             "roofline": {"bound": "mfma", "achieved": round(tf, 2),
                          "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4),
-                         "traffic": None},
+                         "traffic": MEASURED_TRAFFIC.get(
+                             math_runtime.last_kernel())},
         })
         del d_A, d_B, d_C
 

@@ -194,9 +194,10 @@ NMK_DEFINE_MAP2_ALL_T(mul, OpMul)
 // Transcendentals.  log(P/S) and exp(b) are the float32 library routines.
 // The two float64 erf calls and 1.0 / sqrt(z) dominate the instruction count
 // (the kernel is ALU-bound, not HBM-bound), so the float64 path evaluates
-//   erf  by a piecewise degree-9 polynomial on 24 intervals of [0, 6)
-//        (erf_table.inc, absolute error < 1e-14; erf(|x| >= 6) = 1 in
-//        double), coefficients staged in LDS;
+//   0.5 + 0.5 erf(x)  by a piecewise degree-9 polynomial for erf / 2 on 24
+//        intervals of [0, 6) (erf_table.inc, absolute error < 1e-14;
+//        erf(|x| >= 6) = 1 in double), coefficients staged in LDS; halving is
+//        exact, so the sum rounds as 0.5 + 0.5 * erf(x) would;
 //   1/sqrt(z)  by v_rsq_f64 refined with two Newton steps (relative error a
 //        few 1e-16), falling back to 1.0 / sqrt(z) outside [1e-290, 1e290].
 // Both stay within a few ulp of the library results, far inside the
@@ -216,25 +217,30 @@ template <> struct BsMath<double> {
     }
     return y;
   }
-  __device__ static __forceinline__ double erf_(double x, const double *tab) {
-    double ax = __builtin_fabs(x);
-    ax = ax < 6.0 ? ax : 0x1.7ffffffffffffp+2; // largest double below 6
-    int idx = int(ax * 4.0);
-    const double u = __builtin_fma(ax, 8.0, -double(2 * idx + 1));
-    const double *c = tab + idx * NMK_ERF_COEFFS;
+  // 0.5 + 0.5 * erf(x)
+  __device__ static __forceinline__ double cdfTerm(double x, const double *tab) {
+    const double ax = __builtin_fabs(x);
+    const double t = ax * 4.0; // interval index + fraction
+    // int(NaN) is 0 and int(huge) saturates, so the row index is always valid
+    const int idx = min(int(t), NMK_ERF_INTERVALS - 1);
+    // u = 8 |x| - (2 idx + 1) = 2 frac(t) - 1; NaN stays NaN
+    const double u = __builtin_fma(t - double(idx), 2.0, -1.0);
+    const double *c = tab + __mul24(idx, NMK_ERF_ROW);
     double p = c[NMK_ERF_COEFFS - 1];
 #pragma unroll
     for (int k = NMK_ERF_COEFFS - 2; k >= 0; --k)
       p = __builtin_fma(p, u, c[k]);
-    return __builtin_copysign(p, x);
+    // erf(|x| >= 6) rounds to exactly 1 in double (erfc(6) = 2e-17)
+    p = ax >= 6.0 ? 0.5 : p;
+    return 0.5 + __builtin_copysign(p, x);
   }
 };
 template <> struct BsMath<float> {
   __device__ static __forceinline__ float rsqrt_(float z) {
     return 1.0f / sqrtf(z);
   }
-  __device__ static __forceinline__ float erf_(float x, const double *) {
-    return erff(x);
+  __device__ static __forceinline__ float cdfTerm(float x, const double *) {
+    return 0.5f + 0.5f * erff(x);
   }
 };
 
@@ -250,8 +256,8 @@ blackScholesOne(float P, float S, float T, float mr, W sigSigTwo,
   const float amb = a - b;
   const W w1 = (W(amb) + c) * y;
   const W w2 = (W(amb) - c) * y;
-  const W d1 = W(0.5) + W(0.5) * BsMath<W>::erf_(w1, erfTab);
-  const W d2 = W(0.5) + W(0.5) * BsMath<W>::erf_(w2, erfTab);
+  const W d1 = BsMath<W>::cdfTerm(w1, erfTab); // 0.5 + 0.5 * erf(w1)
+  const W d2 = BsMath<W>::cdfTerm(w2, erfTab);
   const float Se = expf(b) * S;
   const W r = W(P) * d1 - W(Se) * d2;
   call = float(r);
@@ -260,7 +266,8 @@ blackScholesOne(float P, float S, float T, float mr, W sigSigTwo,
 
 // VEC options per lane per iteration (float4 or float2 accesses).  The
 // float64 variant is ALU-bound and register-hungry: two options per lane at
-// six waves per SIMD measured fastest; the float32 variant takes four.
+// five to six waves per SIMD measured fastest (no spills at five); the
+// float32 variant takes four.
 template <int VEC> struct BsVec;
 template <> struct BsVec<4> {
   typedef float4_t type;
@@ -275,12 +282,12 @@ blackScholes(const float *__restrict__ price, const float *__restrict__ strike,
              const float *__restrict__ t, float rate, float volatility,
              float *__restrict__ call, float *__restrict__ put, int64_t n) {
   typedef typename BsVec<VEC>::type V;
-  __shared__ double erfTab[sizeof(W) == 8 ? NMK_ERF_INTERVALS * NMK_ERF_COEFFS
-                                          : 1];
+  __shared__ __attribute__((aligned(16))) double
+      erfTab[sizeof(W) == 8 ? NMK_ERF_INTERVALS * NMK_ERF_ROW : 1];
   if (sizeof(W) == 8) {
-    for (int i = threadIdx.x; i < NMK_ERF_INTERVALS * NMK_ERF_COEFFS;
+    for (int i = threadIdx.x; i < NMK_ERF_INTERVALS * NMK_ERF_ROW;
          i += blockDim.x)
-      erfTab[i] = kErfTable[i];
+      erfTab[i] = kHalfErfTable[i];
     __syncthreads();
   }
   const float mr = -rate;

@@ -144,6 +144,27 @@ def test_black_scholes_reference_typing(env, n):
     np.testing.assert_allclose(put, rp, rtol=BS_RTOL, atol=BS_ATOL)
 
 
+def test_black_scholes_special_values(env):
+    """Zero, infinite and NaN inputs take the same IEEE paths as the oracle."""
+    hip, ops, orc = env
+    inf, nan = np.inf, np.nan
+    price = np.array([30, 0, 30, 0, inf, 30, nan, 30, 30, 1e-30, 50, 10], np.float32)
+    strike = np.array([30, 30, 0, 0, 30, inf, 30, nan, 30, 30, 10, 50], np.float32)
+    t = np.array([1.5, 1, 1, 1, 1, 1, 1, 1, 0, 1, 2, 1], np.float32)
+    d = [hip.asarray(x) for x in (price, strike, t, np.zeros(12, np.float32),
+                                  np.zeros(12, np.float32))]
+    ops.black_scholes(d[0], d[1], d[2], np.float32(0.1), np.float32(0.2), d[3], d[4])
+    with np.errstate(all="ignore"):
+        rc, rp = orc.black_scholes(price, strike, t, 0.1, 0.2, wide=True)
+    call, put = d[3].asnumpy(), d[4].asnumpy()
+    assert np.array_equal(np.isnan(call), np.isnan(rc))
+    assert np.array_equal(np.isnan(put), np.isnan(rp))
+    ok = ~np.isnan(rc)
+    np.testing.assert_allclose(call[ok], rc[ok], rtol=BS_RTOL, atol=BS_ATOL)
+    ok = ~np.isnan(rp)
+    np.testing.assert_allclose(put[ok], rp[ok], rtol=BS_RTOL, atol=BS_ATOL)
+
+
 def test_black_scholes_float32_typing(env):
     hip, ops, orc = env
     inp, call, put = _run_bs(hip, ops, 524288, False)
