@@ -57,7 +57,8 @@ void nmrtMathRuntimeInit(void);
 void nmrtMathRuntimeFinalize(void);
 
 /* Name of the device kernel the most recent gemm call on this thread ran
- * ("sgemm_mfma_128x128", "sgemm_generic", ...); for tests and profiling. */
+ * ("sgemm_mfma_256x256", "sgemm_mfma_128x128", "dgemm_mfma_128x128",
+ * "sgemm_generic", "dgemm_generic"); for tests and profiling. */
 const char *nmhipMathLastKernel(void);
 
 #ifdef __cplusplus

@@ -4,8 +4,8 @@
 // Entry points, argument meaning and layout rules follow the oneMKL-backed
 // runtime they replace (reference:
 // numba_mlir/numba_mlir/math_runtime/sycl/lib/NumpyLinalg.cpp:67-183); the
-// arithmetic is a hand-written LDS-tiled fp32 MFMA kernel for gfx950 plus a
-// strided fallback.
+// arithmetic is a hand-written LDS-tiled MFMA kernel for gfx950 (fp32 and
+// fp64 matrix cores) plus a strided fallback.
 #include "numba_mlir_hip/GpuQueueInterface.hpp"
 #include "numba_mlir_hip/MathRuntime.h"
 
@@ -20,6 +20,8 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef double doublex4 __attribute__((ext_vector_type(4)));
+typedef double doublex2 __attribute__((ext_vector_type(2)));
 
 // fatal_failure of the reference prints to stderr and aborts
 // (math_runtime/include/Common.hpp:10-15).
@@ -41,90 +43,123 @@ void checkHip(hipError_t err, const char *what) {
 thread_local const char *lastKernel = "";
 
 // ---------------------------------------------------------------------------
-// C[M,N] = alpha * A[M,K] * B[K,N] + beta * C with C row-major (ldc), fp32 in,
-// fp32 accumulate on the matrix cores.  Each input operand may be stored with
-// either of its two dimensions contiguous:
+// C[M,N] = alpha * A[M,K] * B[K,N] + beta * C with C row-major (ldc) on the
+// matrix cores, float32 (v_mfma_f32_32x32x2_f32) or float64
+// (v_mfma_f64_16x16x4_f64), accumulating in the operand type.  Each input
+// operand may be stored with either of its two dimensions contiguous:
 //   A_KC: A(m,k) = A[m * lda + k]   (row-major A)   else A[k * lda + m]
 //   B_NC: B(k,n) = B[k * ldb + n]   (row-major B)   else B[n * ldb + k]
 // which covers the four transpose cases of a BLAS gemm; a column-major C is
 // handled by the host as C^T = B^T A^T.
 //
-// 256 threads = 4 waves in a 2 x 2 grid; each wave owns TM x TN tiles of
-// v_mfma_f32_32x32x2_f32, so the block tile is (64 TM) x (64 TN) and a wave
-// keeps 16 TM TN accumulator registers.  K advances in slabs of BK = 16.
+// 256 threads = 4 waves in a 2 x 2 grid; each wave owns TM x TN MFMA tiles of
+// edge TILE (32 for float32, 16 for float64), so the block tile is
+// (2 TM TILE) x (2 TN TILE).  K advances in slabs of BK elements (64 bytes).
 //
-// LDS holds both operands K-major ([k][m] and [k][n], rows padded by 4 floats)
-// so that the MFMA operand fetch -- lane l needs element (l % 32) of row
-// (k + l / 32) -- is a conflict-free ds_read_b32.  Global fetches are float4
-// along the operand's contiguous dimension: an operand contiguous in m / n
-// is written to LDS as float4, one contiguous in k is scattered over four LDS
-// rows.  Two LDS stages: the next K slab is fetched from global memory into
-// registers before the MFMAs of the current slab are issued and written to
-// the other stage after them, one barrier per slab.
+// LDS holds both operands K-major ([k][m] and [k][n], rows padded so that the
+// rows one MFMA operand fetch touches fall on different banks): lane l needs
+// element (l % TILE) of row (k + l / TILE), a conflict-free ds_read.  Global
+// fetches are 128-bit along the operand's contiguous dimension: an operand
+// contiguous in m / n is written to LDS as one 128-bit word, one contiguous
+// in k is scattered over LDS rows.  Two LDS stages: the next K slab is
+// fetched from global memory into registers before the MFMAs of the current
+// slab are issued and written to the other stage after them, one barrier per
+// slab.
 //
-// MFMA 32x32x2 operand layout (64 lanes):
-//   A (32 x 2): lane l holds A[l % 32][l / 32]
-//   B (2 x 32): lane l holds B[l / 32][l % 32]
-//   D (32 x 32): lane l, register r holds D[8*(r/4) + 4*(l/32) + r%4][l % 32]
+// MFMA operand layouts (64 lanes):
+//   f32 32x32x2: A[l % 32][l / 32], B[l / 32][l % 32],
+//                D reg r = D[8*(r/4) + 4*(l/32) + r%4][l % 32]   (16 regs)
+//   f64 16x16x4: A[l % 16][l / 16], B[l / 16][l % 16],
+//                D reg r = D[4*r + l/16][l % 16]                  (4 regs)
 //
-// Requirements (checked by the host): M % (64 TM) == 0, N % (64 TN) == 0,
-// K % 16 == 0, lda/ldb % 4 == 0, A and B 16-byte aligned.
-constexpr int BK = 16, PAD = 4;
+// Requirements (checked by the host): M and N multiples of the block tile,
+// K % BK == 0, leading dimensions multiples of the 128-bit vector, A and B
+// 16-byte aligned.
+template <typename T> struct Mfma;
+template <> struct Mfma<float> {
+  typedef floatx4 Vec;   // 128-bit global access
+  typedef floatx16 Acc;  // one MFMA tile per lane
+  static constexpr int TILE = 32, KSTEP = 2, BK = 16, VEC = 4, NACC = 16,
+                       PAD = 4;
+  __device__ static __forceinline__ Acc mma(float a, float b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ int accRow(int r, int lane) {
+    return 8 * (r / 4) + 4 * (lane / 32) + r % 4;
+  }
+};
+template <> struct Mfma<double> {
+  typedef doublex2 Vec;
+  typedef doublex4 Acc;
+  // PAD 16: consecutive k rows land 32 banks apart for a 128-wide tile
+  static constexpr int TILE = 16, KSTEP = 4, BK = 8, VEC = 2, NACC = 4,
+                       PAD = 16;
+  __device__ static __forceinline__ Acc mma(double a, double b, Acc c) {
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ int accRow(int r, int lane) {
+    return 4 * r + lane / 16;
+  }
+};
 
-// One operand's slab of X x 16 (X = BM or BN) on its way from global memory
-// to LDS[stage][k][x].  T float4 per thread.
-template <int X, bool K_CONTIG> struct SlabFetch {
-  static constexpr int T = X / 64;
-  // K_CONTIG: thread -> (x = tid / 4 + 64 i, k = 4 (tid % 4) .. +3)
-  // else    : thread -> (k = tid / (X / 4) + (1024 / X) i, x = 4 (tid % (X/4)) .. +3)
-  static constexpr int K_ROWS = 1024 / X;
+// One operand's slab of X x BK (X = BM or BN) on its way from global memory
+// to LDS[k][x].  NV 128-bit words per thread.
+//   K_CONTIG: thread -> (x = tid / (BK/VEC) + 64 i, k = VEC (tid % (BK/VEC)) ..)
+//   else    : thread -> (k = tid / (X/VEC) + K_ROWS i, x = VEC (tid % (X/VEC)) ..)
+template <typename T, int X, bool K_CONTIG> struct SlabFetch {
+  typedef Mfma<T> M;
+  typedef typename M::Vec Vec;
+  static constexpr int NV = X / 64;
+  static constexpr int K_ROWS = 256 * M::VEC / X;
   int x, k;
-  const float *base;
+  const T *base;
   int64_t ld;
-  floatx4 reg[T];
+  Vec reg[NV];
 
-  __device__ __forceinline__ void init(const float *p, int64_t ld_, int origin,
+  __device__ __forceinline__ void init(const T *p, int64_t ld_, int origin,
                                        int tid) {
     ld = ld_;
     if (K_CONTIG) {
-      x = tid / 4;
-      k = (tid % 4) * 4;
+      x = tid / (M::BK / M::VEC);
+      k = (tid % (M::BK / M::VEC)) * M::VEC;
       base = p + int64_t(origin + x) * ld + k;
     } else {
-      k = tid / (X / 4);
-      x = (tid % (X / 4)) * 4;
+      k = tid / (X / M::VEC);
+      x = (tid % (X / M::VEC)) * M::VEC;
       base = p + int64_t(k) * ld + origin + x;
     }
   }
   __device__ __forceinline__ void fetch(int k0) {
 #pragma unroll
-    for (int i = 0; i < T; ++i)
-      reg[i] = *reinterpret_cast<const floatx4 *>(
+    for (int i = 0; i < NV; ++i)
+      reg[i] = *reinterpret_cast<const Vec *>(
           K_CONTIG ? base + int64_t(64 * i) * ld + k0
                    : base + int64_t(k0 + K_ROWS * i) * ld);
   }
-  __device__ __forceinline__ void stash(float (*lds)[X + PAD]) const {
+  __device__ __forceinline__ void stash(T (*lds)[X + M::PAD]) const {
 #pragma unroll
-    for (int i = 0; i < T; ++i) {
+    for (int i = 0; i < NV; ++i) {
       if (K_CONTIG) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
+        for (int q = 0; q < M::VEC; ++q)
           lds[k + q][x + 64 * i] = reg[i][q];
       } else {
-        *reinterpret_cast<floatx4 *>(&lds[k + K_ROWS * i][x]) = reg[i];
+        *reinterpret_cast<Vec *>(&lds[k + K_ROWS * i][x]) = reg[i];
       }
     }
   }
 };
 
-template <int TM, int TN, bool A_KC, bool B_NC>
+template <typename T, int TM, int TN, bool A_KC, bool B_NC>
 __global__ __launch_bounds__(256) void
-sgemm_mfma(const float *__restrict__ A, const float *__restrict__ B,
-           float *__restrict__ C, int M, int N, int K, int64_t lda, int64_t ldb,
-           int64_t ldc, float alpha, float beta) {
-  constexpr int BM = 64 * TM, BN = 64 * TN;
-  __shared__ float As[2][BK][BM + PAD];
-  __shared__ float Bs[2][BK][BN + PAD];
+gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
+          int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, T alpha,
+          T beta) {
+  typedef Mfma<T> MF;
+  constexpr int TILE = MF::TILE, BK = MF::BK;
+  constexpr int BM = 2 * TM * TILE, BN = 2 * TN * TILE;
+  __shared__ __attribute__((aligned(16))) T As[2][BK][BM + MF::PAD];
+  __shared__ __attribute__((aligned(16))) T Bs[2][BK][BN + MF::PAD];
 
   const int tid = threadIdx.x;
   const int lane = tid % 64;
@@ -133,19 +168,19 @@ sgemm_mfma(const float *__restrict__ A, const float *__restrict__ B,
   const int bm = blockIdx.y * BM;
   const int bn = blockIdx.x * BN;
 
-  SlabFetch<BM, A_KC> fa;
-  SlabFetch<BN, !B_NC> fb;
+  SlabFetch<T, BM, A_KC> fa;
+  SlabFetch<T, BN, !B_NC> fb;
   fa.init(A, lda, bm, tid);
   fb.init(B, ldb, bn, tid);
 
-  floatx16 acc[TM][TN];
+  typename MF::Acc acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        acc[i][j][r] = 0.f;
+      for (int r = 0; r < MF::NACC; ++r)
+        acc[i][j][r] = T(0);
 
   fa.fetch(0);
   fb.fetch(0);
@@ -154,7 +189,7 @@ sgemm_mfma(const float *__restrict__ A, const float *__restrict__ B,
   __syncthreads();
 
   const int nSlabs = K / BK;
-  const int kLane = lane / 32, xLane = lane % 32;
+  const int kLane = lane / TILE, xLane = lane % TILE;
   for (int s = 0; s < nSlabs; ++s) {
     const int cur = s & 1;
     if (s + 1 < nSlabs) {
@@ -162,20 +197,19 @@ sgemm_mfma(const float *__restrict__ A, const float *__restrict__ B,
       fb.fetch((s + 1) * BK);
     }
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 2) {
-      float a[TM], b[TN];
+    for (int kk = 0; kk < BK; kk += MF::KSTEP) {
+      T a[TM], b[TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i)
-        a[i] = As[cur][kk + kLane][wm * (32 * TM) + i * 32 + xLane];
+        a[i] = As[cur][kk + kLane][wm * (TM * TILE) + i * TILE + xLane];
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        b[j] = Bs[cur][kk + kLane][wn * (32 * TN) + j * 32 + xLane];
+        b[j] = Bs[cur][kk + kLane][wn * (TN * TILE) + j * TILE + xLane];
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j],
-                                                           acc[i][j], 0, 0, 0);
+          acc[i][j] = MF::mma(a[i], b[j], acc[i][j]);
     }
     if (s + 1 < nSlabs) {
       fa.stash(As[cur ^ 1]);
@@ -188,14 +222,14 @@ sgemm_mfma(const float *__restrict__ A, const float *__restrict__ B,
   for (int i = 0; i < TM; ++i) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      const int col = bn + wn * (32 * TN) + j * 32 + xLane;
+      const int col = bn + wn * (TN * TILE) + j * TILE + xLane;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
+      for (int r = 0; r < MF::NACC; ++r) {
         const int row =
-            bm + wm * (32 * TM) + i * 32 + 8 * (r / 4) + 4 * kLane + r % 4;
-        float *dst = C + int64_t(row) * ldc + col;
-        float v = alpha * acc[i][j][r];
-        if (beta != 0.f)
+            bm + wm * (TM * TILE) + i * TILE + MF::accRow(r, lane);
+        T *dst = C + int64_t(row) * ldc + col;
+        T v = alpha * acc[i][j][r];
+        if (beta != T(0))
           v += beta * *dst;
         *dst = v;
       }
@@ -310,14 +344,14 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
 
   if (M > 0 && N > 0) {
     bool launched = false;
-    if constexpr (sizeof(T) == 4) {
+    {
       // Operands as the kernel sees them: X(m,k), Y(k,n), Z row-major.  A
       // column-major C is computed as C^T = B^T A^T (swap and transpose the
       // inputs); which dimension of each input is contiguous follows from
       // its unit stride (NumpyLinalg.cpp:87-102).
       const bool cRow = c->strides[1] == 1;
-      const float *X = cRow ? aData : bData;
-      const float *Y = cRow ? bData : aData;
+      const T *X = cRow ? aData : bData;
+      const T *Y = cRow ? bData : aData;
       // strides of X over (m, k) and Y over (k, n)
       const int64_t xm = cRow ? a->strides[0] : b->strides[1];
       const int64_t xk = cRow ? a->strides[1] : b->strides[0];
@@ -327,43 +361,49 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       const int64_t ldz = cRow ? c->strides[0] : c->strides[1];
       const bool xKc = xk == 1, yNc = yn == 1;
       const int64_t ldx = xKc ? xm : xk, ldy = yNc ? yk : yn;
-      // 256 x 256 block tiles (one block per CU on a 4096^2 problem) when the
-      // shape allows and there are enough tiles to fill the 256 CUs; 128 x
-      // 128 otherwise.  Measured within 3 % of each other; the larger tile
-      // halves the operand traffic.
-      const bool big = Mz % 256 == 0 && Nz % 256 == 0 &&
+      constexpr int VEC = Mfma<T>::VEC, BK = Mfma<T>::BK;
+      // float32: 256 x 256 block tiles (one block per CU on a 4096^2
+      // problem) when the shape allows and there are enough tiles to fill the
+      // 256 CUs, 128 x 128 otherwise (measured within 3 % of each other; the
+      // larger tile halves the operand traffic).  float64: 128 x 128.
+      const bool big = sizeof(T) == 4 && Mz % 256 == 0 && Nz % 256 == 0 &&
                        (Mz / 256) * (Nz / 256) >= 192;
       const int BM = big ? 256 : 128, BN = BM;
       const bool unitOk = (xk == 1 || xm == 1) && (yk == 1 || yn == 1);
       if (unitOk && K > 0 && Mz % BM == 0 && Nz % BN == 0 && K % BK == 0 &&
-          ldx % 4 == 0 && ldy % 4 == 0 && ldx > 0 && ldy > 0 && aligned16(X) &&
-          aligned16(Y) && M <= 0x7fffffff && N <= 0x7fffffff &&
+          ldx % VEC == 0 && ldy % VEC == 0 && ldx > 0 && ldy > 0 &&
+          aligned16(X) && aligned16(Y) && M <= 0x7fffffff && N <= 0x7fffffff &&
           K <= 0x7fffffff && Mz / BM <= 65535) {
         dim3 grid(unsigned(Nz / BN), unsigned(Mz / BM), 1);
-#define NMHIP_SGEMM_LAUNCH(TM, TN, XKC, YNC)                                   \
-  hipLaunchKernelGGL((sgemm_mfma<TM, TN, XKC, YNC>), grid, dim3(256), 0,       \
+#define NMHIP_GEMM_LAUNCH(TM, TN, XKC, YNC)                                    \
+  hipLaunchKernelGGL((gemm_mfma<T, TM, TN, XKC, YNC>), grid, dim3(256), 0,     \
                      stream, X, Y, cData, int(Mz), int(Nz), int(K), ldx, ldy,  \
                      ldz, alpha, beta)
-#define NMHIP_SGEMM_LAYOUTS(TM, TN)                                            \
+#define NMHIP_GEMM_LAYOUTS(TM, TN)                                             \
   do {                                                                         \
     if (xKc && yNc)                                                            \
-      NMHIP_SGEMM_LAUNCH(TM, TN, true, true);                                  \
+      NMHIP_GEMM_LAUNCH(TM, TN, true, true);                                   \
     else if (xKc)                                                              \
-      NMHIP_SGEMM_LAUNCH(TM, TN, true, false);                                 \
+      NMHIP_GEMM_LAUNCH(TM, TN, true, false);                                  \
     else if (yNc)                                                              \
-      NMHIP_SGEMM_LAUNCH(TM, TN, false, true);                                 \
+      NMHIP_GEMM_LAUNCH(TM, TN, false, true);                                  \
     else                                                                       \
-      NMHIP_SGEMM_LAUNCH(TM, TN, false, false);                                \
+      NMHIP_GEMM_LAUNCH(TM, TN, false, false);                                 \
   } while (0)
-        if (big) {
-          NMHIP_SGEMM_LAYOUTS(4, 4);
-          lastKernel = "sgemm_mfma_256x256";
+        if constexpr (sizeof(T) == 4) {
+          if (big) {
+            NMHIP_GEMM_LAYOUTS(4, 4);
+            lastKernel = "sgemm_mfma_256x256";
+          } else {
+            NMHIP_GEMM_LAYOUTS(2, 2);
+            lastKernel = "sgemm_mfma_128x128";
+          }
         } else {
-          NMHIP_SGEMM_LAYOUTS(2, 2);
-          lastKernel = "sgemm_mfma_128x128";
+          NMHIP_GEMM_LAYOUTS(4, 4);
+          lastKernel = "dgemm_mfma_128x128";
         }
-#undef NMHIP_SGEMM_LAYOUTS
-#undef NMHIP_SGEMM_LAUNCH
+#undef NMHIP_GEMM_LAYOUTS
+#undef NMHIP_GEMM_LAUNCH
         launched = true;
       }
     }

@@ -173,6 +173,26 @@ def test_identity_and_linearity_full_size(env):
                                atol=1e-4 * 64 * 3)
 
 
+@pytest.mark.parametrize("ta,tb,tc", list(itertools.product([False, True], repeat=3)))
+@pytest.mark.parametrize("m,n,k", [(128, 128, 8), (256, 384, 72), (1024, 1024, 1024)])
+def test_float64_mfma(env, ta, tb, tc, m, n, k):
+    """mkl_gemm_float64_device on the fp64 matrix cores, every layout; the
+    tolerance is rel 1e-5 (float64 bar), met with a wide margin."""
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(m + n + k)
+    a, b = rng.standard_normal((m, k)), rng.standard_normal((k, n))
+    c0 = rng.standard_normal((m, n))
+    lay = lambda x, t: np.asfortranarray(x) if t else x
+    d_c = _to_dev(hip, lay(c0, tc))
+    ops.gemm(_to_dev(hip, lay(a, ta)), _to_dev(hip, lay(b, tb)), d_c, 1.25, -0.5)
+    assert mrt.last_kernel() == "dgemm_mfma_128x128"
+    got = d_c.asnumpy()
+    truth = -0.5 * c0 + 1.25 * (a @ b)
+    bound = 1e-13 * (0.5 * np.abs(c0) + 1.25 * (np.abs(a) @ np.abs(b)))
+    assert (np.abs(got - truth) <= bound).all()
+    np.testing.assert_allclose(got, truth, rtol=1e-5, atol=1e-9)
+
+
 def test_float64_gemm(env):
     hip, ops, _, mrt = env
     rng = np.random.default_rng(4)
