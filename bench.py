@@ -37,7 +37,7 @@ MEASURED_TRAFFIC = {
     "nmk_black_scholes_f32_w64": 335603175,
     "nmk_black_scholes_f32_w32": 335607569,
     "nmk_map2_rowbcast_add_f64": 268483579,
-    "nmk_sum_axis1_f32": 536996441,
+    "nmk_sum_axis1_wide_f32": 536996441,
     "nmk_norm2_f32": 536896400,
     "nmk_sum_axis0_i32_i64": 538012349,
     "nmk_twin_pairwise_f64_rows": 540323459,

@@ -646,7 +646,10 @@ NMHIP_EXPORT void nmhipReduce(void *ctx, int op, int dtype, const void *x,
     if (op == NMHIP_SUM && dtype == NMHIP_F32 && axis == 1 && rowMajor &&
         n0 > 0 && n1 > 0) {
       const int vec = (aligned16(x) && s0 % 4 == 0 && n1 % 4 == 0) ? 1 : 0;
-      c->launch("nmk_sum_axis1_f32", size_t(ceilDiv(n0, 4)), 1, 1, 256, 1, 1,
+      // a block per row for long rows, a wave per row otherwise
+      const bool wide = n1 >= 4096 && n0 <= 0x7fffffff;
+      c->launch(wide ? "nmk_sum_axis1_wide_f32" : "nmk_sum_axis1_f32",
+                size_t(wide ? n0 : ceilDiv(n0, 4)), 1, 1, 256, 1, 1,
                 {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(n0), Arg::I64(n1),
                  Arg::I64(s0), Arg::I32(vec)});
       return;
@@ -727,7 +730,9 @@ NMHIP_EXPORT void nmhipNorm2RowsF32(void *ctx, const float *x, int64_t n0,
     if (n0 == 0)
       return;
     const int vec = (aligned16(x) && s0 % 4 == 0 && n1 % 4 == 0) ? 1 : 0;
-    c->launch("nmk_norm2_axis1_f32", size_t(ceilDiv(n0, 4)), 1, 1, 256, 1, 1,
+    const bool wide = n1 >= 4096 && n0 <= 0x7fffffff;
+    c->launch(wide ? "nmk_norm2_axis1_wide_f32" : "nmk_norm2_axis1_f32",
+              size_t(wide ? n0 : ceilDiv(n0, 4)), 1, 1, 256, 1, 1,
               {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(n0), Arg::I64(n1),
                Arg::I64(s0), Arg::I32(vec)});
   });

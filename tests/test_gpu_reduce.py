@@ -98,7 +98,8 @@ def test_sum_axis1_f32(env, shape):
     rng = np.random.Generator(np.random.PCG64(1003))
     x = rng.standard_normal(shape, dtype=np.float32)
     got = ops.sum(hip.asarray(x), axis=1).asnumpy()
-    assert hip.get_context().last_kernel() == "nmk_sum_axis1_f32"
+    assert hip.get_context().last_kernel() == (
+        "nmk_sum_axis1_wide_f32" if shape[1] >= 4096 else "nmk_sum_axis1_f32")
     x64 = x.astype(np.float64)
     truth, mag = x64.sum(axis=1), np.abs(x64).sum(axis=1)
     assert (np.abs(got - truth) <= 1e-4 * mag).all()
