@@ -34,15 +34,15 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 # counters read for a 256 MiB device copy (FETCH x2.000, WRITE x1.000); the
 # runs and the table are in profiles/bench_all_configs_hbm_counters.txt.
 MEASURED_TRAFFIC = {
-    "nmk_black_scholes_f32_w64": 335603175,
-    "nmk_black_scholes_f32_w32": 335607569,
-    "nmk_map2_rowbcast_add_f64": 268483579,
-    "nmk_sum_axis1_wide_f32": 536996441,
-    "nmk_norm2_f32": 536896400,
-    "nmk_sum_axis0_i32_i64": 538012349,
-    "nmk_twin_pairwise_f64_rows": 540323459,
+    "nmk_black_scholes_f32_w64": 341900506,
+    "nmk_black_scholes_f32_w32": 335602174,
+    "nmk_map2_rowbcast_add_f64": 268479506,
+    "nmk_sum_axis1_wide_f32": 537385291,
+    "nmk_norm2_f32": 536909027,
+    "nmk_sum_axis0_i32_i64": 538012431,
+    "nmk_twin_pairwise_f64_rows": 540334698,
     "nmk_copy_b128": 536870912,
-    "sgemm_mfma_256x256": 709036864,
+    "sgemm_mfma_256x256": 709056652,
 }
 
 

@@ -143,3 +143,10 @@ def test_call_logging_env(native_libs):
          "g.runtime_lib.gpuxQueueDestroy(None)"],
         env=env, capture_output=True, text=True)
     assert proc.stdout.startswith("gpuxQueueDestroy enter\n")
+
+
+def test_bench_refuses_more_than_one_gpu():
+    proc = subprocess.run(["python", os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                          capture_output=True, text=True)
+    assert proc.returncode == 2
+    assert "one GPU" in proc.stderr and proc.stdout == ""
