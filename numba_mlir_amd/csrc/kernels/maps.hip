@@ -191,48 +191,56 @@ NMK_DEFINE_MAP2_ALL_T(mul, OpMul)
 // NumPy computes for the same source, and what the reference computes when
 // the literals are written as np.float32).
 //
-// Transcendentals.  log(P/S) and exp(b) are the float32 library routines.
-// The two float64 erf calls and 1.0 / sqrt(z) dominate the instruction count
-// (the kernel is ALU-bound, not HBM-bound), so the float64 path evaluates
-//   0.5 + 0.5 erf(x)  by a piecewise degree-9 polynomial for erf / 2 on 24
-//        intervals of [0, 6) (erf_table.inc, absolute error < 1e-14;
-//        erf(|x| >= 6) = 1 in double), coefficients staged in LDS; halving is
-//        exact, so the sum rounds as 0.5 + 0.5 * erf(x) would;
-//   1/sqrt(z)  by v_rsq_f64 refined with two Newton steps (relative error a
-//        few 1e-16), falling back to 1.0 / sqrt(z) outside [1e-290, 1e290].
-// Both stay within a few ulp of the library results, far inside the
-// tolerance the path is checked at.
+// Cost.  Arithmetic and HBM traffic take about the same time here (about
+// 40 us of vector-ALU issue against 52 us for the five streams of 2^24
+// options), so every instruction counts:
+//   0.5 + 0.5 erf(x)  is a degree-7 polynomial for erf / 2 around the nearest
+//        of 97 nodes 1/16 apart on [0, 6] (erf_table.inc, absolute error of
+//        erf below 1e-15; erf(|x| >= 5.97) = 1 in double), coefficients
+//        staged in LDS; halving is exact, so the sum rounds as
+//        0.5 + 0.5 * erf(x) would;
+//   1 / sqrt(z)  is v_rsq_f64 with one third-order correction (below one unit
+//        in the last place);
+//   log(P / S) and exp(b)  are the float32 library routines' own operation
+//        sequences without their range handling wherever every lane of the
+//        wave has everyday operands (bit-identical results), and the library
+//        routines otherwise.
 #include "erf_table.inc"
 
 template <typename W> struct BsMath;
 template <> struct BsMath<double> {
+  // 1 / sqrt(z) for z = T * sigSigTwo: the product of a float and of the
+  // double of a float, so z is 0, inf, NaN, negative or a normal double far
+  // from the ends of the range, and neither y * y nor z * y * y can overflow.
+  // The hardware seed (relative error e below 2^-20) gets one third-order
+  // step y (1 + e/2 + 3 e^2 / 8), leaving 5/16 e^3: below 2^-60.
   __device__ static __forceinline__ double rsqrt_(double z) {
-    if (!(z > 1e-290 && z < 1e290))
-      return 1.0 / sqrt(z);
-    double y = __builtin_amdgcn_rsq(z);
-#pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const double r = __builtin_fma(-z, y * y, 1.0); // 1 - z y^2
-      y = __builtin_fma(0.5 * y, r, y);
-    }
-    return y;
+    const double y = __builtin_amdgcn_rsq(z);
+    const double e = __builtin_fma(-z, y * y, 1.0); // 1 - z y^2
+    const double step = __builtin_fma(y * e, __builtin_fma(0.375, e, 0.5), y);
+    // z = 0 -> inf and z = inf -> 0 come from the seed (e is NaN there);
+    // a negative or NaN z gives NaN either way.
+    return __builtin_amdgcn_class(z, 0x260 /* -0 | +0 | +inf */) ? y : step;
   }
-  // 0.5 + 0.5 * erf(x)
+  // 0.5 + 0.5 * erf(x) for a non-NaN x (a NaN x gives a finite value: the
+  // caller tests for it).
   __device__ static __forceinline__ double cdfTerm(double x, const double *tab) {
-    const double ax = __builtin_fabs(x);
-    const double t = ax * 4.0; // interval index + fraction
-    // int(NaN) is 0 and int(huge) saturates, so the row index is always valid
-    const int idx = min(int(t), NMK_ERF_INTERVALS - 1);
-    // u = 8 |x| - (2 idx + 1) = 2 frac(t) - 1; NaN stays NaN
-    const double u = __builtin_fma(t - double(idx), 2.0, -1.0);
-    const double *c = tab + __mul24(idx, NMK_ERF_ROW);
+    const double ax = __builtin_fmin(__builtin_fabs(x), 6.0);
+    // Adding 1.5 * 2^48 rounds ax to the nearest sixteenth and leaves that
+    // count, 0..96, in the low word of the sum.
+    const double magic = 0x1.8p48;
+    const double t = ax + magic;
+    const int node = __double2loint(t);
+    const double u = ax - (t - magic); // exact, |u| <= 1/32
+    const double *c = tab + __mul24(node, NMK_ERF_ROW);
     double p = c[NMK_ERF_COEFFS - 1];
 #pragma unroll
     for (int k = NMK_ERF_COEFFS - 2; k >= 0; --k)
       p = __builtin_fma(p, u, c[k]);
-    // erf(|x| >= 6) rounds to exactly 1 in double (erfc(6) = 2e-17)
-    p = ax >= 6.0 ? 0.5 : p;
     return 0.5 + __builtin_copysign(p, x);
+  }
+  __device__ static __forceinline__ bool eitherNaN(double a, double b) {
+    return __builtin_isunordered(a, b);
   }
 };
 template <> struct BsMath<float> {
@@ -242,14 +250,53 @@ template <> struct BsMath<float> {
   __device__ static __forceinline__ float cdfTerm(float x, const double *) {
     return 0.5f + 0.5f * erff(x);
   }
+  __device__ static __forceinline__ bool eitherNaN(float, float) {
+    return false; // erff propagates NaN by itself
+  }
 };
 
-template <typename W>
+// The float32 steps log(P / S) and exp(b) without the range handling of the
+// general routines: the same operations in the same order, so the results
+// are bit-identical to P / S, logf and expf whenever bsEveryday() holds --
+// P and S positive with exponents in [-60, 60) (the quotient and the
+// reciprocal are then normal numbers) and |b| <= 80 (exp(b) is normal).
+// The division is the reciprocal times P with one residual correction.  It
+// is the general routines' handling of zeros, infinities, NaNs, denormals
+// and overflow that costs two thirds of their instructions.
+__device__ __forceinline__ bool bsEveryday(float P, float S, float b) {
+  const uint32_t lo = 0x21800000u;   // bits of 2^-60
+  const uint32_t span = 0x3C000000u; // up to, not including, 2^60
+  return (__float_as_uint(P) - lo) < span && (__float_as_uint(S) - lo) < span &&
+         __builtin_fabsf(b) <= 80.0f;
+}
+__device__ __forceinline__ float bsDivEveryday(float P, float S) {
+  const float y = __builtin_amdgcn_rcpf(S);
+  const float q = P * y;
+  const float e = __builtin_fmaf(-q, S, P);
+  return __builtin_fmaf(e, y, q);
+}
+__device__ __forceinline__ float bsLogEveryday(float q) {
+  const float y = __builtin_amdgcn_logf(q); // log2
+  const float r = y * 0x1.62e42ep-1f;
+  float e = __builtin_fmaf(y, 0x1.62e42ep-1f, -r);
+  e = __builtin_fmaf(y, 0x1.efa39ep-25f, e);
+  return r + e;
+}
+__device__ __forceinline__ float bsExpEveryday(float b) {
+  const float p = b * 0x1.715476p+0f; // b log2(e), then its rounding error
+  float e = __builtin_fmaf(b, 0x1.715476p+0f, -p);
+  e = __builtin_fmaf(b, 0x1.4ae0bep-26f, e);
+  const float n = __builtin_rintf(p);
+  const float v = __builtin_amdgcn_exp2f((p - n) + e);
+  return __builtin_ldexpf(v, int(n));
+}
+
+template <typename W, bool EVERYDAY>
 __device__ __forceinline__ void
 blackScholesOne(float P, float S, float T, float mr, W sigSigTwo,
                 const double *erfTab, float &call, float &put) {
-  const float a = logf(P / S);
   const float b = T * mr;
+  const float a = EVERYDAY ? bsLogEveryday(bsDivEveryday(P, S)) : logf(P / S);
   const W z = W(T) * sigSigTwo;
   const W c = W(0.25) * z;
   const W y = BsMath<W>::rsqrt_(z);
@@ -258,10 +305,40 @@ blackScholesOne(float P, float S, float T, float mr, W sigSigTwo,
   const W w2 = (W(amb) - c) * y;
   const W d1 = BsMath<W>::cdfTerm(w1, erfTab); // 0.5 + 0.5 * erf(w1)
   const W d2 = BsMath<W>::cdfTerm(w2, erfTab);
-  const float Se = expf(b) * S;
+  const float Se = (EVERYDAY ? bsExpEveryday(b) : expf(b)) * S;
   const W r = W(P) * d1 - W(Se) * d2;
-  call = float(r);
-  put = float(r - W(P) + W(Se));
+  const bool nan = BsMath<W>::eitherNaN(w1, w2);
+  call = nan ? __builtin_nanf("") : float(r);
+  put = nan ? __builtin_nanf("") : float(r - W(P) + W(Se));
+}
+
+// One trip of VEC options per lane.  The everyday forms are taken when every
+// lane of the wave qualifies, so each version stays one straight-line block.
+template <typename W, int VEC, typename V>
+__device__ __forceinline__ void bsTrip(const V &P, const V &S, const V &T,
+                                       float mr, W sigSigTwo,
+                                       const double *erfTab, V &c, V &u) {
+  bool everyday = true;
+#pragma unroll
+  for (int k = 0; k < VEC; ++k)
+    everyday = everyday && bsEveryday(P[k], S[k], T[k] * mr);
+  if (__builtin_amdgcn_ballot_w64(!everyday) == 0) {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      float ck, uk;
+      blackScholesOne<W, true>(P[k], S[k], T[k], mr, sigSigTwo, erfTab, ck, uk);
+      c[k] = ck;
+      u[k] = uk;
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      float ck, uk;
+      blackScholesOne<W, false>(P[k], S[k], T[k], mr, sigSigTwo, erfTab, ck, uk);
+      c[k] = ck;
+      u[k] = uk;
+    }
+  }
 }
 
 // VEC options per lane per iteration (float4 or float2 accesses).  The
@@ -283,9 +360,9 @@ blackScholes(const float *__restrict__ price, const float *__restrict__ strike,
              float *__restrict__ call, float *__restrict__ put, int64_t n) {
   typedef typename BsVec<VEC>::type V;
   __shared__ __attribute__((aligned(16))) double
-      erfTab[sizeof(W) == 8 ? NMK_ERF_INTERVALS * NMK_ERF_ROW : 1];
+      erfTab[sizeof(W) == 8 ? NMK_ERF_NODES * NMK_ERF_ROW : 1];
   if (sizeof(W) == 8) {
-    for (int i = threadIdx.x; i < NMK_ERF_INTERVALS * NMK_ERF_ROW;
+    for (int i = threadIdx.x; i < NMK_ERF_NODES * NMK_ERF_ROW;
          i += blockDim.x)
       erfTab[i] = kHalfErfTable[i];
     __syncthreads();
@@ -305,13 +382,7 @@ blackScholes(const float *__restrict__ price, const float *__restrict__ strike,
     const V S = streamLoad(sv + i);
     const V T = streamLoad(tv + i);
     V c, u;
-#pragma unroll
-    for (int k = 0; k < VEC; ++k) {
-      float ck, uk;
-      blackScholesOne<W>(P[k], S[k], T[k], mr, sigSigTwo, erfTab, ck, uk);
-      c[k] = ck;
-      u[k] = uk;
-    }
+    bsTrip<W, VEC>(P, S, T, mr, sigSigTwo, erfTab, c, u);
     streamStore(c, cv + i);
     streamStore(u, uv + i);
   }
@@ -319,7 +390,7 @@ blackScholes(const float *__restrict__ price, const float *__restrict__ strike,
   const int64_t tail = nvec * VEC + threadIdx.x;
   if (blockIdx.x == 0 && tail < n) {
     float ck, uk;
-    blackScholesOne<W>(price[tail], strike[tail], t[tail], mr, sigSigTwo,
+    blackScholesOne<W, false>(price[tail], strike[tail], t[tail], mr, sigSigTwo,
                        erfTab, ck, uk);
     call[tail] = ck;
     put[tail] = uk;

@@ -165,6 +165,66 @@ def test_black_scholes_special_values(env):
     np.testing.assert_allclose(put[ok], rp[ok], rtol=BS_RTOL, atol=BS_ATOL)
 
 
+def test_black_scholes_out_of_range_operands(env):
+    """Operands outside the everyday range (huge, tiny, denormal, negative, a
+    long-dated option whose discount factor underflows) go through the general
+    routines and still match the oracle."""
+    hip, ops, orc = env
+    price = np.array([1e38, 1e-38, 1e-42, 30, 30, -30, 30, 2.0 ** 60, 2.0 ** -61, 30, 1e20],
+                     np.float32)
+    strike = np.array([1e38, 1e-38, 1e-42, 1e38, 1e-38, 30, -30, 2.0 ** 59, 2.0 ** -60, 30, 1e-20],
+                      np.float32)
+    t = np.array([1, 1, 1, 1, 1, 1, 1, 1.5, 1.5, 1000, 1], np.float32)
+    n = len(price)
+    for wide in (True, False):
+        d = [hip.asarray(x) for x in (price, strike, t, np.zeros(n, np.float32),
+                                      np.zeros(n, np.float32))]
+        ops.black_scholes(d[0], d[1], d[2], np.float32(0.1), np.float32(0.2), d[3], d[4],
+                          float64_literals=wide)
+        with np.errstate(all="ignore"):
+            rc, rp = orc.black_scholes(price, strike, t, 0.1, 0.2, wide=wide)
+        call, put = d[3].asnumpy(), d[4].asnumpy()
+        assert np.array_equal(np.isnan(call), np.isnan(rc)), (wide, call, rc)
+        assert np.array_equal(np.isnan(put), np.isnan(rp)), (wide, put, rp)
+        ok = np.isfinite(rc)
+        np.testing.assert_allclose(call[ok], rc[ok], rtol=1e-4, atol=1e-30)
+        assert np.array_equal(call[~ok & ~np.isnan(rc)], rc[~ok & ~np.isnan(rc)])
+        ok = np.isfinite(rp)
+        np.testing.assert_allclose(put[ok], rp[ok], rtol=1e-4, atol=2e-5 if not wide else 1e-30)
+        assert np.array_equal(put[~ok & ~np.isnan(rp)], rp[~ok & ~np.isnan(rp)])
+
+
+def test_black_scholes_general_and_everyday_forms_agree(env):
+    """One odd lane sends its whole wave through the general routines; every
+    other option of that wave must come out bit-identical to the run without
+    the odd lane."""
+    hip, ops, orc = env
+    n = 1 << 16
+    (price, strike, t, rate, vol), call0, put0 = _run_bs(hip, ops, n, True)
+    for wide in (True, False):
+        d = [hip.asarray(x) for x in (price, strike, t, np.zeros(n, np.float32),
+                                      np.zeros(n, np.float32))]
+        ops.black_scholes(d[0], d[1], d[2], rate, vol, d[3], d[4], float64_literals=wide)
+        base_c, base_p = d[3].asnumpy(), d[4].asnumpy()
+        p2, s2, t2 = price.copy(), strike.copy(), t.copy()
+        odd = np.arange(7, n, 97)          # at least one lane in every wave
+        p2[odd[0::3]] = 0.0
+        s2[odd[1::3]] = np.inf
+        t2[odd[2::3]] = 900.0              # exp(-90) is below the everyday range
+        d = [hip.asarray(x) for x in (p2, s2, t2, np.zeros(n, np.float32),
+                                      np.zeros(n, np.float32))]
+        ops.black_scholes(d[0], d[1], d[2], rate, vol, d[3], d[4], float64_literals=wide)
+        c2, u2 = d[3].asnumpy(), d[4].asnumpy()
+        keep = np.ones(n, bool)
+        keep[odd] = False
+        assert np.array_equal(c2[keep], base_c[keep])
+        assert np.array_equal(u2[keep], base_p[keep])
+        with np.errstate(all="ignore"):
+            rc, rp = orc.black_scholes(p2[odd], s2[odd], t2[odd], rate, vol, wide=wide)
+        np.testing.assert_allclose(c2[odd], rc, rtol=1e-4, atol=2e-5)
+        np.testing.assert_allclose(u2[odd], rp, rtol=1e-4, atol=2e-5)
+
+
 def test_black_scholes_float32_typing(env):
     hip, ops, orc = env
     inp, call, put = _run_bs(hip, ops, 524288, False)
