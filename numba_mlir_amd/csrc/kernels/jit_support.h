@@ -1,0 +1,223 @@
+// Device-side support for kernels generated from Python @kernel bodies
+// (numba_mlir_amd/mlir/kernel_compiler.py).  The generated source includes
+// this header and nothing else; it is compiled for gfx950 on its own.
+//
+// What the reference's lowering provides as GPU-dialect ops and SPIR-V
+// builtins (reference: numba_mlir/mlir_compiler/lib/pipelines/LowerToGpu.cpp:
+// ids 1195-1265, atomics 1404-1465, barriers 1515-1553, group reductions
+// 1564-1780, local/private arrays 1296-1386) are plain device functions here.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fast_math.h"
+
+namespace nmkjit {
+
+// ---- array views ----------------------------------------------------------
+// An N-d strided view: what a memref argument is unpacked into.  Strides are
+// in elements.
+template <typename T, int N> struct View {
+  T *p;
+  int64_t shape[N];
+  int64_t stride[N];
+};
+
+// Python index normalisation: a negative index counts from the end.
+__device__ __forceinline__ int64_t wrap(int64_t i, int64_t n) {
+  return i < 0 ? i + n : i;
+}
+
+// Bounds-checked builds: an index outside [0, n) raises the flag and is
+// redirected to element 0, so the kernel finishes and the host can report it.
+__device__ __forceinline__ int64_t checked(int64_t i, int64_t n, int *flag) {
+  if (i < 0 || i >= n) {
+    *flag = 1;
+    return 0;
+  }
+  return i;
+}
+
+// v[i] on the leading dimension: the view of rank N - 1.
+template <typename T, int N>
+__device__ __forceinline__ View<T, N - 1> sub(const View<T, N> &v, int64_t i) {
+  View<T, N - 1> r;
+  r.p = v.p + i * v.stride[0];
+#pragma unroll
+  for (int k = 1; k < N; ++k) {
+    r.shape[k - 1] = v.shape[k];
+    r.stride[k - 1] = v.stride[k];
+  }
+  return r;
+}
+
+// The same on dimension `dim`.
+template <typename T, int N>
+__device__ __forceinline__ View<T, N - 1> subAt(const View<T, N> &v, int dim,
+                                                int64_t i) {
+  View<T, N - 1> r;
+  r.p = v.p + i * v.stride[dim];
+#pragma unroll
+  for (int k = 0; k < N - 1; ++k) {
+    r.shape[k] = v.shape[k < dim ? k : k + 1];
+    r.stride[k] = v.stride[k < dim ? k : k + 1];
+  }
+  return r;
+}
+
+// v[..., start:stop:step, ...] on dimension `dim`, Python slice semantics;
+// kNone marks an omitted bound.
+constexpr int64_t kNone = INT64_MIN;
+
+template <typename T, int N>
+__device__ __forceinline__ View<T, N> slice(const View<T, N> &v, int dim,
+                                            int64_t start, int64_t stop,
+                                            int64_t step) {
+  const int64_t n = v.shape[dim];
+  if (step == kNone)
+    step = 1;
+  int64_t lo, hi;
+  if (step > 0) {
+    lo = start == kNone ? 0 : (start < 0 ? (start + n < 0 ? 0 : start + n) : (start > n ? n : start));
+    hi = stop == kNone ? n : (stop < 0 ? (stop + n < 0 ? 0 : stop + n) : (stop > n ? n : stop));
+  } else {
+    lo = start == kNone ? n - 1 : (start < 0 ? (start + n < 0 ? -1 : start + n) : (start >= n ? n - 1 : start));
+    hi = stop == kNone ? -1 : (stop < 0 ? (stop + n < 0 ? -1 : stop + n) : (stop >= n ? n - 1 : stop));
+  }
+  int64_t count = 0;
+  if (step > 0 && hi > lo)
+    count = (hi - lo + step - 1) / step;
+  else if (step < 0 && hi < lo)
+    count = (lo - hi - step - 1) / (-step);
+  View<T, N> r = v;
+  r.p = v.p + lo * v.stride[dim];
+  r.shape[dim] = count;
+  r.stride[dim] = v.stride[dim] * step;
+  return r;
+}
+
+// ---- Python arithmetic ----------------------------------------------------
+template <typename T> __device__ __forceinline__ T floordivInt(T a, T b) {
+  if (b == 0)
+    return 0;
+  const T q = a / b;
+  return ((a % b != 0) && ((a < 0) != (b < 0))) ? q - 1 : q;
+}
+template <typename T> __device__ __forceinline__ T modInt(T a, T b) {
+  if (b == 0)
+    return 0;
+  const T r = a % b;
+  return (r != 0 && ((r < 0) != (b < 0))) ? r + b : r;
+}
+// CPython's float_divmod.
+template <typename T> __device__ __forceinline__ T modFloat(T a, T b) {
+  T m = fmod(a, b);
+  if (m != T(0)) {
+    if ((b < T(0)) != (m < T(0)))
+      m += b;
+  } else {
+    m = copysign(T(0), b);
+  }
+  return m;
+}
+template <typename T> __device__ __forceinline__ T floordivFloat(T a, T b) {
+  T m = fmod(a, b);
+  T d = (a - m) / b;
+  if (m != T(0) && ((b < T(0)) != (m < T(0))))
+    d -= T(1);
+  if (d != T(0)) {
+    T f = floor(d);
+    if (d - f > T(0.5))
+      f += T(1);
+    return f;
+  }
+  return copysign(T(0), a / b);
+}
+template <typename T> __device__ __forceinline__ T powInt(T base, T e) {
+  if (e < 0)
+    return base == 1 ? 1 : (base == -1 ? ((e & 1) ? -1 : 1) : 0);
+  T r = 1;
+  while (e > 0) {
+    if (e & 1)
+      r *= base;
+    base *= base;
+    e >>= 1;
+  }
+  return r;
+}
+
+// ---- atomics (return the old value) ---------------------------------------
+__device__ __forceinline__ int32_t atomicAddT(int32_t *p, int32_t v) {
+  return atomicAdd(p, v);
+}
+__device__ __forceinline__ int64_t atomicAddT(int64_t *p, int64_t v) {
+  return int64_t(atomicAdd(reinterpret_cast<unsigned long long *>(p),
+                           static_cast<unsigned long long>(v)));
+}
+__device__ __forceinline__ float atomicAddT(float *p, float v) {
+  return atomicAdd(p, v);
+}
+__device__ __forceinline__ double atomicAddT(double *p, double v) {
+  return atomicAdd(p, v);
+}
+
+// ---- work-group helpers ---------------------------------------------------
+__device__ __forceinline__ int linearLocalId() {
+  return threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z);
+}
+__device__ __forceinline__ int localCount() {
+  return blockDim.x * blockDim.y * blockDim.z;
+}
+
+struct AddOp {
+  template <typename T> __device__ T operator()(T a, T b) const { return a + b; }
+};
+struct MulOp {
+  template <typename T> __device__ T operator()(T a, T b) const { return a * b; }
+};
+struct MinOp {
+  template <typename T> __device__ T operator()(T a, T b) const { return b < a ? b : a; }
+};
+struct MaxOp {
+  template <typename T> __device__ T operator()(T a, T b) const { return a < b ? b : a; }
+};
+
+constexpr int kMaxGroup = 1024;
+
+// Work-group reduction.  Work-items outside the global size never run the
+// kernel body, so they cannot take part: before the body, every lane of the
+// block (in or out) parks the neutral element in its slot (groupInit), and
+// the block learns whether it is clipped.  A full block reduces by an LDS
+// tree; a clipped block, whose members need not be a prefix of the linear
+// ids, has every member fold all slots in order.
+template <typename T>
+__device__ __forceinline__ void groupInit(T *slots, T neutral) {
+  slots[linearLocalId()] = neutral;
+}
+
+template <typename T, typename Op>
+__device__ __forceinline__ T groupReduce(T *slots, T v, bool clipped, Op op) {
+  const int tid = linearLocalId();
+  const int n = localCount();
+  __syncthreads(); // a previous call may still be reading the slots
+  slots[tid] = v;
+  __syncthreads();
+  if (!clipped) {
+    int s = 1;
+    while (s < n)
+      s <<= 1;
+    for (s >>= 1; s > 0; s >>= 1) {
+      if (tid < s && tid + s < n)
+        slots[tid] = op(slots[tid], slots[tid + s]);
+      __syncthreads();
+    }
+    return slots[0];
+  }
+  T r = slots[0];
+  for (int i = 1; i < n; ++i)
+    r = op(r, slots[i]);
+  return r;
+}
+
+} // namespace nmkjit

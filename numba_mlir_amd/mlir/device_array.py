@@ -177,6 +177,33 @@ class HipNdArray:
         return HipNdArray(self._buffer, self.shape[::-1], self.dtype,
                           self.strides[::-1], self._offset)
 
+    def __getitem__(self, key):
+        """Basic indexing (integers and slices): a view of the same
+        allocation, as ``usm_ndarray`` gives."""
+        if not isinstance(key, tuple):
+            key = (key,)
+        if len(key) > self.ndim:
+            raise IndexError("too many indices for device array")
+        shape, strides, offset = [], [], self._offset
+        for dim, k in enumerate(key):
+            n, st = self.shape[dim], self.strides[dim]
+            if isinstance(k, slice):
+                start, stop, step = k.indices(n)
+                shape.append(len(range(start, stop, step)))
+                strides.append(st * step)
+                offset += start * st
+            elif isinstance(k, (int, np.integer)):
+                k = int(k)
+                if not -n <= k < n:
+                    raise IndexError(f"index {k} is out of bounds for axis {dim} "
+                                     f"with size {n}")
+                offset += (k % n) * st
+            else:
+                raise IndexError("only integers and slices index a device array")
+        shape += self.shape[len(key):]
+        strides += self.strides[len(key):]
+        return HipNdArray(self._buffer, shape, self.dtype, strides, offset)
+
     @property
     def __hip_array_interface__(self):
         return {

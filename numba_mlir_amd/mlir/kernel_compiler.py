@@ -1,0 +1,1386 @@
+"""Translates a Python ``@kernel`` body into a gfx950 kernel.
+
+In the reference the body goes through Numba's front end, the plier and GPU
+dialects and SPIR-V (reference: numba_mlir/numba_mlir/mlir/kernel_impl.py:97-206,
+numba_mlir/mlir_compiler/lib/pipelines/LowerToGpu.cpp).  Here the body's
+syntax tree is typed with the same rules and printed as one HIP ``__global__``
+function, which hipcc compiles to a code object for ``gpuxModuleLoad``:
+
+* types: Python ``int``/``float``/``bool`` literals and captured constants are
+  int64/float64/bool; binary operators promote with ``numpy.promote_types``
+  (linalg_builder.py:261-275); ``/`` on integers gives float64; a variable
+  assigned values of several types takes their common type;
+* one work-item per global id, dimension 0 on x, the tail guarded by
+  ``id < global_size`` (LowerToGpu.cpp:1113-1137);
+* the kernel's parameters are what the compiled host code passes
+  (GpuRuntimeToLlvm.cpp:444-628): per array its pointer, shape and strides (in
+  elements), scalars by value, one work-group-memory parameter per
+  ``local.array``, then the three global sizes.
+
+Supported syntax: assignments (also augmented and to array elements), ``if``,
+``for ... in range(...)``, ``while``, ``break``/``continue``/``return``,
+arithmetic with Python semantics for ``//``, ``%`` and ``**``, comparisons,
+``and``/``or``/``not``, conditional expressions, indexing with integers,
+tuples and slices (views), ``math``/``numpy`` scalar functions, casts, calls
+of plain Python functions and lambdas (compiled as device functions), and the
+kernel builtins: ids and sizes, ``atomic.add/sub``, ``barrier``/``mem_fence``,
+``local.array``/``private.array``, ``group.reduce_*``.
+"""
+
+import ast
+import hashlib
+import inspect
+import math
+import os
+import subprocess
+import textwrap
+
+import numpy as np
+
+
+class KernelCompileError(Exception):
+    pass
+
+
+# ---------------------------------------------------------------------------
+# Types
+# ---------------------------------------------------------------------------
+
+class Scalar:
+    def __init__(self, name, ctype, dtype):
+        self.name, self.ctype, self.dtype = name, ctype, np.dtype(dtype)
+        self.kind = self.dtype.kind          # b, i, u, f
+        self.is_float = self.kind == "f"
+        self.is_int = self.kind in "iu"
+        self.is_bool = self.kind == "b"
+
+    def __repr__(self):
+        return self.name
+
+
+BOOL = Scalar("bool", "bool", np.bool_)
+INT8 = Scalar("int8", "int8_t", np.int8)
+INT16 = Scalar("int16", "int16_t", np.int16)
+INT32 = Scalar("int32", "int32_t", np.int32)
+INT64 = Scalar("int64", "int64_t", np.int64)
+UINT8 = Scalar("uint8", "uint8_t", np.uint8)
+UINT16 = Scalar("uint16", "uint16_t", np.uint16)
+UINT32 = Scalar("uint32", "uint32_t", np.uint32)
+UINT64 = Scalar("uint64", "uint64_t", np.uint64)
+FLOAT32 = Scalar("float32", "float", np.float32)
+FLOAT64 = Scalar("float64", "double", np.float64)
+_SCALARS = {s.dtype: s for s in (BOOL, INT8, INT16, INT32, INT64, UINT8, UINT16,
+                                 UINT32, UINT64, FLOAT32, FLOAT64)}
+
+
+def scalar_of(dtype):
+    try:
+        return _SCALARS[np.dtype(dtype)]
+    except (KeyError, TypeError):
+        raise KernelCompileError(f"Unsupported element type: {dtype}")
+
+
+def promote(a, b):
+    return scalar_of(np.promote_types(a.dtype, b.dtype))
+
+
+class Array:
+    """``space``: global (an argument or a view of one), local or private.
+
+    An argument can carry two facts the kernel is specialised on, as Numba
+    specialises on layout: ``layout == "C"`` (dense row-major: the strides
+    follow from the shape) and ``const_shape`` (the extent of a short trailing
+    dimension, so that a loop over it unrolls)."""
+
+    def __init__(self, elem, ndim, space="global", layout="A", const_shape=None):
+        self.elem, self.ndim, self.space = elem, ndim, space
+        self.layout = layout
+        self.const_shape = tuple(const_shape) if const_shape else (None,) * ndim
+
+    def key(self):
+        return ("array", self.elem.name, self.ndim, self.space, self.layout,
+                self.const_shape)
+
+    def ctype(self):
+        return f"nmkjit::View<{self.elem.ctype}, {self.ndim}>"
+
+    def __eq__(self, other):
+        return isinstance(other, Array) and self.key() == other.key()
+
+    def __hash__(self):
+        return hash(self.key())
+
+    def __repr__(self):
+        return f"array({self.elem}, {self.ndim}d, {self.space})"
+
+
+class SliceArg:
+    """A ``slice`` passed as a kernel argument: three int64 parameters."""
+
+    def key(self):
+        return ("slice",)
+
+    def __eq__(self, other):
+        return isinstance(other, SliceArg)
+
+    def __hash__(self):
+        return hash("slice")
+
+
+def type_key(t):
+    return t.name if isinstance(t, Scalar) else t.key()
+
+
+SMALL_DIM = 8      # trailing dimensions up to this extent become constants
+
+
+def type_of_argument(value, specialize=False):
+    """Type of a launch argument (the unboxing of the reference's dispatcher).
+    With ``specialize`` a device array also reports a dense row-major layout
+    and the extents of its short non-leading dimensions."""
+    if hasattr(value, "dtype") and hasattr(value, "ndim") and hasattr(value, "elem_strides"):
+        if specialize and value.ndim >= 1:
+            dense = bool(getattr(value, "is_c_contiguous", lambda: False)()) and \
+                all(n > 0 for n in value.shape)
+            const = [None] + [int(n) if 0 < n <= SMALL_DIM else None
+                              for n in value.shape[1:]]
+            return Array(scalar_of(value.dtype), value.ndim,
+                         layout="C" if dense else "A", const_shape=const)
+        return Array(scalar_of(value.dtype), value.ndim)
+    if isinstance(value, slice):
+        return SliceArg()
+    if isinstance(value, (bool, np.bool_)):
+        return BOOL
+    if isinstance(value, np.generic):
+        return scalar_of(value.dtype)
+    if isinstance(value, int):
+        return INT64
+    if isinstance(value, float):
+        return FLOAT64
+    raise KernelCompileError(f"Unsupported kernel argument type: {type(value)}")
+
+
+class Val:
+    """A typed expression: C++ text, type, and what is known at compile time."""
+
+    def __init__(self, code, type_, const=None, nonneg=False, items=None, pyobj=None,
+                 slice_parts=None):
+        self.code, self.type = code, type_
+        self.const = const            # Python value of a compile-time constant
+        self.nonneg = nonneg or (isinstance(const, (int, float)) and not
+                                 isinstance(const, bool) and const >= 0)
+        self.items = items            # tuple expression: list of Val
+        self.pyobj = pyobj            # a Python object known at compile time
+        self.slice_parts = slice_parts  # (start, stop, step) Vals or None each
+
+
+class _Deferred(Exception):
+    """A name is used before its type is known (resolved by a later pass)."""
+
+
+_UNARY_MATH = {
+    # python name -> C name; results are float32 for float32 input, else float64
+    "sqrt": "sqrt", "exp": "exp", "log": "log", "log2": "log2", "log10": "log10",
+    "log1p": "log1p", "expm1": "expm1", "sin": "sin", "cos": "cos", "tan": "tan",
+    "asin": "asin", "acos": "acos", "atan": "atan", "sinh": "sinh", "cosh": "cosh",
+    "tanh": "tanh", "asinh": "asinh", "acosh": "acosh", "atanh": "atanh",
+    "erf": "erf", "erfc": "erfc", "gamma": "tgamma", "lgamma": "lgamma",
+    "fabs": "fabs", "arcsin": "asin", "arccos": "acos", "arctan": "atan",
+    "arcsinh": "asinh", "arccosh": "acosh", "arctanh": "atanh", "exp2": "exp2",
+    "cbrt": "cbrt", "absolute": "fabs",
+}
+_BINARY_MATH = {"atan2": "atan2", "arctan2": "atan2", "pow": "pow", "power": "pow",
+                "hypot": "hypot", "copysign": "copysign", "fmod": "fmod"}
+_ROUNDING = {"floor": "floor", "ceil": "ceil", "trunc": "trunc"}
+
+_CAST_TYPES = {
+    bool: BOOL, int: INT64, float: FLOAT64, np.bool_: BOOL, np.int8: INT8,
+    np.int16: INT16, np.int32: INT32, np.int64: INT64, np.uint8: UINT8,
+    np.uint16: UINT16, np.uint32: UINT32, np.uint64: UINT64,
+    np.float32: FLOAT32, np.float64: FLOAT64,
+}
+
+_GROUP_NEUTRAL = {
+    "add": lambda t: "0",
+    "mul": lambda t: "1",
+    "min": lambda t: _type_limit(t, True),
+    "max": lambda t: _type_limit(t, False),
+}
+_GROUP_OPS = {"add": "AddOp", "mul": "MulOp", "min": "MinOp", "max": "MaxOp"}
+
+
+def _type_limit(t, largest):
+    if t.is_float:
+        return "__builtin_inf()" if largest else "-__builtin_inf()"
+    info = np.iinfo(t.dtype)
+    v = info.max if largest else info.min
+    if t is INT64 and not largest:
+        return "INT64_MIN"
+    suffix = "ull" if t is UINT64 else "ll"
+    return f"{v}{suffix}"
+
+
+def _float_literal(v, t):
+    if math.isnan(v):
+        return "__builtin_nan(\"\")" if t is FLOAT64 else "__builtin_nanf(\"\")"
+    if math.isinf(v):
+        s = "__builtin_inf()" if t is FLOAT64 else "__builtin_inff()"
+        return s if v > 0 else "-" + s
+    text = float(v).hex()
+    return text if t is FLOAT64 else text + "f"
+
+
+def cast(val, to):
+    if val.type is to:
+        return val
+    if val.const is not None:
+        return constant(_convert_const(val.const, to), to)
+    return Val(f"(({to.ctype})({val.code}))", to, nonneg=val.nonneg and not to.is_bool)
+
+
+def _convert_const(v, to):
+    if to.is_bool:
+        return bool(v)
+    if to.is_float:
+        return float(to.dtype.type(v))
+    if isinstance(v, float):
+        v = int(v) if math.isfinite(v) else 0
+    return int(np.array(int(v), dtype=np.int64 if -2 ** 63 <= int(v) < 2 ** 63
+                        else np.uint64).astype(to.dtype))
+
+
+def constant(v, t=None):
+    if isinstance(v, (bool, np.bool_)):
+        t = t or BOOL
+    elif isinstance(v, (int, np.integer)):
+        t = t or (scalar_of(v.dtype) if isinstance(v, np.generic) else INT64)
+    elif isinstance(v, (float, np.floating)):
+        t = t or (scalar_of(v.dtype) if isinstance(v, np.generic) else FLOAT64)
+    else:
+        raise KernelCompileError(f"Unsupported constant: {v!r}")
+    if t.is_bool:
+        v = bool(v)
+        return Val("true" if v else "false", t, const=v)
+    if t.is_float:
+        v = float(v)
+        return Val(_float_literal(v, t), t, const=v)
+    v = int(v)
+    if t is INT64 and v == -2 ** 63:
+        code = "INT64_MIN"
+    elif t in (INT64,):
+        code = f"((int64_t){v}ll)"
+    elif t is UINT64:
+        code = f"((uint64_t){v}ull)"
+    else:
+        code = f"(({t.ctype}){v})"
+    return Val(code, t, const=v)
+
+
+# ---------------------------------------------------------------------------
+# Module: everything that ends up in one generated source file
+# ---------------------------------------------------------------------------
+
+class Module:
+    def __init__(self, stubs, boundscheck=False):
+        self.stubs = stubs              # kernel_impl module (the stub objects)
+        self.boundscheck = boundscheck  # redirect and report out-of-range indices
+        # set when the body can tell how work-items are grouped (local or
+        # group ids, local sizes, barriers, fences, local arrays, group
+        # reductions): only then does the item-to-lane mapping matter
+        self.communicates = False
+        self.device_funcs = {}          # (id(func), arg type keys) -> (name, ret type)
+        self.device_code = []
+        self.in_progress = set()
+        self.counter = 0
+
+    def fresh(self, prefix):
+        self.counter += 1
+        return f"{prefix}{self.counter}"
+
+
+def _function_ast(func):
+    """The FunctionDef or Lambda node of a Python function object."""
+    try:
+        src = inspect.getsource(func)
+    except (OSError, TypeError) as exc:
+        raise KernelCompileError(
+            f"No source available for {getattr(func, '__name__', func)!r}: {exc}")
+    src = textwrap.dedent(src)
+    try:
+        tree = ast.parse(src)
+    except SyntaxError:
+        # the source lines of a lambda need not be a statement on their own
+        # (a dictionary entry, an argument): parse from each `lambda` keyword
+        found = []
+        start = src.find("lambda")
+        while start >= 0:
+            for end in range(len(src), start + 6, -1):
+                try:
+                    node = ast.parse(src[start:end].strip().rstrip(","), mode="eval").body
+                except SyntaxError:
+                    continue
+                if isinstance(node, ast.Lambda):
+                    found.append(node)
+                    break
+            start = src.find("lambda", start + 6)
+        tree = ast.Module(body=[ast.Expr(value=n) for n in found], type_ignores=[])
+    name = func.__name__
+    if name == "<lambda>":
+        lambdas = [n for n in ast.walk(tree) if isinstance(n, ast.Lambda)]
+        nargs = func.__code__.co_argcount
+        names = func.__code__.co_varnames[:nargs]
+        match = [n for n in lambdas if [a.arg for a in n.args.args] == list(names)]
+        if len(match) != 1:
+            # same parameter names: tell them apart by the names they use
+            used = set(func.__code__.co_names) | set(func.__code__.co_freevars)
+            match = [n for n in match if {x.id for x in ast.walk(n.body)
+                                          if isinstance(x, ast.Name)} - set(names) == used]
+        if len(match) != 1:
+            raise KernelCompileError(
+                "Cannot tell which lambda of the source line is meant; put each "
+                "lambda on a line of its own")
+        return match[0]
+    for n in ast.walk(tree):
+        if isinstance(n, (ast.FunctionDef,)) and n.name == name:
+            return n
+    raise KernelCompileError(f"Cannot find the definition of {name}")
+
+
+class FunctionTranslator:
+    def __init__(self, module, func, arg_types, is_kernel, ndim=0):
+        self.m = module
+        self.func = func
+        self.is_kernel = is_kernel
+        self.ndim = ndim
+        self.node = _function_ast(func)
+        args = self.node.args
+        if args.vararg or args.kwarg or args.kwonlyargs or args.defaults:
+            raise KernelCompileError("Only plain positional parameters are supported")
+        self.params = [a.arg for a in args.args]
+        if len(self.params) != len(arg_types):
+            raise KernelCompileError(
+                f"{func.__name__} takes {len(self.params)} arguments, {len(arg_types)} given")
+        self.arg_types = list(arg_types)
+        cv = inspect.getclosurevars(func)
+        self.outer = {}
+        self.outer.update(cv.builtins)
+        self.outer.update(cv.globals)
+        self.outer.update(cv.nonlocals)
+        # names that inspect does not report (used only inside nested scopes)
+        self.func_globals = getattr(func, "__globals__", {})
+        self.env = dict(zip(self.params, self.arg_types))   # name -> type
+        self.assigned = self._assigned_names()
+        self.ret_type = None
+        self.lines = []
+        self.indent = 1
+        self.emitting = False
+        self.local_arrays = []       # (elem Scalar, shape tuple) in source order
+        self.group_sites = []        # (slot name, Scalar, op)
+        self.private_decls = []
+        self.allow_remap = False     # kernels only: see translate_kernel
+        self.reversed = False
+        self.site_names = {}         # ast node -> stable names
+        self.array_info = {}         # variable name -> Array type (views)
+
+    # -- helpers -----------------------------------------------------------
+    def err(self, node, msg):
+        line = getattr(node, "lineno", "?")
+        raise KernelCompileError(f"{self.func.__name__}, line {line}: {msg}")
+
+    def _assigned_names(self):
+        names = set()
+        self.store_count = {}
+        body = self.node.body if isinstance(self.node.body, list) else []
+        for n in ast.walk(ast.Module(body=body, type_ignores=[])):
+            if isinstance(n, ast.Name) and isinstance(n.ctx, ast.Store):
+                names.add(n.id)
+                self.store_count[n.id] = self.store_count.get(n.id, 0) + 1
+        # a name bound once, at the top level, to a constant is that constant
+        # (array shapes and range bounds written through a local name)
+        self.const_vars = {}
+        self.top_level = {id(s) for s in body}
+        return names - set(self.params)
+
+    def emit(self, text):
+        if self.emitting:
+            self.lines.append("  " * self.indent + text)
+
+    def cname(self, name):
+        return f"v_{name}"
+
+    # -- name resolution ---------------------------------------------------
+    def lookup(self, node):
+        name = node.id
+        if name in self.env:
+            t = self.env[name]
+            if isinstance(t, Scalar):
+                if name in self.const_vars:
+                    return constant(_convert_const(self.const_vars[name], t), t)
+                return Val(self.cname(name), t, nonneg=name in self.nonneg_vars)
+            if isinstance(t, Array):
+                return Val(self.cname(name), t)
+            if isinstance(t, SliceArg):
+                c = self.cname(name)
+                parts = tuple(Val(f"{c}_{k}", INT64) for k in ("start", "stop", "step"))
+                return Val(c, t, slice_parts=parts)
+            if isinstance(t, tuple) and t[0] == "tuple":
+                return Val(None, t, items=self.tuple_vars[name])
+            raise KernelCompileError(f"Unsupported variable type for {name}")
+        if name in self.params or name in self.assigned:
+            raise _Deferred(name)
+        if name in self.outer:
+            return self.from_python(self.outer[name], node)
+        if name in self.func_globals:
+            return self.from_python(self.func_globals[name], node)
+        import builtins
+        if hasattr(builtins, name):
+            return self.from_python(getattr(builtins, name), node)
+        self.err(node, f"Unknown name '{name}'")
+
+    def from_python(self, obj, node):
+        if isinstance(obj, (bool, int, float, np.generic)) and not isinstance(obj, complex):
+            return constant(obj)
+        if isinstance(obj, tuple) and all(isinstance(x, (int, np.integer)) for x in obj):
+            return Val(None, ("tuple",), items=[constant(int(x)) for x in obj])
+        return Val(None, None, pyobj=obj)
+
+    # -- expressions -------------------------------------------------------
+    def expr(self, node):
+        method = getattr(self, "expr_" + type(node).__name__, None)
+        if method is None:
+            self.err(node, f"Unsupported expression: {type(node).__name__}")
+        return method(node)
+
+    def scalar(self, node):
+        v = self.expr(node)
+        if not isinstance(v.type, Scalar):
+            self.err(node, "A scalar value is required here")
+        return v
+
+    def expr_Constant(self, node):
+        v = node.value
+        if v is None:
+            return Val(None, None, pyobj=None)
+        if isinstance(v, (bool, int, float)):
+            return constant(v)
+        self.err(node, f"Unsupported constant {v!r}")
+
+    def expr_Name(self, node):
+        return self.lookup(node)
+
+    def extent(self, base, k):
+        known = base.type.const_shape[k]
+        if known is not None:
+            return constant(known)
+        return Val(f"{base.code}.shape[{k}]", INT64, nonneg=True)
+
+    def expr_Attribute(self, node):
+        base = self.expr(node.value)
+        if isinstance(base.type, Array):
+            if node.attr == "shape":
+                items = [self.extent(base, k) for k in range(base.type.ndim)]
+                return Val(None, ("tuple",), items=items)
+            if node.attr == "ndim":
+                return constant(base.type.ndim)
+            if node.attr == "size":
+                code = " * ".join(self.extent(base, k).code for k in range(base.type.ndim))
+                return Val(f"({code})", INT64, nonneg=True)
+            self.err(node, f"Unsupported array attribute '{node.attr}'")
+        if base.type is None and base.pyobj is not None:
+            try:
+                return self.from_python(getattr(base.pyobj, node.attr), node)
+            except AttributeError:
+                self.err(node, f"{base.pyobj!r} has no attribute '{node.attr}'")
+        self.err(node, f"Unsupported attribute access '.{node.attr}'")
+
+    def expr_Tuple(self, node):
+        return Val(None, ("tuple",), items=[self.expr(e) for e in node.elts])
+
+    def expr_Slice(self, node):
+        parts = tuple(self.scalar(p) if p is not None else None
+                      for p in (node.lower, node.upper, node.step))
+        return Val(None, SliceArg(), slice_parts=parts)
+
+    def expr_UnaryOp(self, node):
+        v = self.scalar(node.operand)
+        if isinstance(node.op, ast.Not):
+            b = self.truth(v)
+            if b.const is not None:
+                return constant(not b.const)
+            return Val(f"(!{b.code})", BOOL)
+        if isinstance(node.op, ast.UAdd):
+            return cast(v, INT64) if v.type.is_bool else v
+        if isinstance(node.op, ast.USub):
+            if v.type.is_bool:
+                v = cast(v, INT64)
+            if v.const is not None:
+                return constant(-v.const, v.type)
+            return Val(f"(-{v.code})", v.type)
+        if isinstance(node.op, ast.Invert):
+            if v.type.is_float:
+                self.err(node, "~ needs an integer")
+            if v.type.is_bool:
+                v = cast(v, INT64)
+            return Val(f"(~{v.code})", v.type)
+        self.err(node, "Unsupported unary operator")
+
+    def truth(self, v):
+        if v.type.is_bool:
+            return v
+        if v.const is not None:
+            return constant(bool(v.const))
+        return Val(f"({v.code} != 0)", BOOL)
+
+    def expr_BoolOp(self, node):
+        vals = [self.truth(self.scalar(e)) for e in node.values]
+        op = " && " if isinstance(node.op, ast.And) else " || "
+        return Val("(" + op.join(v.code for v in vals) + ")", BOOL)
+
+    def expr_Compare(self, node):
+        ops = {ast.Lt: "<", ast.LtE: "<=", ast.Gt: ">", ast.GtE: ">=",
+               ast.Eq: "==", ast.NotEq: "!="}
+        left = self.scalar(node.left)
+        parts = []
+        for op, right_node in zip(node.ops, node.comparators):
+            right = self.scalar(right_node)
+            if type(op) not in ops:
+                self.err(node, "Unsupported comparison")
+            t = self.arith_type(left.type, right.type)
+            a, b = cast(left, t), cast(right, t)
+            parts.append(f"({a.code} {ops[type(op)]} {b.code})")
+            left = right
+        return Val("(" + " && ".join(parts) + ")", BOOL)
+
+    def arith_type(self, a, b):
+        t = promote(a, b)
+        return INT64 if t.is_bool else t
+
+    def expr_IfExp(self, node):
+        c = self.truth(self.scalar(node.test))
+        a, b = self.scalar(node.body), self.scalar(node.orelse)
+        t = promote(a.type, b.type)
+        return Val(f"({c.code} ? {cast(a, t).code} : {cast(b, t).code})", t,
+                   nonneg=a.nonneg and b.nonneg)
+
+    def expr_BinOp(self, node):
+        return self.binop(node.op, self.scalar(node.left), self.scalar(node.right), node)
+
+    def binop(self, op, a, b, node):
+        t = self.arith_type(a.type, b.type)
+        if isinstance(op, ast.Div):
+            if not t.is_float:
+                t = FLOAT64
+            x, y = cast(a, t), cast(b, t)
+            return Val(f"({x.code} / {y.code})", t, nonneg=a.nonneg and b.nonneg)
+        if isinstance(op, ast.Pow):
+            if t.is_float:
+                x, y = cast(a, t), cast(b, t)
+                return Val(f"pow({x.code}, {y.code})", t)
+            x, y = cast(a, t), cast(b, t)
+            return Val(f"nmkjit::powInt<{t.ctype}>({x.code}, {y.code})", t,
+                       nonneg=a.nonneg)
+        if isinstance(op, (ast.BitAnd, ast.BitOr, ast.BitXor, ast.LShift, ast.RShift)):
+            if t.is_float:
+                self.err(node, "Bitwise operators need integers")
+            if a.type.is_bool and b.type.is_bool and not isinstance(op, (ast.LShift, ast.RShift)):
+                t = BOOL
+            sym = {ast.BitAnd: "&", ast.BitOr: "|", ast.BitXor: "^", ast.LShift: "<<",
+                   ast.RShift: ">>"}[type(op)]
+            x, y = cast(a, t), cast(b, t)
+            return Val(f"(({t.ctype})({x.code} {sym} {y.code}))", t,
+                       nonneg=a.nonneg and b.nonneg)
+        x, y = cast(a, t), cast(b, t)
+        if isinstance(op, (ast.Add, ast.Sub, ast.Mult)):
+            sym = {ast.Add: "+", ast.Sub: "-", ast.Mult: "*"}[type(op)]
+            if x.const is not None and y.const is not None and t.is_int:
+                r = {"+": x.const + y.const, "-": x.const - y.const,
+                     "*": x.const * y.const}[sym]
+                if -2 ** 63 <= r < 2 ** 63:
+                    return constant(r, t)
+            nonneg = a.nonneg and b.nonneg and sym != "-"
+            code = f"({x.code} {sym} {y.code})"
+            if t.dtype.itemsize < 4:      # C promotes narrow integers to int
+                code = f"(({t.ctype}){code})"
+            return Val(code, t, nonneg=nonneg)
+        if isinstance(op, ast.FloorDiv):
+            if t.is_float:
+                return Val(f"nmkjit::floordivFloat<{t.ctype}>({x.code}, {y.code})", t)
+            if x.const is not None and y.const is not None and y.const != 0:
+                return constant(x.const // y.const, t)
+            if a.nonneg and b.nonneg and y.const:
+                return Val(f"({x.code} / {y.code})", t, nonneg=True)
+            return Val(f"nmkjit::floordivInt<{t.ctype}>({x.code}, {y.code})", t,
+                       nonneg=a.nonneg and b.nonneg)
+        if isinstance(op, ast.Mod):
+            if t.is_float:
+                return Val(f"nmkjit::modFloat<{t.ctype}>({x.code}, {y.code})", t,
+                           nonneg=b.nonneg)
+            if x.const is not None and y.const is not None and y.const != 0:
+                return constant(x.const % y.const, t)
+            if a.nonneg and b.nonneg and y.const:
+                return Val(f"({x.code} % {y.code})", t, nonneg=True)
+            return Val(f"nmkjit::modInt<{t.ctype}>({x.code}, {y.code})", t, nonneg=b.nonneg)
+        self.err(node, f"Unsupported operator {type(op).__name__}")
+
+    # -- indexing ----------------------------------------------------------
+    def index_items(self, node):
+        v = self.expr(node)
+        return v.items if v.items is not None else [v]
+
+    def normalise_index(self, idx, base, dim):
+        idx = cast(idx, INT64) if idx.type is not INT64 else idx
+        if idx.const is not None:
+            if idx.const < 0:
+                idx = Val(f"({base.code}.shape[{dim}] + {idx.code})", INT64)
+        elif not idx.nonneg:
+            idx = Val(f"nmkjit::wrap({idx.code}, {base.code}.shape[{dim}])", INT64)
+        if self.m.boundscheck:
+            idx = Val(f"nmkjit::checked({idx.code}, {base.code}.shape[{dim}], nmk_oob)",
+                      INT64, nonneg=True)
+        return idx
+
+    def subscript(self, node):
+        """Returns ("elem", lvalue code, elem type) or ("view", Val)."""
+        base = self.expr(node.value)
+        if base.items is not None:            # tuple[constant]
+            k = self.expr(node.slice)
+            if k.const is None:
+                self.err(node, "A tuple can only be indexed by a constant")
+            return ("value", base.items[k.const])
+        if not isinstance(base.type, Array):
+            self.err(node, "Only arrays and tuples can be indexed")
+        items = self.index_items(node.slice)
+        ndim = base.type.ndim
+        if len(items) > ndim:
+            self.err(node, f"Too many indices for a {ndim}-d array")
+        if all(isinstance(i.type, Scalar) for i in items) and len(items) == ndim:
+            terms = []
+            for d, i in enumerate(items):
+                i = self.normalise_index(i, base, d)
+                terms.append(f"{i.code} * {base.code}.stride[{d}]")
+            return ("elem", f"{base.code}.p[{' + '.join(terms)}]", base.type.elem)
+        # a view: integers drop a dimension, slices keep it
+        cur, cur_t, dim = base.code, base.type, 0
+        for i in items:
+            if isinstance(i.type, Scalar):
+                i = self.normalise_index(i, Val(cur, cur_t), dim)
+                cur = f"nmkjit::subAt({cur}, {dim}, {i.code})"
+                cur_t = Array(cur_t.elem, cur_t.ndim - 1, cur_t.space)
+            elif isinstance(i.type, SliceArg):
+                parts = [cast(p, INT64).code if p is not None else "nmkjit::kNone"
+                         for p in i.slice_parts]
+                cur = f"nmkjit::slice({cur}, {dim}, {', '.join(parts)})"
+                dim += 1
+            else:
+                self.err(node, "Unsupported index")
+        if cur_t.ndim == 0:
+            self.err(node, "Too many indices")
+        return ("view", Val(cur, cur_t))
+
+    def expr_Subscript(self, node):
+        kind, *rest = self.subscript(node)
+        if kind == "elem":
+            code, elem = rest
+            return Val(code, elem)
+        return rest[0]
+
+    # -- calls -------------------------------------------------------------
+    def expr_Call(self, node):
+        fn = self.expr(node.func)
+        if fn.type is not None or fn.pyobj is None:
+            self.err(node, "Only functions known at compile time can be called")
+        obj = fn.pyobj
+        kwargs = {k.arg: k.value for k in node.keywords}
+        stubs = self.m.stubs
+        ids = {
+            stubs.get_global_id: ("gid", True), stubs.get_local_id: ("lid", True),
+            stubs.get_group_id: ("grp", True), stubs.get_global_size: ("gsz", True),
+            stubs.get_local_size: ("lsz", True),
+        }
+        if inspect.isfunction(obj) and obj in ids:
+            axis = self.expr(node.args[0])
+            if axis.const is None or not 0 <= axis.const <= 2:
+                self.err(node, "The axis must be a constant 0, 1 or 2")
+            if ids[obj][0] in ("lid", "grp", "lsz"):
+                self.m.communicates = True
+            return Val(f"nmk_{ids[obj][0]}{axis.const}", INT64, nonneg=True)
+        if obj is stubs.atomic.add or obj is stubs.atomic.sub:
+            return self.call_atomic(node, obj is stubs.atomic.sub)
+        if obj is stubs.barrier or obj is stubs.mem_fence:
+            self.m.communicates = True
+            flags = node.args[0] if node.args else kwargs.get("flags")
+            if flags is not None:
+                f = self.expr(flags)
+                if f.const is None and not (f.type is None and f.pyobj is None):
+                    self.err(node, "The fence flags must be a constant")
+            self.emit("__syncthreads();" if obj is stubs.barrier else
+                      "__threadfence_block();")
+            return Val(None, None, pyobj=None)
+        if obj is stubs.local.array or obj is stubs.private.array:
+            self.err(node, "local.array / private.array must be assigned to a variable")
+        for opname in _GROUP_OPS:
+            if obj is getattr(stubs.group, "reduce_" + opname):
+                return self.call_group(node, opname)
+        if obj is stubs.kernel_func:
+            self.err(node, "kernel_func cannot be called inside a kernel")
+        if isinstance(obj, type) and obj in _CAST_TYPES:
+            if len(node.args) != 1:
+                self.err(node, "A cast takes one argument")
+            return cast(self.scalar(node.args[0]), _CAST_TYPES[obj])
+        if obj is abs or obj is np.abs or obj is np.absolute or obj is math.fabs:
+            v = self.scalar(node.args[0])
+            if obj is math.fabs and not v.type.is_float:
+                v = cast(v, FLOAT64)
+            if v.type.is_float:
+                return Val(f"fabs({v.code})", v.type, nonneg=True)
+            if v.type.is_bool or v.type.kind == "u":
+                return v
+            return Val(f"({v.code} < 0 ? ({v.type.ctype})(-{v.code}) : {v.code})", v.type,
+                       nonneg=True)
+        if any(obj is f for f in (min, max, np.minimum, np.maximum)):
+            vals = [self.scalar(a) for a in node.args]
+            if len(vals) < 2:
+                self.err(node, "min/max need at least two scalar arguments")
+            is_min = obj is min or obj is np.minimum
+            acc = vals[0]
+            for v in vals[1:]:
+                t = promote(acc.type, v.type)
+                a, b = cast(acc, t), cast(v, t)
+                cmp = "<" if is_min else ">"
+                # Python keeps the first of equal arguments
+                acc = Val(f"({b.code} {cmp} {a.code} ? {b.code} : {a.code})", t,
+                          nonneg=(acc.nonneg and v.nonneg) if is_min else
+                          (acc.nonneg or v.nonneg))
+            return acc
+        if obj is len:
+            v = self.expr(node.args[0])
+            if isinstance(v.type, Array):
+                return self.extent(v, 0)
+            if v.items is not None:
+                return constant(len(v.items))
+            self.err(node, "len() needs an array or a tuple")
+        if obj is range:
+            self.err(node, "range() is only supported as the iterable of a for loop")
+        name = getattr(obj, "__name__", None)
+        mod = getattr(obj, "__module__", None)
+        is_np = isinstance(obj, np.ufunc) or mod == "numpy"
+        if (mod == "math" or is_np) and name in _UNARY_MATH and len(node.args) == 1:
+            v = self.scalar(node.args[0])
+            t = FLOAT32 if v.type is FLOAT32 else FLOAT64
+            v = cast(v, t)
+            if name == "sqrt" and t is FLOAT64:
+                # same rounding as the library routine at half its cost
+                return Val(f"nmk::sqrtF64({v.code})", t, nonneg=True)
+            return Val(f"{_UNARY_MATH[name]}({v.code})", t)
+        if (mod == "math" or is_np) and name in _ROUNDING and len(node.args) == 1:
+            v = self.scalar(node.args[0])
+            if not v.type.is_float:
+                return cast(v, INT64) if mod == "math" else cast(v, FLOAT64)
+            r = Val(f"{_ROUNDING[name]}({v.code})", v.type)
+            return cast(r, INT64) if mod == "math" else r
+        if (mod == "math" or is_np) and name in _BINARY_MATH and len(node.args) == 2:
+            a, b = self.scalar(node.args[0]), self.scalar(node.args[1])
+            t = promote(a.type, b.type)
+            t = t if t.is_float else FLOAT64
+            return Val(f"{_BINARY_MATH[name]}({cast(a, t).code}, {cast(b, t).code})", t)
+        if mod == "math" and name in ("isnan", "isinf", "isfinite") or \
+                is_np and name in ("isnan", "isinf", "isfinite"):
+            v = self.scalar(node.args[0])
+            if not v.type.is_float:
+                return constant(name == "isfinite")
+            return Val(f"(bool)__builtin_{name}({v.code})", BOOL)
+        if inspect.isfunction(obj):
+            return self.call_device(node, obj)
+        self.err(node, f"Unsupported call target {obj!r}")
+
+    def call_atomic(self, node, negate):
+        if len(node.args) != 3:
+            self.err(node, "atomic.add/sub take (array, index, value)")
+        arr = self.expr(node.args[0])
+        if not isinstance(arr.type, Array):
+            self.err(node, "The first argument of an atomic must be an array")
+        elem = arr.type.elem
+        if elem not in (INT32, INT64, FLOAT32, FLOAT64):
+            self.err(node, f"Atomics on {elem} are not supported")
+        items = self.index_items(node.args[1])
+        if len(items) != arr.type.ndim:
+            self.err(node, "An atomic needs a full index")
+        terms = []
+        for d, i in enumerate(items):
+            i = self.normalise_index(i, arr, d)
+            terms.append(f"{i.code} * {arr.code}.stride[{d}]")
+        val = cast(self.scalar(node.args[2]), elem)
+        v = f"(-{val.code})" if negate else val.code
+        return Val(f"nmkjit::atomicAddT(&{arr.code}.p[{' + '.join(terms)}], "
+                   f"({elem.ctype}){v})", elem)
+
+    def call_group(self, node, opname):
+        self.m.communicates = True
+        if not self.is_kernel:
+            self.err(node, "group reductions are only supported in the kernel body")
+        v = self.scalar(node.args[0])
+        t = INT64 if v.type.is_bool else v.type
+        if t.dtype.itemsize < 4:
+            t = INT32 if t.kind == "i" else UINT32
+        v = cast(v, t)
+        if node not in self.site_names:
+            self.site_names[node] = self.m.fresh("nmk_group")
+        slot = self.site_names[node]
+        if self.emitting and all(s[0] != slot for s in self.group_sites):
+            neutral = _GROUP_NEUTRAL[opname](t)
+            if t is FLOAT32 and "inf" in neutral:
+                neutral = neutral.replace("__builtin_inf()", "__builtin_inff()")
+            self.group_sites.append((slot, t, neutral))
+        tmp = self.m.fresh("nmk_t")
+        self.emit(f"const {t.ctype} {tmp} = nmkjit::groupReduce({slot}, {v.code}, "
+                  f"nmk_clipped != 0, nmkjit::{_GROUP_OPS[opname]}());")
+        return Val(tmp, t)
+
+    def call_device(self, node, obj):
+        if node.keywords:
+            self.err(node, "Keyword arguments are not supported in device calls")
+        args = [self.expr(a) for a in node.args]
+        for a in args:
+            if not isinstance(a.type, (Scalar, Array)):
+                self.err(node, "Device functions take scalars and arrays")
+        key = (obj, tuple(type_key(a.type) for a in args))
+        if key in self.m.in_progress:
+            self.err(node, "Recursive device functions are not supported")
+        if key not in self.m.device_funcs:
+            self.m.in_progress.add(key)
+            try:
+                tr = FunctionTranslator(self.m, obj, [a.type for a in args], False)
+                name = self.m.fresh(f"nmk_dev_{_safe(obj.__name__)}_")
+                code, ret = tr.translate_device(name)
+            finally:
+                self.m.in_progress.discard(key)
+            self.m.device_funcs[key] = (name, ret)
+            self.m.device_code.append(code)
+        name, ret = self.m.device_funcs[key]
+        actual = [a.code for a in args] + (["nmk_oob"] if self.m.boundscheck else [])
+        call = f"{name}({', '.join(actual)})"
+        if ret is None:
+            self.emit(call + ";")
+            return Val(None, None, pyobj=None)
+        return Val(call, ret)
+
+    # -- statements --------------------------------------------------------
+    def stmt(self, node):
+        method = getattr(self, "stmt_" + type(node).__name__, None)
+        if method is None:
+            self.err(node, f"Unsupported statement: {type(node).__name__}")
+        try:
+            method(node)
+        except _Deferred:
+            if self.emitting:
+                raise
+            self.deferred = True
+
+    def block(self, stmts):
+        self.indent += 1
+        for s in stmts:
+            self.stmt(s)
+        self.indent -= 1
+
+    def stmt_Pass(self, node):
+        pass
+
+    def stmt_Expr(self, node):
+        if isinstance(node.value, ast.Constant):
+            return                                     # docstring
+        v = self.expr(node.value)
+        if v.code is not None and isinstance(v.type, Scalar):
+            self.emit(f"(void)({v.code});")
+
+    def bind(self, name, t, node):
+        """Records that ``name`` receives a value of type ``t``."""
+        old = self.env.get(name)
+        if name in self.params and not isinstance(old, Scalar):
+            self.err(node, f"Cannot rebind the array argument '{name}'")
+        if isinstance(t, Scalar):
+            if old is None:
+                new = t
+            elif isinstance(old, Scalar):
+                new = promote(old, t)
+            else:
+                self.err(node, f"'{name}' is used both as a scalar and as an array")
+            if new is not old:
+                self.env[name] = new
+                self.changed = True
+        else:
+            if isinstance(old, Scalar):
+                self.err(node, f"'{name}' is used both as a scalar and as an array")
+            if old is not None and old != t:
+                self.err(node, f"'{name}' is bound to arrays of different types")
+            if old is None:
+                self.env[name] = t
+                self.changed = True
+
+    def special_array_call(self, value):
+        """local.array / private.array call nodes, else None."""
+        if not isinstance(value, ast.Call):
+            return None
+        try:
+            fn = self.expr(value.func)
+        except (_Deferred, KernelCompileError):
+            return None
+        stubs = self.m.stubs
+        if fn.pyobj is stubs.local.array:
+            return "local"
+        if fn.pyobj is stubs.private.array:
+            return "private"
+        return None
+
+    def array_alloc(self, name, node, space):
+        call = node.value
+        args = list(call.args)
+        kwargs = {k.arg: k.value for k in call.keywords}
+        shape_node = args[0] if args else kwargs.get("shape")
+        dtype_node = args[1] if len(args) > 1 else kwargs.get("dtype")
+        if shape_node is None or dtype_node is None:
+            self.err(node, "array(shape, dtype) needs both arguments")
+        shape = self.expr(shape_node)
+        dims = shape.items if shape.items is not None else [shape]
+        if any(d.const is None or isinstance(d.const, float) for d in dims):
+            self.err(node, "The shape of a local or private array must be constant")
+        dims = tuple(int(d.const) for d in dims)
+        if isinstance(dtype_node, ast.Constant) and isinstance(dtype_node.value, str):
+            elem = scalar_of(dtype_node.value)
+        else:
+            dt = self.expr(dtype_node)
+            if dt.pyobj is None:
+                self.err(node, "The dtype must be a NumPy type or its name")
+            elem = scalar_of(dt.pyobj)
+        t = Array(elem, len(dims), space)
+        self.bind(name, t, node)
+        if not self.emitting:
+            return
+        strides = []
+        acc = 1
+        for d in reversed(dims):
+            strides.insert(0, acc)
+            acc *= d
+        total = acc
+        shape_c = ", ".join(str(d) for d in dims)
+        stride_c = ", ".join(str(s) for s in strides)
+        c = self.cname(name)
+        if space == "local":
+            self.m.communicates = True
+            if not self.is_kernel:
+                self.err(node, "local.array is only supported in the kernel body")
+            k = len(self.local_arrays)
+            self.local_arrays.append((elem, dims))
+            self.emit(f"{c} = {{reinterpret_cast<{elem.ctype} *>(nmk_dyn_lds + nmk_lds{k}), "
+                      f"{{{shape_c}}}, {{{stride_c}}}}};")
+        else:
+            store = self.m.fresh("nmk_priv")
+            self.private_decls.append(f"{elem.ctype} {store}[{max(total, 1)}] = {{}};")
+            self.emit(f"{c} = {{{store}, {{{shape_c}}}, {{{stride_c}}}}};")
+
+    def stmt_Assign(self, node):
+        if len(node.targets) != 1:
+            self.err(node, "Chained assignment is not supported")
+        target = node.targets[0]
+        if isinstance(target, ast.Name):
+            space = self.special_array_call(node.value)
+            if space:
+                return self.array_alloc(target.id, node, space)
+            v = self.expr(node.value)
+            self.assign_name(target.id, v, node)
+        elif isinstance(target, ast.Subscript):
+            v = self.expr(node.value)
+            self.assign_subscript(target, v, node)
+        elif isinstance(target, ast.Tuple):
+            v = self.expr(node.value)
+            if v.items is None or len(v.items) != len(target.elts):
+                self.err(node, "Tuple assignment needs a tuple of the same length")
+            if not all(isinstance(e, ast.Name) for e in target.elts):
+                self.err(node, "Only names can be unpacked into")
+            # evaluate everything first (a, b = b, a)
+            tmps = []
+            for e, item in zip(target.elts, v.items):
+                if isinstance(item.type, Scalar) and self.emitting:
+                    tmp = self.m.fresh("nmk_t")
+                    self.emit(f"const {item.type.ctype} {tmp} = {item.code};")
+                    item = Val(tmp, item.type, const=item.const, nonneg=item.nonneg)
+                tmps.append(item)
+            for e, item in zip(target.elts, tmps):
+                self.assign_name(e.id, item, node)
+        else:
+            self.err(node, "Unsupported assignment target")
+
+    def assign_name(self, name, v, node):
+        if v.items is not None:
+            if name in self.env and not (isinstance(self.env[name], tuple)):
+                self.err(node, f"'{name}' changes from a scalar to a tuple")
+            self.tuple_vars[name] = v.items
+            self.env[name] = ("tuple",)
+            return
+        if isinstance(v.type, SliceArg):
+            self.err(node, "Slices cannot be stored in variables")
+        if v.type is None:
+            self.err(node, "This value cannot be assigned to a variable")
+        self.bind(name, v.type, node)
+        if isinstance(v.type, Scalar):
+            if (v.const is not None and self.store_count.get(name) == 1 and
+                    id(node) in self.top_level and name not in self.params):
+                self.const_vars[name] = v.const
+            if not v.nonneg:
+                self.maybe_negative.add(name)
+            if self.emitting:
+                t = self.env[name]
+                self.emit(f"{self.cname(name)} = {cast(v, t).code};")
+        else:
+            self.emit(f"{self.cname(name)} = {v.code};")
+
+    def assign_subscript(self, target, v, node):
+        kind, *rest = self.subscript(target)
+        if kind != "elem":
+            self.err(node, "Only single elements can be assigned")
+        code, elem = rest
+        if not isinstance(v.type, Scalar):
+            self.err(node, "Only scalars can be stored into an array element")
+        self.emit(f"{code} = {cast(v, elem).code};")
+
+    def stmt_AugAssign(self, node):
+        if isinstance(node.target, ast.Name):
+            cur = self.expr(ast.Name(id=node.target.id, ctx=ast.Load(),
+                                     lineno=node.lineno, col_offset=0))
+            if not isinstance(cur.type, Scalar):
+                self.err(node, "Augmented assignment needs a scalar variable")
+            v = self.binop(node.op, cur, self.scalar(node.value), node)
+            self.assign_name(node.target.id, v, node)
+        elif isinstance(node.target, ast.Subscript):
+            kind, *rest = self.subscript(node.target)
+            if kind != "elem":
+                self.err(node, "Only single elements can be updated")
+            code, elem = rest
+            v = self.binop(node.op, Val(code, elem), self.scalar(node.value), node)
+            self.emit(f"{code} = {cast(v, elem).code};")
+        else:
+            self.err(node, "Unsupported augmented assignment target")
+
+    def stmt_If(self, node):
+        c = self.truth(self.scalar(node.test))
+        self.emit(f"if ({c.code}) {{")
+        self.block(node.body)
+        if node.orelse:
+            self.emit("} else {")
+            self.block(node.orelse)
+        self.emit("}")
+
+    def stmt_For(self, node):
+        if node.orelse:
+            self.err(node, "for ... else is not supported")
+        it = node.iter
+        if not (isinstance(it, ast.Call) and isinstance(it.func, ast.Name) and
+                it.func.id == "range" and it.func.id not in self.env and
+                not it.keywords and 1 <= len(it.args) <= 3):
+            self.err(node, "Only 'for x in range(...)' loops are supported")
+        if not isinstance(node.target, ast.Name):
+            self.err(node, "The loop variable must be a name")
+        a = [cast(self.scalar(x), INT64) for x in it.args]
+        start = a[0] if len(a) > 1 else constant(0)
+        stop = a[1] if len(a) > 1 else a[0]
+        step = a[2] if len(a) > 2 else constant(1)
+        name = node.target.id
+        self.bind(name, INT64, node)
+        if not (start.nonneg and step.const is not None and step.const > 0):
+            self.maybe_negative.add(name)
+        itv = self.m.fresh("nmk_it")
+        stopv, stepv = self.m.fresh("nmk_stop"), self.m.fresh("nmk_step")
+        self.emit("{")
+        self.indent += 1
+        self.emit(f"const int64_t {stopv} = {stop.code}, {stepv} = {step.code};")
+        if step.const is not None and step.const > 0:
+            cond = f"{itv} < {stopv}"
+        elif step.const is not None and step.const < 0:
+            cond = f"{itv} > {stopv}"
+        else:
+            cond = f"({stepv} > 0 ? {itv} < {stopv} : {itv} > {stopv})"
+        self.emit(f"for (int64_t {itv} = {start.code}; {cond}; {itv} += {stepv}) {{")
+        self.indent += 1
+        if self.emitting:
+            t = self.env[name]
+            self.emit(f"{self.cname(name)} = ({t.ctype}){itv};")
+        self.indent -= 1
+        self.block(node.body)
+        self.emit("}")
+        self.indent -= 1
+        self.emit("}")
+
+    def stmt_While(self, node):
+        if node.orelse:
+            self.err(node, "while ... else is not supported")
+        c = self.truth(self.scalar(node.test))
+        self.emit(f"while ({c.code}) {{")
+        self.block(node.body)
+        self.emit("}")
+
+    def stmt_Break(self, node):
+        self.emit("break;")
+
+    def stmt_Continue(self, node):
+        self.emit("continue;")
+
+    def stmt_Return(self, node):
+        if node.value is None or (isinstance(node.value, ast.Constant) and
+                                  node.value.value is None):
+            if not self.is_kernel and self.ret_type is not None:
+                self.err(node, "A device function must return a value on every path")
+            self.emit("return;")
+            return
+        if self.is_kernel:
+            self.err(node, "A kernel cannot return a value")
+        v = self.scalar(node.value)
+        new = v.type if self.ret_type is None else promote(self.ret_type, v.type)
+        if new is not self.ret_type:
+            self.ret_type = new
+            self.changed = True
+        self.emit(f"return {cast(v, self.ret_type).code};")
+
+    # -- driving -----------------------------------------------------------
+    def infer(self, body):
+        """Fixed point of the variable types."""
+        self.tuple_vars = {}
+        self.maybe_negative = set(self.params)
+        self.nonneg_vars = set()
+        for _ in range(12):
+            self.changed = False
+            self.deferred = False
+            self.emitting = False
+            for s in body:
+                self.stmt(s)
+            if not self.changed:
+                break
+        else:
+            raise KernelCompileError("Type inference did not converge")
+        missing = [n for n in self.assigned if n not in self.env]
+        if self.deferred and missing:
+            raise KernelCompileError(
+                f"{self.func.__name__}: cannot type {', '.join(sorted(missing))} "
+                "(used before assignment?)")
+        # Which integer variables can never be negative (their indices need no
+        # wrap-around): the greatest fixed point, starting from "all of them".
+        scalars = {n for n, t in self.env.items()
+                   if isinstance(t, Scalar) and n not in self.params}
+        self.nonneg_vars = set(scalars)
+        for _ in range(12):
+            self.maybe_negative = set(self.params)
+            for s in body:
+                self.stmt(s)
+            new = scalars - self.maybe_negative
+            if new == self.nonneg_vars:
+                break
+            self.nonneg_vars = new
+        else:
+            self.nonneg_vars = set()
+
+    def body_stmts(self):
+        if isinstance(self.node, ast.Lambda):
+            return [ast.Return(value=self.node.body, lineno=self.node.lineno,
+                               col_offset=0)]
+        return self.node.body
+
+    def declarations(self):
+        out = []
+        for name in sorted(self.assigned):
+            t = self.env.get(name)
+            if isinstance(t, Scalar):
+                out.append(f"{t.ctype} {self.cname(name)} = 0;")
+            elif isinstance(t, Array):
+                out.append(f"{t.ctype()} {self.cname(name)} = {{}};")
+        return out
+
+    def run_emit(self, body):
+        self.emitting = True
+        self.lines = []
+        self.group_sites = []
+        self.local_arrays = []
+        self.private_decls = []
+        self.indent = 2 if self.is_kernel else 1
+        for s in body:
+            self.stmt(s)
+        return self.lines
+
+    def translate_device(self, cname):
+        body = self.body_stmts()
+        self.infer(body)
+        lines = self.run_emit(body)
+        ret = self.ret_type
+        params = []
+        for p, t in zip(self.params, self.arg_types):
+            ct = t.ctype if isinstance(t, Scalar) else t.ctype()
+            params.append(f"{ct} {self.cname(p)}")
+        if self.m.boundscheck:
+            params.append("int *nmk_oob")
+        head = (f"__device__ __forceinline__ {ret.ctype if ret else 'void'} "
+                f"{cname}({', '.join(params)}) {{")
+        decls = ["  " + d for d in self.declarations() + self.private_decls]
+        return "\n".join([head] + decls + lines + ["}"]), ret
+
+    def translate_kernel(self, cname):
+        body = self.body_stmts()
+        self.infer(body)
+        lines = self.run_emit(body)
+        params, views = [], []
+        for p, t in zip(self.params, self.arg_types):
+            c = self.cname(p)
+            if isinstance(t, Array):
+                params.append(f"{t.elem.ctype} *{c}_p")
+                params += [f"int64_t {c}_s{k}" for k in range(t.ndim)]
+                params += [f"int64_t {c}_t{k}" for k in range(t.ndim)]
+                if t.ndim == 0:
+                    self.err(self.node, "0-d array arguments are not supported")
+                dims = [str(t.const_shape[k]) if t.const_shape[k] is not None
+                        else f"{c}_s{k}" for k in range(t.ndim)]
+                if t.layout == "C":
+                    # dense row-major: the strides follow from the extents
+                    strides = ["1"] * t.ndim
+                    for k in range(t.ndim - 2, -1, -1):
+                        strides[k] = f"{strides[k + 1]} * {dims[k + 1]}"
+                else:
+                    strides = [f"{c}_t{k}" for k in range(t.ndim)]
+                views.append(f"{t.ctype()} {c} = {{{c}_p, {{{', '.join(dims)}}}, "
+                             f"{{{', '.join(strides)}}}}};")
+            elif isinstance(t, SliceArg):
+                params += [f"int64_t {c}_start", f"int64_t {c}_stop", f"int64_t {c}_step"]
+            else:
+                if p in self.assigned:
+                    params.append(f"{t.ctype} {c}_arg")
+                    views.append(f"{self.env[p].ctype} {c} = {c}_arg;")
+                else:
+                    params.append(f"{t.ctype} {c}")
+        params += [f"uint64_t nmk_lds{k}" for k in range(len(self.local_arrays))]
+        params += ["int64_t nmk_gsz0", "int64_t nmk_gsz1", "int64_t nmk_gsz2"]
+        if self.m.boundscheck:
+            params.append("int *nmk_oob")
+        out = [f'extern "C" __global__ __launch_bounds__(1024) void {cname}(',
+               "    " + ", ".join(params) + ") {"]
+        # Work-items that cannot tell how they are grouped may be laid out on
+        # the lanes in any order: put the LAST global dimension on x, so that
+        # adjacent lanes touch adjacent elements of row-major arrays.
+        self.reversed = (self.allow_remap and not self.m.communicates and self.ndim > 1)
+        hw = "xyz"
+        dim = [hw[self.ndim - 1 - k] if (self.reversed and k < self.ndim) else hw[k]
+               for k in range(3)]
+        out += [
+            "  const int64_t " + ", ".join(f"nmk_lid{k} = threadIdx.{dim[k]}" for k in range(3)) + ";",
+            "  const int64_t " + ", ".join(f"nmk_grp{k} = blockIdx.{dim[k]}" for k in range(3)) + ";",
+            "  const int64_t " + ", ".join(f"nmk_lsz{k} = blockDim.{dim[k]}" for k in range(3)) + ";",
+            "  const int64_t nmk_gid0 = nmk_grp0 * nmk_lsz0 + nmk_lid0;",
+            "  const int64_t nmk_gid1 = nmk_grp1 * nmk_lsz1 + nmk_lid1;",
+            "  const int64_t nmk_gid2 = nmk_grp2 * nmk_lsz2 + nmk_lid2;",
+            "  const bool nmk_active = nmk_gid0 < nmk_gsz0 && nmk_gid1 < nmk_gsz1 && "
+            "nmk_gid2 < nmk_gsz2;",
+            "  (void)nmk_lid0; (void)nmk_lid1; (void)nmk_lid2; (void)nmk_grp0; (void)nmk_grp1;",
+            "  (void)nmk_grp2; (void)nmk_lsz0; (void)nmk_lsz1; (void)nmk_lsz2;",
+        ]
+        if self.group_sites:
+            out.append("  __shared__ int nmk_clipped;")
+            for slot, t, _ in self.group_sites:
+                out.append(f"  __shared__ {t.ctype} {slot}[nmkjit::kMaxGroup];")
+            out.append("  if (nmkjit::linearLocalId() == 0) nmk_clipped = 0;")
+            out.append("  __syncthreads();")
+            out.append("  if (!nmk_active) nmk_clipped = 1;")
+            for slot, t, neutral in self.group_sites:
+                out.append(f"  nmkjit::groupInit<{t.ctype}>({slot}, ({t.ctype}){neutral});")
+            out.append("  __syncthreads();")
+        out.append("  if (nmk_active) {")
+        out += ["    " + v for v in views]
+        out += ["    " + d for d in self.declarations() + self.private_decls]
+        out += lines
+        out.append("  }")
+        out.append("}")
+        return "\n".join(out)
+
+
+def _safe(name):
+    return "".join(ch if ch.isalnum() else "_" for ch in name)
+
+
+HEADER = """// Generated from the Python @kernel '{name}'; do not edit.
+#include "jit_support.h"
+extern __shared__ __attribute__((aligned(16))) unsigned char nmk_dyn_lds[];
+"""
+
+
+class CompiledKernel:
+    def __init__(self, name, source, local_arrays):
+        self.name, self.source = name, source
+        # bytes of each work-group-memory parameter, in parameter order
+        self.local_bytes = [int(np.prod(shape, dtype=np.int64)) * elem.dtype.itemsize
+                            for elem, shape in local_arrays]
+
+
+def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False):
+    """Python function + argument types -> CompiledKernel (source only).
+
+    With ``boundscheck`` every index is tested against its dimension: an
+    index outside it is replaced by 0 and the flag the kernel's last
+    parameter points at is set, so the launch can raise IndexError instead
+    of faulting the GPU.  With ``remap`` a body whose work-items cannot
+    observe their grouping gets global dimension ``ndim - 1`` on x
+    (``reversed_dims`` of the result tells the launcher)."""
+    module = Module(stubs, boundscheck)
+    tr = FunctionTranslator(module, func, arg_types, True, ndim)
+    tr.allow_remap = remap
+    digest = hashlib.sha256()
+    body = tr.translate_kernel("NMK_KERNEL_NAME")
+    text = "\n\n".join(module.device_code + [body])
+    digest.update(text.encode())
+    name = f"nmkjit_{_safe(func.__name__)}_{digest.hexdigest()[:12]}"
+    source = HEADER.format(name=func.__name__) + "\n" + text.replace("NMK_KERNEL_NAME", name) + "\n"
+    compiled = CompiledKernel(name, source, tr.local_arrays)
+    compiled.boundscheck = boundscheck
+    compiled.reversed_dims = tr.reversed
+    return compiled
+
+
+# ---------------------------------------------------------------------------
+# Source -> code object
+# ---------------------------------------------------------------------------
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_KERNELS_DIR = os.path.join(os.path.dirname(_HERE), "csrc", "kernels")
+CACHE_DIR = os.environ.get(
+    "NUMBA_MLIR_KERNEL_CACHE", os.path.join(os.path.dirname(_HERE), "kernel_cache"))
+
+
+def _hipcc():
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    return os.environ.get("HIPCC", os.path.join(rocm, "bin", "hipcc"))
+
+
+_FLAGS = ["--genco", "--no-gpu-bundle-output", "--offload-arch=gfx950", "-O3",
+          "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang",
+          "-packed-fp32-ops", "-std=c++17"]
+
+
+def build_code_object(compiled):
+    """Compiles the generated source with hipcc; code objects are cached on
+    disk under the hash of (source, support header, flags)."""
+    support = b""
+    for header in ("jit_support.h", "fast_math.h"):
+        with open(os.path.join(_KERNELS_DIR, header), "rb") as f:
+            support += f.read()
+    digest = hashlib.sha256()
+    for part in (compiled.source.encode(), support, " ".join(_FLAGS).encode()):
+        digest.update(part)
+    key = digest.hexdigest()[:24]
+    os.makedirs(CACHE_DIR, exist_ok=True)
+    obj = os.path.join(CACHE_DIR, f"{compiled.name}_{key}.hsaco")
+    if not os.path.exists(obj):
+        src = os.path.join(CACHE_DIR, f"{compiled.name}_{key}.hip")
+        with open(src, "w") as f:
+            f.write(compiled.source)
+        tmp = obj + f".tmp{os.getpid()}"
+        proc = subprocess.run([_hipcc(), *_FLAGS, f"-I{_KERNELS_DIR}", "-o", tmp, src],
+                              capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise KernelCompileError(
+                f"hipcc failed for {compiled.name}:\n{proc.stderr}\n--- source ---\n"
+                f"{compiled.source}")
+        os.replace(tmp, obj)
+    with open(obj, "rb") as f:
+        return f.read()

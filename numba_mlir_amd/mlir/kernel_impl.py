@@ -2,11 +2,14 @@
 
 In the reference ``Kernel.__call__`` hands the Python body to the compiler,
 which wraps it in one ``_gpu_range`` loop per dimension and emits a GPU kernel
-(reference: numba_mlir/numba_mlir/mlir/kernel_impl.py:97-206).  Without the
-compiler the body cannot be translated, so a kernel is bound to a hand-written
-gfx950 twin of the same body (``twin=`` names its symbol in the built-in
-"twins" code object; ``{dtype}`` and ``{rank}`` are filled from the first
-array argument).  Everything around the body is the reference's behaviour:
+(reference: numba_mlir/numba_mlir/mlir/kernel_impl.py:97-206).  Here the body is translated to HIP by ``kernel_compiler`` (types inferred from
+the launch arguments, one specialisation per signature), compiled to a gfx950
+code object and launched through ``gpuxModuleLoad`` / ``gpuxKernelGet`` /
+``gpuxLaunchKernel``.  A kernel may instead be bound to a hand-written twin of
+its body (``twin=`` names a symbol of the built-in "twins" code object;
+``{dtype}`` and ``{rank}`` are filled from the first array argument): the
+benchmark's pairwise kernel uses one whose work-items are remapped for
+coalesced stores.  Everything around the body is the reference's behaviour:
 
 * launch geometry: ``grid_k = ceil(global_k / local_k)``, tail guarded
   in-kernel, dimension 0 <-> x (reference: LowerToGpu.cpp:1113-1137);
@@ -18,10 +21,13 @@ is an error, as in the reference.
 """
 
 import ctypes
+import weakref
 
 import numpy as np
 
-from . import lowered
+from . import kernel_compiler, lowered
+from .gpu_runtime import runtime_lib
+from .utils import readenv
 from .device_array import HipNdArray
 from .kernel_base import KernelBase
 from .lowered import GPUParamDesc, lib
@@ -117,8 +123,8 @@ class group(Stub):
 
 def kernel_func(func):
     """Device function callable from kernels (``mlir_njit(mlir_force_inline=
-    True)`` in the reference, kernel_impl.py:209); a plain function here, the
-    twin inlines it by construction."""
+    True)`` in the reference, kernel_impl.py:209); a plain function here: the
+    kernel compiler translates whatever Python function a kernel calls."""
     return func
 
 
@@ -158,20 +164,38 @@ class _ParamList:
     def add_local(self, nbytes):
         self._slots.append((None, nbytes))
 
+    _SCALAR_PARAMS = {
+        np.dtype(np.bool_): (ctypes.c_bool, lowered.PARAM_BOOL),
+        np.dtype(np.int8): (ctypes.c_int8, lowered.PARAM_INT8),
+        np.dtype(np.uint8): (ctypes.c_uint8, lowered.PARAM_INT8),
+        np.dtype(np.int16): (ctypes.c_int16, lowered.PARAM_INT16),
+        np.dtype(np.uint16): (ctypes.c_uint16, lowered.PARAM_INT16),
+        np.dtype(np.int32): (ctypes.c_int32, lowered.PARAM_INT32),
+        np.dtype(np.uint32): (ctypes.c_uint32, lowered.PARAM_INT32),
+        np.dtype(np.int64): (ctypes.c_int64, lowered.PARAM_INT64),
+        np.dtype(np.uint64): (ctypes.c_uint64, lowered.PARAM_INT64),
+        np.dtype(np.float32): (ctypes.c_float, lowered.PARAM_FLOAT32),
+        np.dtype(np.float64): (ctypes.c_double, lowered.PARAM_FLOAT64),
+    }
+
     def add_scalar(self, value):
         if isinstance(value, (bool, np.bool_)):
             self._add(ctypes.c_bool(bool(value)), lowered.PARAM_BOOL)
-        elif isinstance(value, (int, np.integer)) and not isinstance(
-                value, np.int32):
-            self._add(ctypes.c_int64(int(value)), lowered.PARAM_INT64)
-        elif isinstance(value, np.int32):
-            self._add(ctypes.c_int32(int(value)), lowered.PARAM_INT32)
-        elif isinstance(value, np.float32):
-            self._add(ctypes.c_float(float(value)), lowered.PARAM_FLOAT32)
-        elif isinstance(value, (float, np.floating)):
-            self._add(ctypes.c_double(float(value)), lowered.PARAM_FLOAT64)
+        elif isinstance(value, np.generic) and value.dtype in self._SCALAR_PARAMS:
+            ctype, ptype = self._SCALAR_PARAMS[value.dtype]
+            self._add(ctype(value.item()), ptype)
+        elif isinstance(value, int):
+            self._add(ctypes.c_int64(value), lowered.PARAM_INT64)
+        elif isinstance(value, float):
+            self._add(ctypes.c_double(value), lowered.PARAM_FLOAT64)
         else:
             raise TypeError(f"Unsupported kernel argument type: {type(value)}")
+
+    def add_slice(self, value):
+        none = -2 ** 63           # an omitted bound
+        for part in (value.start, value.stop, value.step):
+            self._add(ctypes.c_int64(none if part is None else int(part)),
+                      lowered.PARAM_INT64)
 
     def build(self):
         descs = (GPUParamDesc * (len(self._slots) + 1))()
@@ -190,25 +214,101 @@ class _ParamList:
         return descs
 
 
+NO_DEPS = (ctypes.c_void_p * 1)(None)
+MAX_SPECIALISATIONS = 16   # per kernel, before new shapes get the general form
+
+
+def _release_handles(handles):
+    for kern, module in handles:
+        runtime_lib.gpuxKernelDestroy(kern)
+        runtime_lib.gpuxModuleDestroy(module)
+
+
+def _loaded_kernel(ctx, compiled):
+    """gpuxModuleLoad + gpuxKernelGet once per context and code object; the
+    handles are released before the context's queue (finalizers run last in,
+    first out)."""
+    table = getattr(ctx, "_jit_kernels", None)
+    if table is None:
+        table = ctx._jit_kernels = {}
+        ctx._jit_handles = []
+        weakref.finalize(ctx, _release_handles, ctx._jit_handles)
+    kern = table.get(compiled.name)
+    if kern is None:
+        blob = kernel_compiler.build_code_object(compiled)
+        module = runtime_lib.gpuxModuleLoad(ctx.queue, blob, len(blob))
+        kern = runtime_lib.gpuxKernelGet(module, compiled.name.encode())
+        table[compiled.name] = kern
+        ctx._jit_handles.append((kern, module))
+    return kern
+
+
+def _bounds_flag(ctx):
+    """One zeroed int32 per context for bounds-checked launches."""
+    flag = getattr(ctx, "_jit_bounds_flag", None)
+    if flag is None:
+        flag = ctx._jit_bounds_flag = HipNdArray.from_numpy(np.zeros(1, np.int32),
+                                                               device=ctx.device)
+    return flag
+
+
 class Kernel(KernelBase):
     def __init__(self, func, kwargs):
         super().__init__(func)
         self.twin = kwargs.get("twin")
-        # local.array sizes of the body in bytes: a list, or a callable
+        # local.array sizes of a twin's body in bytes: a list, or a callable
         # (global_size, local_size) -> list.  Each becomes a workgroup-memory
         # parameter after the user arguments (GpuRuntimeToLlvm.cpp:507-536).
+        # Compiled kernels know their own.
         self.local_bytes = kwargs.get("local_bytes", ())
+        # boundscheck=True (or NUMBA_MLIR_KERNEL_BOUNDSCHECK=1, cf. Numba's
+        # NUMBA_BOUNDSCHECK): an out-of-range index raises IndexError after the
+        # launch instead of reading or writing foreign memory.
+        self.boundscheck = bool(kwargs.get(
+            "boundscheck", readenv("NUMBA_MLIR_KERNEL_BOUNDSCHECK", int, 0)))
         self.last_launch = None
+        self._compiled = {}
 
     def _twin_name(self, args):
-        if self.twin is None:
-            raise NotImplementedError(
-                f"@kernel '{self.py_func.__name__}' has no hand-written gfx950 "
-                "twin; compiling arbitrary kernel bodies needs the ROCDL "
-                "lowering of the compiler")
         first = next((a for a in args if isinstance(a, HipNdArray)), None)
         tag = _DTYPE_TAGS.get(first.dtype) if first is not None else None
         return self.twin.format(dtype=tag, rank=len(self.global_size))
+
+    def compile(self, args, ndim, remap=False):
+        """The specialisation of the body for these arguments (translated on
+        first use; constants captured by the body are part of the key)."""
+        import sys
+        # Specialised on dense layouts and short trailing extents; a kernel
+        # that keeps meeting new ones gets the general form for the rest.
+        captured = self._captured_constants()
+        for specialize in (True, False):
+            types = [kernel_compiler.type_of_argument(a, specialize) for a in args]
+            key = (ndim, tuple(kernel_compiler.type_key(t) for t in types),
+                   captured, self.boundscheck, remap)
+            compiled = self._compiled.get(key)
+            if compiled is not None or len(self._compiled) < MAX_SPECIALISATIONS:
+                break
+        if compiled is None:
+            compiled = kernel_compiler.translate(self.py_func, types, ndim,
+                                                 sys.modules[__name__],
+                                                 self.boundscheck, remap)
+            self._compiled[key] = compiled
+        return compiled
+
+    def _captured_constants(self):
+        func = self.py_func
+        cells = []
+        for cell in func.__closure__ or ():
+            try:
+                v = cell.cell_contents
+            except ValueError:
+                continue
+            cells.append(v if isinstance(v, (bool, int, float, np.generic, tuple))
+                         else id(v))
+        try:
+            return hash(tuple(cells))
+        except TypeError:
+            return id(func)
 
     def __call__(self, *args, **kwargs):
         self.check_call_args(args, kwargs)
@@ -216,41 +316,92 @@ class Kernel(KernelBase):
 
         ndim = len(self.global_size)
         assert 1 <= ndim <= 3, f"Invalid dim count: {ndim}"
-        name = self._twin_name(args)
-
-        if len(self.local_size) != 0:
-            block = list(self.local_size)
-        else:
-            gsize = (ctypes.c_uint32 * ndim)(*[min(int(g), 0xFFFFFFFF)
-                                               for g in self.global_size])
-            bsize = (ctypes.c_uint32 * ndim)()
-            lib.nmhipSuggestBlockSize(ctx.handle, name.encode(), gsize, bsize,
-                                      ndim)
-            block = list(bsize)
-        block += [1] * (3 - ndim)
         gsize3 = [int(g) for g in self.global_size] + [1] * (3 - ndim)
-        grid = [(g + b - 1) // b for g, b in zip(gsize3, block)]
+
+        def geometry(compiled, kern):
+            """Block and grid in hardware order (x, y, z)."""
+            order = list(range(ndim))
+            if compiled is not None and compiled.reversed_dims:
+                order.reverse()
+            sizes = [gsize3[k] for k in order]
+            if len(self.local_size) != 0:
+                block = [int(self.local_size[k]) for k in order]
+            else:
+                gsize = (ctypes.c_uint32 * ndim)(*[min(g, 0xFFFFFFFF) for g in sizes])
+                bsize = (ctypes.c_uint32 * ndim)()
+                if kern is None:
+                    lib.nmhipSuggestBlockSize(ctx.handle, name.encode(), gsize, bsize, ndim)
+                else:
+                    runtime_lib.gpuxSuggestBlockSize(ctx.queue, kern, gsize, bsize, ndim)
+                block = list(bsize)
+            sizes += [1] * (3 - ndim)
+            block += [1] * (3 - ndim)
+            return block, [(g + b - 1) // b for g, b in zip(sizes, block)]
+
+        if self.twin is not None:
+            name = self._twin_name(args)
+            compiled = kern = None
+            block, grid = geometry(None, None)
+        else:
+            # With a runtime-chosen block a body that cannot observe its
+            # grouping is laid out for coalescing (last dimension on x), unless
+            # that pushes a long dimension past the y / z grid limit.
+            remap = len(self.local_size) == 0 and ndim > 1
+            compiled = self.compile(args, ndim, remap)
+            name = compiled.name
+            kern = _loaded_kernel(ctx, compiled)
+            block, grid = geometry(compiled, kern)
+            if compiled.reversed_dims and max(grid[1:]) > 65535:
+                compiled = self.compile(args, ndim, False)
+                name = compiled.name
+                kern = _loaded_kernel(ctx, compiled)
+                block, grid = geometry(compiled, kern)
 
         params = _ParamList()
         for a in args:
             if isinstance(a, HipNdArray):
                 params.add_array(a)
+            elif isinstance(a, slice):
+                params.add_slice(a)
             else:
                 params.add_scalar(a)
-        local_bytes = self.local_bytes
-        if callable(local_bytes):
-            local_bytes = local_bytes(tuple(gsize3[:ndim]), tuple(block[:ndim]))
+        if compiled is not None:
+            local_bytes = compiled.local_bytes
+        else:
+            local_bytes = self.local_bytes
+            if callable(local_bytes):
+                local_bytes = local_bytes(tuple(gsize3[:ndim]), tuple(block[:ndim]))
         for nbytes in local_bytes:
             params.add_local(int(nbytes))
         for g in gsize3:
             params.add_scalar(int(g))
+        flag = None
+        if compiled is not None and compiled.boundscheck:
+            flag = _bounds_flag(ctx)
+            params._add(ctypes.c_void_p(flag.ptr), lowered.PARAM_PTR)
         descs = params.build()
 
         self.last_launch = {"kernel": name, "grid": tuple(grid),
                             "block": tuple(block)}
-        lib.nmhipLaunch(ctx.handle, name.encode(),
-                        (ctypes.c_size_t * 3)(*grid),
-                        (ctypes.c_size_t * 3)(*block), descs)
+        if 0 in gsize3:
+            return
+        if kern is None:
+            lib.nmhipLaunch(ctx.handle, name.encode(),
+                            (ctypes.c_size_t * 3)(*grid),
+                            (ctypes.c_size_t * 3)(*block), descs)
+        else:
+            # the compiled host code's sequence: launch, wait, destroy event
+            # (GpuRuntimeToLlvm.cpp:577-628)
+            queue = ctx.queue
+            event = runtime_lib.gpuxLaunchKernel(queue, kern, *grid, *block,
+                                                 NO_DEPS, descs)
+            runtime_lib.gpuxWait(queue, event)
+            runtime_lib.gpuxDestroyEvent(queue, event)
+            if flag is not None and flag.asnumpy()[0] != 0:
+                flag.copy_from_host(np.zeros(1, np.int32))
+                raise IndexError(
+                    f"kernel '{self.py_func.__name__}' indexed an array out of "
+                    "bounds (the access was redirected to element 0)")
 
 
 def kernel(func=None, **kwargs):

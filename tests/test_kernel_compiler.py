@@ -1,0 +1,249 @@
+"""CPU tests of the @kernel translator: typing rules, generated source, error
+reporting, and that the generated HIP compiles for gfx950 (no GPU needed)."""
+
+import math
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+from numba_mlir_amd.mlir import kernel_compiler as kc
+
+
+@pytest.fixture(scope="module")
+def K(native_libs):
+    from numba_mlir_amd.mlir import kernel_impl
+    return kernel_impl
+
+
+F32_1D = kc.Array(kc.FLOAT32, 1)
+F64_1D = kc.Array(kc.FLOAT64, 1)
+I32_1D = kc.Array(kc.INT32, 1)
+I64_1D = kc.Array(kc.INT64, 1)
+
+
+def source_of(K, func, types, ndim=1, **kw):
+    return kc.translate(func, types, ndim, K, **kw).source
+
+
+def declared_type(src, name):
+    m = re.search(r"^\s*([\w:<>, ]+?) v_%s = " % name, src, re.M)
+    assert m, f"{name} is not declared in\n{src}"
+    return m.group(1).strip()
+
+
+def test_argument_types():
+    class Dev:
+        dtype, ndim, elem_strides = np.dtype(np.float32), 2, (4, 1)
+
+    assert kc.type_of_argument(Dev()) == kc.Array(kc.FLOAT32, 2)
+    assert kc.type_of_argument(3) is kc.INT64
+    assert kc.type_of_argument(3.0) is kc.FLOAT64
+    assert kc.type_of_argument(True) is kc.BOOL
+    assert kc.type_of_argument(np.int32(3)) is kc.INT32
+    assert kc.type_of_argument(np.float32(3)) is kc.FLOAT32
+    assert isinstance(kc.type_of_argument(slice(1, 2)), kc.SliceArg)
+    with pytest.raises(kc.KernelCompileError):
+        kc.type_of_argument("text")
+
+
+def test_promotion_follows_numpy():
+    assert kc.promote(kc.INT32, kc.FLOAT32) is kc.FLOAT64
+    assert kc.promote(kc.INT32, kc.INT64) is kc.INT64
+    assert kc.promote(kc.FLOAT32, kc.FLOAT32) is kc.FLOAT32
+    assert kc.promote(kc.INT16, kc.FLOAT32) is kc.FLOAT32
+    assert kc.promote(kc.BOOL, kc.INT8) is kc.INT8
+
+
+def test_variable_types(K):
+    get_global_id = K.get_global_id
+
+    def func(a, f, out):
+        i = get_global_id(0)
+        lit_i = 7                  # int64
+        lit_f = 0.5                # float64
+        x = a[i] + lit_i           # int32 + int64 -> int64
+        y = f[i] * f[i]            # float32
+        z = f[i] + lit_f           # float32 + float64 -> float64
+        q = a[i] / a[i]            # true division -> float64
+        r = a[i] // 2              # int64 (literal)
+        acc = 0                    # int64, then widened by the float32 store
+        acc = acc + y
+        b = a[i] > 2 and not y < 1.0
+        out[i] = x + y + z + q + r + acc + b
+
+    src = source_of(K, func, [I32_1D, F32_1D, F64_1D])
+    assert declared_type(src, "i") == "int64_t"
+    assert declared_type(src, "x") == "int64_t"
+    assert declared_type(src, "y") == "float"
+    assert declared_type(src, "z") == "double"
+    assert declared_type(src, "q") == "double"
+    assert declared_type(src, "r") == "int64_t"
+    assert declared_type(src, "acc") == "double"      # int64 joined with float32
+    assert declared_type(src, "b") == "bool"
+    # a name bound once, at the top level, to a constant is used as that constant
+    assert "+ ((int64_t)7ll))" in src and "+ v_lit_i" not in src
+
+
+def test_known_non_negative_indices_need_no_wrap(K):
+    get_global_id, get_local_id = K.get_global_id, K.get_local_id
+
+    def func(a, out):
+        i = get_global_id(0)
+        j = i + get_local_id(0) * 2
+        k = i - 1
+        out[i] = a[j] + a[k] + a[-1] + a[i % 4]
+
+    src = source_of(K, func, [F32_1D, F32_1D])
+    body = src.split("if (nmk_active)")[1]
+    assert body.count("nmkjit::wrap(") == 1            # only a[k]
+    assert "v_a.shape[0] + ((int64_t)-1ll)" in body     # a[-1]
+
+
+def test_kernel_signature_matches_the_launch_abi(K):
+    get_global_id, local, barrier = K.get_global_id, K.local, K.barrier
+
+    def func(a, n, s, b):
+        lm = local.array((4, 8), np.float64)
+        i = get_global_id(0)
+        lm[0, 0] = a[i, 0]
+        barrier()
+        b[s][i] = lm[0, 0] + n
+
+    ck = kc.translate(func, [kc.Array(kc.FLOAT32, 2), kc.INT64, kc.SliceArg(), F64_1D], 1, K)
+    sig = ck.source[ck.source.index("void " + ck.name):ck.source.index(") {")]
+    params = [p.strip() for p in sig.split("(", 1)[1].split(",")]
+    assert params == [
+        "float *v_a_p", "int64_t v_a_s0", "int64_t v_a_s1", "int64_t v_a_t0", "int64_t v_a_t1",
+        "int64_t v_n", "int64_t v_s_start", "int64_t v_s_stop", "int64_t v_s_step",
+        "double *v_b_p", "int64_t v_b_s0", "int64_t v_b_t0",
+        "uint64_t nmk_lds0", "int64_t nmk_gsz0", "int64_t nmk_gsz1", "int64_t nmk_gsz2"]
+    assert ck.local_bytes == [4 * 8 * 8]
+    assert ck.name.startswith("nmkjit_func_")
+    # same body, same name; another signature, another name
+    assert kc.translate(func, [kc.Array(kc.FLOAT32, 2), kc.INT64, kc.SliceArg(), F64_1D],
+                        1, K).name == ck.name
+    assert kc.translate(func, [kc.Array(kc.FLOAT64, 2), kc.INT64, kc.SliceArg(), F64_1D],
+                        1, K).name != ck.name
+
+
+def test_bounds_checked_build_adds_the_flag(K):
+    get_global_id = K.get_global_id
+
+    def helper(a, i):
+        return a[i]
+
+    def func(a, b):
+        i = get_global_id(0)
+        b[i] = helper(a, i + 1)
+
+    plain = source_of(K, func, [F32_1D, F32_1D])
+    checked = source_of(K, func, [F32_1D, F32_1D], boundscheck=True)
+    assert "nmk_oob" not in plain and "checked(" not in plain
+    assert checked.count("nmkjit::checked(") == 2
+    assert "int64_t nmk_gsz2, int *nmk_oob)" in checked
+    assert re.search(r"nmk_dev_helper_\d+\(v_a, \(v_i \+ \(\(int64_t\)1ll\)\), nmk_oob\)", checked)
+
+
+def test_device_functions_are_specialised_per_signature(K):
+    get_global_id = K.get_global_id
+    square = K.kernel_func(lambda v: v * v)
+
+    def func(a, b, c):
+        i = get_global_id(0)
+        c[i] = square(a[i]) + square(b[i]) + square(a[i])
+
+    src = source_of(K, func, [F32_1D, I32_1D, F64_1D])
+    devs = re.findall(r"__device__ __forceinline__ (\w+) (nmk_dev__lambda__\d+)\((\w+) v_v\)", src)
+    assert sorted((r, p) for r, _, p in devs) == [("float", "float"), ("int32_t", "int32_t")]
+
+
+@pytest.mark.parametrize("body,message", [
+    ("x = [1, 2]", "Unsupported expression: List"),
+    ("x = a[i]\n    x = a", "both as a scalar and as an array"),
+    ("for v in a:\n        pass", "Only 'for x in range"),
+    ("x = undefined_name + 1", "Unknown name 'undefined_name'"),
+    ("lm = local.array(i, np.float32)", "must be constant"),
+    ("return 3", "A kernel cannot return a value"),
+    ("x = 'text'", "Unsupported constant"),
+    ("a[i, 0] = 1", "Too many indices"),
+    ("import os", "Unsupported statement: Import"),
+    ("x = y + 1\n    y = 2", None),          # used before assignment in a straight line
+])
+def test_errors_name_the_line(K, body, message, tmp_path):
+    src = ("import numpy as np\n"
+           "from numba_mlir_amd.mlir.kernel_impl import get_global_id, local\n"
+           "def func(a):\n    i = get_global_id(0)\n    " + body + "\n")
+    path = tmp_path / "kern_mod.py"
+    path.write_text(src)
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("kern_mod", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    if message is None:
+        kc.translate(mod.func, [F32_1D], 1, K)       # legal for the translator: y is typed later
+        return
+    with pytest.raises(kc.KernelCompileError) as err:
+        kc.translate(mod.func, [F32_1D], 1, K)
+    assert message in str(err.value)
+    assert "func" in str(err.value)
+
+
+def test_lambdas_are_found_in_their_source_line(K):
+    table = {
+        "add": lambda a, b: a + b,
+        "hyp": lambda a, b: math.sqrt(a * a + b * b),
+    }
+    get_global_id = K.get_global_id
+    for name, expect in (("add", "(v_a + v_b)"), ("hyp", "sqrtF64(")):
+        f = table[name]
+
+        def func(x, y, out):
+            i = get_global_id(0)
+            out[i] = f(x[i], y[i])
+
+        assert expect in source_of(K, func, [F64_1D, F64_1D, F64_1D])
+
+
+def test_generated_source_compiles_for_gfx950(K, tmp_path, monkeypatch):
+    """hipcc cross-compiles without a GPU; the cache is keyed on the source."""
+    monkeypatch.setattr(kc, "CACHE_DIR", str(tmp_path))
+    get_global_id, atomic, group, private = K.get_global_id, K.atomic, K.group, K.private
+    barrier = K.barrier
+
+    def func(a, s, out, hist):
+        i = get_global_id(0)
+        scratch = private.array(4, np.float64)
+        for k in range(4):
+            scratch[k] = a[i] ** k
+        total = group.reduce_add(scratch[3] % 7.0)
+        barrier()
+        view = out[s]
+        view[i] = total + max(scratch[0], scratch[1]) + abs(a[i]) // 2
+        atomic.add(hist, (i % 2, 0), 1)
+
+    ck = kc.translate(func, [F64_1D, kc.SliceArg(), F64_1D, kc.Array(kc.INT32, 2)], 1, K)
+    blob = kc.build_code_object(ck)
+    assert blob[:4] == b"\x7fELF"
+    files = sorted(os.listdir(tmp_path))
+    assert len(files) == 2 and files[0].endswith(".hip") and files[1].endswith(".hsaco")
+    stamp = os.path.getmtime(tmp_path / files[1])
+    assert kc.build_code_object(ck) == blob                       # from the cache
+    assert os.path.getmtime(tmp_path / files[1]) == stamp
+    # the code object exports exactly the kernel
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    nm = os.path.join(rocm, "llvm", "bin", "llvm-nm")
+    if os.path.exists(nm):
+        out = subprocess.run([nm, str(tmp_path / files[1])], capture_output=True, text=True).stdout
+        assert re.search(r" T %s\b" % ck.name, out)
+
+
+def test_compile_failure_shows_the_compiler_output(K, tmp_path, monkeypatch):
+    monkeypatch.setattr(kc, "CACHE_DIR", str(tmp_path))
+    bad = kc.CompiledKernel("nmkjit_bad", "this is not HIP\n", [])
+    with pytest.raises(kc.KernelCompileError) as err:
+        kc.build_code_object(bad)
+    assert "hipcc failed" in str(err.value) and "this is not HIP" in str(err.value)
+    assert not [f for f in os.listdir(tmp_path) if f.endswith(".hsaco")]
