@@ -19,3 +19,4 @@ from .mlir.kernel_impl import (
     mem_fence,
     private,
 )
+from .mlir.kernel_compiler import KernelCompileError  # noqa: F401

@@ -228,7 +228,10 @@ def test_kernel_argument_checks(env):
         k[(4,), ()](hip.asarray(np.zeros(4, np.int32)), x=1)
     with pytest.raises(ValueError):
         k[(4,), ()](3)
-    with pytest.raises(NotImplementedError):
-        kapi.kernel(lambda c: None)[(4,), ()](hip.asarray(np.zeros(4, np.int32)))
+    def unsupported(c):
+        c[0] = [1, 2][0]
+
+    with pytest.raises(kapi.KernelCompileError, match="line 2: Unsupported expression: List"):
+        kapi.kernel(unsupported)[(4,), ()](hip.asarray(np.zeros(4, np.int32)))
     with pytest.raises(NotImplementedError):
         kapi.get_global_id(0)
