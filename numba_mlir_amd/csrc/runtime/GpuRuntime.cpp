@@ -192,30 +192,111 @@ struct Event {
   Event *next = nullptr;
 };
 
-// Kind of every live pointer handed out by gpuxAlloc, so gpuxDeAlloc can pick
-// hipFree or hipHostFree.  DeAlloc may arrive from any thread.
+// Kind, size and device of every live pointer handed out by gpuxAlloc, so
+// gpuxDeAlloc can pick hipFree or hipHostFree.  DeAlloc may arrive from any
+// thread.
+struct AllocInfo {
+  int kind = -1;
+  size_t bytes = 0;
+  int device = 0;
+};
+
 struct AllocRegistry {
   std::mutex mutex;
-  std::unordered_map<void *, int> kinds;
+  std::unordered_map<void *, AllocInfo> live;
 
-  void add(void *ptr, int kind) {
+  void add(void *ptr, AllocInfo info) {
     std::lock_guard<std::mutex> lock(mutex);
-    kinds[ptr] = kind;
+    live[ptr] = info;
   }
-  int take(void *ptr) {
+  AllocInfo take(void *ptr) {
     std::lock_guard<std::mutex> lock(mutex);
-    auto it = kinds.find(ptr);
-    if (it == kinds.end())
-      return -1;
-    int kind = it->second;
-    kinds.erase(it);
-    return kind;
+    auto it = live.find(ptr);
+    if (it == live.end())
+      return AllocInfo();
+    AllocInfo info = it->second;
+    live.erase(it);
+    return info;
   }
 };
 
 AllocRegistry &allocRegistry() {
   static AllocRegistry *reg = new AllocRegistry; // outlives late DeAllocs
   return *reg;
+}
+
+// Device blocks given back by gpuxDeAlloc are kept for the next gpuxAlloc of
+// the same size on the same device: hipMalloc / hipFree of the arrays a
+// compiled function returns cost several kernel times each (hipFree also
+// synchronises the device).  As with hipFree in the reference's sequence, the
+// caller has waited for the work that used a block before giving it back.
+// Blocks below 64 KiB are not worth keeping; the total kept is capped
+// (NUMBA_MLIR_GPU_ALLOC_CACHE_MB, default 16384, 0 = off) and everything is
+// released when an allocation fails.
+class DeviceBlockCache {
+public:
+  static constexpr size_t kMinBytes = 64 * 1024;
+
+  void *take(int device, size_t bytes) {
+    std::lock_guard<std::mutex> lock(mutex);
+    auto it = blocks.find(key(device, bytes));
+    if (it == blocks.end() || it->second.empty())
+      return nullptr;
+    void *ptr = it->second.back();
+    it->second.pop_back();
+    kept -= bytes;
+    return ptr;
+  }
+
+  // False when the block should be freed for real.
+  bool put(int device, void *ptr, size_t bytes) {
+    if (bytes < kMinBytes)
+      return false;
+    std::lock_guard<std::mutex> lock(mutex);
+    if (kept + bytes > limit())
+      return false;
+    blocks[key(device, bytes)].push_back(ptr);
+    kept += bytes;
+    return true;
+  }
+
+  // Hands every kept block of `device` to `release`.
+  template <typename F> void flush(int device, F release) {
+    std::vector<void *> all;
+    {
+      std::lock_guard<std::mutex> lock(mutex);
+      for (auto &entry : blocks) {
+        if (int(entry.first >> 48) != device)
+          continue;
+        kept -= (entry.first & ((uint64_t(1) << 48) - 1)) * entry.second.size();
+        all.insert(all.end(), entry.second.begin(), entry.second.end());
+        entry.second.clear();
+      }
+    }
+    for (void *ptr : all)
+      release(ptr);
+  }
+
+private:
+  static uint64_t key(int device, size_t bytes) {
+    return (uint64_t(device) << 48) | uint64_t(bytes);
+  }
+  static size_t limit() {
+    static size_t value = [] {
+      const char *env = std::getenv("NUMBA_MLIR_GPU_ALLOC_CACHE_MB");
+      const long long mb = env ? std::atoll(env) : 16384;
+      return size_t(mb > 0 ? mb : 0) << 20;
+    }();
+    return value;
+  }
+  std::mutex mutex;
+  std::unordered_map<uint64_t, std::vector<void *>> blocks;
+  size_t kept = 0;
+};
+
+DeviceBlockCache &deviceBlockCache() {
+  static DeviceBlockCache *cache = new DeviceBlockCache; // never destroyed
+  return *cache;
 }
 
 struct Kernel {
@@ -439,11 +520,20 @@ public:
 
     makeCurrent();
     void *ptr = nullptr;
-    const size_t bytes = size ? size : 1;
+    // device blocks come in multiples of 256 bytes, so equal requests match
+    const size_t bytes =
+        type == GPUX_ALLOC_DEVICE ? ((size ? size : 1) + 255) / 256 * 256
+                                  : (size ? size : 1);
     switch (type) {
     case GPUX_ALLOC_DEVICE:
-      if (hipApi().malloc_(&ptr, bytes) != hipSuccess || !ptr)
-        fail("Failed to allocate device memory");
+      ptr = deviceBlockCache().take(device, bytes);
+      if (!ptr && (hipApi().malloc_(&ptr, bytes) != hipSuccess || !ptr)) {
+        // give back what is kept and try once more
+        ptr = nullptr;
+        deviceBlockCache().flush(device, [](void *p) { (void)hipApi().free_(p); });
+        if (hipApi().malloc_(&ptr, bytes) != hipSuccess || !ptr)
+          fail("Failed to allocate device memory");
+      }
       break;
     case GPUX_ALLOC_SHARED:
       if (hipApi().mallocManaged(&ptr, bytes, hipMemAttachGlobal) !=
@@ -463,7 +553,7 @@ public:
       fail("Invalid allocation type");
     }
     if (ptr)
-      allocRegistry().add(ptr, type);
+      allocRegistry().add(ptr, AllocInfo{type, bytes, device});
 
     // The allocation is synchronous, so its event is complete already
     // (position 0), as the reference's default-constructed event is
@@ -476,13 +566,14 @@ public:
 
   void dealloc(void *ptr) {
     if (ptr) {
-      int kind = allocRegistry().take(ptr);
-      if (kind < 0)
+      const AllocInfo info = allocRegistry().take(ptr);
+      if (info.kind < 0)
         fail("gpuxDeAlloc: pointer %p was not allocated by gpuxAlloc", ptr);
       makeCurrent();
-      if (kind == GPUX_ALLOC_HOST)
+      if (info.kind == GPUX_ALLOC_HOST)
         check(hipApi().hostFree(ptr), "hipHostFree");
-      else
+      else if (info.kind != GPUX_ALLOC_DEVICE ||
+               !deviceBlockCache().put(info.device, ptr, info.bytes))
         check(hipApi().free_(ptr), "hipFree");
     }
     release(); // taken in alloc()

@@ -1,0 +1,296 @@
+"""``njit`` / ``vectorize`` / ``prange`` for functions over device arrays.
+
+In the reference ``@njit`` hands the function to Numba and the MLIR pipeline,
+which fuses whole-array expressions into parallel loops and offloads them
+(reference: numba_mlir/numba_mlir/decorators.py:24-120; the fused
+Black-Scholes test, numba_mlir/numba_mlir/mlir/tests/test_numpy.py:2796-2866).
+Here a call is served in one of three ways, tried in this order:
+
+1. *library lowering*: a function whose body is one ``return`` of a map,
+   reduction or contraction the hand-written kernels cover -- ``a + b``
+   (also ``-``, ``*``) with broadcasting, ``np.sum/prod/min/max(x[, axis])``,
+   ``np.sqrt(np.sum(x * x))``, ``np.dot(a, b)`` / ``a @ b`` -- goes to that
+   kernel, which is what the linalg lowering does with these patterns;
+2. *one parallel loop*: assignments followed by a single top-level
+   ``for i in prange(...)`` become one kernel, one work-item per iteration;
+3. *elementwise fusion*: any other function built from whole-array
+   arithmetic, ``math``/``numpy`` scalar functions, ``vectorize``d functions and
+   ``out[:] = ...`` stores becomes one fused kernel over the broadcast shape.
+
+Anything else (scalar indexing outside a loop, reductions mixed with maps,
+several loops) is reported as unsupported rather than run on the host.
+NumPy arguments are copied to the device for the call and back afterwards.
+"""
+
+import ast
+import functools
+import inspect
+import sys
+
+import numpy as np
+
+from .mlir import device_array as hip
+from .mlir import kernel_compiler, kernel_impl, ops
+from .mlir.device_array import HipNdArray
+from .mlir.utils import readenv
+
+
+def prange(*args):
+    """``range`` on the host; the grid of the offloaded loop under ``njit``."""
+    return range(*args)
+
+
+prange._nmk_prange = True
+
+
+class _Vectorized:
+    """A scalar function applied elementwise (reference:
+    numba_mlir/numba_mlir/mlir/vectorize.py:16-20).  Inside ``njit`` functions
+    it is inlined as a device function; called directly it maps over NumPy
+    arrays on the host."""
+
+    def __init__(self, func):
+        self.py_func = self._nmk_vectorized = func
+        functools.update_wrapper(self, func)
+
+    def __call__(self, *args):
+        return np.vectorize(self.py_func)(*args)
+
+
+def vectorize(arg_or_function=(), **kws):
+    if inspect.isfunction(arg_or_function):
+        return _Vectorized(arg_or_function)
+    return _Vectorized
+
+
+_BINARY = {ast.Add: ops.add, ast.Sub: ops.subtract, ast.Mult: ops.multiply}
+_REDUCE = {"sum": ops.sum, "prod": ops.prod, "min": ops.amin, "max": ops.amax,
+           "amin": ops.amin, "amax": ops.amax}
+
+
+class Dispatcher:
+    def __init__(self, py_func, parallel=False, boundscheck=None, **options):
+        self.py_func = py_func
+        self.parallel = parallel
+        if boundscheck is None:
+            boundscheck = readenv("NUMBA_MLIR_KERNEL_BOUNDSCHECK", int, 0)
+        self.boundscheck = bool(boundscheck)
+        self.options = options
+        self.last_launch = None          # what served the most recent call
+        self._compiled = {}
+        try:
+            node = kernel_compiler._function_ast(py_func)
+        except kernel_compiler.KernelCompileError:
+            node = None
+        self._node = node
+        functools.update_wrapper(self, py_func)
+
+    # -- entry ---------------------------------------------------------------
+    def __call__(self, *args, **kwargs):
+        if kwargs:
+            raise ValueError("kwargs not supported")
+        host = [isinstance(a, np.ndarray) for a in args]
+        if any(host):
+            dev = [hip.asarray(a) if h else a for a, h in zip(args, host)]
+            result = self._run(dev)
+            for a, d, h in zip(args, dev, host):
+                if h and a.flags.writeable:
+                    a[...] = d.asnumpy()
+            return result.asnumpy() if isinstance(result, HipNdArray) else result
+        return self._run(list(args))
+
+    def _run(self, args):
+        if self._node is None:
+            raise kernel_compiler.KernelCompileError(
+                f"No source available for {self.py_func!r}")
+        served = self._library(args)
+        if served is not NotImplemented:
+            return served
+        if self._has_parallel_loop():
+            return self._parallel(args)
+        return self._elementwise(args)
+
+    # -- 1. library lowering -------------------------------------------------
+    def _params(self):
+        return [a.arg for a in self._node.args.args]
+
+    def _library(self, args):
+        body = self._node.body
+        expr = body if isinstance(self._node, ast.Lambda) else None
+        if expr is None:
+            stmts = [s for s in body if not (isinstance(s, ast.Expr) and
+                                             isinstance(s.value, ast.Constant))]
+            if len(stmts) != 1 or not isinstance(stmts[0], ast.Return) or \
+                    stmts[0].value is None:
+                return NotImplemented
+            expr = stmts[0].value
+        by_name = dict(zip(self._params(), args))
+
+        def array(node):
+            if isinstance(node, ast.Name) and isinstance(by_name.get(node.id), HipNdArray):
+                return by_name[node.id]
+            return None
+
+        def np_call(node, names):
+            """np.<name>(...) or <array>.<name>(...): (name, positional, keywords)."""
+            if not isinstance(node, ast.Call) or not isinstance(node.func, ast.Attribute):
+                return None
+            if node.func.attr not in names:
+                return None
+            base = node.func.value
+            if isinstance(base, ast.Name) and self._resolve(base.id) is np:
+                return node.func.attr, list(node.args), node.keywords
+            if array(base) is not None:
+                return node.func.attr, [base] + list(node.args), node.keywords
+            return None
+
+        try:
+            # a (+|-|*) b
+            if isinstance(expr, ast.BinOp) and type(expr.op) in _BINARY:
+                a, b = array(expr.left), array(expr.right)
+                if a is not None and b is not None and a.dtype == b.dtype and \
+                        a.ndim <= 2 and b.ndim <= 2:
+                    return self._served("library", _BINARY[type(expr.op)](a, b), a.ctx)
+            # a @ b, np.dot(a, b)
+            if isinstance(expr, ast.BinOp) and isinstance(expr.op, ast.MatMult):
+                a, b = array(expr.left), array(expr.right)
+                if a is not None and b is not None:
+                    return self._served("library", ops.dot(a, b), a.ctx)
+            call = np_call(expr, ("dot",))
+            if call and len(call[1]) == 2 and not call[2]:
+                a, b = array(call[1][0]), array(call[1][1])
+                if a is not None and b is not None and a.ndim == b.ndim == 2:
+                    return self._served("library", ops.dot(a, b), a.ctx)
+            # np.sum(x, axis=k) and friends
+            call = np_call(expr, tuple(_REDUCE))
+            if call:
+                name, pos, kws = call
+                x = array(pos[0]) if pos else None
+                axis = None
+                ok = x is not None and len(pos) <= 2 and all(k.arg == "axis" for k in kws)
+                for node in pos[1:] + [k.value for k in kws]:
+                    if isinstance(node, ast.Constant) and (node.value is None or
+                                                           isinstance(node.value, int)):
+                        axis = node.value
+                    else:
+                        ok = False
+                if ok:
+                    return self._served("library", _REDUCE[name](x, axis=axis), x.ctx)
+            # np.sqrt(np.sum(x * x))
+            call = np_call(expr, ("sqrt",))
+            if call and len(call[1]) == 1 and not call[2]:
+                inner = np_call(call[1][0], ("sum",))
+                if inner and len(inner[1]) == 1 and not inner[2]:
+                    prod = inner[1][0]
+                    if isinstance(prod, ast.BinOp) and isinstance(prod.op, ast.Mult) and \
+                            isinstance(prod.left, ast.Name) and \
+                            isinstance(prod.right, ast.Name) and \
+                            prod.left.id == prod.right.id:
+                        x = array(prod.left)
+                        if x is not None and x.dtype == np.float32:
+                            return self._served("library", ops.sqrt_sum_squares(x), x.ctx)
+        except (TypeError, ValueError, NotImplementedError):
+            return NotImplemented       # outside what the kernel covers: fuse instead
+        return NotImplemented
+
+    def _resolve(self, name):
+        cv = inspect.getclosurevars(self.py_func)
+        for table in (cv.nonlocals, cv.globals, cv.builtins):
+            if name in table:
+                return table[name]
+        return getattr(self.py_func, "__globals__", {}).get(name)
+
+    def _served(self, how, result, ctx):
+        self.last_launch = {"path": how, "kernel": ctx.last_kernel()}
+        return result
+
+    # -- 2. one parallel loop ------------------------------------------------
+    def _has_parallel_loop(self):
+        if isinstance(self._node, ast.Lambda):
+            return False
+        for stmt in self._node.body:
+            if isinstance(stmt, ast.For) and isinstance(stmt.iter, ast.Call) and \
+                    isinstance(stmt.iter.func, ast.Name):
+                target = self._resolve(stmt.iter.func.id)
+                if getattr(target, "_nmk_prange", False):
+                    return True
+        return False
+
+    def _compile(self, mode, args, ndim, remap):
+        captured = kernel_impl.Kernel._captured_constants(self)
+        for specialize in (True, False):
+            types = [kernel_compiler.type_of_argument(a, specialize) for a in args]
+            key = (mode, ndim, tuple(kernel_compiler.type_key(t) for t in types),
+                   captured, remap)
+            compiled = self._compiled.get(key)
+            if compiled is not None or len(self._compiled) < kernel_impl.MAX_SPECIALISATIONS:
+                break
+        if compiled is None:
+            compiled = kernel_compiler.translate(
+                self.py_func, types, ndim, kernel_impl, self.boundscheck, remap, mode)
+            self._compiled[key] = compiled
+        return compiled
+
+    def _parallel(self, args):
+        ctx = kernel_impl.check_device_args(args)
+        compiled = self._compile("parallel", args, 1, False)
+        scope = dict(getattr(self.py_func, "__globals__", {}))
+        scope.update(inspect.getclosurevars(self.py_func).nonlocals)
+        scope.update(zip(self._params(), args))
+        for src in compiled.preamble_source:
+            try:                      # scalars the loop bounds may be built from
+                exec(src, scope)      # noqa: S102
+            except Exception:         # noqa: BLE001 -- device-only values
+                pass
+        bounds = [eval(src, scope) for src in compiled.range_source]   # noqa: S307
+        count = len(range(*[int(b) for b in bounds]))
+        info = kernel_impl.launch_compiled(ctx, compiled, self.py_func.__name__,
+                                           (count,), args)
+        self.last_launch = dict(info, path="parallel loop")
+        return None
+
+    # -- 3. elementwise fusion -----------------------------------------------
+    def _elementwise(self, args):
+        ctx = kernel_impl.check_device_args(args)
+        arrays = [a for a in args if isinstance(a, HipNdArray)]
+        shape = np.broadcast_shapes(*[a.shape for a in arrays])
+        views = [a.broadcast_to(shape) if isinstance(a, HipNdArray) else a for a in args]
+        dense = all(v.is_c_contiguous() for v in views if isinstance(v, HipNdArray))
+        if dense:                         # one long row: the cheapest indexing
+            run_shape = (int(np.prod(shape, dtype=np.int64)),)
+            views = [v.reshape(run_shape) if isinstance(v, HipNdArray) else v
+                     for v in views]
+        else:
+            run_shape = shape
+        if not 1 <= len(run_shape) <= 3:
+            raise kernel_compiler.KernelCompileError(
+                f"{self.py_func.__name__}: elementwise functions over strided arrays "
+                "support up to three dimensions")
+        compiled = self._compile("elementwise", views, len(run_shape), len(run_shape) > 1)
+        for name, a, v in zip(self._params(), args, views):
+            if isinstance(a, HipNdArray) and f"v_{name}" in compiled.written and \
+                    a.shape != tuple(shape):
+                raise ValueError(f"'{name}' is assigned but has shape {a.shape}, not the "
+                                 f"broadcast shape {tuple(shape)}")
+        ret = None
+        if compiled.ret_dtype is not None:
+            ret = HipNdArray.empty(shape, compiled.ret_dtype, device=ctx.device)
+        ret_view = ret.reshape(run_shape) if (ret is not None and dense) else ret
+        info = kernel_impl.launch_compiled(ctx, compiled, self.py_func.__name__,
+                                           run_shape, views, ret_view)
+        self.last_launch = dict(info, path="elementwise")
+        return ret
+
+
+def njit(signature_or_function=None, parallel=False, **options):
+    """``@njit`` / ``@njit(parallel=True)``."""
+    if inspect.isfunction(signature_or_function):
+        return Dispatcher(signature_or_function, parallel=parallel, **options)
+
+    def wrap(func):
+        return Dispatcher(func, parallel=parallel, **options)
+
+    return wrap
+
+
+jit = njit

@@ -177,6 +177,28 @@ class HipNdArray:
         return HipNdArray(self._buffer, self.shape[::-1], self.dtype,
                           self.strides[::-1], self._offset)
 
+    def __len__(self):
+        if not self.shape:
+            raise TypeError("len() of a 0-d device array")
+        return self.shape[0]
+
+    def broadcast_to(self, shape):
+        """Read-only style view with stride 0 along broadcast dimensions
+        (NumPy's rules: trailing dimensions align, extents are equal or 1)."""
+        shape = tuple(int(n) for n in shape)
+        if len(shape) < self.ndim:
+            raise ValueError(f"cannot broadcast {self.shape} to {shape}")
+        pad = len(shape) - self.ndim
+        strides = [0] * pad
+        for n, st, want in zip(self.shape, self.strides, shape[pad:]):
+            if n == want:
+                strides.append(st)
+            elif n == 1:
+                strides.append(0)
+            else:
+                raise ValueError(f"cannot broadcast {self.shape} to {shape}")
+        return HipNdArray(self._buffer, shape, self.dtype, strides, self._offset)
+
     def __getitem__(self, key):
         """Basic indexing (integers and slices): a view of the same
         allocation, as ``usm_ndarray`` gives."""

@@ -377,8 +377,16 @@ class FunctionTranslator:
         self.local_arrays = []       # (elem Scalar, shape tuple) in source order
         self.group_sites = []        # (slot name, Scalar, op)
         self.private_decls = []
+        # "kernel": an @kernel body; "elementwise": an @njit function of whole
+        # arrays fused into one map (an array used as a value means its
+        # element at the work-item's index); "parallel": an @njit function
+        # whose top-level prange loop becomes the grid; "device" otherwise
+        self.mode = "kernel" if is_kernel else "device"
+        self.range_source = None     # parallel mode: source of the prange arguments
         self.allow_remap = False     # kernels only: see translate_kernel
         self.reversed = False
+        self.written_arrays = set()  # elementwise mode: arrays stored through [:]
+        self._lambda_body = None
         self.site_names = {}         # ast node -> stable names
         self.array_info = {}         # variable name -> Array type (views)
 
@@ -453,9 +461,30 @@ class FunctionTranslator:
 
     def scalar(self, node):
         v = self.expr(node)
+        if isinstance(v.type, Array) and self.mode == "elementwise":
+            return self.element_here(v, node)
         if not isinstance(v.type, Scalar):
             self.err(node, "A scalar value is required here")
         return v
+
+    def element_here(self, arr, node):
+        """Elementwise mode: the element of ``arr`` at this work-item's index
+        (every array argument arrives broadcast to the iteration space)."""
+        if arr.type.ndim != self.ndim:
+            self.err(node, "Only whole arrays of the iteration space can be used "
+                           "in an elementwise function")
+        terms = [f"nmk_gid{d} * {arr.code}.stride[{d}]" for d in range(self.ndim)]
+        return Val(f"{arr.code}.p[{' + '.join(terms)}]", arr.type.elem)
+
+    @staticmethod
+    def is_whole_slice(node):
+        def full(n):
+            return (isinstance(n, ast.Slice) and n.lower is None and n.upper is None
+                    and n.step is None) or \
+                   (isinstance(n, ast.Constant) and n.value is Ellipsis)
+        if isinstance(node, ast.Tuple):
+            return all(full(e) for e in node.elts)
+        return full(node)
 
     def expr_Constant(self, node):
         v = node.value
@@ -678,6 +707,8 @@ class FunctionTranslator:
         return ("view", Val(cur, cur_t))
 
     def expr_Subscript(self, node):
+        if self.mode == "elementwise" and self.is_whole_slice(node.slice):
+            return self.expr(node.value)          # a[:] is a itself
         kind, *rest = self.subscript(node)
         if kind == "elem":
             code, elem = rest
@@ -789,6 +820,20 @@ class FunctionTranslator:
             if not v.type.is_float:
                 return constant(name == "isfinite")
             return Val(f"(bool)__builtin_{name}({v.code})", BOOL)
+        if is_np and name == "where" and len(node.args) == 3:
+            c = self.truth(self.scalar(node.args[0]))
+            a, b = self.scalar(node.args[1]), self.scalar(node.args[2])
+            t = promote(a.type, b.type)
+            return Val(f"({c.code} ? {cast(a, t).code} : {cast(b, t).code})", t,
+                       nonneg=a.nonneg and b.nonneg)
+        if is_np and name == "square" and len(node.args) == 1:
+            v = self.scalar(node.args[0])
+            return self.binop(ast.Mult(), v, v, node)
+        if is_np and name == "negative" and len(node.args) == 1:
+            v = self.scalar(node.args[0])
+            return Val(f"(-{v.code})", INT64 if v.type.is_bool else v.type)
+        if getattr(obj, "_nmk_vectorized", None) is not None:
+            return self.call_device(node, obj._nmk_vectorized)
         if inspect.isfunction(obj):
             return self.call_device(node, obj)
         self.err(node, f"Unsupported call target {obj!r}")
@@ -840,6 +885,9 @@ class FunctionTranslator:
         if node.keywords:
             self.err(node, "Keyword arguments are not supported in device calls")
         args = [self.expr(a) for a in node.args]
+        if self.mode == "elementwise":
+            args = [self.element_here(a, node) if isinstance(a.type, Array) else a
+                    for a in args]
         for a in args:
             if not isinstance(a.type, (Scalar, Array)):
                 self.err(node, "Device functions take scalars and arrays")
@@ -1034,6 +1082,16 @@ class FunctionTranslator:
             self.emit(f"{self.cname(name)} = {v.code};")
 
     def assign_subscript(self, target, v, node):
+        if self.mode == "elementwise" and self.is_whole_slice(target.slice):
+            arr = self.expr(target.value)
+            if not isinstance(arr.type, Array):
+                self.err(node, "Only arrays can be assigned through [:]")
+            if isinstance(v.type, Array):
+                v = self.element_here(v, node)
+            dst = self.element_here(arr, node)
+            self.written_arrays.add(arr.code)
+            self.emit(f"{dst.code} = {cast(v, arr.type.elem).code};")
+            return
         kind, *rest = self.subscript(target)
         if kind != "elem":
             self.err(node, "Only single elements can be assigned")
@@ -1073,9 +1131,16 @@ class FunctionTranslator:
         if node.orelse:
             self.err(node, "for ... else is not supported")
         it = node.iter
-        if not (isinstance(it, ast.Call) and isinstance(it.func, ast.Name) and
-                it.func.id == "range" and it.func.id not in self.env and
-                not it.keywords and 1 <= len(it.args) <= 3):
+        is_range = is_prange = False
+        if isinstance(it, ast.Call) and not it.keywords and 1 <= len(it.args) <= 3:
+            try:
+                fn = self.expr(it.func)
+            except KernelCompileError:
+                fn = None
+            if fn is not None and fn.type is None:
+                is_range = fn.pyobj is range
+                is_prange = bool(getattr(fn.pyobj, "_nmk_prange", False))
+        if not (is_range or is_prange):
             self.err(node, "Only 'for x in range(...)' loops are supported")
         if not isinstance(node.target, ast.Name):
             self.err(node, "The loop variable must be a name")
@@ -1084,6 +1149,22 @@ class FunctionTranslator:
         stop = a[1] if len(a) > 1 else a[0]
         step = a[2] if len(a) > 2 else constant(1)
         name = node.target.id
+        if is_prange and self.mode == "parallel" and id(node) in self.top_level:
+            # the parallel loop is the grid: work-item g runs iteration g
+            if self.range_source is not None and self.range_source[0] is not node:
+                self.err(node, "Only one top-level prange loop is offloaded")
+            if step.const is None or step.const <= 0:
+                self.err(node, "A prange step must be a positive constant")
+            self.range_source = (node, [ast.unparse(x) for x in it.args])
+            self.bind(name, INT64, node)
+            if not start.nonneg:
+                self.maybe_negative.add(name)
+            if self.emitting:
+                self.emit(f"{self.cname(name)} = {start.code} + nmk_gid0 * {step.code};")
+            self.indent -= 1
+            self.block(node.body)
+            self.indent += 1
+            return
         self.bind(name, INT64, node)
         if not (start.nonneg and step.const is not None and step.const > 0):
             self.maybe_negative.add(name)
@@ -1129,6 +1210,18 @@ class FunctionTranslator:
             if not self.is_kernel and self.ret_type is not None:
                 self.err(node, "A device function must return a value on every path")
             self.emit("return;")
+            return
+        if self.mode == "elementwise":
+            if id(node) not in self.top_level:
+                self.err(node, "An elementwise function returns at its end only")
+            v = self.scalar(node.value)
+            if self.ret_type is None:
+                self.ret_type = v.type
+                self.changed = True
+            elif self.ret_type is not v.type:
+                self.err(node, "An elementwise function has one return statement")
+            terms = [f"nmk_gid{d} * nmk_ret.stride[{d}]" for d in range(self.ndim)]
+            self.emit(f"nmk_ret.p[{' + '.join(terms)}] = {v.code};")
             return
         if self.is_kernel:
             self.err(node, "A kernel cannot return a value")
@@ -1178,8 +1271,11 @@ class FunctionTranslator:
 
     def body_stmts(self):
         if isinstance(self.node, ast.Lambda):
-            return [ast.Return(value=self.node.body, lineno=self.node.lineno,
-                               col_offset=0)]
+            if self._lambda_body is None:
+                self._lambda_body = [ast.Return(value=self.node.body,
+                                                lineno=self.node.lineno, col_offset=0)]
+                self.top_level.add(id(self._lambda_body[0]))
+            return self._lambda_body
         return self.node.body
 
     def declarations(self):
@@ -1251,6 +1347,16 @@ class FunctionTranslator:
                     views.append(f"{self.env[p].ctype} {c} = {c}_arg;")
                 else:
                     params.append(f"{t.ctype} {c}")
+        if self.mode == "elementwise" and self.ret_type is not None:
+            # the array an elementwise function returns: allocated by the
+            # caller, passed after the function's own arguments
+            n = self.ndim
+            params.append(f"{self.ret_type.ctype} *nmk_ret_p")
+            params += [f"int64_t nmk_ret_s{k}" for k in range(n)]
+            params += [f"int64_t nmk_ret_t{k}" for k in range(n)]
+            views.append(f"nmkjit::View<{self.ret_type.ctype}, {n}> nmk_ret = {{nmk_ret_p, "
+                         f"{{{', '.join(f'nmk_ret_s{k}' for k in range(n))}}}, "
+                         f"{{{', '.join(f'nmk_ret_t{k}' for k in range(n))}}}}};")
         params += [f"uint64_t nmk_lds{k}" for k in range(len(self.local_arrays))]
         params += ["int64_t nmk_gsz0", "int64_t nmk_gsz1", "int64_t nmk_gsz2"]
         if self.m.boundscheck:
@@ -1313,7 +1419,8 @@ class CompiledKernel:
                             for elem, shape in local_arrays]
 
 
-def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False):
+def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
+              mode="kernel"):
     """Python function + argument types -> CompiledKernel (source only).
 
     With ``boundscheck`` every index is tested against its dimension: an
@@ -1321,10 +1428,19 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False):
     parameter points at is set, so the launch can raise IndexError instead
     of faulting the GPU.  With ``remap`` a body whose work-items cannot
     observe their grouping gets global dimension ``ndim - 1`` on x
-    (``reversed_dims`` of the result tells the launcher)."""
+    (``reversed_dims`` of the result tells the launcher).
+
+    ``mode``: "kernel" for an @kernel body; "elementwise" for a function of
+    whole arrays fused into one map over ``ndim`` dimensions (``ret_dtype`` of
+    the result is the dtype of the returned array, if any); "parallel" for a
+    function whose top-level prange loop becomes a 1-d grid (``range_source``
+    holds the source text of the prange arguments for the host to evaluate)."""
     module = Module(stubs, boundscheck)
     tr = FunctionTranslator(module, func, arg_types, True, ndim)
     tr.allow_remap = remap
+    tr.mode = mode
+    if mode == "parallel":
+        _check_parallel_shape(tr)
     digest = hashlib.sha256()
     body = tr.translate_kernel("NMK_KERNEL_NAME")
     text = "\n\n".join(module.device_code + [body])
@@ -1334,7 +1450,38 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False):
     compiled = CompiledKernel(name, source, tr.local_arrays)
     compiled.boundscheck = boundscheck
     compiled.reversed_dims = tr.reversed
+    compiled.ret_dtype = tr.ret_type.dtype if (mode == "elementwise" and tr.ret_type) else None
+    compiled.range_source = tr.range_source[1] if tr.range_source else None
+    compiled.written = sorted(tr.written_arrays)
+    # parallel mode: what precedes the loop, for the host to evaluate the
+    # loop bounds that depend on it (n = len(x); for i in prange(n))
+    compiled.preamble_source = []
+    if tr.range_source:
+        for stmt in tr.body_stmts():
+            if stmt is tr.range_source[0]:
+                break
+            compiled.preamble_source.append(ast.unparse(stmt))
+    if mode == "parallel" and compiled.range_source is None:
+        raise KernelCompileError(f"{func.__name__}: no top-level prange loop to offload")
     return compiled
+
+
+def _check_parallel_shape(tr):
+    """A parallel function is: simple statements, one prange loop, nothing
+    after it (what follows a loop runs once, not per work-item)."""
+    body = tr.body_stmts()
+    seen = False
+    for stmt in body:
+        if isinstance(stmt, ast.For):
+            if seen:
+                tr.err(stmt, "Only one top-level loop is offloaded")
+            seen = True
+        elif seen and not (isinstance(stmt, ast.Return) and stmt.value is None) and \
+                not isinstance(stmt, ast.Pass):
+            tr.err(stmt, "Statements after the parallel loop are not supported")
+        elif not seen and not isinstance(stmt, (ast.Assign, ast.AugAssign, ast.Expr,
+                                               ast.Pass)):
+            tr.err(stmt, "Only assignments may precede the parallel loop")
 
 
 # ---------------------------------------------------------------------------

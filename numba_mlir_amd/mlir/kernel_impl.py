@@ -318,90 +318,122 @@ class Kernel(KernelBase):
         assert 1 <= ndim <= 3, f"Invalid dim count: {ndim}"
         gsize3 = [int(g) for g in self.global_size] + [1] * (3 - ndim)
 
-        def geometry(compiled, kern):
-            """Block and grid in hardware order (x, y, z)."""
-            order = list(range(ndim))
-            if compiled is not None and compiled.reversed_dims:
-                order.reverse()
-            sizes = [gsize3[k] for k in order]
-            if len(self.local_size) != 0:
-                block = [int(self.local_size[k]) for k in order]
-            else:
-                gsize = (ctypes.c_uint32 * ndim)(*[min(g, 0xFFFFFFFF) for g in sizes])
-                bsize = (ctypes.c_uint32 * ndim)()
-                if kern is None:
-                    lib.nmhipSuggestBlockSize(ctx.handle, name.encode(), gsize, bsize, ndim)
-                else:
-                    runtime_lib.gpuxSuggestBlockSize(ctx.queue, kern, gsize, bsize, ndim)
-                block = list(bsize)
-            sizes += [1] * (3 - ndim)
-            block += [1] * (3 - ndim)
-            return block, [(g + b - 1) // b for g, b in zip(sizes, block)]
-
         if self.twin is not None:
             name = self._twin_name(args)
             compiled = kern = None
-            block, grid = geometry(None, None)
+            if len(self.local_size) != 0:
+                block = [int(n) for n in self.local_size]
+            else:
+                gsize = (ctypes.c_uint32 * ndim)(*[min(g, 0xFFFFFFFF) for g in gsize3[:ndim]])
+                bsize = (ctypes.c_uint32 * ndim)()
+                lib.nmhipSuggestBlockSize(ctx.handle, name.encode(), gsize, bsize, ndim)
+                block = list(bsize)
+            block += [1] * (3 - ndim)
+            grid = [(g + b - 1) // b for g, b in zip(gsize3, block)]
         else:
             # With a runtime-chosen block a body that cannot observe its
             # grouping is laid out for coalescing (last dimension on x), unless
             # that pushes a long dimension past the y / z grid limit.
             remap = len(self.local_size) == 0 and ndim > 1
             compiled = self.compile(args, ndim, remap)
-            name = compiled.name
             kern = _loaded_kernel(ctx, compiled)
-            block, grid = geometry(compiled, kern)
+            block, grid = _geometry(ctx, compiled, kern, gsize3[:ndim], self.local_size)
             if compiled.reversed_dims and max(grid[1:]) > 65535:
                 compiled = self.compile(args, ndim, False)
-                name = compiled.name
                 kern = _loaded_kernel(ctx, compiled)
-                block, grid = geometry(compiled, kern)
+                block, grid = _geometry(ctx, compiled, kern, gsize3[:ndim],
+                                        self.local_size)
+            name = compiled.name
+
+        if compiled is not None:
+            _launch_loaded(ctx, compiled, kern, self.py_func.__name__, grid, block,
+                           gsize3, args)
+            self.last_launch = {"kernel": name, "grid": tuple(grid), "block": tuple(block)}
+            return
 
         params = _ParamList()
         for a in args:
             if isinstance(a, HipNdArray):
                 params.add_array(a)
-            elif isinstance(a, slice):
-                params.add_slice(a)
             else:
                 params.add_scalar(a)
-        if compiled is not None:
-            local_bytes = compiled.local_bytes
-        else:
-            local_bytes = self.local_bytes
-            if callable(local_bytes):
-                local_bytes = local_bytes(tuple(gsize3[:ndim]), tuple(block[:ndim]))
+        local_bytes = self.local_bytes
+        if callable(local_bytes):
+            local_bytes = local_bytes(tuple(gsize3[:ndim]), tuple(block[:ndim]))
         for nbytes in local_bytes:
             params.add_local(int(nbytes))
         for g in gsize3:
             params.add_scalar(int(g))
-        flag = None
-        if compiled is not None and compiled.boundscheck:
-            flag = _bounds_flag(ctx)
-            params._add(ctypes.c_void_p(flag.ptr), lowered.PARAM_PTR)
         descs = params.build()
-
-        self.last_launch = {"kernel": name, "grid": tuple(grid),
-                            "block": tuple(block)}
+        self.last_launch = {"kernel": name, "grid": tuple(grid), "block": tuple(block)}
         if 0 in gsize3:
             return
-        if kern is None:
-            lib.nmhipLaunch(ctx.handle, name.encode(),
-                            (ctypes.c_size_t * 3)(*grid),
-                            (ctypes.c_size_t * 3)(*block), descs)
+        lib.nmhipLaunch(ctx.handle, name.encode(), (ctypes.c_size_t * 3)(*grid),
+                        (ctypes.c_size_t * 3)(*block), descs)
+
+
+def _geometry(ctx, compiled, kern, global_size, local_size):
+    """Block and grid of a compiled kernel in hardware order (x, y, z)."""
+    ndim = len(global_size)
+    order = list(range(ndim))
+    if compiled.reversed_dims:
+        order.reverse()
+    sizes = [int(global_size[k]) for k in order]
+    if len(local_size) != 0:
+        block = [int(local_size[k]) for k in order]
+    else:
+        gsize = (ctypes.c_uint32 * ndim)(*[min(g, 0xFFFFFFFF) for g in sizes])
+        bsize = (ctypes.c_uint32 * ndim)()
+        runtime_lib.gpuxSuggestBlockSize(ctx.queue, kern, gsize, bsize, ndim)
+        block = list(bsize)
+    sizes += [1] * (3 - ndim)
+    block += [1] * (3 - ndim)
+    return block, [(g + b - 1) // b for g, b in zip(sizes, block)]
+
+
+def _launch_loaded(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret=None):
+    """The compiled host code's sequence for one kernel: parameters, launch,
+    wait, destroy event (GpuRuntimeToLlvm.cpp:444-628)."""
+    params = _ParamList()
+    for a in args:
+        if isinstance(a, HipNdArray):
+            params.add_array(a)
+        elif isinstance(a, slice):
+            params.add_slice(a)
         else:
-            # the compiled host code's sequence: launch, wait, destroy event
-            # (GpuRuntimeToLlvm.cpp:577-628)
-            queue = ctx.queue
-            event = runtime_lib.gpuxLaunchKernel(queue, kern, *grid, *block,
-                                                 NO_DEPS, descs)
-            runtime_lib.gpuxWait(queue, event)
-            runtime_lib.gpuxDestroyEvent(queue, event)
-            if flag is not None and flag.asnumpy()[0] != 0:
-                flag.copy_from_host(np.zeros(1, np.int32))
-                raise IndexError(
-                    f"kernel '{self.py_func.__name__}' indexed an array out of "
-                    "bounds (the access was redirected to element 0)")
+            params.add_scalar(a)
+    if ret is not None:
+        params.add_array(ret)
+    for nbytes in compiled.local_bytes:
+        params.add_local(int(nbytes))
+    for g in gsize3:
+        params.add_scalar(int(g))
+    flag = None
+    if compiled.boundscheck:
+        flag = _bounds_flag(ctx)
+        params._add(ctypes.c_void_p(flag.ptr), lowered.PARAM_PTR)
+    descs = params.build()
+    if 0 in gsize3:
+        return
+    queue = ctx.queue
+    event = runtime_lib.gpuxLaunchKernel(queue, kern, *grid, *block, NO_DEPS, descs)
+    runtime_lib.gpuxWait(queue, event)
+    runtime_lib.gpuxDestroyEvent(queue, event)
+    if flag is not None and flag.asnumpy()[0] != 0:
+        flag.copy_from_host(np.zeros(1, np.int32))
+        raise IndexError(
+            f"kernel '{func_name}' indexed an array out of bounds (the access was "
+            "redirected to element 0)")
+
+
+def launch_compiled(ctx, compiled, func_name, global_size, args, ret=None):
+    """Loads (once) and launches a translated function over ``global_size``
+    with a runtime-chosen block; returns the launch geometry."""
+    kern = _loaded_kernel(ctx, compiled)
+    block, grid = _geometry(ctx, compiled, kern, global_size, ())
+    gsize3 = [int(g) for g in global_size] + [1] * (3 - len(global_size))
+    _launch_loaded(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret)
+    return {"kernel": compiled.name, "grid": tuple(grid), "block": tuple(block)}
 
 
 def kernel(func=None, **kwargs):

@@ -35,7 +35,7 @@ struct State {
   int expectParams = 0;
   LaunchRecord last{};
   std::unordered_map<void *, int> allocs; // ptr -> 0 device, 1 managed, 2 host
-  long freesDevice = 0, freesHost = 0;
+  long freesDevice = 0, freesHost = 0, mallocsDevice = 0;
   uintptr_t nextHandle = 0x1000;
   std::unordered_map<void *, std::string> functionNames;
 };
@@ -112,7 +112,10 @@ hipError_t allocKind(void **p, size_t n, int kind) {
   *p = mem;
   return hipSuccess;
 }
-hipError_t mMalloc(void **p, size_t n) { return allocKind(p, n, 0); }
+hipError_t mMalloc(void **p, size_t n) {
+  st().mallocsDevice++;
+  return allocKind(p, n, 0);
+}
 hipError_t mMallocManaged(void **p, size_t n, unsigned) {
   return allocKind(p, n, 1);
 }
@@ -215,6 +218,7 @@ MOCK_EXPORT long mockCounter(const char *name) {
   if (n == "launches") return s.launches;
   if (n == "allocs_live") return long(s.allocs.size());
   if (n == "frees_device") return s.freesDevice;
+  if (n == "mallocs_device") return s.mallocsDevice;
   if (n == "frees_host") return s.freesHost;
   if (n == "modules_live") return s.modulesLoaded - s.modulesUnloaded;
   if (n == "current_device") return s.currentDevice;

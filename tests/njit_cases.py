@@ -1,0 +1,124 @@
+"""Functions shared by the CPU (translate + compile) and GPU (run) tests of
+``njit``.  The Black-Scholes bodies restate the formula of the reference's
+fused-loop test (numba_mlir/numba_mlir/mlir/tests/test_numpy.py:2827-2852),
+once over whole arrays and once as a prange loop."""
+
+import math
+
+import numpy as np
+
+from numba_mlir_amd.decorators import prange, vectorize
+
+
+@vectorize(nopython=True)
+def _erf(x):
+    return math.erf(x)
+
+
+def black_scholes_arrays(price, strike, t, rate, volatility, call, put):
+    mr = -rate
+    sig_sig_two = volatility * volatility * 2
+    P = price
+    S = strike
+    T = t
+    a = np.log(P / S)
+    b = T * mr
+    z = T * sig_sig_two
+    c = 0.25 * z
+    y = 1.0 / np.sqrt(z)
+    w1 = (a - b + c) * y
+    w2 = (a - b - c) * y
+    d1 = 0.5 + 0.5 * _erf(w1)
+    d2 = 0.5 + 0.5 * _erf(w2)
+    Se = np.exp(b) * S
+    r = P * d1 - Se * d2
+    call[:] = r
+    put[:] = r - P + Se
+
+
+def black_scholes_loop(nopt, price, strike, t, rate, volatility, call, put):
+    mr = -rate
+    sig_sig_two = volatility * volatility * 2
+    for i in prange(nopt):
+        P = price[i]
+        S = strike[i]
+        T = t[i]
+        a = math.log(P / S)
+        b = T * mr
+        z = T * sig_sig_two
+        c = 0.25 * z
+        y = 1.0 / math.sqrt(z)
+        w1 = (a - b + c) * y
+        w2 = (a - b - c) * y
+        d1 = 0.5 + 0.5 * math.erf(w1)
+        d2 = 0.5 + 0.5 * math.erf(w2)
+        Se = math.exp(b) * S
+        r = P * d1 - Se * d2
+        call[i] = r
+        put[i] = r - P + Se
+
+
+def add(a, b):
+    return a + b
+
+
+def fused_map(a, b, c, scale):
+    t = a * scale + np.sin(b)
+    u = np.where(t > c, t, c) / (1.0 + np.abs(c))
+    return np.maximum(u, 0.25) ** 2 - t
+
+
+def fused_store(x, y, out_f, out_i):
+    s = x + y
+    out_f[:] = np.sqrt(np.abs(s)) * 0.5
+    out_i[...] = x // 3 + y % 5
+
+
+def saxpy_loop(alpha, x, y, out):
+    n = len(x)
+    for i in prange(n):
+        out[i] = alpha * x[i] + y[i]
+
+
+def strided_loop(x, out):
+    for i in prange(1, x.shape[0] - 1, 2):
+        acc = 0.0
+        for k in range(x.shape[1]):
+            acc += x[i, k] * (x[i - 1, k] + x[i + 1, k])
+        out[i] = acc
+
+
+def row_sums(x):
+    return np.sum(x, axis=1)
+
+
+def col_sums(x):
+    return x.sum(axis=0)
+
+
+def norm(x):
+    return np.sqrt(np.sum(x * x))
+
+
+def matmul(a, b):
+    return a @ b
+
+
+def dot(a, b):
+    return np.dot(a, b)
+
+
+def statements_after_loop(x, out):
+    for i in prange(len(x)):
+        out[i] = x[i]
+    out[0] = 0.0
+
+
+def two_returns(a):
+    if True:
+        return a + 1
+    return a
+
+
+def no_loop(x):
+    y = 1

@@ -1,0 +1,180 @@
+"""GPU parity: ``njit`` over device arrays -- library lowering, one parallel
+loop, elementwise fusion -- against NumPy / the oracle."""
+
+import numpy as np
+import pytest
+
+import njit_cases as cases
+from numba_mlir_amd.decorators import njit
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def env(hip):
+    from numba_mlir_amd import workloads
+    from numba_mlir_amd.mlir import ops
+    from oracle import oracle as orc
+    return hip, ops, orc, workloads
+
+
+def _bs_inputs(hip, workloads, n):
+    price, strike, t, rate, vol, call, put = workloads.black_scholes(n)
+    dev = [hip.asarray(x) for x in (price, strike, t)]
+    return (price, strike, t, rate, vol), dev, hip.asarray(call), hip.asarray(put)
+
+
+@pytest.mark.parametrize("n", [1, 1000, 524288])
+def test_black_scholes_whole_array_body(env, n):
+    """The reference's fused-loop test (test_numpy.py:2796-2866): the body over
+    whole arrays becomes one kernel; results against the oracle at the path's
+    tolerance and against the reference's own bar."""
+    hip, ops, orc, workloads = env
+    inp, dev, call, put = _bs_inputs(hip, workloads, n)
+    f = njit(cases.black_scholes_arrays)
+    f(dev[0], dev[1], dev[2], inp[3], inp[4], call, put)
+    assert f.last_launch["path"] == "elementwise"
+    rc, rp = orc.black_scholes(*inp, wide=True)
+    np.testing.assert_allclose(call.asnumpy(), rc, rtol=1e-4, atol=1e-7)
+    np.testing.assert_allclose(put.asnumpy(), rp, rtol=1e-4, atol=1e-7)
+    # and against the hand-written kernel of the same formula
+    c2, p2 = hip.asarray(np.zeros(n, np.float32)), hip.asarray(np.zeros(n, np.float32))
+    ops.black_scholes(dev[0], dev[1], dev[2], inp[3], inp[4], c2, p2)
+    np.testing.assert_allclose(call.asnumpy(), c2.asnumpy(), rtol=2e-6, atol=1e-6)
+    np.testing.assert_allclose(put.asnumpy(), p2.asnumpy(), rtol=2e-6, atol=2e-6)
+
+
+def test_black_scholes_prange_body(env):
+    hip, ops, orc, workloads = env
+    n = 100003
+    inp, dev, call, put = _bs_inputs(hip, workloads, n)
+    f = njit(parallel=True)(cases.black_scholes_loop)
+    f(n, dev[0], dev[1], dev[2], inp[3], inp[4], call, put)
+    assert f.last_launch["path"] == "parallel loop"
+    rc, rp = orc.black_scholes(*inp, wide=True)
+    np.testing.assert_allclose(call.asnumpy(), rc, rtol=1e-4, atol=1e-7)
+    np.testing.assert_allclose(put.asnumpy(), rp, rtol=1e-4, atol=1e-7)
+
+
+def test_numpy_arguments_round_trip(env):
+    """Host arrays are copied in and out, as calling the jitted function on
+    NumPy arrays behaves in the reference."""
+    hip, ops, orc, workloads = env
+    price, strike, t, rate, vol, call, put = workloads.black_scholes(4096)
+    njit(cases.black_scholes_arrays)(price, strike, t, rate, vol, call, put)
+    rc, rp = orc.black_scholes(price, strike, t, rate, vol, wide=True)
+    np.testing.assert_allclose(call, rc, rtol=1e-4, atol=1e-7)
+    np.testing.assert_allclose(put, rp, rtol=1e-4, atol=1e-7)
+    out = njit(cases.add)(np.arange(6.0).reshape(2, 3), np.ones((1, 3)))
+    np.testing.assert_array_equal(out, np.arange(6.0).reshape(2, 3) + 1)
+
+
+def test_broadcast_add_goes_to_the_hand_written_kernel(env):
+    hip, ops, orc, workloads = env
+    a, b = workloads.broadcast_add(512, 1024)
+    f = njit(parallel=True)(cases.add)
+    out = f(hip.asarray(a), hip.asarray(b))
+    assert f.last_launch == {"path": "library", "kernel": "nmk_map2_rowbcast_add_f64"}
+    assert np.array_equal(out.asnumpy(), a + b)
+    # operands the map kernels do not cover are fused instead
+    x = np.arange(24, dtype=np.int16).reshape(2, 3, 4)
+    out = f(hip.asarray(x), hip.asarray(x[:1]))
+    assert f.last_launch["path"] == "elementwise"
+    assert np.array_equal(out.asnumpy(), x + x[:1])
+    out = f(hip.asarray(np.arange(5, dtype=np.int32)), hip.asarray(np.arange(5.0)))
+    assert out.dtype == np.float64 and np.array_equal(out.asnumpy(), 2.0 * np.arange(5))
+
+
+@pytest.mark.parametrize("shapes", [((40, 50), (40, 50), (40, 50)),
+                                    ((40, 1), (1, 50), (40, 50)),
+                                    ((50,), (40, 50), (1, 1)),
+                                    ((3, 4, 5), (4, 1), (5,))])
+def test_elementwise_fusion_with_broadcasting(env, shapes):
+    hip, ops, orc, workloads = env
+    rng = np.random.default_rng(11)
+    a, b, c = (rng.uniform(-2, 2, s) for s in shapes)
+    f = njit(cases.fused_map)
+    out = f(hip.asarray(a), hip.asarray(b), hip.asarray(c), 1.5)
+    assert f.last_launch["path"] == "elementwise"
+    np.testing.assert_allclose(out.asnumpy(), cases.fused_map(a, b, c, 1.5), rtol=1e-13)
+    assert out.shape == np.broadcast_shapes(*shapes)
+
+
+def test_elementwise_fusion_over_strided_views(env):
+    hip, ops, orc, workloads = env
+    rng = np.random.default_rng(12)
+    base = rng.uniform(-2, 2, (3, 64, 96))
+    dev = hip.asarray(base)
+    views = [dev[k, ::2, 1::3] for k in range(3)]
+    host = [base[k, ::2, 1::3] for k in range(3)]
+    f = njit(cases.fused_map)
+    out = f(*views, 0.5)
+    np.testing.assert_allclose(out.asnumpy(), cases.fused_map(*host, 0.5), rtol=1e-13)
+    out = f(views[0].T, views[1].T, views[2].T, 0.5)
+    np.testing.assert_allclose(out.asnumpy(), cases.fused_map(*[h.T for h in host], 0.5),
+                               rtol=1e-13)
+
+
+def test_stores_into_several_outputs(env):
+    hip, ops, orc, workloads = env
+    x = np.arange(-50, 50, dtype=np.int32)
+    y = np.arange(100, 0, -1, dtype=np.int32)
+    out_f, out_i = hip.asarray(np.zeros(100)), hip.asarray(np.zeros(100, np.int64))
+    njit(cases.fused_store)(hip.asarray(x), hip.asarray(y), out_f, out_i)
+    ref_f, ref_i = np.zeros(100), np.zeros(100, np.int64)
+    cases.fused_store(x.astype(np.int64), y.astype(np.int64), ref_f, ref_i)
+    np.testing.assert_allclose(out_f.asnumpy(), ref_f, rtol=1e-15)
+    np.testing.assert_array_equal(out_i.asnumpy(), ref_i)
+    with pytest.raises(ValueError, match="broadcast shape"):
+        njit(cases.fused_store)(hip.asarray(x), hip.asarray(y), out_f,
+                                hip.asarray(np.zeros(1, np.int64)))
+
+
+def test_prange_loops(env):
+    hip, ops, orc, workloads = env
+    rng = np.random.default_rng(13)
+    x, y = rng.standard_normal(10007).astype(np.float32), rng.standard_normal(10007).astype(np.float32)
+    out = hip.asarray(np.zeros(10007, np.float32))
+    njit(parallel=True)(cases.saxpy_loop)(np.float32(2.5), hip.asarray(x), hip.asarray(y), out)
+    np.testing.assert_array_equal(out.asnumpy(), np.float32(2.5) * x + y)
+    m = rng.standard_normal((101, 7))
+    out = hip.asarray(np.zeros(101))
+    njit(parallel=True)(cases.strided_loop)(hip.asarray(m), out)
+    ref = np.zeros(101)
+    cases.strided_loop(m, ref)
+    np.testing.assert_allclose(out.asnumpy(), ref, rtol=1e-13)
+
+
+def test_reductions_and_contractions_go_to_the_library(env):
+    hip, ops, orc, workloads = env
+    x = workloads.reduce_f32(256, 4096)
+    xi = workloads.reduce_i32(256, 512)
+    f = njit(cases.row_sums)
+    got = f(hip.asarray(x))
+    assert f.last_launch == {"path": "library", "kernel": "nmk_sum_axis1_wide_f32"}
+    np.testing.assert_allclose(got.asnumpy(), x.astype(np.float64).sum(axis=1), rtol=1e-4,
+                               atol=1e-3)
+    f = njit(cases.col_sums)
+    got = f(hip.asarray(xi))
+    assert f.last_launch["kernel"] == "nmk_sum_axis0_i32_i64"
+    assert np.array_equal(got.asnumpy(), xi.sum(axis=0, dtype=np.int64))
+    f = njit(cases.norm)
+    got = f(hip.asarray(x))
+    assert f.last_launch["kernel"] == "nmk_norm2_f32"
+    np.testing.assert_allclose(got.asnumpy()[0], np.sqrt((x.astype(np.float64) ** 2).sum()),
+                               rtol=1e-5)
+    a, b = workloads.matmul(256)
+    for fn in (cases.matmul, cases.dot):
+        got = njit(fn)(hip.asarray(a), hip.asarray(b))
+        np.testing.assert_allclose(got.asnumpy(), orc.gemm_f32_truth(a, b), rtol=1e-4,
+                                   atol=1e-3)
+
+
+def test_unsupported_functions_are_reported(env):
+    hip, ops, orc, workloads = env
+    from numba_mlir_amd.kernel import KernelCompileError
+    x = hip.asarray(np.arange(8.0))
+    with pytest.raises(KernelCompileError, match="after the parallel loop"):
+        njit(parallel=True)(cases.statements_after_loop)(x, hip.asarray(np.zeros(8)))
+    with pytest.raises(ValueError, match="at least one device array"):
+        njit(cases.add)(1.0, 2.0)

@@ -247,3 +247,55 @@ def test_compile_failure_shows_the_compiler_output(K, tmp_path, monkeypatch):
         kc.build_code_object(bad)
     assert "hipcc failed" in str(err.value) and "this is not HIP" in str(err.value)
     assert not [f for f in os.listdir(tmp_path) if f.endswith(".hsaco")]
+
+
+# ---- njit: whole-array functions and prange loops ---------------------------
+
+def _njit_types(case):
+    f32 = lambda n: kc.Array(kc.FLOAT32, n, layout="C")      # noqa: E731
+    f64 = lambda n: kc.Array(kc.FLOAT64, n, layout="C")      # noqa: E731
+    return {
+        "black_scholes_arrays": ("elementwise", 1, [f32(1)] * 3 + [kc.FLOAT32] * 2 + [f32(1)] * 2),
+        "black_scholes_loop": ("parallel", 1, [kc.INT64] + [f32(1)] * 3 + [kc.FLOAT32] * 2 + [f32(1)] * 2),
+        "fused_map": ("elementwise", 2, [kc.Array(kc.FLOAT64, 2)] * 3 + [kc.FLOAT64]),
+        "fused_store": ("elementwise", 1, [kc.Array(kc.INT32, 1, layout="C")] * 2 +
+                        [f64(1), kc.Array(kc.INT64, 1, layout="C")]),
+        "saxpy_loop": ("parallel", 1, [kc.FLOAT32, f32(1), f32(1), f32(1)]),
+        "strided_loop": ("parallel", 1, [kc.Array(kc.FLOAT64, 2), f64(1)]),
+    }[case]
+
+
+@pytest.mark.parametrize("case", ["black_scholes_arrays", "black_scholes_loop", "fused_map",
+                                  "fused_store", "saxpy_loop", "strided_loop"])
+def test_njit_functions_translate_and_compile(K, case, tmp_path, monkeypatch):
+    import njit_cases
+    monkeypatch.setattr(kc, "CACHE_DIR", str(tmp_path))
+    mode, ndim, types = _njit_types(case)
+    ck = kc.translate(getattr(njit_cases, case), types, ndim, K, mode=mode)
+    assert kc.build_code_object(ck)[:4] == b"\x7fELF"
+    if case == "black_scholes_arrays":
+        # the reference's typing falls out of the rules: literal-bearing
+        # intermediates are float64, log(P / S), T * mr and exp(b) * S float32
+        for name, ctype in (("a", "float"), ("b", "float"), ("Se", "float"),
+                            ("sig_sig_two", "double"), ("z", "double"), ("c", "double"),
+                            ("y", "double"), ("w1", "double"), ("d1", "double"),
+                            ("r", "double")):
+            assert declared_type(ck.source, name) == ctype, name
+        assert ck.written == ["v_call", "v_put"] and ck.ret_dtype is None
+    if case == "fused_map":
+        assert ck.ret_dtype == np.float64 and "nmk_ret_p" in ck.source
+    if case == "strided_loop":
+        assert ck.range_source == ["1", "x.shape[0] - 1", "2"]
+    if case == "saxpy_loop":
+        assert ck.range_source == ["n"] or ck.range_source == ["len(x)"]
+
+
+def test_njit_rejects_what_it_cannot_offload(K):
+    import njit_cases
+    f64 = kc.Array(kc.FLOAT64, 1, layout="C")
+    with pytest.raises(kc.KernelCompileError, match="after the parallel loop"):
+        kc.translate(njit_cases.statements_after_loop, [f64, f64], 1, K, mode="parallel")
+    with pytest.raises(kc.KernelCompileError, match="returns at its end only"):
+        kc.translate(njit_cases.two_returns, [f64], 1, K, mode="elementwise")
+    with pytest.raises(kc.KernelCompileError, match="no top-level prange loop"):
+        kc.translate(njit_cases.no_loop, [f64], 1, K, mode="parallel")

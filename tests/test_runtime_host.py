@@ -295,6 +295,39 @@ def test_allocation_kinds(rt, qk):
     rt.gpuxDeAlloc(q, res.ptr)
 
 
+def test_large_device_blocks_are_kept_for_reuse(rt, qk):
+    """gpuxDeAlloc keeps device blocks of 64 KiB and more; the next gpuxAlloc
+    of the same (256-byte rounded) size takes one without calling hipMalloc."""
+    q, _, _ = qk
+    res = AllocResult()
+
+    def alloc(nbytes, kind=0):
+        rt.gpuxAlloc(q, nbytes, 64, kind, NO_DEPS, ctypes.byref(res))
+        rt.gpuxDestroyEvent(q, res.event)
+        return res.ptr
+
+    mallocs, frees = counter(rt, "mallocs_device"), counter(rt, "frees_device")
+    a = alloc(1 << 20)
+    b = alloc(1 << 20)
+    assert a != b and counter(rt, "mallocs_device") == mallocs + 2
+    rt.gpuxDeAlloc(q, a)
+    rt.gpuxDeAlloc(q, b)
+    assert counter(rt, "frees_device") == frees            # kept, not freed
+    c = alloc((1 << 20) - 100)                               # rounds to the same size
+    d = alloc(1 << 20)
+    assert {c, d} == {a, b} and counter(rt, "mallocs_device") == mallocs + 2
+    e = alloc(2 << 20)                                       # another size: a new block
+    assert e not in (a, b) and counter(rt, "mallocs_device") == mallocs + 3
+    small = alloc(4096)                                      # below the threshold
+    rt.gpuxDeAlloc(q, small)
+    assert counter(rt, "frees_device") == frees + 1
+    shared = alloc(1 << 20, kind=1)                          # only device memory is kept
+    rt.gpuxDeAlloc(q, shared)
+    assert counter(rt, "frees_device") == frees + 2
+    for p in (c, d, e):
+        rt.gpuxDeAlloc(q, p)
+
+
 def test_event_pool_reuses_events(rt, qk):
     """Cross-queue use creates a device event once per pooled slot."""
     q, _, k = qk
