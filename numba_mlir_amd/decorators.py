@@ -25,7 +25,6 @@ NumPy arguments are copied to the device for the call and back afterwards.
 import ast
 import functools
 import inspect
-import sys
 
 import numpy as np
 
@@ -217,7 +216,7 @@ class Dispatcher:
         return False
 
     def _compile(self, mode, args, ndim, remap):
-        captured = kernel_impl.Kernel._captured_constants(self)
+        captured = kernel_impl.captured_constants(self.py_func)
         for specialize in (True, False):
             types = [kernel_compiler.type_of_argument(a, specialize) for a in args]
             key = (mode, ndim, tuple(kernel_compiler.type_key(t) for t in types),

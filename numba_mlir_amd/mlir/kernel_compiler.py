@@ -414,6 +414,9 @@ class FunctionTranslator:
             self.lines.append("  " * self.indent + text)
 
     def cname(self, name):
+        if "." in name:                      # element k of the tuple variable
+            base, k = name.split(".")
+            return f"vt_{base}_{k}"
         return f"v_{name}"
 
     # -- name resolution ---------------------------------------------------
@@ -432,7 +435,9 @@ class FunctionTranslator:
                 parts = tuple(Val(f"{c}_{k}", INT64) for k in ("start", "stop", "step"))
                 return Val(c, t, slice_parts=parts)
             if isinstance(t, tuple) and t[0] == "tuple":
-                return Val(None, t, items=self.tuple_vars[name])
+                items = [Val(self.cname(i), self.env[i], nonneg=i in self.nonneg_vars)
+                         if isinstance(i, str) else i for i in self.tuple_vars[name]]
+                return Val(None, t, items=items)
             raise KernelCompileError(f"Unsupported variable type for {name}")
         if name in self.params or name in self.assigned:
             raise _Deferred(name)
@@ -561,7 +566,10 @@ class FunctionTranslator:
         return Val(f"({v.code} != 0)", BOOL)
 
     def expr_BoolOp(self, node):
-        vals = [self.truth(self.scalar(e)) for e in node.values]
+        vals = [self.scalar(e) for e in node.values]
+        if not all(v.type.is_bool for v in vals):
+            # Python's and / or return one of the operands, not a truth value
+            self.err(node, "'and' / 'or' are supported between boolean values only")
         op = " && " if isinstance(node.op, ast.And) else " || "
         return Val("(" + op.join(v.code for v in vals) + ")", BOOL)
 
@@ -1061,7 +1069,26 @@ class FunctionTranslator:
         if v.items is not None:
             if name in self.env and not (isinstance(self.env[name], tuple)):
                 self.err(node, f"'{name}' changes from a scalar to a tuple")
-            self.tuple_vars[name] = v.items
+            # the scalar elements are stored now (a later change of what they
+            # were computed from must not show); views and slices are kept as
+            # expressions
+            items = []
+            for k, item in enumerate(v.items):
+                if isinstance(item.type, Scalar) and item.const is None:
+                    slot = f"{name}.{k}"
+                    self.assigned.add(slot)
+                    self.bind(slot, item.type, node)
+                    if not item.nonneg:
+                        self.maybe_negative.add(slot)
+                    if self.emitting:
+                        self.emit(f"{self.cname(slot)} = {cast(item, self.env[slot]).code};")
+                    items.append(slot)
+                else:
+                    items.append(item)
+            old = self.tuple_vars.get(name)
+            if old is not None and len(old) != len(items):
+                self.err(node, f"'{name}' is bound to tuples of different lengths")
+            self.tuple_vars[name] = items
             self.env[name] = ("tuple",)
             return
         if isinstance(v.type, SliceArg):

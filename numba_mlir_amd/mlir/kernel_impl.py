@@ -252,6 +252,22 @@ def _bounds_flag(ctx):
     return flag
 
 
+def captured_constants(func):
+    """Hash of what a function's closure holds: constants a body captures are
+    compiled in, so they belong to the key of its specialisations."""
+    cells = []
+    for cell in func.__closure__ or ():
+        try:
+            v = cell.cell_contents
+        except ValueError:
+            continue
+        cells.append(v if isinstance(v, (bool, int, float, np.generic, tuple)) else id(v))
+    try:
+        return hash(tuple(cells))
+    except TypeError:
+        return id(func)
+
+
 class Kernel(KernelBase):
     def __init__(self, func, kwargs):
         super().__init__(func)
@@ -280,7 +296,7 @@ class Kernel(KernelBase):
         import sys
         # Specialised on dense layouts and short trailing extents; a kernel
         # that keeps meeting new ones gets the general form for the rest.
-        captured = self._captured_constants()
+        captured = captured_constants(self.py_func)
         for specialize in (True, False):
             types = [kernel_compiler.type_of_argument(a, specialize) for a in args]
             key = (ndim, tuple(kernel_compiler.type_key(t) for t in types),
@@ -294,21 +310,6 @@ class Kernel(KernelBase):
                                                  self.boundscheck, remap)
             self._compiled[key] = compiled
         return compiled
-
-    def _captured_constants(self):
-        func = self.py_func
-        cells = []
-        for cell in func.__closure__ or ():
-            try:
-                v = cell.cell_contents
-            except ValueError:
-                continue
-            cells.append(v if isinstance(v, (bool, int, float, np.generic, tuple))
-                         else id(v))
-        try:
-            return hash(tuple(cells))
-        except TypeError:
-            return id(func)
 
     def __call__(self, *args, **kwargs):
         self.check_call_args(args, kwargs)

@@ -674,6 +674,30 @@ def test_device_functions_and_tuples(env):
           exact=False, rtol=1e-12)
 
 
+def test_tuple_elements_are_values(env):
+    def func(out):
+        i = get_global_id(0)
+        pair = (i, i * 2)
+        i = i + 100                         # must not show through the tuple
+        if pair[1] > 6:
+            pair = (pair[0], -pair[1])
+        out[pair[0]] = pair[1] + i
+
+    check(env, func, 8, DEFAULT_LOCAL_SIZE, [np.zeros(8, np.int64)])
+
+
+def test_and_or_need_booleans(env):
+    hip, sim = env
+
+    def func(a, out):
+        i = get_global_id(0)
+        out[i] = a[i] or 7                  # Python would store a[i] or 7
+
+    with pytest.raises(K.KernelCompileError, match="boolean values only"):
+        K.kernel(func)[4, DEFAULT_LOCAL_SIZE](hip.asarray(np.arange(4)),
+                                              hip.asarray(np.zeros(4, np.int64)))
+
+
 def test_strided_and_transposed_arguments(env):
     hip, sim = env
 
