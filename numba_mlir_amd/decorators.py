@@ -25,6 +25,7 @@ NumPy arguments are copied to the device for the call and back afterwards.
 import ast
 import functools
 import inspect
+import math
 
 import numpy as np
 
@@ -62,6 +63,28 @@ def vectorize(arg_or_function=(), **kws):
     return _Vectorized
 
 
+ELEMENTS_PER_THREAD = 4     # of a fused 1-d map or prange loop
+
+
+def _disjoint(arrays):
+    """True when no two of the device arrays share a byte (then the kernel may
+    reorder their loads and stores freely)."""
+    spans = []
+    for a in arrays:
+        lo = hi = a.ptr
+        for n, st in zip(a.shape, a.strides):
+            if n == 0:
+                lo = hi = a.ptr
+                break
+            if st >= 0:
+                hi += (n - 1) * st
+            else:
+                lo += (n - 1) * st
+        spans.append((lo, hi + a.dtype.itemsize))
+    spans.sort()
+    return all(spans[k][1] <= spans[k + 1][0] for k in range(len(spans) - 1))
+
+
 _BINARY = {ast.Add: ops.add, ast.Sub: ops.subtract, ast.Mult: ops.multiply}
 _REDUCE = {"sum": ops.sum, "prod": ops.prod, "min": ops.amin, "max": ops.amax,
            "amin": ops.amin, "amax": ops.amax}
@@ -82,6 +105,9 @@ class Dispatcher:
         except kernel_compiler.KernelCompileError:
             node = None
         self._node = node
+        self._names = None             # what the body's free names are bound to
+        self._parallel_loop = None     # whether the body has a top-level prange loop
+        self._library_form = None      # the one-expression pattern, parsed once
         functools.update_wrapper(self, py_func)
 
     # -- entry ---------------------------------------------------------------
@@ -113,16 +139,25 @@ class Dispatcher:
     def _params(self):
         return [a.arg for a in self._node.args.args]
 
+    def _single_expression(self):
+        """The expression of a body that is one ``return``, else None."""
+        if self._library_form is None:
+            body = self._node.body
+            expr = body if isinstance(self._node, ast.Lambda) else None
+            if expr is None:
+                stmts = [s for s in body if not (isinstance(s, ast.Expr) and
+                                                 isinstance(s.value, ast.Constant))]
+                if len(stmts) == 1 and isinstance(stmts[0], ast.Return) and \
+                        stmts[0].value is not None:
+                    expr = stmts[0].value
+            shapes = (ast.BinOp, ast.Call)
+            self._library_form = (expr if isinstance(expr, shapes) else False,)
+        return self._library_form[0]
+
     def _library(self, args):
-        body = self._node.body
-        expr = body if isinstance(self._node, ast.Lambda) else None
-        if expr is None:
-            stmts = [s for s in body if not (isinstance(s, ast.Expr) and
-                                             isinstance(s.value, ast.Constant))]
-            if len(stmts) != 1 or not isinstance(stmts[0], ast.Return) or \
-                    stmts[0].value is None:
-                return NotImplemented
-            expr = stmts[0].value
+        expr = self._single_expression()
+        if expr is False or expr is None:
+            return NotImplemented
         by_name = dict(zip(self._params(), args))
 
         def array(node):
@@ -193,11 +228,12 @@ class Dispatcher:
         return NotImplemented
 
     def _resolve(self, name):
-        cv = inspect.getclosurevars(self.py_func)
-        for table in (cv.nonlocals, cv.globals, cv.builtins):
-            if name in table:
-                return table[name]
-        return getattr(self.py_func, "__globals__", {}).get(name)
+        if self._names is None:
+            cv = inspect.getclosurevars(self.py_func)
+            self._names = dict(getattr(self.py_func, "__globals__", {}))
+            for table in (cv.builtins, cv.globals, cv.nonlocals):
+                self._names.update(table)
+        return self._names.get(name)
 
     def _served(self, how, result, ctx):
         self.last_launch = {"path": how, "kernel": ctx.last_kernel()}
@@ -205,28 +241,31 @@ class Dispatcher:
 
     # -- 2. one parallel loop ------------------------------------------------
     def _has_parallel_loop(self):
-        if isinstance(self._node, ast.Lambda):
-            return False
-        for stmt in self._node.body:
-            if isinstance(stmt, ast.For) and isinstance(stmt.iter, ast.Call) and \
-                    isinstance(stmt.iter.func, ast.Name):
-                target = self._resolve(stmt.iter.func.id)
-                if getattr(target, "_nmk_prange", False):
-                    return True
-        return False
+        if self._parallel_loop is None:
+            self._parallel_loop = False
+            if not isinstance(self._node, ast.Lambda):
+                for stmt in self._node.body:
+                    if isinstance(stmt, ast.For) and isinstance(stmt.iter, ast.Call) and \
+                            isinstance(stmt.iter.func, ast.Name):
+                        target = self._resolve(stmt.iter.func.id)
+                        if getattr(target, "_nmk_prange", False):
+                            self._parallel_loop = True
+        return self._parallel_loop
 
     def _compile(self, mode, args, ndim, remap):
         captured = kernel_impl.captured_constants(self.py_func)
+        noalias = _disjoint([a for a in args if isinstance(a, HipNdArray)])
         for specialize in (True, False):
             types = [kernel_compiler.type_of_argument(a, specialize) for a in args]
             key = (mode, ndim, tuple(kernel_compiler.type_key(t) for t in types),
-                   captured, remap)
+                   captured, remap, noalias)
             compiled = self._compiled.get(key)
             if compiled is not None or len(self._compiled) < kernel_impl.MAX_SPECIALISATIONS:
                 break
         if compiled is None:
             compiled = kernel_compiler.translate(
-                self.py_func, types, ndim, kernel_impl, self.boundscheck, remap, mode)
+                self.py_func, types, ndim, kernel_impl, self.boundscheck, remap, mode,
+                noalias=noalias, elements_per_thread=ELEMENTS_PER_THREAD)
             self._compiled[key] = compiled
         return compiled
 
@@ -256,7 +295,7 @@ class Dispatcher:
         views = [a.broadcast_to(shape) if isinstance(a, HipNdArray) else a for a in args]
         dense = all(v.is_c_contiguous() for v in views if isinstance(v, HipNdArray))
         if dense:                         # one long row: the cheapest indexing
-            run_shape = (int(np.prod(shape, dtype=np.int64)),)
+            run_shape = (math.prod(shape),)
             views = [v.reshape(run_shape) if isinstance(v, HipNdArray) else v
                      for v in views]
         else:

@@ -12,6 +12,7 @@ view dies, as the reference's NRT MemInfo destructor does
 """
 
 import ctypes
+import math
 import weakref
 
 import numpy as np
@@ -162,7 +163,7 @@ class HipNdArray:
 
     @property
     def size(self):
-        return int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
+        return math.prod(self.shape)
 
     @property
     def nbytes(self):
@@ -257,7 +258,7 @@ class HipNdArray:
         if not self.is_c_contiguous():
             raise ValueError("reshape needs a C-contiguous device array")
         strides = _dense_strides(shape, self.dtype.itemsize)
-        if int(np.prod(shape, dtype=np.int64)) != self.size:
+        if math.prod(int(n) for n in shape) != self.size:
             raise ValueError("cannot reshape: size mismatch")
         return HipNdArray(self._buffer, shape, self.dtype, strides, self._offset)
 

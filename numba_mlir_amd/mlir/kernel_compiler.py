@@ -386,6 +386,9 @@ class FunctionTranslator:
         self.allow_remap = False     # kernels only: see translate_kernel
         self.reversed = False
         self.written_arrays = set()  # elementwise mode: arrays stored through [:]
+        self.read_arrays = set()     # elementwise mode: arrays loaded as values
+        self.noalias = False         # no two array arguments overlap (host-checked)
+        self.elements_per_thread = 1
         self._lambda_body = None
         self.site_names = {}         # ast node -> stable names
         self.array_info = {}         # variable name -> Array type (views)
@@ -478,8 +481,20 @@ class FunctionTranslator:
         if arr.type.ndim != self.ndim:
             self.err(node, "Only whole arrays of the iteration space can be used "
                            "in an elementwise function")
+        self.read_arrays.add(arr.code)
         terms = [f"nmk_gid{d} * {arr.code}.stride[{d}]" for d in range(self.ndim)]
         return Val(f"{arr.code}.p[{' + '.join(terms)}]", arr.type.elem)
+
+    def store_here(self, arr_code, elem, value_code):
+        """Elementwise mode: the store of this work-item's element.  An array
+        that is only written, and that no other argument overlaps, is streamed
+        past the caches."""
+        terms = [f"nmk_gid{d} * {arr_code}.stride[{d}]" for d in range(self.ndim)]
+        dst = f"{arr_code}.p[{' + '.join(terms)}]"
+        if self.noalias and arr_code not in self.read_arrays:
+            self.emit(f"__builtin_nontemporal_store(({elem.ctype})({value_code}), &{dst});")
+        else:
+            self.emit(f"{dst} = {value_code};")
 
     @staticmethod
     def is_whole_slice(node):
@@ -1115,9 +1130,10 @@ class FunctionTranslator:
                 self.err(node, "Only arrays can be assigned through [:]")
             if isinstance(v.type, Array):
                 v = self.element_here(v, node)
-            dst = self.element_here(arr, node)
+            if arr.type.ndim != self.ndim:
+                self.err(node, "Only whole arrays of the iteration space can be assigned")
             self.written_arrays.add(arr.code)
-            self.emit(f"{dst.code} = {cast(v, arr.type.elem).code};")
+            self.store_here(arr.code, arr.type.elem, cast(v, arr.type.elem).code)
             return
         kind, *rest = self.subscript(target)
         if kind != "elem":
@@ -1247,8 +1263,7 @@ class FunctionTranslator:
                 self.changed = True
             elif self.ret_type is not v.type:
                 self.err(node, "An elementwise function has one return statement")
-            terms = [f"nmk_gid{d} * nmk_ret.stride[{d}]" for d in range(self.ndim)]
-            self.emit(f"nmk_ret.p[{' + '.join(terms)}] = {v.code};")
+            self.store_here("nmk_ret", self.ret_type, v.code)
             return
         if self.is_kernel:
             self.err(node, "A kernel cannot return a value")
@@ -1347,10 +1362,11 @@ class FunctionTranslator:
         self.infer(body)
         lines = self.run_emit(body)
         params, views = [], []
+        restrict = "__restrict__ " if self.noalias else ""
         for p, t in zip(self.params, self.arg_types):
             c = self.cname(p)
             if isinstance(t, Array):
-                params.append(f"{t.elem.ctype} *{c}_p")
+                params.append(f"{t.elem.ctype} *{restrict}{c}_p")
                 params += [f"int64_t {c}_s{k}" for k in range(t.ndim)]
                 params += [f"int64_t {c}_t{k}" for k in range(t.ndim)]
                 if t.ndim == 0:
@@ -1378,7 +1394,7 @@ class FunctionTranslator:
             # the array an elementwise function returns: allocated by the
             # caller, passed after the function's own arguments
             n = self.ndim
-            params.append(f"{self.ret_type.ctype} *nmk_ret_p")
+            params.append(f"{self.ret_type.ctype} *{restrict}nmk_ret_p")
             params += [f"int64_t nmk_ret_s{k}" for k in range(n)]
             params += [f"int64_t nmk_ret_t{k}" for k in range(n)]
             views.append(f"nmkjit::View<{self.ret_type.ctype}, {n}> nmk_ret = {{nmk_ret_p, "
@@ -1397,13 +1413,31 @@ class FunctionTranslator:
         hw = "xyz"
         dim = [hw[self.ndim - 1 - k] if (self.reversed and k < self.ndim) else hw[k]
                for k in range(3)]
+        # A 1-d map whose work-items cannot observe their grouping may give
+        # several elements to a lane, a block apart (coalesced); unrolled, with
+        # non-overlapping arrays, their loads are in flight together.
+        ept = self.elements_per_thread
+        if self.m.communicates or self.ndim != 1 or self.mode == "kernel":
+            ept = self.elements_per_thread = 1
         out += [
             "  const int64_t " + ", ".join(f"nmk_lid{k} = threadIdx.{dim[k]}" for k in range(3)) + ";",
             "  const int64_t " + ", ".join(f"nmk_grp{k} = blockIdx.{dim[k]}" for k in range(3)) + ";",
             "  const int64_t " + ", ".join(f"nmk_lsz{k} = blockDim.{dim[k]}" for k in range(3)) + ";",
-            "  const int64_t nmk_gid0 = nmk_grp0 * nmk_lsz0 + nmk_lid0;",
-            "  const int64_t nmk_gid1 = nmk_grp1 * nmk_lsz1 + nmk_lid1;",
-            "  const int64_t nmk_gid2 = nmk_grp2 * nmk_lsz2 + nmk_lid2;",
+        ]
+        if ept > 1:
+            out += [
+                "#pragma unroll",
+                f"  for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep) {{",
+                f"  const int64_t nmk_gid0 = (nmk_grp0 * {ept} + nmk_rep) * nmk_lsz0 + nmk_lid0;",
+                "  const int64_t nmk_gid1 = 0, nmk_gid2 = 0;",
+            ]
+        else:
+            out += [
+                "  const int64_t nmk_gid0 = nmk_grp0 * nmk_lsz0 + nmk_lid0;",
+                "  const int64_t nmk_gid1 = nmk_grp1 * nmk_lsz1 + nmk_lid1;",
+                "  const int64_t nmk_gid2 = nmk_grp2 * nmk_lsz2 + nmk_lid2;",
+            ]
+        out += [
             "  const bool nmk_active = nmk_gid0 < nmk_gsz0 && nmk_gid1 < nmk_gsz1 && "
             "nmk_gid2 < nmk_gsz2;",
             "  (void)nmk_lid0; (void)nmk_lid1; (void)nmk_lid2; (void)nmk_grp0; (void)nmk_grp1;",
@@ -1424,6 +1458,8 @@ class FunctionTranslator:
         out += ["    " + d for d in self.declarations() + self.private_decls]
         out += lines
         out.append("  }")
+        if ept > 1:
+            out.append("  }")
         out.append("}")
         return "\n".join(out)
 
@@ -1447,7 +1483,7 @@ class CompiledKernel:
 
 
 def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
-              mode="kernel"):
+              mode="kernel", noalias=False, elements_per_thread=1):
     """Python function + argument types -> CompiledKernel (source only).
 
     With ``boundscheck`` every index is tested against its dimension: an
@@ -1461,11 +1497,18 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     whole arrays fused into one map over ``ndim`` dimensions (``ret_dtype`` of
     the result is the dtype of the returned array, if any); "parallel" for a
     function whose top-level prange loop becomes a 1-d grid (``range_source``
-    holds the source text of the prange arguments for the host to evaluate)."""
+    holds the source text of the prange arguments for the host to evaluate).
+    For these two modes ``noalias`` promises that no two array arguments
+    overlap, and ``elements_per_thread`` asks for that many elements per lane
+    of a 1-d grid (the result says what it got: the launcher divides the grid
+    by it)."""
     module = Module(stubs, boundscheck)
     tr = FunctionTranslator(module, func, arg_types, True, ndim)
     tr.allow_remap = remap
     tr.mode = mode
+    if mode != "kernel":
+        tr.noalias = noalias
+        tr.elements_per_thread = max(1, int(elements_per_thread))
     if mode == "parallel":
         _check_parallel_shape(tr)
     digest = hashlib.sha256()
@@ -1480,6 +1523,7 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     compiled.ret_dtype = tr.ret_type.dtype if (mode == "elementwise" and tr.ret_type) else None
     compiled.range_source = tr.range_source[1] if tr.range_source else None
     compiled.written = sorted(tr.written_arrays)
+    compiled.elements_per_thread = tr.elements_per_thread
     # parallel mode: what precedes the loop, for the host to evaluate the
     # loop bounds that depend on it (n = len(x); for i in prange(n))
     compiled.preamble_source = []

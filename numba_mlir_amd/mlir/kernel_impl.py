@@ -431,7 +431,9 @@ def launch_compiled(ctx, compiled, func_name, global_size, args, ret=None):
     """Loads (once) and launches a translated function over ``global_size``
     with a runtime-chosen block; returns the launch geometry."""
     kern = _loaded_kernel(ctx, compiled)
-    block, grid = _geometry(ctx, compiled, kern, global_size, ())
+    per_lane = getattr(compiled, "elements_per_thread", 1)
+    lanes = [-(-int(global_size[0]) // per_lane)] + [int(g) for g in global_size[1:]]
+    block, grid = _geometry(ctx, compiled, kern, lanes, ())
     gsize3 = [int(g) for g in global_size] + [1] * (3 - len(global_size))
     _launch_loaded(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret)
     return {"kernel": compiled.name, "grid": tuple(grid), "block": tuple(block)}

@@ -299,3 +299,26 @@ def test_njit_rejects_what_it_cannot_offload(K):
         kc.translate(njit_cases.two_returns, [f64], 1, K, mode="elementwise")
     with pytest.raises(kc.KernelCompileError, match="no top-level prange loop"):
         kc.translate(njit_cases.no_loop, [f64], 1, K, mode="parallel")
+
+
+def test_fused_maps_take_several_elements_per_lane(K, tmp_path, monkeypatch):
+    import njit_cases
+    monkeypatch.setattr(kc, "CACHE_DIR", str(tmp_path))
+    mode, ndim, types = _njit_types("black_scholes_arrays")
+    ck = kc.translate(njit_cases.black_scholes_arrays, types, ndim, K, mode=mode,
+                      noalias=True, elements_per_thread=4)
+    assert ck.elements_per_thread == 4
+    assert "for (int nmk_rep = 0; nmk_rep < 4; ++nmk_rep)" in ck.source
+    assert "float *__restrict__ v_price_p" in ck.source
+    # call and put are only written: streamed
+    assert ck.source.count("__builtin_nontemporal_store(") == 2
+    assert kc.build_code_object(ck)[:4] == b"\x7fELF"
+    # overlapping arguments: plain pointers and stores
+    ck = kc.translate(njit_cases.black_scholes_arrays, types, ndim, K, mode=mode,
+                      noalias=False, elements_per_thread=4)
+    assert "__restrict__" not in ck.source and "nontemporal" not in ck.source
+    # more than one dimension, or an @kernel body: one element per lane
+    mode, ndim, types = _njit_types("fused_map")
+    ck = kc.translate(njit_cases.fused_map, types, ndim, K, mode=mode, noalias=True,
+                      elements_per_thread=4)
+    assert ck.elements_per_thread == 1 and "nmk_rep" not in ck.source
