@@ -220,4 +220,28 @@ __device__ __forceinline__ T groupReduce(T *slots, T v, bool clipped, Op op) {
   return r;
 }
 
+// Reduction of one value per lane over the whole block (every lane calls it,
+// lanes outside the global size with the neutral element); lane 0 stores the
+// block's result at partial[block index].  The tree is fixed by the block
+// shape, so repeated launches give the same bits.
+template <typename T, typename Op>
+__device__ __forceinline__ void blockReduceStore(T v, Op op, T *partial) {
+  __shared__ T slots[kMaxGroup];
+  const int tid = linearLocalId();
+  const int n = localCount();
+  __syncthreads(); // the slots may serve several reductions in a row
+  slots[tid] = v;
+  __syncthreads();
+  int s = 1;
+  while (s < n)
+    s <<= 1;
+  for (s >>= 1; s > 0; s >>= 1) {
+    if (tid < s && tid + s < n)
+      slots[tid] = op(slots[tid], slots[tid + s]);
+    __syncthreads();
+  }
+  if (tid == 0)
+    partial[blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)] = slots[0];
+}
+
 } // namespace nmkjit

@@ -13,6 +13,8 @@ Here a call is served in one of three ways, tried in this order:
    kernel, which is what the linalg lowering does with these patterns;
 2. *one parallel loop*: assignments followed by a single top-level
    ``for i in prange(...)`` become one kernel, one work-item per iteration;
+   scalars the loop only updates with ``+=`` / ``*=`` are reductions (lanes,
+   blocks, then the host fold their shares) and may be returned;
 3. *elementwise fusion*: any other function built from whole-array
    arithmetic, ``math``/``numpy`` scalar functions, ``vectorize``d functions and
    ``out[:] = ...`` stores becomes one fused kernel over the broadcast shape.
@@ -282,9 +284,31 @@ class Dispatcher:
                 pass
         bounds = [eval(src, scope) for src in compiled.range_source]   # noqa: S307
         count = len(range(*[int(b) for b in bounds]))
-        info = kernel_impl.launch_compiled(ctx, compiled, self.py_func.__name__,
-                                           (count,), args)
+        partials = []
+
+        def make_partials(blocks):
+            for _, dtype, _ in compiled.reductions:
+                partials.append(HipNdArray.empty((max(blocks, 1),), dtype,
+                                                 device=ctx.device))
+            return partials
+
+        if count == 0 and compiled.reductions:
+            info = {"kernel": compiled.name, "grid": (0, 0, 0), "block": (0, 0, 0)}
+        else:
+            info = kernel_impl.launch_compiled(
+                ctx, compiled, self.py_func.__name__, (count,), args,
+                make_partials=make_partials if compiled.reductions else None)
         self.last_launch = dict(info, path="parallel loop")
+        # fold the per-block partial results, in block order, onto the values
+        # the reduction variables had before the loop
+        for (name, dtype, op), part in zip(compiled.reductions, partials):
+            blocks = part.asnumpy()
+            start = np.dtype(dtype).type(scope[name])
+            with np.errstate(over="ignore"):
+                fold = blocks.sum(dtype=dtype) if op == "add" else blocks.prod(dtype=dtype)
+                scope[name] = start + fold if op == "add" else start * fold
+        if compiled.return_source is not None:
+            return eval(compiled.return_source, scope)                   # noqa: S307
         return None
 
     # -- 3. elementwise fusion -----------------------------------------------

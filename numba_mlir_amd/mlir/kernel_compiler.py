@@ -383,6 +383,8 @@ class FunctionTranslator:
         # whose top-level prange loop becomes the grid; "device" otherwise
         self.mode = "kernel" if is_kernel else "device"
         self.range_source = None     # parallel mode: source of the prange arguments
+        self.reductions = {}         # parallel mode: reduction variable -> "add" | "mul"
+        self.return_node = None      # parallel mode: the return after the loop
         self.allow_remap = False     # kernels only: see translate_kernel
         self.reversed = False
         self.written_arrays = set()  # elementwise mode: arrays stored through [:]
@@ -390,6 +392,7 @@ class FunctionTranslator:
         self.noalias = False         # no two array arguments overlap (host-checked)
         self.elements_per_thread = 1
         self._lambda_body = None
+        self.reduction_types = []    # (name, Scalar) in parameter order
         self.site_names = {}         # ast node -> stable names
         self.array_info = {}         # variable name -> Array type (views)
 
@@ -1052,6 +1055,12 @@ class FunctionTranslator:
         if len(node.targets) != 1:
             self.err(node, "Chained assignment is not supported")
         target = node.targets[0]
+        if isinstance(target, ast.Name) and target.id in self.reductions and \
+                id(node) in self.top_level:
+            v = self.scalar(node.value)           # the host applies the start value
+            self.bind(target.id, v.type, node)
+            self.maybe_negative.add(target.id)
+            return
         if isinstance(target, ast.Name):
             space = self.special_array_call(node.value)
             if space:
@@ -1248,6 +1257,8 @@ class FunctionTranslator:
         self.emit("continue;")
 
     def stmt_Return(self, node):
+        if node is self.return_node:
+            return                                 # evaluated by the host
         if node.value is None or (isinstance(node.value, ast.Constant) and
                                   node.value.value is None):
             if not self.is_kernel and self.ret_type is not None:
@@ -1324,6 +1335,8 @@ class FunctionTranslator:
         out = []
         for name in sorted(self.assigned):
             t = self.env.get(name)
+            if name in self.reductions:
+                continue                           # lives at kernel scope
             if isinstance(t, Scalar):
                 out.append(f"{t.ctype} {self.cname(name)} = 0;")
             elif isinstance(t, Array):
@@ -1400,6 +1413,18 @@ class FunctionTranslator:
             views.append(f"nmkjit::View<{self.ret_type.ctype}, {n}> nmk_ret = {{nmk_ret_p, "
                          f"{{{', '.join(f'nmk_ret_s{k}' for k in range(n))}}}, "
                          f"{{{', '.join(f'nmk_ret_t{k}' for k in range(n))}}}}};")
+        # one partial result per block and reduction variable, after the
+        # function's own arguments (the host folds them in block order)
+        red = []
+        for name in sorted(self.reductions):
+            t = self.env.get(name)
+            if not isinstance(t, Scalar):
+                self.err(self.node, f"The reduction variable '{name}' has no scalar type")
+            t = INT64 if t.is_bool else t
+            neutral = "0" if self.reductions[name] == "add" else "1"
+            red.append((name, t, neutral))
+            params.append(f"{t.ctype} *nmk_part_{name}")
+        self.reduction_types = [(n, t) for n, t, _ in red]
         params += [f"uint64_t nmk_lds{k}" for k in range(len(self.local_arrays))]
         params += ["int64_t nmk_gsz0", "int64_t nmk_gsz1", "int64_t nmk_gsz2"]
         if self.m.boundscheck:
@@ -1424,6 +1449,8 @@ class FunctionTranslator:
             "  const int64_t " + ", ".join(f"nmk_grp{k} = blockIdx.{dim[k]}" for k in range(3)) + ";",
             "  const int64_t " + ", ".join(f"nmk_lsz{k} = blockDim.{dim[k]}" for k in range(3)) + ";",
         ]
+        for name, t, neutral in red:
+            out.append(f"  {t.ctype} {self.cname(name)} = ({t.ctype}){neutral};")
         if ept > 1:
             out += [
                 "#pragma unroll",
@@ -1460,6 +1487,10 @@ class FunctionTranslator:
         out.append("  }")
         if ept > 1:
             out.append("  }")
+        for name, t, _ in red:
+            op = "AddOp" if self.reductions[name] == "add" else "MulOp"
+            out.append(f"  nmkjit::blockReduceStore<{t.ctype}>({self.cname(name)}, "
+                       f"nmkjit::{op}(), nmk_part_{name});")
         out.append("}")
         return "\n".join(out)
 
@@ -1524,6 +1555,11 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     compiled.range_source = tr.range_source[1] if tr.range_source else None
     compiled.written = sorted(tr.written_arrays)
     compiled.elements_per_thread = tr.elements_per_thread
+    # parallel mode: (name, dtype, "add" | "mul") per reduction, in the order
+    # of their partial-result parameters, and the source of the final return
+    compiled.reductions = [(n, t.dtype, tr.reductions[n]) for n, t in tr.reduction_types]
+    compiled.return_source = (ast.unparse(tr.return_node.value)
+                              if tr.return_node is not None else None)
     # parallel mode: what precedes the loop, for the host to evaluate the
     # loop bounds that depend on it (n = len(x); for i in prange(n))
     compiled.preamble_source = []
@@ -1538,21 +1574,53 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
 
 
 def _check_parallel_shape(tr):
-    """A parallel function is: simple statements, one prange loop, nothing
-    after it (what follows a loop runs once, not per work-item)."""
+    """A parallel function is: assignments, one prange loop, then at most a
+    ``return``.  Scalars that the loop only updates with ``+=`` / ``*=`` and
+    that are set before it are reductions: every lane accumulates its share,
+    blocks reduce theirs, the host folds the per-block partials and evaluates
+    the ``return`` expression."""
     body = tr.body_stmts()
-    seen = False
+    loop = None
+    before = set()
     for stmt in body:
         if isinstance(stmt, ast.For):
-            if seen:
+            if loop is not None:
                 tr.err(stmt, "Only one top-level loop is offloaded")
-            seen = True
-        elif seen and not (isinstance(stmt, ast.Return) and stmt.value is None) and \
-                not isinstance(stmt, ast.Pass):
-            tr.err(stmt, "Statements after the parallel loop are not supported")
-        elif not seen and not isinstance(stmt, (ast.Assign, ast.AugAssign, ast.Expr,
-                                               ast.Pass)):
+            loop = stmt
+        elif loop is not None:
+            if isinstance(stmt, ast.Return) and tr.return_node is None:
+                tr.return_node = stmt if stmt.value is not None else None
+            elif not isinstance(stmt, ast.Pass):
+                tr.err(stmt, "Statements after the parallel loop are not supported")
+        elif isinstance(stmt, ast.Assign):
+            before |= {t.id for t in stmt.targets if isinstance(t, ast.Name)}
+        elif not isinstance(stmt, (ast.AugAssign, ast.Expr, ast.Pass)):
             tr.err(stmt, "Only assignments may precede the parallel loop")
+    if loop is None:
+        return
+    ops = {ast.Add: "add", ast.Mult: "mul"}
+    for node in ast.walk(loop):
+        if isinstance(node, ast.AugAssign) and isinstance(node.target, ast.Name) and \
+                node.target.id in before:
+            name = node.target.id
+            if type(node.op) not in ops or tr.reductions.get(name, ops[type(node.op)]) != \
+                    ops[type(node.op)]:
+                tr.err(node, f"'{name}' is set before the parallel loop and updated in it: "
+                             "only '+=' or only '*=' make it a reduction")
+            tr.reductions[name] = ops[type(node.op)]
+    for node in ast.walk(loop):
+        if isinstance(node, ast.Name) and node.id in tr.reductions and \
+                isinstance(node.ctx, ast.Load):
+            tr.err(node, f"The reduction variable '{node.id}' cannot be read inside the loop")
+        if isinstance(node, ast.Assign) and any(isinstance(t, ast.Name) and
+                                                t.id in tr.reductions for t in node.targets):
+            tr.err(node, "A reduction variable can only be updated with '+=' or '*='")
+    if tr.return_node is not None:
+        for node in ast.walk(tr.return_node.value):
+            if isinstance(node, ast.Name) and node.id in tr.assigned and \
+                    node.id not in tr.reductions and node.id not in before:
+                tr.err(node, f"'{node.id}' is computed inside the loop; only reductions and "
+                             "what precedes the loop can be returned")
 
 
 # ---------------------------------------------------------------------------

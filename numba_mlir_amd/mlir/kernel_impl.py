@@ -392,7 +392,8 @@ def _geometry(ctx, compiled, kern, global_size, local_size):
     return block, [(g + b - 1) // b for g, b in zip(sizes, block)]
 
 
-def _launch_loaded(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret=None):
+def _launch_loaded(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret=None,
+                   partials=()):
     """The compiled host code's sequence for one kernel: parameters, launch,
     wait, destroy event (GpuRuntimeToLlvm.cpp:444-628)."""
     params = _ParamList()
@@ -405,6 +406,8 @@ def _launch_loaded(ctx, compiled, kern, func_name, grid, block, gsize3, args, re
             params.add_scalar(a)
     if ret is not None:
         params.add_array(ret)
+    for part in partials:                 # one pointer per reduction variable
+        params._add(ctypes.c_void_p(part.ptr), lowered.PARAM_PTR)
     for nbytes in compiled.local_bytes:
         params.add_local(int(nbytes))
     for g in gsize3:
@@ -427,15 +430,20 @@ def _launch_loaded(ctx, compiled, kern, func_name, grid, block, gsize3, args, re
             "redirected to element 0)")
 
 
-def launch_compiled(ctx, compiled, func_name, global_size, args, ret=None):
+def launch_compiled(ctx, compiled, func_name, global_size, args, ret=None,
+                    make_partials=None):
     """Loads (once) and launches a translated function over ``global_size``
-    with a runtime-chosen block; returns the launch geometry."""
+    with a runtime-chosen block; returns the launch geometry.
+    ``make_partials(blocks)`` supplies the per-block result arrays of a
+    function with reductions once the grid is known."""
     kern = _loaded_kernel(ctx, compiled)
     per_lane = getattr(compiled, "elements_per_thread", 1)
     lanes = [-(-int(global_size[0]) // per_lane)] + [int(g) for g in global_size[1:]]
     block, grid = _geometry(ctx, compiled, kern, lanes, ())
     gsize3 = [int(g) for g in global_size] + [1] * (3 - len(global_size))
-    _launch_loaded(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret)
+    partials = make_partials(grid[0] * grid[1] * grid[2]) if make_partials else ()
+    _launch_loaded(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret,
+                   partials)
     return {"kernel": compiled.name, "grid": tuple(grid), "block": tuple(block)}
 
 

@@ -122,3 +122,43 @@ def two_returns(a):
 
 def no_loop(x):
     y = 1
+
+
+def sum_of_squares(x):
+    s = 0.0
+    for i in prange(len(x)):
+        s += x[i] * x[i]
+    return math.sqrt(s)
+
+
+def mean_and_count(x, threshold):
+    total = 0.0
+    above = 0
+    n = x.shape[0]
+    for i in prange(n):
+        total += x[i]
+        if x[i] > threshold:
+            above += 1
+    return total / n, above
+
+
+def int_dot(a, b):
+    acc = 10
+    for i in prange(len(a)):
+        acc += a[i] * b[i]
+    return acc
+
+
+def product(x):
+    p = 2.0
+    for i in prange(x.shape[0]):
+        p *= x[i]
+    return p
+
+
+def reduction_read_in_loop(x):
+    s = 0.0
+    for i in prange(len(x)):
+        s += x[i]
+        x[i] = s
+    return s

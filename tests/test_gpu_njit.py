@@ -145,6 +145,32 @@ def test_prange_loops(env):
     np.testing.assert_allclose(out.asnumpy(), ref, rtol=1e-13)
 
 
+def test_prange_reductions(env):
+    """Scalars a prange loop only updates with += / *= are reductions: lanes,
+    blocks, then the host fold their shares; the return runs on the host."""
+    hip, ops, orc, workloads = env
+    rng = np.random.default_rng(14)
+    x = rng.standard_normal(1000003).astype(np.float32)
+    got = njit(parallel=True)(cases.sum_of_squares)(hip.asarray(x))
+    # x[i] * x[i] is a float32 product; the accumulator is float64
+    np.testing.assert_allclose(got, np.sqrt((x * x).astype(np.float64).sum()), rtol=1e-12)
+    mean, above = njit(parallel=True)(cases.mean_and_count)(hip.asarray(x), 0.5)
+    np.testing.assert_allclose(mean, x.astype(np.float64).mean(), rtol=1e-9, atol=1e-12)
+    assert above == int((x > 0.5).sum())
+    a = rng.integers(-1000, 1000, 70001).astype(np.int32)
+    b = rng.integers(-1000, 1000, 70001).astype(np.int32)
+    f = njit(parallel=True)(cases.int_dot)
+    assert f(hip.asarray(a), hip.asarray(b)) == 10 + int((a.astype(np.int64) * b).sum())
+    assert f(hip.asarray(a[:0]), hip.asarray(b[:0])) == 10       # empty loop: start value
+    # repeated launches fold in the same order: same bits
+    g = njit(parallel=True)(cases.sum_of_squares)
+    dx = hip.asarray(x)
+    assert len({g(dx) for _ in range(5)}) == 1
+    p = rng.uniform(0.9, 1.1, 5000)
+    np.testing.assert_allclose(njit(parallel=True)(cases.product)(hip.asarray(p)),
+                               2.0 * np.prod(p), rtol=1e-12)
+
+
 def test_reductions_and_contractions_go_to_the_library(env):
     hip, ops, orc, workloads = env
     x = workloads.reduce_f32(256, 4096)

@@ -322,3 +322,22 @@ def test_fused_maps_take_several_elements_per_lane(K, tmp_path, monkeypatch):
     ck = kc.translate(njit_cases.fused_map, types, ndim, K, mode=mode, noalias=True,
                       elements_per_thread=4)
     assert ck.elements_per_thread == 1 and "nmk_rep" not in ck.source
+
+
+def test_prange_reductions(K, tmp_path, monkeypatch):
+    import njit_cases
+    monkeypatch.setattr(kc, "CACHE_DIR", str(tmp_path))
+    f32 = kc.Array(kc.FLOAT32, 1, layout="C")
+    ck = kc.translate(njit_cases.mean_and_count, [f32, kc.FLOAT64], 1, K, mode="parallel",
+                      noalias=True, elements_per_thread=4)
+    assert ck.reductions == [("above", np.dtype(np.int64), "add"),
+                             ("total", np.dtype(np.float64), "add")]
+    assert ck.return_source == "(total / n, above)"
+    assert "int64_t *nmk_part_above, double *nmk_part_total" in ck.source
+    assert ck.source.count("nmkjit::blockReduceStore<") == 2
+    assert kc.build_code_object(ck)[:4] == b"\x7fELF"
+    ck = kc.translate(njit_cases.product, [f32], 1, K, mode="parallel")
+    assert ck.reductions == [("p", np.dtype(np.float64), "mul")]
+    assert "double v_p = (double)1;" in ck.source
+    with pytest.raises(kc.KernelCompileError, match="cannot be read inside the loop"):
+        kc.translate(njit_cases.reduction_read_in_loop, [f32], 1, K, mode="parallel")
