@@ -211,7 +211,10 @@ class Dispatcher:
                     else:
                         ok = False
                 if ok:
-                    return self._served("library", _REDUCE[name](x, axis=axis), x.ctx)
+                    result = _REDUCE[name](x, axis=axis)
+                    if axis is None and isinstance(result, HipNdArray):
+                        result = result.asnumpy().reshape(-1)[0]   # a scalar, as NumPy's
+                    return self._served("library", result, x.ctx)
             # np.sqrt(np.sum(x * x))
             call = np_call(expr, ("sqrt",))
             if call and len(call[1]) == 1 and not call[2]:
@@ -224,7 +227,9 @@ class Dispatcher:
                             prod.left.id == prod.right.id:
                         x = array(prod.left)
                         if x is not None and x.dtype == np.float32:
-                            return self._served("library", ops.sqrt_sum_squares(x), x.ctx)
+                            return self._served(
+                                "library", ops.sqrt_sum_squares(x).asnumpy().reshape(-1)[0],
+                                x.ctx)
         except (TypeError, ValueError, NotImplementedError):
             return NotImplemented       # outside what the kernel covers: fuse instead
         return NotImplemented

@@ -162,3 +162,32 @@ def reduction_read_in_loop(x):
         s += x[i]
         x[i] = s
     return s
+
+
+def parfor_add(a, b, c):
+    for i in prange(len(a)):
+        c[i] = a[i] + b[i]
+
+
+def parfor_scalar(a, b, c, d):
+    for i in prange(len(a)):
+        c[i] = a[i] + b[i] + d
+
+
+def nested_prange(a):
+    ah, aw = a.shape
+    for h in prange(ah):
+        for w in prange(aw):
+            a[h, w] = w + h * aw
+
+
+def scale_into(a, b):
+    b[:] = a * 2
+
+
+def add_into(a, b, c):
+    c[:] = a + b
+
+
+def fill(a):
+    a[:] = 42

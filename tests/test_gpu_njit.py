@@ -145,6 +145,44 @@ def test_prange_loops(env):
     np.testing.assert_allclose(out.asnumpy(), ref, rtol=1e-13)
 
 
+SCALARS = [True, False, -3, -2, -1, 0, 1, 2, 3, -2.5, -1.0, -0.5, -0.0, 0.0, 0.5, 1.0, 2.5]
+
+
+def test_reference_parfor_and_array_statement_tests(env):
+    """test_gpu.py:1518-1700: prange loops over device and shared arrays, a
+    scalar argument or captured value of every kind, b[:] = a * 2, c[:] = a + b,
+    nested prange with the shape unpacked before the loop."""
+    hip, ops, orc, workloads = env
+    a = np.arange(1024, dtype=np.float32)
+    b = np.arange(1024, dtype=np.float32) * 3
+    da, db = hip.asarray(a), hip.asarray(b, usm_type="shared")
+    out = hip.asarray(np.zeros(1024, np.float32))
+    njit(cases.parfor_add)(da, db, out)
+    np.testing.assert_array_equal(out.asnumpy(), a + b)
+    for val in SCALARS:
+        ref = np.zeros(1024, np.float32)
+        cases.parfor_scalar(a, b, ref, val)
+        njit(cases.parfor_scalar)(da, db, out, val)
+        np.testing.assert_array_equal(out.asnumpy(), ref)
+
+        def captured(a, b, c):
+            for i in cases.prange(len(a)):
+                c[i] = a[i] + b[i] + val
+
+        njit(captured)(da, db, out)
+        np.testing.assert_array_equal(out.asnumpy(), ref)
+    njit(cases.scale_into)(da, out)
+    np.testing.assert_array_equal(out.asnumpy(), a * 2)
+    njit(cases.add_into)(da, db, out)
+    np.testing.assert_array_equal(out.asnumpy(), a + b)
+    njit(cases.fill)(out)
+    np.testing.assert_array_equal(out.asnumpy(), np.full(1024, 42, np.float32))
+    grid = hip.asarray(np.zeros((2, 3), np.float32))
+    for options in ({}, {"gpu_use_64bit_index": True}, {"fastmath": True}):
+        njit(cases.nested_prange, **options)(grid)
+        np.testing.assert_array_equal(grid.asnumpy(), [[0, 1, 2], [3, 4, 5]])
+
+
 def test_prange_reductions(env):
     """Scalars a prange loop only updates with += / *= are reductions: lanes,
     blocks, then the host fold their shares; the return runs on the host."""
@@ -187,8 +225,34 @@ def test_reductions_and_contractions_go_to_the_library(env):
     f = njit(cases.norm)
     got = f(hip.asarray(x))
     assert f.last_launch["kernel"] == "nmk_norm2_f32"
-    np.testing.assert_allclose(got.asnumpy()[0], np.sqrt((x.astype(np.float64) ** 2).sum()),
-                               rtol=1e-5)
+    assert isinstance(got, np.float32)
+    np.testing.assert_allclose(got, np.sqrt((x.astype(np.float64) ** 2).sum()), rtol=1e-5)
+    # the reference's reduce tests (test_gpu.py:2045-2098): sizes, shapes, forms
+    for size in (7, 16, 64, 65, 256, 512, 1024 * 1024):
+        v = np.arange(size, dtype=np.float32)
+        np.testing.assert_allclose(njit(lambda a: a.sum())(hip.asarray(v)), v.sum(), rtol=1e-5)
+    forms = [                                  # one lambda per source line
+        lambda a: a.sum(),
+        lambda a: a.sum(axis=0),
+        lambda a: a.sum(axis=1),
+        lambda a: np.prod(a),
+        lambda a: np.prod(a, axis=0),
+        lambda a: np.prod(a, axis=1),
+        lambda a: np.amin(a),
+        lambda a: np.amax(a),
+    ]
+    for k, form in enumerate(forms):
+        for shape in ((7, 16), (25, 64), (65, 7)):
+            for dtype in (np.int32, np.int64, np.float32):
+                count = shape[0] * shape[1]
+                if count > 30 and 3 <= k <= 5:
+                    continue                   # products overflow (skipped there too)
+                v = np.arange(1, count + 1, dtype=dtype).reshape(shape).copy()
+                f = njit(form)
+                got = f(hip.asarray(v))
+                assert f.last_launch["path"] == "library"
+                got = got.asnumpy() if hasattr(got, "asnumpy") else got
+                np.testing.assert_allclose(got, form(v), rtol=1e-5)
     a, b = workloads.matmul(256)
     for fn in (cases.matmul, cases.dot):
         got = njit(fn)(hip.asarray(a), hip.asarray(b))
