@@ -110,6 +110,7 @@ class Dispatcher:
         self._names = None             # what the body's free names are bound to
         self._parallel_loop = None     # whether the body has a top-level prange loop
         self._library_form = None      # the one-expression pattern, parsed once
+        self._rank = None              # grid dimensions of the prange nest
         functools.update_wrapper(self, py_func)
 
     # -- entry ---------------------------------------------------------------
@@ -276,9 +277,30 @@ class Dispatcher:
             self._compiled[key] = compiled
         return compiled
 
+    def _grid_rank(self):
+        """Depth of the perfect nest of prange loops at the top level (up to
+        three; inner bounds must not depend on outer loop variables)."""
+        if self._rank is None:
+            loop = next(s for s in self._node.body if isinstance(s, ast.For))
+            rank, seen = 1, {loop.target.id} if isinstance(loop.target, ast.Name) else set()
+            while rank < 3 and len(loop.body) == 1 and isinstance(loop.body[0], ast.For):
+                inner = loop.body[0]
+                it = inner.iter
+                if not (isinstance(it, ast.Call) and isinstance(it.func, ast.Name) and
+                        getattr(self._resolve(it.func.id), "_nmk_prange", False)):
+                    break
+                used = {n.id for a in it.args for n in ast.walk(a) if isinstance(n, ast.Name)}
+                if used & seen or not isinstance(inner.target, ast.Name):
+                    break
+                seen.add(inner.target.id)
+                loop, rank = inner, rank + 1
+            self._rank = rank
+        return self._rank
+
     def _parallel(self, args):
         ctx = kernel_impl.check_device_args(args)
-        compiled = self._compile("parallel", args, 1, False)
+        rank = self._grid_rank()
+        compiled = self._compile("parallel", args, rank, rank > 1)
         scope = dict(getattr(self.py_func, "__globals__", {}))
         scope.update(inspect.getclosurevars(self.py_func).nonlocals)
         scope.update(zip(self._params(), args))
@@ -287,8 +309,20 @@ class Dispatcher:
                 exec(src, scope)      # noqa: S102
             except Exception:         # noqa: BLE001 -- device-only values
                 pass
-        bounds = [eval(src, scope) for src in compiled.range_source]   # noqa: S307
-        count = len(range(*[int(b) for b in bounds]))
+        def trip_counts(kernel):
+            out = []
+            for sources in kernel.grid_sources:
+                bounds = [eval(src, scope) for src in sources]         # noqa: S307
+                out.append(len(range(*[int(b) for b in bounds])))
+            return out
+
+        counts = trip_counts(compiled)
+        if rank > 1 and max(counts[:-1]) > 65535:
+            # the outer loops land on grid y / z, which are 16-bit: keep only
+            # the outermost loop as the grid
+            compiled = self._compile("parallel", args, 1, False)
+            counts = trip_counts(compiled)
+        count = math.prod(counts)
         partials = []
 
         def make_partials(blocks):
@@ -301,7 +335,7 @@ class Dispatcher:
             info = {"kernel": compiled.name, "grid": (0, 0, 0), "block": (0, 0, 0)}
         else:
             info = kernel_impl.launch_compiled(
-                ctx, compiled, self.py_func.__name__, (count,), args,
+                ctx, compiled, self.py_func.__name__, tuple(counts), args,
                 make_partials=make_partials if compiled.reductions else None)
         self.last_launch = dict(info, path="parallel loop")
         # fold the per-block partial results, in block order, onto the values

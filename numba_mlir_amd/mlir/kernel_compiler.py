@@ -383,6 +383,8 @@ class FunctionTranslator:
         # whose top-level prange loop becomes the grid; "device" otherwise
         self.mode = "kernel" if is_kernel else "device"
         self.range_source = None     # parallel mode: source of the prange arguments
+        self.grid_loops = []         # parallel mode: the perfectly nested prange loops
+        self.grid_sources = []       # ... and the source of their range arguments
         self.reductions = {}         # parallel mode: reduction variable -> "add" | "mul"
         self.return_node = None      # parallel mode: the return after the loop
         self.allow_remap = False     # kernels only: see translate_kernel
@@ -1201,18 +1203,25 @@ class FunctionTranslator:
         stop = a[1] if len(a) > 1 else a[0]
         step = a[2] if len(a) > 2 else constant(1)
         name = node.target.id
-        if is_prange and self.mode == "parallel" and id(node) in self.top_level:
-            # the parallel loop is the grid: work-item g runs iteration g
-            if self.range_source is not None and self.range_source[0] is not node:
-                self.err(node, "Only one top-level prange loop is offloaded")
+        depth = self.grid_depth(node) if (is_prange and self.mode == "parallel") else None
+        if depth is not None:
+            # a grid loop: work-item g of dimension `depth` runs iteration g
             if step.const is None or step.const <= 0:
                 self.err(node, "A prange step must be a positive constant")
-            self.range_source = (node, [ast.unparse(x) for x in it.args])
+            if depth == 0:
+                if self.range_source is not None and self.range_source[0] is not node:
+                    self.err(node, "Only one top-level prange loop is offloaded")
+                self.range_source = (node, [ast.unparse(x) for x in it.args])
+                self.grid_loops = [node]
+                self.grid_sources = [self.range_source[1]]
+            elif node not in self.grid_loops:
+                self.grid_loops.append(node)
+                self.grid_sources.append([ast.unparse(x) for x in it.args])
             self.bind(name, INT64, node)
             if not start.nonneg:
                 self.maybe_negative.add(name)
             if self.emitting:
-                self.emit(f"{self.cname(name)} = {start.code} + nmk_gid0 * {step.code};")
+                self.emit(f"{self.cname(name)} = {start.code} + nmk_gid{depth} * {step.code};")
             self.indent -= 1
             self.block(node.body)
             self.indent += 1
@@ -1241,6 +1250,18 @@ class FunctionTranslator:
         self.emit("}")
         self.indent -= 1
         self.emit("}")
+
+    def grid_depth(self, node):
+        """Which grid dimension a prange loop is, or None for a sequential one:
+        the top-level loop is dimension 0; a prange loop that is the whole body
+        of grid loop k is dimension k + 1 (a perfect nest), while the launch
+        has that many dimensions."""
+        if id(node) in self.top_level:
+            return 0
+        for k, outer in enumerate(self.grid_loops):
+            if k + 1 < self.ndim and len(outer.body) == 1 and outer.body[0] is node:
+                return k + 1
+        return None
 
     def stmt_While(self, node):
         if node.orelse:
@@ -1553,6 +1574,7 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     compiled.reversed_dims = tr.reversed
     compiled.ret_dtype = tr.ret_type.dtype if (mode == "elementwise" and tr.ret_type) else None
     compiled.range_source = tr.range_source[1] if tr.range_source else None
+    compiled.grid_sources = list(tr.grid_sources)   # per grid dimension
     compiled.written = sorted(tr.written_arrays)
     compiled.elements_per_thread = tr.elements_per_thread
     # parallel mode: (name, dtype, "add" | "mul") per reduction, in the order

@@ -179,8 +179,21 @@ def test_reference_parfor_and_array_statement_tests(env):
     np.testing.assert_array_equal(out.asnumpy(), np.full(1024, 42, np.float32))
     grid = hip.asarray(np.zeros((2, 3), np.float32))
     for options in ({}, {"gpu_use_64bit_index": True}, {"fastmath": True}):
-        njit(cases.nested_prange, **options)(grid)
+        f = njit(cases.nested_prange, **options)
+        f(grid)
         np.testing.assert_array_equal(grid.asnumpy(), [[0, 1, 2], [3, 4, 5]])
+    # the perfect nest is a 2-d grid with the inner loop on x ...
+    big = hip.asarray(np.zeros((300, 1000), np.float32))
+    f(big)
+    assert f.last_launch["grid"][1] == 300 and f.last_launch["block"][1] == 1
+    np.testing.assert_array_equal(big.asnumpy(),
+                                  np.arange(300000, dtype=np.float32).reshape(300, 1000))
+    # ... unless the outer loop is too long for grid y: then it alone is the grid
+    tall = hip.asarray(np.zeros((70000, 4), np.float32))
+    f(tall)
+    assert f.last_launch["grid"][1] == 1
+    np.testing.assert_array_equal(tall.asnumpy(),
+                                  np.arange(280000, dtype=np.float32).reshape(70000, 4))
 
 
 def test_prange_reductions(env):
