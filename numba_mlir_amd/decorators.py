@@ -95,6 +95,9 @@ _REDUCE = {"sum": ops.sum, "prod": ops.prod, "min": ops.amin, "max": ops.amax,
 class Dispatcher:
     def __init__(self, py_func, parallel=False, boundscheck=None, **options):
         self.py_func = py_func
+        # inside another compiled function or kernel a call of this one is
+        # inlined as a device function of its scalar arguments
+        self._nmk_vectorized = py_func
         self.parallel = parallel
         if boundscheck is None:
             boundscheck = readenv("NUMBA_MLIR_KERNEL_BOUNDSCHECK", int, 0)

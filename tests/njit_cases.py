@@ -191,3 +191,9 @@ def add_into(a, b, c):
 
 def fill(a):
     a[:] = 42
+
+
+def _smoothstep(x, lo, hi):
+    t = min(max((x - lo) / (hi - lo), 0.0), 1.0)
+    return t * t * (3.0 - 2.0 * t)
+

@@ -273,6 +273,33 @@ def test_reductions_and_contractions_go_to_the_library(env):
                                    atol=1e-3)
 
 
+def test_compiled_functions_call_each_other(env):
+    """An njit function called from a prange loop or a kernel is inlined as a
+    device function of its scalar arguments."""
+    hip, ops, orc, workloads = env
+    from numba_mlir_amd import kernel as K
+    smooth = njit(cases._smoothstep)
+    x = np.linspace(-0.5, 1.5, 1001)
+
+    def loop(x, out):
+        for i in cases.prange(len(x)):
+            out[i] = smooth(x[i], 0.25, 0.75)
+
+    def body(x, out):
+        i = K.get_global_id(0)
+        out[i] = smooth(x[i], 0.25, 0.75) * 2.0
+
+    ref = np.array([cases._smoothstep(v, 0.25, 0.75) for v in x])
+    out = hip.asarray(np.zeros_like(x))
+    njit(parallel=True)(loop)(hip.asarray(x), out)
+    np.testing.assert_allclose(out.asnumpy(), ref, rtol=1e-15)
+    K.kernel(body)[len(x), K.DEFAULT_LOCAL_SIZE](hip.asarray(x), out)
+    np.testing.assert_allclose(out.asnumpy(), 2.0 * ref, rtol=1e-15)
+    # whole-array form: the same function maps over arrays
+    f = njit(lambda x: smooth(x, 0.25, 0.75))
+    np.testing.assert_allclose(f(hip.asarray(x)).asnumpy(), ref, rtol=1e-15)
+
+
 def test_unsupported_functions_are_reported(env):
     hip, ops, orc, workloads = env
     from numba_mlir_amd.kernel import KernelCompileError
