@@ -92,7 +92,10 @@ template <> struct Mfma<double> {
   typedef doublex2 Vec;
   typedef doublex4 Acc;
   // PAD 16: consecutive k rows land 32 banks apart for a 128-wide tile
-  static constexpr int TILE = 16, KSTEP = 4, BK = 8, VEC = 2, NACC = 4,
+#ifndef NMHIP_DGEMM_BK
+#define NMHIP_DGEMM_BK 16
+#endif
+  static constexpr int TILE = 16, KSTEP = 4, BK = NMHIP_DGEMM_BK, VEC = 2, NACC = 4,
                        PAD = 16;
   __device__ static __forceinline__ Acc mma(double a, double b, Acc c) {
     return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
@@ -104,13 +107,14 @@ template <> struct Mfma<double> {
 
 // One operand's slab of X x BK (X = BM or BN) on its way from global memory
 // to LDS[k][x].  NV 128-bit words per thread.
-//   K_CONTIG: thread -> (x = tid / (BK/VEC) + 64 i, k = VEC (tid % (BK/VEC)) ..)
+//   K_CONTIG: thread -> (x = tid / (BK/VEC) + X_STEP i, k = VEC (tid % (BK/VEC)) ..)
 //   else    : thread -> (k = tid / (X/VEC) + K_ROWS i, x = VEC (tid % (X/VEC)) ..)
 template <typename T, int X, bool K_CONTIG> struct SlabFetch {
   typedef Mfma<T> M;
   typedef typename M::Vec Vec;
-  static constexpr int NV = X / 64;
-  static constexpr int K_ROWS = 256 * M::VEC / X;
+  static constexpr int NV = X * M::BK / (M::VEC * 256);
+  static constexpr int X_STEP = 256 * M::VEC / M::BK; // K_CONTIG: x rows per pass
+  static constexpr int K_ROWS = 256 * M::VEC / X;     // else: k rows per pass
   int x, k;
   const T *base;
   int64_t ld;
@@ -133,7 +137,7 @@ template <typename T, int X, bool K_CONTIG> struct SlabFetch {
 #pragma unroll
     for (int i = 0; i < NV; ++i)
       reg[i] = *reinterpret_cast<const Vec *>(
-          K_CONTIG ? base + int64_t(64 * i) * ld + k0
+          K_CONTIG ? base + int64_t(X_STEP * i) * ld + k0
                    : base + int64_t(k0 + K_ROWS * i) * ld);
   }
   __device__ __forceinline__ void stash(T (*lds)[X + M::PAD]) const {
@@ -142,7 +146,7 @@ template <typename T, int X, bool K_CONTIG> struct SlabFetch {
       if (K_CONTIG) {
 #pragma unroll
         for (int q = 0; q < M::VEC; ++q)
-          lds[k + q][x + 64 * i] = reg[i][q];
+          lds[k + q][x + X_STEP * i] = reg[i][q];
       } else {
         *reinterpret_cast<Vec *>(&lds[k + K_ROWS * i][x]) = reg[i];
       }

@@ -174,7 +174,7 @@ def test_identity_and_linearity_full_size(env):
 
 
 @pytest.mark.parametrize("ta,tb,tc", list(itertools.product([False, True], repeat=3)))
-@pytest.mark.parametrize("m,n,k", [(128, 128, 8), (256, 384, 72), (1024, 1024, 1024)])
+@pytest.mark.parametrize("m,n,k", [(128, 128, 16), (256, 384, 80), (1024, 1024, 1024)])
 def test_float64_mfma(env, ta, tb, tc, m, n, k):
     """mkl_gemm_float64_device on the fp64 matrix cores, every layout; the
     tolerance is rel 1e-5 (float64 bar), met with a wide margin."""
