@@ -66,6 +66,7 @@ def vectorize(arg_or_function=(), **kws):
 
 
 ELEMENTS_PER_THREAD = 4     # of a fused 1-d map or prange loop
+MAX_PLANS = kernel_impl.MAX_PLANS   # stored launches per compiled function
 
 
 def _disjoint(arrays):
@@ -105,6 +106,8 @@ class Dispatcher:
         self.options = options
         self.last_launch = None          # what served the most recent call
         self._compiled = {}
+        self._plans = {}
+        self._loop_plans = {}
         try:
             node = kernel_compiler._function_ast(py_func)
         except kernel_compiler.KernelCompileError:
@@ -300,30 +303,66 @@ class Dispatcher:
             self._rank = rank
         return self._rank
 
+    def _host_scope(self, args):
+        """The names the body's host-side statements see."""
+        func = self.py_func
+        scope = dict(getattr(func, "__globals__", {}))
+        for name, cell in zip(func.__code__.co_freevars, func.__closure__ or ()):
+            try:
+                scope[name] = cell.cell_contents
+            except ValueError:            # not yet bound
+                pass
+        scope.update(zip(self._params(), args))
+        return scope
+
+    @staticmethod
+    def _host_code(compiled):
+        """A translated loop's host-side sources as code objects (once)."""
+        code = getattr(compiled, "_host_code", None)
+        if code is None:
+            code = compiled._host_code = (
+                [compile(src, "<loop preamble>", "exec") for src in compiled.preamble_source],
+                [[compile(src, "<loop bound>", "eval") for src in sources]
+                 for sources in compiled.grid_sources],
+                None if compiled.return_source is None else
+                compile(compiled.return_source, "<loop result>", "eval"))
+        return code
+
     def _parallel(self, args):
         ctx = kernel_impl.check_device_args(args)
-        rank = self._grid_rank()
-        compiled = self._compile("parallel", args, rank, rank > 1)
-        scope = dict(getattr(self.py_func, "__globals__", {}))
-        scope.update(inspect.getclosurevars(self.py_func).nonlocals)
-        scope.update(zip(self._params(), args))
-        for src in compiled.preamble_source:
-            try:                      # scalars the loop bounds may be built from
-                exec(src, scope)      # noqa: S102
-            except Exception:         # noqa: BLE001 -- device-only values
-                pass
-        def trip_counts(kernel):
-            out = []
-            for sources in kernel.grid_sources:
-                bounds = [eval(src, scope) for src in sources]         # noqa: S307
-                out.append(len(range(*[int(b) for b in bounds])))
-            return out
+        arrays = [a for a in args if isinstance(a, HipNdArray)]
+        # what the choice of kernel depends on: types, shapes, strides, aliasing
+        key = (ctx, kernel_impl.plan_key(args),
+               kernel_impl.captured_constants(self.py_func), _disjoint(arrays))
+        entry = self._loop_plans.get(key)
+        if entry is None:
+            if len(self._loop_plans) >= MAX_PLANS:
+                self._loop_plans.clear()
+            rank = self._grid_rank()
+            entry = self._loop_plans[key] = {
+                "nest": self._compile("parallel", args, rank, rank > 1),
+                "flat": None, "plans": {}}
+        scope = self._host_scope(args)
 
+        def trip_counts(kernel):
+            preamble, bounds, _ = self._host_code(kernel)
+            for code in preamble:
+                try:                      # scalars the loop bounds may be built from
+                    exec(code, scope)     # noqa: S102
+                except Exception:         # noqa: BLE001 -- device-only values
+                    pass
+            return tuple(len(range(*[int(eval(code, scope)) for code in codes]))  # noqa: S307
+                         for codes in bounds)
+
+        compiled = entry["nest"]
         counts = trip_counts(compiled)
-        if rank > 1 and max(counts[:-1]) > 65535:
+        if len(counts) > 1 and max(counts[:-1]) > 65535:
             # the outer loops land on grid y / z, which are 16-bit: keep only
             # the outermost loop as the grid
-            compiled = self._compile("parallel", args, 1, False)
+            if entry["flat"] is None:
+                entry["flat"] = self._compile("parallel", args, 1, False)
+            compiled = entry["flat"]
+            scope = self._host_scope(args)
             counts = trip_counts(compiled)
         count = math.prod(counts)
         partials = []
@@ -337,9 +376,20 @@ class Dispatcher:
         if count == 0 and compiled.reductions:
             info = {"kernel": compiled.name, "grid": (0, 0, 0), "block": (0, 0, 0)}
         else:
-            info = kernel_impl.launch_compiled(
-                ctx, compiled, self.py_func.__name__, tuple(counts), args,
-                make_partials=make_partials if compiled.reductions else None)
+            plan = entry["plans"].get((compiled.name, counts))
+            if plan is None:
+                plan = kernel_impl.plan_compiled(
+                    ctx, compiled, self.py_func.__name__, counts, args,
+                    make_partials=make_partials if compiled.reductions else None)
+                plan.run()
+                if len(entry["plans"]) >= MAX_PLANS:
+                    entry["plans"].clear()
+                entry["plans"][(compiled.name, counts)] = plan
+            else:
+                if compiled.reductions:
+                    make_partials(math.prod(plan.grid))
+                plan.run(args, partials=partials)
+            info = plan.info
         self.last_launch = dict(info, path="parallel loop")
         # fold the per-block partial results, in block order, onto the values
         # the reduction variables had before the loop
@@ -349,13 +399,33 @@ class Dispatcher:
             with np.errstate(over="ignore"):
                 fold = blocks.sum(dtype=dtype) if op == "add" else blocks.prod(dtype=dtype)
                 scope[name] = start + fold if op == "add" else start * fold
-        if compiled.return_source is not None:
-            return eval(compiled.return_source, scope)                   # noqa: S307
+        return_code = self._host_code(compiled)[2]
+        if return_code is not None:
+            return eval(return_code, scope)                              # noqa: S307
         return None
 
     # -- 3. elementwise fusion -----------------------------------------------
     def _elementwise(self, args):
         ctx = kernel_impl.check_device_args(args)
+        # Everything but addresses and scalar values is fixed by the argument
+        # types, shapes and strides: such a call replays a stored launch.
+        key = (ctx, kernel_impl.plan_key(args),
+               kernel_impl.captured_constants(self.py_func))
+        entry = self._plans.get(key)
+        if entry is not None:
+            plan = entry["plan"]
+            if plan is None:              # an argument is written: aliasing decides
+                plan = entry["by_alias"].get(
+                    _disjoint([a for a in args if isinstance(a, HipNdArray)]))
+            if plan is not None:
+                ret = None
+                if entry["ret_dtype"] is not None:
+                    ret = HipNdArray.empty(entry["shape"], entry["ret_dtype"],
+                                           device=ctx.device)
+                plan.run(args, ret)
+                self.last_launch = dict(plan.info, path="elementwise")
+                return ret
+
         arrays = [a for a in args if isinstance(a, HipNdArray)]
         shape = np.broadcast_shapes(*[a.shape for a in arrays])
         views = [a.broadcast_to(shape) if isinstance(a, HipNdArray) else a for a in args]
@@ -380,9 +450,21 @@ class Dispatcher:
         if compiled.ret_dtype is not None:
             ret = HipNdArray.empty(shape, compiled.ret_dtype, device=ctx.device)
         ret_view = ret.reshape(run_shape) if (ret is not None and dense) else ret
-        info = kernel_impl.launch_compiled(ctx, compiled, self.py_func.__name__,
-                                           run_shape, views, ret_view)
-        self.last_launch = dict(info, path="elementwise")
+        plan = kernel_impl.plan_compiled(ctx, compiled, self.py_func.__name__,
+                                         run_shape, views, ret_view)
+        plan.run()
+        self.last_launch = dict(plan.info, path="elementwise")
+
+        if len(self._plans) >= MAX_PLANS:
+            self._plans.clear()
+        writes = any(f"v_{name}" in compiled.written for name in self._params())
+        entry = self._plans.setdefault(key, {
+            "plan": None, "by_alias": {}, "shape": tuple(shape),
+            "ret_dtype": compiled.ret_dtype})
+        if writes:
+            entry["by_alias"][_disjoint(arrays)] = plan
+        else:
+            entry["plan"] = plan
         return ret
 
 

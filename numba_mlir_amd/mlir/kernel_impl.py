@@ -21,6 +21,7 @@ is an error, as in the reference.
 """
 
 import ctypes
+import threading
 import weakref
 
 import numpy as np
@@ -153,13 +154,16 @@ class _ParamList:
 
     def _add(self, cvalue, ptype):
         self._slots.append((cvalue, ptype))
+        return cvalue
 
     def add_array(self, arr):
-        self._add(ctypes.c_void_p(arr.ptr), lowered.PARAM_PTR)
+        """Returns the pointer slot (a launch plan rewrites it per call)."""
+        slot = self._add(ctypes.c_void_p(arr.ptr), lowered.PARAM_PTR)
         for n in arr.shape:
             self._add(ctypes.c_int64(n), lowered.PARAM_INT64)
         for s in arr.elem_strides:
             self._add(ctypes.c_int64(s), lowered.PARAM_INT64)
+        return slot
 
     def add_local(self, nbytes):
         self._slots.append((None, nbytes))
@@ -179,23 +183,25 @@ class _ParamList:
     }
 
     def add_scalar(self, value):
+        """Returns the value slot."""
         if isinstance(value, (bool, np.bool_)):
-            self._add(ctypes.c_bool(bool(value)), lowered.PARAM_BOOL)
-        elif isinstance(value, np.generic) and value.dtype in self._SCALAR_PARAMS:
+            return self._add(ctypes.c_bool(bool(value)), lowered.PARAM_BOOL)
+        if isinstance(value, np.generic) and value.dtype in self._SCALAR_PARAMS:
             ctype, ptype = self._SCALAR_PARAMS[value.dtype]
-            self._add(ctype(value.item()), ptype)
-        elif isinstance(value, int):
-            self._add(ctypes.c_int64(value), lowered.PARAM_INT64)
-        elif isinstance(value, float):
-            self._add(ctypes.c_double(value), lowered.PARAM_FLOAT64)
-        else:
-            raise TypeError(f"Unsupported kernel argument type: {type(value)}")
+            return self._add(ctype(value.item()), ptype)
+        if isinstance(value, int):
+            return self._add(ctypes.c_int64(value), lowered.PARAM_INT64)
+        if isinstance(value, float):
+            return self._add(ctypes.c_double(value), lowered.PARAM_FLOAT64)
+        raise TypeError(f"Unsupported kernel argument type: {type(value)}")
+
+    SLICE_NONE = -2 ** 63         # an omitted bound
 
     def add_slice(self, value):
-        none = -2 ** 63           # an omitted bound
-        for part in (value.start, value.stop, value.step):
-            self._add(ctypes.c_int64(none if part is None else int(part)),
-                      lowered.PARAM_INT64)
+        """Returns the three slots (start, stop, step)."""
+        return [self._add(ctypes.c_int64(self.SLICE_NONE if part is None else int(part)),
+                          lowered.PARAM_INT64)
+                for part in (value.start, value.stop, value.step)]
 
     def build(self):
         descs = (GPUParamDesc * (len(self._slots) + 1))()
@@ -216,6 +222,7 @@ class _ParamList:
 
 NO_DEPS = (ctypes.c_void_p * 1)(None)
 MAX_SPECIALISATIONS = 16   # per kernel, before new shapes get the general form
+MAX_PLANS = 64             # stored launches per kernel
 
 
 def _release_handles(handles):
@@ -284,6 +291,7 @@ class Kernel(KernelBase):
             "boundscheck", readenv("NUMBA_MLIR_KERNEL_BOUNDSCHECK", int, 0)))
         self.last_launch = None
         self._compiled = {}
+        self._plans = {}       # stored launches (shared by configured copies)
 
     def _twin_name(self, args):
         first = next((a for a in args if isinstance(a, HipNdArray)), None)
@@ -332,6 +340,14 @@ class Kernel(KernelBase):
             block += [1] * (3 - ndim)
             grid = [(g + b - 1) // b for g, b in zip(gsize3, block)]
         else:
+            # Types, shapes and strides seen before replay a stored launch.
+            key = (ctx, plan_key(args), captured_constants(self.py_func),
+                   tuple(gsize3[:ndim]), tuple(self.local_size))
+            plan = self._plans.get(key)
+            if plan is not None:
+                plan.run(args)
+                self.last_launch = plan.info
+                return
             # With a runtime-chosen block a body that cannot observe its
             # grouping is laid out for coalescing (last dimension on x), unless
             # that pushes a long dimension past the y / z grid limit.
@@ -347,9 +363,13 @@ class Kernel(KernelBase):
             name = compiled.name
 
         if compiled is not None:
-            _launch_loaded(ctx, compiled, kern, self.py_func.__name__, grid, block,
-                           gsize3, args)
-            self.last_launch = {"kernel": name, "grid": tuple(grid), "block": tuple(block)}
+            plan = LaunchPlan(ctx, compiled, kern, self.py_func.__name__, grid, block,
+                              gsize3, args)
+            plan.run()
+            if len(self._plans) >= MAX_PLANS:
+                self._plans.clear()
+            self._plans[key] = plan
+            self.last_launch = plan.info
             return
 
         params = _ParamList()
@@ -392,59 +412,113 @@ def _geometry(ctx, compiled, kern, global_size, local_size):
     return block, [(g + b - 1) // b for g, b in zip(sizes, block)]
 
 
+class LaunchPlan:
+    """One kernel launch with everything that depends only on the arguments'
+    types, shapes and strides already done: the kernel handle, the geometry
+    and the GPUParamDesc array.  ``run`` rewrites the pointer and scalar slots
+    and replays the compiled host code's sequence for one kernel: launch,
+    wait, destroy event (GpuRuntimeToLlvm.cpp:444-628)."""
+
+    def __init__(self, ctx, compiled, kern, func_name, grid, block, gsize3, args,
+                 ret=None, partials=()):
+        self.ctx, self.compiled, self.kern, self.func_name = ctx, compiled, kern, func_name
+        self.grid, self.block = tuple(grid), tuple(block)
+        self.info = {"kernel": compiled.name, "grid": self.grid, "block": self.block}
+        self.empty = 0 in gsize3
+        params = _ParamList()
+        self._arg_slots = []
+        for a in args:
+            if isinstance(a, HipNdArray):
+                self._arg_slots.append(params.add_array(a))
+            elif isinstance(a, slice):
+                self._arg_slots.append(params.add_slice(a))
+            else:
+                self._arg_slots.append(params.add_scalar(a))
+        self._ret_slot = params.add_array(ret) if ret is not None else None
+        # one pointer per reduction variable
+        self._partial_slots = [params._add(ctypes.c_void_p(part.ptr), lowered.PARAM_PTR)
+                               for part in partials]
+        for nbytes in compiled.local_bytes:
+            params.add_local(int(nbytes))
+        for g in gsize3:
+            params.add_scalar(int(g))
+        self._flag = None
+        if compiled.boundscheck:
+            self._flag = _bounds_flag(ctx)
+            params._add(ctypes.c_void_p(self._flag.ptr), lowered.PARAM_PTR)
+        self._params = params             # owns the slots the descriptors point at
+        self._descs = params.build()
+        self._lock = threading.Lock()     # slots are rewritten per call
+        self._launch = (ctx.queue, kern, *self.grid, *self.block, NO_DEPS, self._descs)
+
+    def run(self, args=None, ret=None, partials=()):
+        """Launches; ``args`` (same types, shapes and strides as the plan was
+        built for) refresh the pointer and scalar slots first."""
+        if self.empty:
+            return
+        queue = self.ctx.queue
+        with self._lock:                  # the launch call copies the values out
+            if args is not None:
+                for slot, a in zip(self._arg_slots, args):
+                    if isinstance(a, HipNdArray):
+                        slot.value = a.ptr
+                    elif isinstance(a, slice):
+                        for part_slot, part in zip(slot, (a.start, a.stop, a.step)):
+                            part_slot.value = (_ParamList.SLICE_NONE if part is None
+                                               else int(part))
+                    else:
+                        slot.value = a.item() if isinstance(a, np.generic) else a
+                if ret is not None:
+                    self._ret_slot.value = ret.ptr
+                for slot, part in zip(self._partial_slots, partials):
+                    slot.value = part.ptr
+            event = runtime_lib.gpuxLaunchKernel(*self._launch)
+        runtime_lib.gpuxWait(queue, event)
+        runtime_lib.gpuxDestroyEvent(queue, event)
+        flag = self._flag
+        if flag is not None and flag.asnumpy()[0] != 0:
+            flag.copy_from_host(np.zeros(1, np.int32))
+            raise IndexError(
+                f"kernel '{self.func_name}' indexed an array out of bounds (the access "
+                "was redirected to element 0)")
+
+
+def plan_key(args):
+    """What a launch plan depends on besides the kernel: per argument its
+    type, and for arrays dtype, shape and strides (not the address)."""
+    return tuple((a.dtype, a.shape, a.strides) if isinstance(a, HipNdArray)
+                 else (a.dtype if isinstance(a, np.generic) else type(a))
+                 for a in args)
+
+
 def _launch_loaded(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret=None,
                    partials=()):
-    """The compiled host code's sequence for one kernel: parameters, launch,
-    wait, destroy event (GpuRuntimeToLlvm.cpp:444-628)."""
-    params = _ParamList()
-    for a in args:
-        if isinstance(a, HipNdArray):
-            params.add_array(a)
-        elif isinstance(a, slice):
-            params.add_slice(a)
-        else:
-            params.add_scalar(a)
-    if ret is not None:
-        params.add_array(ret)
-    for part in partials:                 # one pointer per reduction variable
-        params._add(ctypes.c_void_p(part.ptr), lowered.PARAM_PTR)
-    for nbytes in compiled.local_bytes:
-        params.add_local(int(nbytes))
-    for g in gsize3:
-        params.add_scalar(int(g))
-    flag = None
-    if compiled.boundscheck:
-        flag = _bounds_flag(ctx)
-        params._add(ctypes.c_void_p(flag.ptr), lowered.PARAM_PTR)
-    descs = params.build()
-    if 0 in gsize3:
-        return
-    queue = ctx.queue
-    event = runtime_lib.gpuxLaunchKernel(queue, kern, *grid, *block, NO_DEPS, descs)
-    runtime_lib.gpuxWait(queue, event)
-    runtime_lib.gpuxDestroyEvent(queue, event)
-    if flag is not None and flag.asnumpy()[0] != 0:
-        flag.copy_from_host(np.zeros(1, np.int32))
-        raise IndexError(
-            f"kernel '{func_name}' indexed an array out of bounds (the access was "
-            "redirected to element 0)")
+    LaunchPlan(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret,
+               partials).run()
 
 
-def launch_compiled(ctx, compiled, func_name, global_size, args, ret=None,
-                    make_partials=None):
-    """Loads (once) and launches a translated function over ``global_size``
-    with a runtime-chosen block; returns the launch geometry.
-    ``make_partials(blocks)`` supplies the per-block result arrays of a
-    function with reductions once the grid is known."""
+def plan_compiled(ctx, compiled, func_name, global_size, args, ret=None,
+                  make_partials=None):
+    """Loads a translated function (once) and prepares its launch over
+    ``global_size`` with a runtime-chosen block.  ``make_partials(blocks)``
+    supplies the per-block result arrays of a function with reductions once
+    the grid is known."""
     kern = _loaded_kernel(ctx, compiled)
     per_lane = getattr(compiled, "elements_per_thread", 1)
     lanes = [-(-int(global_size[0]) // per_lane)] + [int(g) for g in global_size[1:]]
     block, grid = _geometry(ctx, compiled, kern, lanes, ())
     gsize3 = [int(g) for g in global_size] + [1] * (3 - len(global_size))
     partials = make_partials(grid[0] * grid[1] * grid[2]) if make_partials else ()
-    _launch_loaded(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret,
-                   partials)
-    return {"kernel": compiled.name, "grid": tuple(grid), "block": tuple(block)}
+    return LaunchPlan(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret,
+                      partials)
+
+
+def launch_compiled(ctx, compiled, func_name, global_size, args, ret=None,
+                    make_partials=None):
+    """plan_compiled + one launch; returns the launch geometry."""
+    plan = plan_compiled(ctx, compiled, func_name, global_size, args, ret, make_partials)
+    plan.run()
+    return plan.info
 
 
 def kernel(func=None, **kwargs):

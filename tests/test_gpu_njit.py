@@ -308,3 +308,54 @@ def test_unsupported_functions_are_reported(env):
         njit(parallel=True)(cases.statements_after_loop)(x, hip.asarray(np.zeros(8)))
     with pytest.raises(ValueError, match="at least one device array"):
         njit(cases.add)(1.0, 2.0)
+
+
+def test_repeated_calls_replay_stored_launches(env):
+    """A call whose argument types, shapes and strides were seen before reuses
+    the prepared launch: new addresses, new scalar values and a change of
+    aliasing must all still be honoured."""
+    hip, ops, orc, workloads = env
+    rng = np.random.default_rng(11)
+    f = njit(cases.fused_map)
+    for scale in (0.5, -3.0, 7.25):
+        a, b, c = (rng.standard_normal(1000) for _ in range(3))
+        got = f(hip.asarray(a), hip.asarray(b), hip.asarray(c), scale)
+        np.testing.assert_allclose(got.asnumpy(), cases.fused_map(a, b, c, scale), rtol=1e-12)
+    assert len(f._plans) == 1
+    # a different length is a different launch
+    a, b, c = (rng.standard_normal(77) for _ in range(3))
+    got = f(hip.asarray(a), hip.asarray(b), hip.asarray(c), 2.0)
+    np.testing.assert_allclose(got.asnumpy(), cases.fused_map(a, b, c, 2.0), rtol=1e-12)
+    assert len(f._plans) == 2
+
+    g = njit(parallel=True)(cases.saxpy_loop)
+    for alpha in (2.0, -1.5, 0.0):
+        x, y = rng.standard_normal(5000), rng.standard_normal(5000)
+        out = hip.asarray(np.zeros(5000))
+        g(alpha, hip.asarray(x), hip.asarray(y), out)
+        np.testing.assert_array_equal(out.asnumpy(), alpha * x + y)
+    # the output aliasing an input: same shapes, another kernel variant
+    x, y = rng.standard_normal(5000), rng.standard_normal(5000)
+    dx = hip.asarray(x)
+    g(3.0, dx, hip.asarray(y), dx)
+    np.testing.assert_array_equal(dx.asnumpy(), 3.0 * x + y)
+    x2 = rng.standard_normal(5000)
+    out = hip.asarray(np.zeros(5000))
+    g(3.0, hip.asarray(x2), hip.asarray(y), out)
+    np.testing.assert_array_equal(out.asnumpy(), 3.0 * x2 + y)
+
+    h = njit(parallel=True)(cases.sum_of_squares)
+    for n in (4096, 4096, 100, 4096):
+        v = rng.standard_normal(n).astype(np.float32)
+        np.testing.assert_allclose(h(hip.asarray(v)), np.sqrt(np.sum(v.astype(np.float64) ** 2)),
+                                   rtol=1e-6)
+
+    k = njit(cases.add_into)
+    for _ in range(3):
+        a, b = rng.standard_normal(300), rng.standard_normal(300)
+        dc = hip.asarray(np.zeros(300))
+        k(hip.asarray(a), hip.asarray(b), dc)
+        np.testing.assert_array_equal(dc.asnumpy(), a + b)
+    da_ = hip.asarray(a)
+    k(da_, hip.asarray(b), da_)             # in place
+    np.testing.assert_array_equal(da_.asnumpy(), a + b)
