@@ -244,4 +244,17 @@ __device__ __forceinline__ void blockReduceStore(T v, Op op, T *partial) {
     partial[blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)] = slots[0];
 }
 
+// A store of a value that no work-item of the launch reads back.  `unit`:
+// adjacent lanes write adjacent elements, so a wave completes whole lines in
+// one instruction and they can stream past the caches; any other pattern is
+// left to L2 to combine.  `unit` is uniform over the launch.
+template <typename T>
+__device__ __forceinline__ void streamStore(T *p, T v, bool unit) {
+  if (unit)
+    __builtin_nontemporal_store(v, p);
+  else
+    *p = v;
+}
+__device__ __forceinline__ void streamStore(bool *p, bool v, bool) { *p = v; }
+
 } // namespace nmkjit

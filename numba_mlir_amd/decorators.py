@@ -69,25 +69,6 @@ ELEMENTS_PER_THREAD = 4     # of a fused 1-d map or prange loop
 MAX_PLANS = kernel_impl.MAX_PLANS   # stored launches per compiled function
 
 
-def _disjoint(arrays):
-    """True when no two of the device arrays share a byte (then the kernel may
-    reorder their loads and stores freely)."""
-    spans = []
-    for a in arrays:
-        lo = hi = a.ptr
-        for n, st in zip(a.shape, a.strides):
-            if n == 0:
-                lo = hi = a.ptr
-                break
-            if st >= 0:
-                hi += (n - 1) * st
-            else:
-                lo += (n - 1) * st
-        spans.append((lo, hi + a.dtype.itemsize))
-    spans.sort()
-    return all(spans[k][1] <= spans[k + 1][0] for k in range(len(spans) - 1))
-
-
 _BINARY = {ast.Add: ops.add, ast.Sub: ops.subtract, ast.Mult: ops.multiply}
 _REDUCE = {"sum": ops.sum, "prod": ops.prod, "min": ops.amin, "max": ops.amax,
            "amin": ops.amin, "amax": ops.amax}
@@ -268,7 +249,7 @@ class Dispatcher:
 
     def _compile(self, mode, args, ndim, remap):
         captured = kernel_impl.captured_constants(self.py_func)
-        noalias = _disjoint([a for a in args if isinstance(a, HipNdArray)])
+        noalias = hip.disjoint([a for a in args if isinstance(a, HipNdArray)])
         for specialize in (True, False):
             types = [kernel_compiler.type_of_argument(a, specialize) for a in args]
             key = (mode, ndim, tuple(kernel_compiler.type_key(t) for t in types),
@@ -333,7 +314,7 @@ class Dispatcher:
         arrays = [a for a in args if isinstance(a, HipNdArray)]
         # what the choice of kernel depends on: types, shapes, strides, aliasing
         key = (ctx, kernel_impl.plan_key(args),
-               kernel_impl.captured_constants(self.py_func), _disjoint(arrays))
+               kernel_impl.captured_constants(self.py_func), hip.disjoint(arrays))
         entry = self._loop_plans.get(key)
         if entry is None:
             if len(self._loop_plans) >= MAX_PLANS:
@@ -416,7 +397,7 @@ class Dispatcher:
             plan = entry["plan"]
             if plan is None:              # an argument is written: aliasing decides
                 plan = entry["by_alias"].get(
-                    _disjoint([a for a in args if isinstance(a, HipNdArray)]))
+                    hip.disjoint([a for a in args if isinstance(a, HipNdArray)]))
             if plan is not None:
                 ret = None
                 if entry["ret_dtype"] is not None:
@@ -462,7 +443,7 @@ class Dispatcher:
             "plan": None, "by_alias": {}, "shape": tuple(shape),
             "ret_dtype": compiled.ret_dtype})
         if writes:
-            entry["by_alias"][_disjoint(arrays)] = plan
+            entry["by_alias"][hip.disjoint(arrays)] = plan
         else:
             entry["plan"] = plan
         return ret

@@ -322,3 +322,22 @@ def asnumpy(arr):
 
 def empty(shape, dtype, usm_type="device", device=None):
     return HipNdArray.empty(shape, dtype, usm_type, device)
+
+
+def disjoint(arrays):
+    """True when no two of the device arrays share a byte (then the kernel may
+    reorder their loads and stores freely)."""
+    spans = []
+    for a in arrays:
+        lo = hi = a.ptr
+        for n, st in zip(a.shape, a.strides):
+            if n == 0:
+                lo = hi = a.ptr
+                break
+            if st >= 0:
+                hi += (n - 1) * st
+            else:
+                lo += (n - 1) * st
+        spans.append((lo, hi + a.dtype.itemsize))
+    spans.sort()
+    return all(spans[k][1] <= spans[k + 1][0] for k in range(len(spans) - 1))

@@ -172,6 +172,7 @@ class Val:
         self.items = items            # tuple expression: list of Val
         self.pyobj = pyobj            # a Python object known at compile time
         self.slice_parts = slice_parts  # (start, stop, step) Vals or None each
+        self.gid = None               # k: the value is global id k plus a constant
 
 
 class _Deferred(Exception):
@@ -392,6 +393,9 @@ class FunctionTranslator:
         self.written_arrays = set()  # elementwise mode: arrays stored through [:]
         self.read_arrays = set()     # elementwise mode: arrays loaded as values
         self.noalias = False         # no two array arguments overlap (host-checked)
+        self._store_only = None      # array parameters the body never reads
+        self.last_elem_gid = None    # of the element subscript() resolved last
+        self.last_elem_unit = "false"
         self.elements_per_thread = 1
         self._lambda_body = None
         self.reduction_types = []    # (name, Scalar) in parameter order
@@ -414,6 +418,9 @@ class FunctionTranslator:
         # a name bound once, at the top level, to a constant is that constant
         # (array shapes and range bounds written through a local name)
         self.const_vars = {}
+        # ... and one bound once, at the top level, to a global id (plus a
+        # constant) is known to run along that grid dimension
+        self.gid_vars = {}
         self.top_level = {id(s) for s in body}
         return names - set(self.params)
 
@@ -435,7 +442,9 @@ class FunctionTranslator:
             if isinstance(t, Scalar):
                 if name in self.const_vars:
                     return constant(_convert_const(self.const_vars[name], t), t)
-                return Val(self.cname(name), t, nonneg=name in self.nonneg_vars)
+                v = Val(self.cname(name), t, nonneg=name in self.nonneg_vars)
+                v.gid = self.gid_vars.get(name)
+                return v
             if isinstance(t, Array):
                 return Val(self.cname(name), t)
             if isinstance(t, SliceArg):
@@ -497,7 +506,9 @@ class FunctionTranslator:
         terms = [f"nmk_gid{d} * {arr_code}.stride[{d}]" for d in range(self.ndim)]
         dst = f"{arr_code}.p[{' + '.join(terms)}]"
         if self.noalias and arr_code not in self.read_arrays:
-            self.emit(f"__builtin_nontemporal_store(({elem.ctype})({value_code}), &{dst});")
+            last = self.ndim - 1
+            self.emit(f"NMK_STORE_ALONG{last}(&{dst}, ({elem.ctype})({value_code}), "
+                      f"{arr_code}.stride[{last}] == 1);")
         else:
             self.emit(f"{dst} = {value_code};")
 
@@ -656,9 +667,17 @@ class FunctionTranslator:
                     return constant(r, t)
             nonneg = a.nonneg and b.nonneg and sym != "-"
             code = f"({x.code} {sym} {y.code})"
+            gid = None
+            if t is INT64:                # id + constant still runs along the id
+                if sym in "+-" and a.gid is not None and y.const is not None:
+                    gid = a.gid
+                elif sym == "+" and b.gid is not None and x.const is not None:
+                    gid = b.gid
             if t.dtype.itemsize < 4:      # C promotes narrow integers to int
                 code = f"(({t.ctype}){code})"
-            return Val(code, t, nonneg=nonneg)
+            v = Val(code, t, nonneg=nonneg)
+            v.gid = gid
+            return v
         if isinstance(op, ast.FloorDiv):
             if t.is_float:
                 return Val(f"nmkjit::floordivFloat<{t.ctype}>({x.code}, {y.code})", t)
@@ -715,6 +734,9 @@ class FunctionTranslator:
             for d, i in enumerate(items):
                 i = self.normalise_index(i, base, d)
                 terms.append(f"{i.code} * {base.code}.stride[{d}]")
+            # the grid dimension the innermost index runs along, if any
+            self.last_elem_gid = i.gid
+            self.last_elem_unit = f"{base.code}.stride[{ndim - 1}] == 1"
             return ("elem", f"{base.code}.p[{' + '.join(terms)}]", base.type.elem)
         # a view: integers drop a dimension, slices keep it
         cur, cur_t, dim = base.code, base.type, 0
@@ -762,7 +784,10 @@ class FunctionTranslator:
                 self.err(node, "The axis must be a constant 0, 1 or 2")
             if ids[obj][0] in ("lid", "grp", "lsz"):
                 self.m.communicates = True
-            return Val(f"nmk_{ids[obj][0]}{axis.const}", INT64, nonneg=True)
+            v = Val(f"nmk_{ids[obj][0]}{axis.const}", INT64, nonneg=True)
+            if ids[obj][0] == "gid":
+                v.gid = axis.const
+            return v
         if obj is stubs.atomic.add or obj is stubs.atomic.sub:
             return self.call_atomic(node, obj is stubs.atomic.sub)
         if obj is stubs.barrier or obj is stubs.mem_fence:
@@ -1126,6 +1151,9 @@ class FunctionTranslator:
             if (v.const is not None and self.store_count.get(name) == 1 and
                     id(node) in self.top_level and name not in self.params):
                 self.const_vars[name] = v.const
+            if (v.gid is not None and self.store_count.get(name) == 1 and
+                    id(node) in self.top_level and name not in self.params):
+                self.gid_vars[name] = v.gid
             if not v.nonneg:
                 self.maybe_negative.add(name)
             if self.emitting:
@@ -1152,7 +1180,50 @@ class FunctionTranslator:
         code, elem = rest
         if not isinstance(v.type, Scalar):
             self.err(node, "Only scalars can be stored into an array element")
+        if self.noalias and self.last_elem_gid is not None and \
+                isinstance(target.value, ast.Name) and \
+                target.value.id in self.store_only_params():
+            # read by nobody in this launch: past the caches when adjacent
+            # lanes write adjacent elements (see translate_kernel)
+            self.emit(f"NMK_STORE_ALONG{self.last_elem_gid}(&{code}, "
+                      f"({elem.ctype})({cast(v, elem).code}), {self.last_elem_unit});")
+            return
         self.emit(f"{code} = {cast(v, elem).code};")
+
+    def store_only_params(self):
+        """Array parameters of a kernel (or loop function) that the body only
+        stores elements into: every use is ``p[...] = value``, ``p.shape`` /
+        ``p.size`` / ``p.ndim`` / ``p.dtype`` or ``len(p)``.  Handing the array
+        to anything else (a view, another name, a call, an atomic, ``+=``)
+        counts as reading it."""
+        if self._store_only is not None:
+            return self._store_only
+        names = {p for p, t in zip(self.params, self.arg_types)
+                 if isinstance(t, Array) and t.space == "global"}
+        if not self.is_kernel:
+            names = set()
+        parents = {}
+        for parent in ast.walk(self.node):
+            for child in ast.iter_child_nodes(parent):
+                parents[id(child)] = parent
+        for n in ast.walk(self.node):
+            if not (isinstance(n, ast.Name) and n.id in names):
+                continue
+            parent = parents.get(id(n))
+            if isinstance(n.ctx, ast.Load):
+                if isinstance(parent, ast.Subscript) and parent.value is n and \
+                        isinstance(parent.ctx, ast.Store) and \
+                        isinstance(parents.get(id(parent)), ast.Assign):
+                    continue
+                if isinstance(parent, ast.Attribute) and \
+                        parent.attr in ("shape", "size", "ndim", "dtype"):
+                    continue
+                if isinstance(parent, ast.Call) and isinstance(parent.func, ast.Name) and \
+                        parent.func.id == "len" and len(parent.args) == 1:
+                    continue
+            names.discard(n.id)
+        self._store_only = names
+        return names
 
     def stmt_AugAssign(self, node):
         if isinstance(node.target, ast.Name):
@@ -1220,6 +1291,8 @@ class FunctionTranslator:
             self.bind(name, INT64, node)
             if not start.nonneg:
                 self.maybe_negative.add(name)
+            if step.const == 1 and self.store_count.get(name) == 1:
+                self.gid_vars[name] = depth
             if self.emitting:
                 self.emit(f"{self.cname(name)} = {start.code} + nmk_gid{depth} * {step.code};")
             self.indent -= 1
@@ -1396,7 +1469,10 @@ class FunctionTranslator:
         self.infer(body)
         lines = self.run_emit(body)
         params, views = [], []
-        restrict = "__restrict__ " if self.noalias else ""
+        # (a kernel whose work-items exchange data through memory keeps plain
+        # pointers)
+        restrict = "__restrict__ " if self.noalias and not (
+            self.mode == "kernel" and self.m.communicates) else ""
         for p, t in zip(self.params, self.arg_types):
             c = self.cname(p)
             if isinstance(t, Array):
@@ -1459,6 +1535,12 @@ class FunctionTranslator:
         hw = "xyz"
         dim = [hw[self.ndim - 1 - k] if (self.reversed and k < self.ndim) else hw[k]
                for k in range(3)]
+        # Stores nobody reads back go past the caches only along the grid
+        # dimension that lies on x (adjacent lanes), and only into unit-stride
+        # rows: scattered stores are left for L2 to combine.
+        out = [f"#define NMK_STORE_ALONG{k}(p, v, unit) " +
+               ("nmkjit::streamStore(p, v, unit)" if dim[k] == "x" else "(*(p) = (v))")
+               for k in range(3)] + out
         # A 1-d map whose work-items cannot observe their grouping may give
         # several elements to a lane, a block apart (coalesced); unrolled, with
         # non-overlapping arrays, their loads are in flight together.
@@ -1550,16 +1632,17 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     the result is the dtype of the returned array, if any); "parallel" for a
     function whose top-level prange loop becomes a 1-d grid (``range_source``
     holds the source text of the prange arguments for the host to evaluate).
-    For these two modes ``noalias`` promises that no two array arguments
-    overlap, and ``elements_per_thread`` asks for that many elements per lane
-    of a 1-d grid (the result says what it got: the launcher divides the grid
+    ``noalias`` promises that no two array arguments overlap (pointers become
+    ``__restrict__``; arrays the body only stores into are written past the
+    caches).  For the last two modes ``elements_per_thread`` asks for that
+    many elements per lane of a 1-d grid (the result says what it got: the launcher divides the grid
     by it)."""
     module = Module(stubs, boundscheck)
     tr = FunctionTranslator(module, func, arg_types, True, ndim)
     tr.allow_remap = remap
     tr.mode = mode
+    tr.noalias = noalias
     if mode != "kernel":
-        tr.noalias = noalias
         tr.elements_per_thread = max(1, int(elements_per_thread))
     if mode == "parallel":
         _check_parallel_shape(tr)

@@ -29,7 +29,7 @@ import numpy as np
 from . import kernel_compiler, lowered
 from .gpu_runtime import runtime_lib
 from .utils import readenv
-from .device_array import HipNdArray
+from .device_array import HipNdArray, disjoint
 from .kernel_base import KernelBase
 from .lowered import GPUParamDesc, lib
 
@@ -298,9 +298,10 @@ class Kernel(KernelBase):
         tag = _DTYPE_TAGS.get(first.dtype) if first is not None else None
         return self.twin.format(dtype=tag, rank=len(self.global_size))
 
-    def compile(self, args, ndim, remap=False):
+    def compile(self, args, ndim, remap=False, noalias=False):
         """The specialisation of the body for these arguments (translated on
-        first use; constants captured by the body are part of the key)."""
+        first use; constants captured by the body are part of the key).
+        ``noalias``: the caller found no two array arguments overlapping."""
         import sys
         # Specialised on dense layouts and short trailing extents; a kernel
         # that keeps meeting new ones gets the general form for the rest.
@@ -308,14 +309,15 @@ class Kernel(KernelBase):
         for specialize in (True, False):
             types = [kernel_compiler.type_of_argument(a, specialize) for a in args]
             key = (ndim, tuple(kernel_compiler.type_key(t) for t in types),
-                   captured, self.boundscheck, remap)
+                   captured, self.boundscheck, remap, noalias)
             compiled = self._compiled.get(key)
             if compiled is not None or len(self._compiled) < MAX_SPECIALISATIONS:
                 break
         if compiled is None:
             compiled = kernel_compiler.translate(self.py_func, types, ndim,
                                                  sys.modules[__name__],
-                                                 self.boundscheck, remap)
+                                                 self.boundscheck, remap,
+                                                 noalias=noalias)
             self._compiled[key] = compiled
         return compiled
 
@@ -341,8 +343,9 @@ class Kernel(KernelBase):
             grid = [(g + b - 1) // b for g, b in zip(gsize3, block)]
         else:
             # Types, shapes and strides seen before replay a stored launch.
+            noalias = disjoint([a for a in args if isinstance(a, HipNdArray)])
             key = (ctx, plan_key(args), captured_constants(self.py_func),
-                   tuple(gsize3[:ndim]), tuple(self.local_size))
+                   tuple(gsize3[:ndim]), tuple(self.local_size), noalias)
             plan = self._plans.get(key)
             if plan is not None:
                 plan.run(args)
@@ -352,11 +355,11 @@ class Kernel(KernelBase):
             # grouping is laid out for coalescing (last dimension on x), unless
             # that pushes a long dimension past the y / z grid limit.
             remap = len(self.local_size) == 0 and ndim > 1
-            compiled = self.compile(args, ndim, remap)
+            compiled = self.compile(args, ndim, remap, noalias)
             kern = _loaded_kernel(ctx, compiled)
             block, grid = _geometry(ctx, compiled, kern, gsize3[:ndim], self.local_size)
             if compiled.reversed_dims and max(grid[1:]) > 65535:
-                compiled = self.compile(args, ndim, False)
+                compiled = self.compile(args, ndim, False, noalias)
                 kern = _loaded_kernel(ctx, compiled)
                 block, grid = _geometry(ctx, compiled, kern, gsize3[:ndim],
                                         self.local_size)

@@ -311,7 +311,8 @@ def test_fused_maps_take_several_elements_per_lane(K, tmp_path, monkeypatch):
     assert "for (int nmk_rep = 0; nmk_rep < 4; ++nmk_rep)" in ck.source
     assert "float *__restrict__ v_price_p" in ck.source
     # call and put are only written: streamed
-    assert ck.source.count("__builtin_nontemporal_store(") == 2
+    assert ck.source.count("NMK_STORE_ALONG0(&") == 2
+    assert "#define NMK_STORE_ALONG0(p, v, unit) nmkjit::streamStore(p, v, unit)" in ck.source
     assert kc.build_code_object(ck)[:4] == b"\x7fELF"
     # overlapping arguments: plain pointers and stores
     ck = kc.translate(njit_cases.black_scholes_arrays, types, ndim, K, mode=mode,
@@ -341,3 +342,70 @@ def test_prange_reductions(K, tmp_path, monkeypatch):
     assert "double v_p = (double)1;" in ck.source
     with pytest.raises(kc.KernelCompileError, match="cannot be read inside the loop"):
         kc.translate(njit_cases.reduction_read_in_loop, [f32], 1, K, mode="parallel")
+
+
+def test_kernels_stream_stores_nobody_reads_back(K):
+    """With arguments the host found disjoint, an array the body only stores
+    into is written past the caches -- where the innermost index runs along
+    the grid dimension that lies on x."""
+    get_global_id = K.get_global_id
+    f64_2d = kc.Array(kc.FLOAT64, 2, layout="C")
+
+    def pairwise(X1, X2, D):
+        i = get_global_id(0)
+        j = get_global_id(1)
+        d = 0.0
+        for k in range(X1.shape[1]):
+            tmp = X1[i, k] - X2[j, k]
+            d += tmp * tmp
+        D[i, j] = np.sqrt(d)
+
+    def stream(src):
+        return [k for k in range(3)
+                if f"#define NMK_STORE_ALONG{k}(p, v, unit) nmkjit::streamStore" in src]
+
+    src = source_of(K, pairwise, [f64_2d] * 3, ndim=2, remap=True, noalias=True)
+    assert "NMK_STORE_ALONG1(&v_D.p[" in src and stream(src) == [1]
+    assert "double *__restrict__ v_D_p" in src
+    # as written (dimension 0 on x) lanes write a column apart: plain stores
+    src = source_of(K, pairwise, [f64_2d] * 3, ndim=2, remap=False, noalias=True)
+    assert "NMK_STORE_ALONG1(&v_D.p[" in src and stream(src) == [0]
+    # arguments that may overlap: nothing changes
+    src = source_of(K, pairwise, [f64_2d] * 3, ndim=2, remap=True)
+    assert "NMK_STORE_ALONG1(&" not in src and "__restrict__" not in src
+
+    def reads_back(a, out):
+        i = get_global_id(0)
+        out[i] = a[i]
+        out[i] += 1.0
+
+    def shifted(a, out):
+        i = get_global_id(0)
+        out[i + 1] = a[i]
+
+    def scattered(a, idx, out):
+        i = get_global_id(0)
+        out[idx[i]] = a[i]
+
+    def handed_on(a, out):
+        i = get_global_id(0)
+        view = out[1:]
+        view[i] = a[i]
+        out[i] = 0.0
+
+    assert "NMK_STORE_ALONG0(&" not in source_of(K, reads_back, [F64_1D] * 2, noalias=True)
+    assert "NMK_STORE_ALONG0(&" in source_of(K, shifted, [F64_1D] * 2, noalias=True)
+    assert "NMK_STORE_ALONG0(&" not in source_of(K, scattered, [F64_1D, I64_1D, F64_1D],
+                                                  noalias=True)
+    assert "NMK_STORE_ALONG0(&" not in source_of(K, handed_on, [F64_1D] * 2, noalias=True)
+
+    # work-items that exchange data through memory keep plain pointers
+    barrier = K.barrier
+
+    def exchanging(a, out):
+        i = get_global_id(0)
+        out[i] = a[i]
+        barrier()
+        a[i] = 1.0
+
+    assert "__restrict__" not in source_of(K, exchanging, [F64_1D] * 2, noalias=True)
