@@ -190,8 +190,21 @@ _UNARY_MATH = {
     "arcsinh": "asinh", "arccosh": "acosh", "arctanh": "atanh", "exp2": "exp2",
     "cbrt": "cbrt", "absolute": "fabs",
 }
-_BINARY_MATH = {"atan2": "atan2", "arctan2": "atan2", "pow": "pow", "power": "pow",
+_BINARY_MATH = {"atan2": "atan2", "arctan2": "atan2", "pow": "pow",
                 "hypot": "hypot", "copysign": "copysign", "fmod": "fmod"}
+# NumPy's named forms of the operators (reference: numpy/funcs.py:362-383 and
+# 457-562 register the same bodies under both names)
+_UFUNC_BINOPS = {
+    "add": ast.Add, "subtract": ast.Sub, "multiply": ast.Mult, "divide": ast.Div,
+    "true_divide": ast.Div, "power": ast.Pow, "floor_divide": ast.FloorDiv,
+    "remainder": ast.Mod, "mod": ast.Mod, "bitwise_and": ast.BitAnd,
+    "bitwise_or": ast.BitOr, "bitwise_xor": ast.BitXor, "left_shift": ast.LShift,
+    "right_shift": ast.RShift}
+_UFUNC_COMPARE = {
+    "less": ast.Lt, "less_equal": ast.LtE, "greater": ast.Gt, "greater_equal": ast.GtE,
+    "equal": ast.Eq, "not_equal": ast.NotEq}
+_UFUNC_UNARY = {"positive": ast.UAdd, "invert": ast.Invert, "bitwise_not": ast.Invert,
+                "logical_not": ast.Not}
 _ROUNDING = {"floor": "floor", "ceil": "ceil", "trunc": "trunc"}
 
 _CAST_TYPES = {
@@ -862,6 +875,32 @@ class FunctionTranslator:
                 return cast(v, INT64) if mod == "math" else cast(v, FLOAT64)
             r = Val(f"{_ROUNDING[name]}({v.code})", v.type)
             return cast(r, INT64) if mod == "math" else r
+        if is_np and name in _UFUNC_BINOPS and len(node.args) == 2:
+            return self.binop(_UFUNC_BINOPS[name](), self.scalar(node.args[0]),
+                              self.scalar(node.args[1]), node)
+        if is_np and name in _UFUNC_COMPARE and len(node.args) == 2:
+            return self.expr(ast.copy_location(ast.Compare(
+                left=node.args[0], ops=[_UFUNC_COMPARE[name]()],
+                comparators=[node.args[1]]), node))
+        if is_np and name in _UFUNC_UNARY and len(node.args) == 1:
+            return self.expr(ast.copy_location(ast.UnaryOp(
+                op=_UFUNC_UNARY[name](), operand=node.args[0]), node))
+        if is_np and name in ("logical_and", "logical_or", "logical_xor") and \
+                len(node.args) == 2:
+            a = self.truth(self.scalar(node.args[0]))
+            b = self.truth(self.scalar(node.args[1]))
+            sym = {"logical_and": "&&", "logical_or": "||", "logical_xor": "!="}[name]
+            return Val(f"({a.code} {sym} {b.code})", BOOL)
+        if is_np and name == "clip" and len(node.args) == 3:
+            # min(a_max, max(a, a_min)) in the operands' common type
+            # (reference: numpy/funcs.py:571-578)
+            a, lo, hi = (self.scalar(x) for x in node.args)
+            t = self.arith_type(promote(a.type, lo.type), hi.type)
+            a, lo, hi = cast(a, t), cast(lo, t), cast(hi, t)
+            # (a NaN element stays NaN, as in NumPy)
+            inner = f"({a.code} < {lo.code} ? {lo.code} : {a.code})"
+            return Val(f"({inner} > {hi.code} ? {hi.code} : {inner})", t,
+                       nonneg=hi.nonneg and (a.nonneg or lo.nonneg))
         if (mod == "math" or is_np) and name in _BINARY_MATH and len(node.args) == 2:
             a, b = self.scalar(node.args[0]), self.scalar(node.args[1])
             t = promote(a.type, b.type)

@@ -197,3 +197,60 @@ def _smoothstep(x, lo, hi):
     t = min(max((x - lo) / (hi - lo), 0.0), 1.0)
     return t * t * (3.0 - 2.0 * t)
 
+
+
+# NumPy's named forms of the operators (the reference registers each body under
+# both names, numpy/funcs.py:362-383 and 457-562), one per line so that each
+# lambda's source is found.  (name, function, operand kinds)
+NAMED_UFUNCS = [
+    ("add", lambda a, b: np.add(a, b), "fi"),
+    ("subtract", lambda a, b: np.subtract(a, b), "fi"),
+    ("multiply", lambda a, b: np.multiply(a, b), "fi"),
+    ("true_divide", lambda a, b: np.true_divide(a, b), "fi"),
+    ("power", lambda a, b: np.power(a, b), "p"),
+    ("arctan2", lambda a, b: np.arctan2(a, b), "f"),
+    ("minimum", lambda a, b: np.minimum(a, b), "fi"),
+    ("maximum", lambda a, b: np.maximum(a, b), "fi"),
+    ("logical_and", lambda a, b: np.logical_and(a, b), "fib"),
+    ("logical_or", lambda a, b: np.logical_or(a, b), "fib"),
+    ("logical_xor", lambda a, b: np.logical_xor(a, b), "fib"),
+    ("less", lambda a, b: np.less(a, b), "fi"),
+    ("greater", lambda a, b: np.greater(a, b), "fi"),
+    ("less_equal", lambda a, b: np.less_equal(a, b), "fi"),
+    ("greater_equal", lambda a, b: np.greater_equal(a, b), "fi"),
+    ("equal", lambda a, b: np.equal(a, b), "fib"),
+    ("not_equal", lambda a, b: np.not_equal(a, b), "fib"),
+    ("bitwise_and", lambda a, b: np.bitwise_and(a, b), "ib"),
+    ("bitwise_or", lambda a, b: np.bitwise_or(a, b), "ib"),
+    ("bitwise_xor", lambda a, b: np.bitwise_xor(a, b), "ib"),
+    ("left_shift", lambda a, b: np.left_shift(a, b), "s"),
+    ("right_shift", lambda a, b: np.right_shift(a, b), "s"),
+    ("floor_divide", lambda a, b: np.floor_divide(a, b), "fi"),
+    ("remainder", lambda a, b: np.remainder(a, b), "fi"),
+]
+
+NAMED_UNARY = [
+    ("sqrt", lambda a: np.sqrt(a), "p"),
+    ("square", lambda a: np.square(a), "fi"),
+    ("log", lambda a: np.log(a), "p"),
+    ("sin", lambda a: np.sin(a), "f"),
+    ("cos", lambda a: np.cos(a), "f"),
+    ("exp", lambda a: np.exp(a), "f"),
+    ("tanh", lambda a: np.tanh(a), "f"),
+    ("abs", lambda a: np.abs(a), "fi"),
+    ("negative", lambda a: np.negative(a), "fi"),
+    ("positive", lambda a: np.positive(a), "fi"),
+    ("logical_not", lambda a: np.logical_not(a), "fib"),
+    ("invert", lambda a: np.invert(a), "i"),
+    ("neg", lambda a: -a, "fi"),
+    ("pos", lambda a: +a, "fi"),
+    ("inv", lambda a: ~a, "i"),
+]
+
+
+def clip_scalars(a):
+    return np.clip(a, -0.5, 0.75)
+
+
+def clip_arrays(a, lo, hi):
+    return np.clip(a, lo, hi)

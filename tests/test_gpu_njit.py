@@ -359,3 +359,78 @@ def test_repeated_calls_replay_stored_launches(env):
     da_ = hip.asarray(a)
     k(da_, hip.asarray(b), da_)             # in place
     np.testing.assert_array_equal(da_.asnumpy(), a + b)
+
+
+def _operands(kind, rng, n=257):
+    if kind == "f":
+        return rng.uniform(-3, 3, n), rng.uniform(-3, 3, n)
+    if kind == "p":                       # positive floats
+        return rng.uniform(0.1, 9, n), rng.uniform(0.1, 9, n)
+    if kind == "i":
+        b = rng.integers(-9, 10, n)
+        return rng.integers(-50, 50, n), np.where(b == 0, 3, b)
+    if kind == "s":                       # shift counts
+        return rng.integers(-1000, 1000, n), rng.integers(0, 20, n)
+    return rng.integers(0, 2, n).astype(bool), rng.integers(0, 2, n).astype(bool)
+
+
+@pytest.mark.parametrize("name,func,kinds", cases.NAMED_UFUNCS,
+                         ids=[c[0] for c in cases.NAMED_UFUNCS])
+def test_named_binary_ufuncs(env, name, func, kinds):
+    """test_numpy.py:148-199 compares each registered binary function with
+    NumPy over float, integer and boolean operands."""
+    hip = env[0]
+    rng = np.random.default_rng(5)
+    f = njit(func)
+    for kind in kinds:
+        a, b = _operands(kind, rng)
+        got = f(hip.asarray(a), hip.asarray(b)).asnumpy()
+        want = func(a, b)
+        assert got.dtype == want.dtype, (name, kind)
+        if want.dtype.kind == "f":
+            np.testing.assert_allclose(got, want, rtol=1e-13, err_msg=f"{name} {kind}")
+        else:
+            np.testing.assert_array_equal(got, want, err_msg=f"{name} {kind}")
+        # an array against a scalar broadcasts
+        got = f(hip.asarray(a), b[3]).asnumpy()
+        want = func(a, b[3])
+        if want.dtype.kind == "f":
+            np.testing.assert_allclose(got, want, rtol=1e-13, err_msg=f"{name} {kind}")
+        else:
+            np.testing.assert_array_equal(got, want, err_msg=f"{name} {kind}")
+
+
+@pytest.mark.parametrize("name,func,kinds", cases.NAMED_UNARY,
+                         ids=[c[0] for c in cases.NAMED_UNARY])
+def test_named_unary_ufuncs(env, name, func, kinds):
+    """test_numpy.py:107-145 (unary functions against NumPy)."""
+    hip = env[0]
+    rng = np.random.default_rng(6)
+    f = njit(func)
+    for kind in kinds:
+        a, _ = _operands(kind, rng)
+        got = f(hip.asarray(a)).asnumpy()
+        want = func(a)
+        assert got.dtype == want.dtype, (name, kind)
+        if want.dtype.kind == "f":
+            np.testing.assert_allclose(got, want, rtol=1e-13, err_msg=f"{name} {kind}")
+        else:
+            np.testing.assert_array_equal(got, want, err_msg=f"{name} {kind}")
+
+
+def test_clip(env):
+    """numpy.clip (numpy/funcs.py:571-578; test_numpy.py's clip cases): scalar
+    and array bounds, NaN kept."""
+    hip = env[0]
+    rng = np.random.default_rng(7)
+    a = rng.uniform(-2, 2, 1000)
+    a[::97] = np.nan
+    got = njit(cases.clip_scalars)(hip.asarray(a)).asnumpy()
+    np.testing.assert_array_equal(got, np.clip(a, -0.5, 0.75))
+    lo, hi = rng.uniform(-1, 0, 1000), rng.uniform(0, 1, 1000)
+    got = njit(cases.clip_arrays)(hip.asarray(a), hip.asarray(lo), hip.asarray(hi)).asnumpy()
+    np.testing.assert_array_equal(got, np.clip(a, lo, hi))
+    ai = rng.integers(-100, 100, 500).astype(np.int32)
+    got = njit(cases.clip_arrays)(hip.asarray(ai), np.int32(-7), np.int32(11)).asnumpy()
+    np.testing.assert_array_equal(got, np.clip(ai, -7, 11))
+    assert got.dtype == np.int32
