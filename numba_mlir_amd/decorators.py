@@ -74,6 +74,21 @@ _REDUCE = {"sum": ops.sum, "prod": ops.prod, "min": ops.amin, "max": ops.amax,
            "amin": ops.amin, "amax": ops.amax}
 
 
+_DIVIDE = []
+
+
+def _mean(x, axis):
+    total = ops.sum(x, axis=axis)
+    float_t = x.dtype.type if x.dtype.kind == "f" else np.float64
+    if axis is None:
+        if isinstance(total, HipNdArray):
+            total = total.asnumpy().reshape(-1)[0]
+        return float_t(float_t(total) / float_t(x.size))
+    if not _DIVIDE:
+        _DIVIDE.append(Dispatcher(lambda s, n: s / n))
+    return _DIVIDE[0](total, float_t(x.shape[axis]))
+
+
 class Dispatcher:
     def __init__(self, py_func, parallel=False, boundscheck=None, **options):
         self.py_func = py_func
@@ -203,6 +218,22 @@ class Dispatcher:
                     if axis is None and isinstance(result, HipNdArray):
                         result = result.asnumpy().reshape(-1)[0]   # a scalar, as NumPy's
                     return self._served("library", result, x.ctx)
+            # np.mean(x[, axis]): the sum over the count, in the array's float
+            # type (float64 for integers; reference numpy/funcs.py:306-328)
+            call = np_call(expr, ("mean",))
+            if call:
+                name, pos, kws = call
+                x = array(pos[0]) if pos else None
+                axis = None
+                ok = x is not None and len(pos) <= 2 and all(k.arg == "axis" for k in kws)
+                for node in pos[1:] + [k.value for k in kws]:
+                    if isinstance(node, ast.Constant) and (node.value is None or
+                                                           isinstance(node.value, int)):
+                        axis = node.value
+                    else:
+                        ok = False
+                if ok:
+                    return self._served("library", _mean(x, axis), x.ctx)
             # np.sqrt(np.sum(x * x))
             call = np_call(expr, ("sqrt",))
             if call and len(call[1]) == 1 and not call[2]:

@@ -254,3 +254,15 @@ def clip_scalars(a):
 
 def clip_arrays(a, lo, hi):
     return np.clip(a, lo, hi)
+
+
+def mean_all(x):
+    return np.mean(x)
+
+
+def mean_rows(x):
+    return x.mean(axis=1)
+
+
+def mean_cols(x):
+    return np.mean(x, axis=0)

@@ -434,3 +434,22 @@ def test_clip(env):
     got = njit(cases.clip_arrays)(hip.asarray(ai), np.int32(-7), np.int32(11)).asnumpy()
     np.testing.assert_array_equal(got, np.clip(ai, -7, 11))
     assert got.dtype == np.int32
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32])
+def test_mean(env, dtype):
+    """numpy.mean / array.mean (numpy/funcs.py:306-328): the sum over the
+    count in the array's float type, float64 for integers."""
+    hip = env[0]
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((300, 170)) * 10).astype(dtype)
+    rtol = 2e-6 if dtype == np.float32 else 1e-12
+    dx = hip.asarray(x)
+    for func, want in ((cases.mean_all, np.mean(x)), (cases.mean_rows, x.mean(axis=1)),
+                       (cases.mean_cols, np.mean(x, axis=0))):
+        f = njit(func)
+        got = f(dx)
+        assert f.last_launch["path"] == "library"
+        got = got.asnumpy() if hasattr(got, "asnumpy") else got
+        assert np.asarray(got).dtype == np.asarray(want).dtype
+        np.testing.assert_allclose(got, want, rtol=rtol, atol=1e-6 if dtype == np.float32 else 0)
