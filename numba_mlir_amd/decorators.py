@@ -32,7 +32,7 @@ import math
 import numpy as np
 
 from .mlir import device_array as hip
-from .mlir import kernel_compiler, kernel_impl, ops
+from .mlir import kernel_compiler, kernel_impl, ops, staging
 from .mlir.device_array import HipNdArray
 from .mlir.utils import readenv
 
@@ -89,6 +89,24 @@ def _mean(x, axis):
     return _DIVIDE[0](total, float_t(x.shape[axis]))
 
 
+def _dot(a, b):
+    """numpy.dot of device arrays of rank 1 or 2 through the matrix kernels."""
+    if not (isinstance(a, HipNdArray) and isinstance(b, HipNdArray)):
+        raise TypeError("both operands must be device arrays")
+    if a.ndim == 2 and b.ndim == 2:
+        return ops.dot(a, b)
+    if a.ndim == 1 and b.ndim == 1:
+        if a.shape != b.shape:
+            raise ValueError(f"shapes {a.shape} and {b.shape} do not match")
+        total = ops.sum(ops.multiply(a, b))
+        return total.asnumpy().reshape(-1)[0] if isinstance(total, HipNdArray) else total
+    if a.ndim == 2 and b.ndim == 1:
+        return ops.dot(a, b.reshape((b.shape[0], 1))).reshape((a.shape[0],))
+    if a.ndim == 1 and b.ndim == 2:
+        return ops.dot(a.reshape((1, a.shape[0])), b).reshape((b.shape[1],))
+    raise NotImplementedError("np.dot is implemented for rank 1 and 2")
+
+
 class Dispatcher:
     def __init__(self, py_func, parallel=False, boundscheck=None, **options):
         self.py_func = py_func
@@ -104,6 +122,8 @@ class Dispatcher:
         self._compiled = {}
         self._plans = {}
         self._loop_plans = {}
+        self._stage_plan = None        # (staging.Plan or None,) once analysed
+        self._stage_funcs = {}         # (stage index, captured constants) -> Dispatcher
         try:
             node = kernel_compiler._function_ast(py_func)
         except kernel_compiler.KernelCompileError:
@@ -138,6 +158,9 @@ class Dispatcher:
             return served
         if self._has_parallel_loop():
             return self._parallel(args)
+        plan = self._plan()
+        if plan is not None:
+            return self._staged(plan, args)
         return self._elementwise(args)
 
     # -- 1. library lowering -------------------------------------------------
@@ -416,7 +439,92 @@ class Dispatcher:
             return eval(return_code, scope)                              # noqa: S307
         return None
 
-    # -- 3. elementwise fusion -----------------------------------------------
+    # -- 3. straight-line bodies split at reductions and contractions -------
+    def _plan(self):
+        if self._stage_plan is None:
+            plan = None
+            if isinstance(self._node, (ast.FunctionDef, ast.Lambda)):
+                plan = staging.plan_of(self._node, lambda name: self._resolve(name) is np)
+            self._stage_plan = (plan,)
+        return self._stage_plan[0]
+
+    def _staged(self, plan, args):
+        if len(args) != len(plan.params):
+            raise TypeError(f"{self.py_func.__name__}() takes {len(plan.params)} arguments")
+        env = dict(zip(plan.params, args))
+        scope = None
+        launches = []
+        for k, stage in enumerate(plan.stages):
+            if stage.kind == "lib":
+                env[stage.target] = self._stage_library(
+                    stage, [env[n] for n in stage.operands], launches)
+                continue
+            if stage.kind != "store" and isinstance(stage.expr, ast.Name) and \
+                    stage.expr.id in env:
+                value = env[stage.expr.id]            # another name for a value
+            else:
+                if scope is None:
+                    scope = self._host_scope(())
+                value = self._stage_map(k, stage, env, scope, launches)
+            if stage.kind == "return":
+                self.last_launch = {"path": "staged", "stages": launches}
+                return value
+            if stage.kind == "map":
+                env[stage.target] = value
+        self.last_launch = {"path": "staged", "stages": launches}
+        return None
+
+    def _stage_map(self, k, stage, env, scope, launches):
+        missing = [n for n in stage.inputs if n not in env]
+        if missing:
+            raise kernel_compiler.KernelCompileError(
+                f"{self.py_func.__name__}, line {stage.node.lineno}: '{missing[0]}' is "
+                "used before it is assigned")
+        if not any(isinstance(env[n], HipNdArray) for n in stage.inputs) and \
+                not (stage.kind == "store" and isinstance(env.get(stage.target), HipNdArray)):
+            # scalars only (the result of a full reduction, say): on the host
+            expr = ast.fix_missing_locations(ast.Expression(body=stage.expr))
+            value = eval(compile(expr, "<scalar stage>", "eval"), scope, dict(env))  # noqa: S307
+            launches.append({"path": "host scalar"})
+            return value
+        key = (k, kernel_impl.captured_constants(self.py_func))
+        entry = self._stage_funcs.get(key)
+        if entry is None:
+            func, params = staging.stage_function(
+                stage, f"{self.py_func.__name__}_stage{k}", scope)
+            entry = self._stage_funcs[key] = (
+                Dispatcher(func, boundscheck=self.boundscheck), params)
+        sub, params = entry
+        value = sub._run([env[p] for p in params])
+        launches.append(sub.last_launch)
+        return value
+
+    def _stage_library(self, stage, vals, launches):
+        op, axis = stage.op, stage.kwargs.get("axis")
+        where = f"{self.py_func.__name__}, line {stage.node.lineno}"
+        try:
+            if not any(isinstance(v, HipNdArray) for v in vals):
+                launches.append({"path": "host scalar"})
+                return getattr(np, op)(*vals, **stage.kwargs)
+            ctx = next(v.ctx for v in vals if isinstance(v, HipNdArray))
+            if op == "dot":
+                result = _dot(*vals)
+            else:
+                x = vals[0]
+                if axis is None and x.ndim > 2 and x.is_c_contiguous():
+                    x = x.reshape((x.size,))
+                if op == "mean":
+                    result = _mean(x, axis)
+                else:
+                    result = _REDUCE[op](x, axis=axis)
+                    if axis is None and isinstance(result, HipNdArray):
+                        result = result.asnumpy().reshape(-1)[0]
+            launches.append({"path": "library", "kernel": ctx.last_kernel()})
+            return result
+        except (TypeError, ValueError, NotImplementedError) as exc:
+            raise kernel_compiler.KernelCompileError(f"{where}: np.{op}: {exc}") from exc
+
+    # -- 4. elementwise fusion -----------------------------------------------
     def _elementwise(self, args):
         ctx = kernel_impl.check_device_args(args)
         # Everything but addresses and scalar values is fixed by the argument

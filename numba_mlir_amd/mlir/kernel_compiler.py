@@ -314,6 +314,9 @@ class Module:
 
 def _function_ast(func):
     """The FunctionDef or Lambda node of a Python function object."""
+    node = getattr(func, "__nmk_ast__", None)    # a function built from a tree
+    if node is not None:
+        return node
     try:
         src = inspect.getsource(func)
     except (OSError, TypeError) as exc:

@@ -1,0 +1,218 @@
+"""Splits a straight-line function of whole-array expressions at its
+reductions and contractions.
+
+The reference lowers ``np.sqrt(np.sum(a * b, axis=1)) / n`` to a chain of
+linalg.generic ops -- a map, a reduction, a map -- and fuses what it can
+(numba_mlir/mlir/numpy/funcs.py:163-229 builds the reductions,
+linalg_builder.py:297-325 the maps).  Here the same chain is made explicit:
+every ``np.sum / prod / min / max / mean`` (function or array method),
+``np.dot`` and ``@`` becomes a *library* stage served by a hand-written
+kernel, and the expressions between them become *map* stages, each fused into
+one generated kernel.  Operands of a library stage that are expressions are
+materialised by a map stage first.
+
+Only straight-line bodies qualify: assignments to names, whole-array stores
+(``out[:] = ...``), augmented assignments of names and one final ``return``.
+"""
+
+import ast
+
+REDUCTIONS = ("sum", "prod", "min", "max", "amin", "amax", "mean")
+CONTRACTIONS = ("dot",)
+
+
+class Stage:
+    """kind: "map" (target = expr), "store" (target[...] = expr), "lib"
+    (target = op(operands, **kwargs)), "return" (expr is a Name or a constant
+    expression of names)."""
+
+    def __init__(self, kind, target=None, expr=None, op=None, operands=(), kwargs=None,
+                 node=None):
+        self.kind, self.target, self.expr = kind, target, expr
+        self.op, self.operands, self.kwargs = op, list(operands), kwargs or {}
+        self.node = node            # the source node, for messages
+        self.inputs = []            # local names the expression reads (map / store)
+
+    def __repr__(self):
+        if self.kind == "lib":
+            return f"{self.target} = {self.op}({', '.join(self.operands)}, {self.kwargs})"
+        text = ast.unparse(self.expr) if self.expr is not None else ""
+        return " ".join(part for part in (self.kind, self.target, text) if part)
+
+
+class NotStraightLine(Exception):
+    pass
+
+
+def _is_whole_slice(node):
+    def full(n):
+        return (isinstance(n, ast.Slice) and n.lower is None and n.upper is None
+                and n.step is None) or \
+               (isinstance(n, ast.Constant) and n.value is Ellipsis)
+    if isinstance(node, ast.Tuple):
+        return len(node.elts) > 0 and all(full(e) for e in node.elts)
+    return full(node)
+
+
+class _Splitter(ast.NodeTransformer):
+    def __init__(self, plan):
+        self.plan = plan
+
+    def _operand(self, node):
+        """A name holding the operand's value (materialised if needed)."""
+        if isinstance(node, ast.Name):
+            return node.id
+        name = self.plan.fresh()
+        self.plan.add(Stage("map", name, node, node=node))
+        return name
+
+    def _literal_kwargs(self, node, positional, keywords):
+        kwargs = {}
+        for key, value in list(zip(("axis",), positional)) + \
+                [(k.arg, k.value) for k in keywords]:
+            if key != "axis":
+                raise NotStraightLine(f"line {node.lineno}: only 'axis' is supported here")
+            try:
+                kwargs[key] = ast.literal_eval(value)
+            except ValueError:
+                raise NotStraightLine(f"line {node.lineno}: the axis must be a literal")
+            if not (kwargs[key] is None or isinstance(kwargs[key], int)):
+                raise NotStraightLine(f"line {node.lineno}: the axis must be one integer")
+        return kwargs
+
+    def visit_Call(self, node):
+        self.generic_visit(node)              # innermost stages first
+        func = node.func
+        if not isinstance(func, ast.Attribute):
+            return node
+        name = func.attr
+        if name not in REDUCTIONS + CONTRACTIONS:
+            return node
+        base = func.value
+        if isinstance(base, ast.Name) and base.id not in self.plan.locals:
+            if not self.plan.is_numpy(base.id):
+                return node                   # math.prod, some other module
+            args = list(node.args)            # np.<name>(x, ...)
+        else:
+            args = [base] + list(node.args)   # <expr>.<name>(...)
+        count = 2 if name in CONTRACTIONS else 1
+        if len(args) < count:
+            return node
+        operands = [self._operand(a) for a in args[:count]]
+        kwargs = {} if name in CONTRACTIONS else \
+            self._literal_kwargs(node, args[count:], node.keywords)
+        if name in CONTRACTIONS and (len(args) > count or node.keywords):
+            raise NotStraightLine(f"line {node.lineno}: np.dot takes two arrays here")
+        target = self.plan.fresh()
+        self.plan.add(Stage("lib", target, op=name, operands=operands, kwargs=kwargs,
+                            node=node))
+        self.plan.library_stages += 1
+        return ast.copy_location(ast.Name(id=target, ctx=ast.Load()), node)
+
+    def visit_BinOp(self, node):
+        self.generic_visit(node)
+        if not isinstance(node.op, ast.MatMult):
+            return node
+        operands = [self._operand(node.left), self._operand(node.right)]
+        target = self.plan.fresh()
+        self.plan.add(Stage("lib", target, op="dot", operands=operands, node=node))
+        self.plan.library_stages += 1
+        return ast.copy_location(ast.Name(id=target, ctx=ast.Load()), node)
+
+
+class Plan:
+    """The stages of one function, in execution order."""
+
+    def __init__(self, node, is_numpy):
+        self.is_numpy = is_numpy            # name -> bool: bound to the numpy module
+        self.stages = []
+        self.library_stages = 0
+        self.counter = 0
+        self.params = [a.arg for a in node.args.args]
+        self.locals = set(self.params)
+        body = node.body if isinstance(node.body, list) else [ast.Return(value=node.body)]
+        for stmt in body:
+            for n in ast.walk(stmt):
+                if isinstance(n, ast.Name) and isinstance(n.ctx, ast.Store):
+                    self.locals.add(n.id)
+        splitter = _Splitter(self)
+        returned = False
+        for stmt in body:
+            if returned:
+                raise NotStraightLine("statements after the return")
+            if isinstance(stmt, ast.Expr) and isinstance(stmt.value, ast.Constant):
+                continue                                       # a docstring
+            if isinstance(stmt, ast.AugAssign) and isinstance(stmt.target, ast.Name):
+                load = ast.copy_location(ast.Name(id=stmt.target.id, ctx=ast.Load()), stmt)
+                value = ast.copy_location(ast.BinOp(left=load, op=stmt.op, right=stmt.value),
+                                          stmt)
+                stmt = ast.copy_location(ast.Assign(targets=[stmt.target], value=value), stmt)
+            if isinstance(stmt, ast.Assign) and len(stmt.targets) == 1:
+                target = stmt.targets[0]
+                value = splitter.visit(stmt.value)
+                if isinstance(target, ast.Name):
+                    self.add(Stage("map", target.id, value, node=stmt))
+                    continue
+                if isinstance(target, ast.Subscript) and isinstance(target.value, ast.Name) \
+                        and _is_whole_slice(target.slice):
+                    self.add(Stage("store", target.value.id, value, node=stmt))
+                    continue
+            elif isinstance(stmt, ast.Return):
+                if stmt.value is not None:
+                    self.add(Stage("return", None, splitter.visit(stmt.value), node=stmt))
+                returned = True
+                continue
+            raise NotStraightLine(f"line {stmt.lineno}: not an assignment, a whole-array "
+                                  "store or a return")
+        for stage in self.stages:
+            if stage.expr is not None:
+                seen = []
+                for n in ast.walk(stage.expr):
+                    if isinstance(n, ast.Name) and n.id in self.locals and n.id not in seen:
+                        seen.append(n.id)
+                stage.inputs = seen
+
+    def fresh(self):
+        self.counter += 1
+        name = f"_nmk_t{self.counter}"
+        self.locals.add(name)
+        return name
+
+    def add(self, stage):
+        self.stages.append(stage)
+
+
+def plan_of(node, is_numpy):
+    """The Plan of a FunctionDef / Lambda node, or None when the body is not
+    straight-line or holds no reduction or contraction to split at."""
+    try:
+        import copy
+        plan = Plan(copy.deepcopy(node), is_numpy)
+    except NotStraightLine:
+        return None
+    return plan if plan.library_stages else None
+
+
+def stage_function(stage, name, scope):
+    """A Python function computing one map or store stage (its source is
+    attached as ``__nmk_ast__`` for the kernel compiler)."""
+    args = ast.arguments(posonlyargs=[], args=[], kwonlyargs=[], kw_defaults=[], defaults=[])
+    params = list(stage.inputs)
+    if stage.kind == "store":
+        params = [stage.target] + [p for p in params if p != stage.target]
+        body = ast.Assign(
+            targets=[ast.Subscript(value=ast.Name(id=stage.target, ctx=ast.Load()),
+                                   slice=ast.Constant(value=Ellipsis), ctx=ast.Store())],
+            value=stage.expr)
+    else:
+        body = ast.Return(value=stage.expr)
+    args.args = [ast.arg(arg=p) for p in params]
+    fn = ast.FunctionDef(name=name, args=args, body=[body], decorator_list=[])
+    ast.copy_location(fn, stage.node)
+    ast.copy_location(body, stage.node)
+    module = ast.fix_missing_locations(ast.Module(body=[fn], type_ignores=[]))
+    namespace = dict(scope)
+    exec(compile(module, f"<stage of {name}>", "exec"), namespace)    # noqa: S102
+    func = namespace[name]
+    func.__nmk_ast__ = fn
+    return func, params

@@ -266,3 +266,45 @@ def mean_rows(x):
 
 def mean_cols(x):
     return np.mean(x, axis=0)
+
+
+# straight-line bodies that mix maps with reductions / contractions
+def l2_norm_rows(a):
+    return np.sqrt(np.square(a).sum(axis=1))
+
+
+def softmax(x):
+    e = np.exp(x - np.max(x))
+    return e / np.sum(e)
+
+
+def standardise(x):
+    m = np.mean(x, axis=0)
+    d = x - m
+    return d / np.sqrt(np.mean(d * d, axis=0))
+
+
+def affine(a, b, c):
+    return np.dot(a, b) + c
+
+
+def chain(a, b, c):
+    return a @ b @ c
+
+
+def cosine(x, y):
+    return np.dot(x, y) / (np.sqrt(np.sum(x * x)) * np.sqrt(np.sum(y * y)))
+
+
+def weighted_rows(a, w, out):
+    s = np.sum(a * w, axis=1)
+    s += 1.0
+    out[:] = s * 2.0
+
+
+def matvec(a, v):
+    return np.dot(a, v * 2.0) - 1.0
+
+
+def column_range(x):
+    return x.max(axis=0) - np.min(x, axis=0)

@@ -453,3 +453,48 @@ def test_mean(env, dtype):
         got = got.asnumpy() if hasattr(got, "asnumpy") else got
         assert np.asarray(got).dtype == np.asarray(want).dtype
         np.testing.assert_allclose(got, want, rtol=rtol, atol=1e-6 if dtype == np.float32 else 0)
+
+
+def test_bodies_mixing_maps_reductions_and_products(env):
+    """Straight-line bodies are split at their reductions and matrix products:
+    maps run as fused kernels, the rest on the hand-written kernels
+    (test_l2_norm, test_gpu.py:2198-2223, is the first case)."""
+    hip = env[0]
+    rng = np.random.default_rng(21)
+
+    def run(func, *host, rtol=1e-12):
+        f = njit(func)
+        dev = [hip.asarray(h) if isinstance(h, np.ndarray) else h for h in host]
+        got = f(*dev)
+        assert f.last_launch["path"] == "staged"
+        want = func(*[h.copy() if isinstance(h, np.ndarray) else h for h in host])
+        if want is not None:
+            got = got.asnumpy() if hasattr(got, "asnumpy") else got
+            np.testing.assert_allclose(got, want, rtol=rtol)
+            assert np.asarray(got).shape == np.asarray(want).shape
+        return f, dev
+
+    a32 = rng.standard_normal((65, 25)).astype(np.float32)
+    f, _ = run(cases.l2_norm_rows, a32, rtol=1e-5)
+    assert [s["path"] for s in f.last_launch["stages"]] == ["elementwise", "library",
+                                                            "elementwise"]
+    x = rng.standard_normal(1000)
+    run(cases.softmax, x)
+    m = rng.standard_normal((200, 33))
+    run(cases.standardise, m)
+    run(cases.column_range, m)
+    a, b, c = (rng.standard_normal(s) for s in ((40, 30), (30, 20), (20,)))
+    run(cases.affine, a, b, c)
+    run(cases.chain, a, b, rng.standard_normal((20, 10)))
+    run(cases.cosine, x, rng.standard_normal(1000))
+    run(cases.matvec, a, rng.standard_normal(30))
+    w = rng.standard_normal(30)
+    out = np.zeros(40)
+    f, dev = run(cases.weighted_rows, a, w, out)
+    want = np.zeros(40)
+    cases.weighted_rows(a, w, want)
+    np.testing.assert_allclose(dev[2].asnumpy(), want, rtol=1e-12)
+    # a second call reuses the stage functions
+    f(*dev)
+    np.testing.assert_allclose(dev[2].asnumpy(), want, rtol=1e-12)
+    assert len(f._stage_funcs) == 3

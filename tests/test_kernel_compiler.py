@@ -409,3 +409,47 @@ def test_kernels_stream_stores_nobody_reads_back(K):
         a[i] = 1.0
 
     assert "__restrict__" not in source_of(K, exchanging, [F64_1D] * 2, noalias=True)
+
+
+def test_bodies_are_split_at_reductions_and_contractions():
+    """A straight-line body becomes map stages (one fused kernel each) around
+    library stages (the reductions and matrix products)."""
+    import ast
+    import njit_cases
+    from numba_mlir_amd.mlir import staging
+
+    def plan(func):
+        node = kc._function_ast(func)
+        return staging.plan_of(node, lambda name: name == "np")
+
+    p = plan(njit_cases.l2_norm_rows)
+    assert [s.kind for s in p.stages] == ["map", "lib", "return"]
+    assert ast.unparse(p.stages[0].expr) == "np.square(a)"
+    assert (p.stages[1].op, p.stages[1].kwargs) == ("sum", {"axis": 1})
+    assert ast.unparse(p.stages[2].expr) == "np.sqrt(_nmk_t2)"
+
+    p = plan(njit_cases.softmax)
+    assert [repr(s) for s in p.stages] == [
+        "_nmk_t1 = max(x, {})", "map e np.exp(x - _nmk_t1)",
+        "_nmk_t2 = sum(e, {})", "return e / _nmk_t2"]
+    assert p.stages[1].inputs == ["x", "_nmk_t1"]
+
+    p = plan(njit_cases.chain)
+    assert [(s.kind, s.op, s.operands) for s in p.stages[:2]] == [
+        ("lib", "dot", ["a", "b"]), ("lib", "dot", ["_nmk_t1", "c"])]
+
+    p = plan(njit_cases.weighted_rows)
+    assert [s.kind for s in p.stages] == ["map", "lib", "map", "map", "store"]
+    assert p.stages[3].target == "s" and ast.unparse(p.stages[3].expr) == "s + 1.0"
+
+    # nothing to split at, or not straight-line: left to the other paths
+    assert plan(njit_cases.fused_map) is None
+    assert plan(njit_cases.saxpy_loop) is None
+    assert plan(njit_cases.sum_of_squares) is None
+
+    # a stage's function carries its own tree for the kernel compiler
+    func, params = staging.stage_function(plan(njit_cases.softmax).stages[1],
+                                          "softmax_stage1", {"np": np})
+    assert params == ["x", "_nmk_t1"]
+    assert kc._function_ast(func).name == "softmax_stage1"
+    np.testing.assert_allclose(func(np.array([0.0, 1.0]), 1.0), np.exp([-1.0, 0.0]))
