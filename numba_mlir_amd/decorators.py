@@ -89,12 +89,17 @@ def _mean(x, axis):
     return _DIVIDE[0](total, float_t(x.shape[axis]))
 
 
-def _dot(a, b):
+def _dot(a, b, out=None):
     """numpy.dot of device arrays of rank 1 or 2 through the matrix kernels."""
     if not (isinstance(a, HipNdArray) and isinstance(b, HipNdArray)):
         raise TypeError("both operands must be device arrays")
     if a.ndim == 2 and b.ndim == 2:
-        return ops.dot(a, b)
+        if out is not None and (not isinstance(out, HipNdArray) or
+                                out.shape != (a.shape[0], b.shape[1])):
+            raise ValueError("out must be a device array of the product's shape")
+        return ops.dot(a, b, out=out)
+    if out is not None:
+        raise NotImplementedError("out= is implemented for 2-d operands")
     if a.ndim == 1 and b.ndim == 1:
         if a.shape != b.shape:
             raise ValueError(f"shapes {a.shape} and {b.shape} do not match")
@@ -223,6 +228,14 @@ class Dispatcher:
                 a, b = array(call[1][0]), array(call[1][1])
                 if a is not None and b is not None and a.ndim == b.ndim == 2:
                     return self._served("library", ops.dot(a, b), a.ctx)
+            # np.dot(a, b, c), np.dot(a, b, out=c) (test_gpu.py:2101-2138)
+            if call and len(call[1]) + len(call[2]) == 3 and \
+                    all(k.arg == "out" for k in call[2]):
+                nodes = call[1] + [k.value for k in call[2]]
+                a, b, c = (array(n) for n in nodes)
+                if a is not None and b is not None and c is not None and \
+                        a.ndim == b.ndim == 2:
+                    return self._served("library", _dot(a, b, out=c), a.ctx)
             # np.sum(x, axis=k) and friends
             call = np_call(expr, tuple(_REDUCE))
             if call:
@@ -444,7 +457,9 @@ class Dispatcher:
         if self._stage_plan is None:
             plan = None
             if isinstance(self._node, (ast.FunctionDef, ast.Lambda)):
-                plan = staging.plan_of(self._node, lambda name: self._resolve(name) is np)
+                plan = staging.plan_of(
+                    self._node, lambda name: self._resolve(name) is np,
+                    lambda name: isinstance(self._resolve(name), Dispatcher))
             self._stage_plan = (plan,)
         return self._stage_plan[0]
 
@@ -457,7 +472,19 @@ class Dispatcher:
         for k, stage in enumerate(plan.stages):
             if stage.kind == "lib":
                 env[stage.target] = self._stage_library(
-                    stage, [env[n] for n in stage.operands], launches)
+                    stage, [env[n] for n in stage.operands], launches, env)
+                continue
+            if stage.kind == "view":
+                if scope is None:
+                    scope = self._host_scope(())
+                env[stage.target] = self._stage_view(stage, env, scope)
+                continue
+            if stage.kind == "call":
+                callee = self._resolve(stage.op)
+                value = callee._run([env[n] for n in stage.args])
+                launches.append(callee.last_launch)
+                if stage.target is not None:
+                    env[stage.target] = value
                 continue
             if stage.kind != "store" and isinstance(stage.expr, ast.Name) and \
                     stage.expr.id in env:
@@ -499,16 +526,39 @@ class Dispatcher:
         launches.append(sub.last_launch)
         return value
 
-    def _stage_library(self, stage, vals, launches):
+    def _stage_view(self, stage, env, scope):
+        x = env[stage.operands[0]]
+        where = f"{self.py_func.__name__}, line {stage.node.lineno}"
+        args = []
+        for node in stage.args:
+            expr = ast.fix_missing_locations(ast.Expression(body=node))
+            args.append(eval(compile(expr, "<view argument>", "eval"), scope, dict(env)))  # noqa: S307
+        if not isinstance(x, HipNdArray):
+            return getattr(np, stage.op)(x, *args)
+        try:
+            if stage.op == "reshape":
+                return x.reshape(*args)
+            if stage.op == "ravel":
+                return x.reshape((x.size,))
+            if args and args != [None] and tuple(args[0] if len(args) == 1 else args) != \
+                    tuple(range(x.ndim))[::-1]:
+                raise NotImplementedError("only the full reversal of the axes is supported")
+            return x.T
+        except (TypeError, ValueError, NotImplementedError) as exc:
+            raise kernel_compiler.KernelCompileError(f"{where}: {stage.op}: {exc}") from exc
+
+    def _stage_library(self, stage, vals, launches, env):
         op, axis = stage.op, stage.kwargs.get("axis")
         where = f"{self.py_func.__name__}, line {stage.node.lineno}"
         try:
+            out = env[stage.kwargs["out"]] if "out" in stage.kwargs else None
             if not any(isinstance(v, HipNdArray) for v in vals):
                 launches.append({"path": "host scalar"})
-                return getattr(np, op)(*vals, **stage.kwargs)
+                kwargs = dict(stage.kwargs, out=out) if out is not None else stage.kwargs
+                return getattr(np, op)(*vals, **kwargs)
             ctx = next(v.ctx for v in vals if isinstance(v, HipNdArray))
             if op == "dot":
-                result = _dot(*vals)
+                result = _dot(*vals, out=out)
             else:
                 x = vals[0]
                 if axis is None and x.ndim > 2 and x.is_c_contiguous():

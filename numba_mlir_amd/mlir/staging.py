@@ -19,12 +19,15 @@ import ast
 
 REDUCTIONS = ("sum", "prod", "min", "max", "amin", "amax", "mean")
 CONTRACTIONS = ("dot",)
+VIEWS = ("reshape", "transpose", "ravel")    # no data moves
 
 
 class Stage:
     """kind: "map" (target = expr), "store" (target[...] = expr), "lib"
-    (target = op(operands, **kwargs)), "return" (expr is a Name or a constant
-    expression of names)."""
+    (target = op(operands, **kwargs)), "view" (target = operand reshaped or
+    transposed; ``args`` are expressions of host values), "call" (target =
+    another compiled function applied to whole arrays; ``args`` are names),
+    "return" (expr is a Name or an expression of names)."""
 
     def __init__(self, kind, target=None, expr=None, op=None, operands=(), kwargs=None,
                  node=None):
@@ -32,6 +35,7 @@ class Stage:
         self.op, self.operands, self.kwargs = op, list(operands), kwargs or {}
         self.node = node            # the source node, for messages
         self.inputs = []            # local names the expression reads (map / store)
+        self.args = []              # view / call stages: see above
 
     def __repr__(self):
         if self.kind == "lib":
@@ -86,6 +90,8 @@ class _Splitter(ast.NodeTransformer):
         if not isinstance(func, ast.Attribute):
             return node
         name = func.attr
+        if name in VIEWS:
+            return self._view(node, name)
         if name not in REDUCTIONS + CONTRACTIONS:
             return node
         base = func.value
@@ -99,15 +105,50 @@ class _Splitter(ast.NodeTransformer):
         if len(args) < count:
             return node
         operands = [self._operand(a) for a in args[:count]]
-        kwargs = {} if name in CONTRACTIONS else \
-            self._literal_kwargs(node, args[count:], node.keywords)
-        if name in CONTRACTIONS and (len(args) > count or node.keywords):
-            raise NotStraightLine(f"line {node.lineno}: np.dot takes two arrays here")
+        if name in CONTRACTIONS:
+            # np.dot(a, b, c) / np.dot(a, b, out=c) write into an existing array
+            extra = list(args[count:]) + [k.value for k in node.keywords if k.arg == "out"]
+            if len(extra) > 1 or any(k.arg != "out" for k in node.keywords) or \
+                    not all(isinstance(e, ast.Name) for e in extra):
+                raise NotStraightLine(f"line {node.lineno}: np.dot takes two arrays and "
+                                      "an optional out array here")
+            kwargs = {"out": extra[0].id} if extra else {}
+        else:
+            kwargs = self._literal_kwargs(node, args[count:], node.keywords)
         target = self.plan.fresh()
         self.plan.add(Stage("lib", target, op=name, operands=operands, kwargs=kwargs,
                             node=node))
         self.plan.library_stages += 1
         return ast.copy_location(ast.Name(id=target, ctx=ast.Load()), node)
+
+    def _view(self, node, name):
+        base = node.func.value
+        if isinstance(base, ast.Name) and base.id not in self.plan.locals:
+            if not self.plan.is_numpy(base.id) or not node.args:
+                return node
+            array, args = node.args[0], list(node.args[1:])    # np.reshape(x, shape)
+        else:
+            array, args = base, list(node.args)                # x.reshape(...)
+        if node.keywords:
+            raise NotStraightLine(f"line {node.lineno}: keywords are not supported here")
+        stage = Stage("view", self.plan.fresh(), op=name, operands=[self._operand(array)],
+                      node=node)
+        stage.args = args
+        self.plan.add(stage)
+        self.plan.library_stages += 1
+        return ast.copy_location(ast.Name(id=stage.target, ctx=ast.Load()), node)
+
+    def visit_Attribute(self, node):
+        self.generic_visit(node)
+        if node.attr != "T" or not isinstance(node.ctx, ast.Load):
+            return node
+        if isinstance(node.value, ast.Name) and node.value.id not in self.plan.locals:
+            return node
+        stage = Stage("view", self.plan.fresh(), op="transpose",
+                      operands=[self._operand(node.value)], node=node)
+        self.plan.add(stage)
+        self.plan.library_stages += 1
+        return ast.copy_location(ast.Name(id=stage.target, ctx=ast.Load()), node)
 
     def visit_BinOp(self, node):
         self.generic_visit(node)
@@ -123,8 +164,9 @@ class _Splitter(ast.NodeTransformer):
 class Plan:
     """The stages of one function, in execution order."""
 
-    def __init__(self, node, is_numpy):
+    def __init__(self, node, is_numpy, is_compiled=lambda name: False):
         self.is_numpy = is_numpy            # name -> bool: bound to the numpy module
+        self.is_compiled = is_compiled      # name -> bool: another compiled function
         self.stages = []
         self.library_stages = 0
         self.counter = 0
@@ -147,6 +189,19 @@ class Plan:
                 value = ast.copy_location(ast.BinOp(left=load, op=stmt.op, right=stmt.value),
                                           stmt)
                 stmt = ast.copy_location(ast.Assign(targets=[stmt.target], value=value), stmt)
+            call = stmt.value if isinstance(stmt, (ast.Expr, ast.Assign)) else None
+            if isinstance(call, ast.Call) and isinstance(call.func, ast.Name) and \
+                    call.func.id not in self.locals and self.is_compiled(call.func.id) and \
+                    not call.keywords and \
+                    (isinstance(stmt, ast.Expr) or
+                     (len(stmt.targets) == 1 and isinstance(stmt.targets[0], ast.Name))):
+                # another compiled function applied to whole arrays
+                target = stmt.targets[0].id if isinstance(stmt, ast.Assign) else None
+                stage = Stage("call", target, op=call.func.id, node=stmt)
+                stage.args = [splitter._operand(splitter.visit(a)) for a in call.args]
+                self.add(stage)
+                self.library_stages += 1
+                continue
             if isinstance(stmt, ast.Assign) and len(stmt.targets) == 1:
                 target = stmt.targets[0]
                 value = splitter.visit(stmt.value)
@@ -182,12 +237,13 @@ class Plan:
         self.stages.append(stage)
 
 
-def plan_of(node, is_numpy):
+def plan_of(node, is_numpy, is_compiled=lambda name: False):
     """The Plan of a FunctionDef / Lambda node, or None when the body is not
-    straight-line or holds no reduction or contraction to split at."""
+    straight-line or holds nothing to split at (a reduction, a contraction, a
+    view, a call of another compiled function)."""
     try:
         import copy
-        plan = Plan(copy.deepcopy(node), is_numpy)
+        plan = Plan(copy.deepcopy(node), is_numpy, is_compiled)
     except NotStraightLine:
         return None
     return plan if plan.library_stages else None

@@ -308,3 +308,34 @@ def matvec(a, v):
 
 def column_range(x):
     return x.max(axis=0) - np.min(x, axis=0)
+
+
+def dot_out_positional(a, b, c):
+    return np.dot(a, b, c)
+
+
+def dot_out_keyword(a, b, c):
+    return np.dot(a, b, out=c)
+
+
+def reshape_fill(a):
+    b = a.reshape(17, 23, 56)
+    b[:] = 42
+
+
+def transposed_sum(a):
+    return np.sum(a.T * 2.0, axis=1)
+
+
+def pairwise_loop(X1, X2, D):
+    X1_rows = X1.shape[0]
+    X2_rows = X2.shape[0]
+    X1_cols = X1.shape[1]
+
+    for i in prange(X1_rows):
+        for j in prange(X2_rows):
+            d = 0.0
+            for k in range(X1_cols):
+                tmp = X1[i, k] - X2[j, k]
+                d += tmp * tmp
+            D[i, j] = np.sqrt(d)

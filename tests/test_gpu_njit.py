@@ -498,3 +498,64 @@ def test_bodies_mixing_maps_reductions_and_products(env):
     f(*dev)
     np.testing.assert_allclose(dev[2].asnumpy(), want, rtol=1e-12)
     assert len(f._stage_funcs) == 3
+
+
+def test_compiled_functions_apply_others_to_whole_arrays(env):
+    """test_cfd_indirect / test_cfd_reshape (test_gpu.py:1737-1768, 1934-1964):
+    a compiled function whose statement is a call of another one, and a
+    reshape of an argument that is then filled."""
+    hip = env[0]
+    inner = njit(cases.scale_into)
+
+    def outer(a, b):
+        inner(a, b)
+
+    a = np.arange(1024, dtype=np.float32)
+    da, db = hip.asarray(a), hip.asarray(np.zeros_like(a))
+    f = njit(outer)
+    f(da, db)
+    assert f.last_launch["path"] == "staged"
+    np.testing.assert_array_equal(db.asnumpy(), a * 2)
+
+    fill = njit(cases.reshape_fill)
+
+    def outer2(a):
+        fill(a)
+
+    x = np.arange(17 * 23 * 56, dtype=np.float32).reshape(23, 56, 17).copy()
+    dx = hip.asarray(x)
+    njit(outer2)(dx)
+    np.testing.assert_array_equal(dx.asnumpy(), np.full_like(x, 42))
+
+    m = np.random.default_rng(3).standard_normal((30, 50))
+    got = njit(cases.transposed_sum)(hip.asarray(m))
+    np.testing.assert_allclose(got.asnumpy(), cases.transposed_sum(m), rtol=1e-12)
+
+
+@pytest.mark.parametrize("func", [cases.dot_out_positional, cases.dot_out_keyword])
+def test_dot_into_an_existing_array(env, func):
+    """test_cfd_dot (test_gpu.py:2101-2138): the reference's exact fixture."""
+    hip = env[0]
+    a = np.array([[1, 2, 3], [4, 5, 6]], np.float32)
+    b = np.array([[1, 2], [3, 4], [5, 6]], np.float32)
+    dc = hip.asarray(np.zeros((2, 2), np.float32))
+    f = njit(func)
+    res = f(hip.asarray(a), hip.asarray(b), dc)
+    assert f.last_launch["path"] == "library"
+    np.testing.assert_array_equal(dc.asnumpy(), [[22, 28], [49, 64]])
+    np.testing.assert_array_equal(res.asnumpy(), [[22, 28], [49, 64]])
+
+
+def test_pairwise_as_nested_prange_loops(env):
+    """test_pairwise2 (test_gpu.py:2226-2266): the distance body as two
+    prange loops around a serial one, on the reference's fixture."""
+    hip = env[0]
+    a = np.arange(128 * 3, dtype=np.float32).reshape(128, 3)
+    b = a + 5
+    want = np.zeros((128, 128), np.float32)
+    cases.pairwise_loop(a, b, want)
+    dD = hip.asarray(np.zeros_like(want))
+    f = njit(parallel=True)(cases.pairwise_loop)
+    f(hip.asarray(a), hip.asarray(b), dD)
+    assert f.last_launch["path"] == "parallel loop"
+    np.testing.assert_allclose(dD.asnumpy(), want, rtol=1e-5)
