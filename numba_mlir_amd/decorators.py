@@ -74,11 +74,71 @@ _REDUCE = {"sum": ops.sum, "prod": ops.prod, "min": ops.amin, "max": ops.amax,
            "amin": ops.amin, "amax": ops.amax}
 
 
+def _collapse(shape, views):
+    """Merges adjacent dimensions of an iteration space that every array
+    walks with one stride (a dimension's stride equals the next one's stride
+    times its extent; broadcast dimensions, stride 0, merge with each other)
+    and drops dimensions of extent 1.  Returns the new shape and the views."""
+    arrays = [v for v in views if isinstance(v, HipNdArray)]
+    if 0 in shape or not shape:
+        return tuple(shape), views
+    dims = [(n, [a.strides[d] for a in arrays]) for d, n in enumerate(shape) if n != 1]
+    if not dims:
+        dims = [(1, [0] * len(arrays))]
+    merged = [dims[0]]
+    for n, strides in dims[1:]:
+        before_n, before = merged[-1]
+        if all(b == s * n for b, s in zip(before, strides)):
+            merged[-1] = (before_n * n, strides)
+        else:
+            merged.append((n, strides))
+    new_shape = tuple(n for n, _ in merged)
+    out, k = [], 0
+    for v in views:
+        if isinstance(v, HipNdArray):
+            strides = tuple(st[k] for _, st in merged)
+            out.append(HipNdArray(v._buffer, new_shape, v.dtype, strides, v._offset))
+            k += 1
+        else:
+            out.append(v)
+    return new_shape, out
+
+
+def _reduce_nd(op, x, axis):
+    """A reduction kernel applied to a dense array of any rank along its first
+    or last axis (or all of it), through a 2-d view."""
+    if x.ndim <= 2 or not x.is_c_contiguous():
+        return op(x, axis=axis)
+    if axis is None:
+        return op(x.reshape((x.size,)), axis=None)
+    axis = axis + x.ndim if axis < 0 else axis
+    if axis == 0:
+        return op(x.reshape((x.shape[0], x.size // max(x.shape[0], 1))),
+                  axis=0).reshape(x.shape[1:])
+    if axis == x.ndim - 1:
+        return op(x.reshape((x.size // max(x.shape[-1], 1), x.shape[-1])),
+                  axis=1).reshape(x.shape[:-1])
+    raise NotImplementedError("reductions of arrays of rank > 2 run along the first or "
+                              "the last axis")
+
+
 _DIVIDE = []
+_FILL = []
+
+
+def _fill_body(a, value):
+    a[:] = value
+
+
+def _fill(array, value):
+    if not _FILL:
+        _FILL.append(Dispatcher(_fill_body))
+    _FILL[0]._run([array, value])
+
 
 
 def _mean(x, axis):
-    total = ops.sum(x, axis=axis)
+    total = _reduce_nd(ops.sum, x, axis)
     float_t = x.dtype.type if x.dtype.kind == "f" else np.float64
     if axis is None:
         if isinstance(total, HipNdArray):
@@ -250,7 +310,7 @@ class Dispatcher:
                     else:
                         ok = False
                 if ok:
-                    result = _REDUCE[name](x, axis=axis)
+                    result = _reduce_nd(_REDUCE[name], x, axis)
                     if axis is None and isinstance(result, HipNdArray):
                         result = result.asnumpy().reshape(-1)[0]   # a scalar, as NumPy's
                     return self._served("library", result, x.ctx)
@@ -479,6 +539,11 @@ class Dispatcher:
                     scope = self._host_scope(())
                 env[stage.target] = self._stage_view(stage, env, scope)
                 continue
+            if stage.kind == "alloc":
+                if scope is None:
+                    scope = self._host_scope(())
+                env[stage.target] = self._stage_alloc(stage, env, scope, args)
+                continue
             if stage.kind == "call":
                 callee = self._resolve(stage.op)
                 value = callee._run([env[n] for n in stage.args])
@@ -526,6 +591,36 @@ class Dispatcher:
         launches.append(sub.last_launch)
         return value
 
+    def _stage_alloc(self, stage, env, scope, call_args):
+        """np.empty / zeros / ones (and *_like) on the device of the call's
+        arrays (reference: numpy/funcs.py:581-640)."""
+        def host(node):
+            expr = ast.fix_missing_locations(ast.Expression(body=node))
+            return eval(compile(expr, "<allocation argument>", "eval"), scope, dict(env))  # noqa: S307
+
+        pos = [host(n) for n in stage.args[0]]
+        kws = {k.arg: host(k.value) for k in stage.args[1]}
+        where = f"{self.py_func.__name__}, line {stage.node.lineno}"
+        unknown = set(kws) - {"shape", "dtype"}
+        if unknown or len(pos) > 2:
+            raise kernel_compiler.KernelCompileError(
+                f"{where}: np.{stage.op}: only shape and dtype are supported")
+        ctx = kernel_impl.check_device_args(
+            [a for a in list(call_args) + list(env.values()) if isinstance(a, HipNdArray)])
+        if stage.op.endswith("_like"):
+            like = pos[0]
+            shape = like.shape
+            dtype = kws.get("dtype", pos[1] if len(pos) > 1 else None) or like.dtype
+        else:
+            shape = pos[0] if pos else kws["shape"]
+            dtype = kws.get("dtype", pos[1] if len(pos) > 1 else None) or np.float64
+        if isinstance(shape, (int, np.integer)):
+            shape = (int(shape),)
+        out = HipNdArray.empty(tuple(int(n) for n in shape), dtype, device=ctx.device)
+        if not stage.op.startswith("empty") and out.size:
+            _fill(out, out.dtype.type(1 if stage.op.startswith("ones") else 0))
+        return out
+
     def _stage_view(self, stage, env, scope):
         x = env[stage.operands[0]]
         where = f"{self.py_func.__name__}, line {stage.node.lineno}"
@@ -561,12 +656,10 @@ class Dispatcher:
                 result = _dot(*vals, out=out)
             else:
                 x = vals[0]
-                if axis is None and x.ndim > 2 and x.is_c_contiguous():
-                    x = x.reshape((x.size,))
                 if op == "mean":
                     result = _mean(x, axis)
                 else:
-                    result = _REDUCE[op](x, axis=axis)
+                    result = _reduce_nd(_REDUCE[op], x, axis)
                     if axis is None and isinstance(result, HipNdArray):
                         result = result.asnumpy().reshape(-1)[0]
             launches.append({"path": "library", "kernel": ctx.last_kernel()})
@@ -605,7 +698,7 @@ class Dispatcher:
             views = [v.reshape(run_shape) if isinstance(v, HipNdArray) else v
                      for v in views]
         else:
-            run_shape = shape
+            run_shape, views = _collapse(shape, views)
         if not 1 <= len(run_shape) <= 3:
             raise kernel_compiler.KernelCompileError(
                 f"{self.py_func.__name__}: elementwise functions over strided arrays "
@@ -619,7 +712,7 @@ class Dispatcher:
         ret = None
         if compiled.ret_dtype is not None:
             ret = HipNdArray.empty(shape, compiled.ret_dtype, device=ctx.device)
-        ret_view = ret.reshape(run_shape) if (ret is not None and dense) else ret
+        ret_view = ret.reshape(run_shape) if ret is not None else ret
         plan = kernel_impl.plan_compiled(ctx, compiled, self.py_func.__name__,
                                          run_shape, views, ret_view)
         plan.run()

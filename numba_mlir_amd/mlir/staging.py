@@ -20,11 +20,25 @@ import ast
 REDUCTIONS = ("sum", "prod", "min", "max", "amin", "amax", "mean")
 CONTRACTIONS = ("dot",)
 VIEWS = ("reshape", "transpose", "ravel")    # no data moves
+ALLOCATIONS = ("empty", "zeros", "ones", "empty_like", "zeros_like", "ones_like")
+# NumPy functions that take an `out` array after this many operands
+# (reference: numpy/funcs.py registers them with out="out")
+OUT_AFTER = dict(
+    [(n, 1) for n in ("sqrt", "square", "log", "sin", "cos", "exp", "tanh", "abs",
+                      "absolute", "negative", "positive", "logical_not", "invert")] +
+    [(n, 2) for n in ("add", "subtract", "multiply", "true_divide", "divide", "power",
+                      "arctan2", "minimum", "maximum", "logical_and", "logical_or",
+                      "logical_xor", "less", "greater", "less_equal", "greater_equal",
+                      "equal", "not_equal", "bitwise_and", "bitwise_or", "bitwise_xor",
+                      "left_shift", "right_shift", "floor_divide", "remainder", "mod")] +
+    [("clip", 3)])
 
 
 class Stage:
     """kind: "map" (target = expr), "store" (target[...] = expr), "lib"
-    (target = op(operands, **kwargs)), "view" (target = operand reshaped or
+    (target = op(operands, **kwargs)), "alloc" (target = a new array; ``args``
+    are the call's positional and keyword expressions, of host values), "view"
+    (target = operand reshaped or
     transposed; ``args`` are expressions of host values), "call" (target =
     another compiled function applied to whole arrays; ``args`` are names),
     "return" (expr is a Name or an expression of names)."""
@@ -92,6 +106,16 @@ class _Splitter(ast.NodeTransformer):
         name = func.attr
         if name in VIEWS:
             return self._view(node, name)
+        numpy_function = isinstance(func.value, ast.Name) and \
+            func.value.id not in self.plan.locals and self.plan.is_numpy(func.value.id)
+        if numpy_function and name in ALLOCATIONS:
+            stage = Stage("alloc", self.plan.fresh(), op=name, node=node)
+            stage.args = (list(node.args), list(node.keywords))
+            self.plan.add(stage)
+            self.plan.library_stages += 1
+            return ast.copy_location(ast.Name(id=stage.target, ctx=ast.Load()), node)
+        if numpy_function and name in OUT_AFTER:
+            return self._with_out(node, OUT_AFTER[name])
         if name not in REDUCTIONS + CONTRACTIONS:
             return node
         base = func.value
@@ -120,6 +144,24 @@ class _Splitter(ast.NodeTransformer):
                             node=node))
         self.plan.library_stages += 1
         return ast.copy_location(ast.Name(id=target, ctx=ast.Load()), node)
+
+    def _with_out(self, node, operands):
+        """np.add(a, b, out) / np.add(a, b, out=out): a store into ``out``,
+        whose value the call then is."""
+        out = [k.value for k in node.keywords if k.arg == "out"]
+        if len(node.args) == operands + 1 and not out:
+            out, args = [node.args[-1]], node.args[:-1]
+        else:
+            args = node.args
+        if not out or (isinstance(out[0], ast.Constant) and out[0].value is None):
+            return node
+        if not isinstance(out[0], ast.Name) or len(args) != operands or \
+                any(k.arg != "out" for k in node.keywords):
+            raise NotStraightLine(f"line {node.lineno}: out must be a named array")
+        value = ast.copy_location(ast.Call(func=node.func, args=list(args), keywords=[]), node)
+        self.plan.add(Stage("store", out[0].id, value, node=node))
+        self.plan.library_stages += 1
+        return ast.copy_location(ast.Name(id=out[0].id, ctx=ast.Load()), node)
 
     def _view(self, node, name):
         base = node.func.value

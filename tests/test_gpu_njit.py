@@ -559,3 +559,59 @@ def test_pairwise_as_nested_prange_loops(env):
     f(hip.asarray(a), hip.asarray(b), dD)
     assert f.last_launch["path"] == "parallel loop"
     np.testing.assert_allclose(dD.asnumpy(), want, rtol=1e-5)
+
+
+def test_batchnorm(env):
+    """test_batchnorm (test_numpy.py): allocations, reductions along the
+    first axis of a 4-d array, broadcast stores and maps in one body."""
+    hip = env[0]
+    rng = np.random.default_rng(42)
+    x = rng.random((8, 14, 14, 32), dtype=np.float32)
+    f = njit(cases.batchnorm4, parallel=True)
+    got = f(hip.asarray(x), 1e-5)
+    assert f.last_launch["path"] == "staged"
+    np.testing.assert_allclose(got.asnumpy(), cases.batchnorm(x), rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("a_shape, b_shape",
+                         [((2, 3, 4), (2, 1, 4)), ((1, 2, 3), (1, 1)), ((2, 3, 4), (3, 4)),
+                          ((5, 6, 7, 8), (1, 7, 8)), ((3, 4, 5, 6, 7), (5, 6, 7))])
+def test_broadcast_setitem(env, a_shape, b_shape):
+    """test_broadcast_setitem (test_numpy.py), plus ranks above three whose
+    dimensions merge."""
+    import math
+    hip = env[0]
+    a = np.zeros(a_shape)
+    b = np.arange(math.prod(b_shape)).reshape(b_shape)
+    da = hip.asarray(a)
+    got = njit(cases.broadcast_setitem)(da, hip.asarray(b))
+    want = cases.broadcast_setitem(a.copy(), b)
+    np.testing.assert_array_equal(got.asnumpy(), want)
+    np.testing.assert_array_equal(da.asnumpy(), want)
+
+
+@pytest.mark.parametrize("name,func", cases.OUT_FORMS, ids=[c[0] for c in cases.OUT_FORMS])
+def test_functions_with_an_out_array(env, name, func):
+    """test_binary_inplace (test_numpy.py): the third argument receives the
+    result and is what the call returns."""
+    hip = env[0]
+    rng = np.random.default_rng(9)
+    a, b = rng.uniform(0.5, 3, (6, 7)), rng.uniform(0.5, 3, (7,))
+    want = np.zeros((6, 7))
+    func(a, b, want)
+    dc = hip.asarray(np.zeros((6, 7)))
+    res = njit(func)(hip.asarray(a), hip.asarray(b), dc)
+    np.testing.assert_allclose(dc.asnumpy(), want, rtol=1e-13)
+    assert res is dc
+
+
+def test_clip_with_out_and_allocations(env):
+    hip = env[0]
+    rng = np.random.default_rng(10)
+    a, lo, hi = rng.uniform(-2, 2, 50), rng.uniform(-1, 0, 50), rng.uniform(0, 1, 50)
+    out = hip.asarray(np.zeros(50))
+    njit(cases.clip_out)(hip.asarray(a), hip.asarray(lo), hip.asarray(hi), out)
+    np.testing.assert_array_equal(out.asnumpy(), np.clip(a, lo, hi))
+    x = rng.uniform(-2, 2, (9, 11))
+    got = njit(cases.zeros_ones)(hip.asarray(x))
+    np.testing.assert_allclose(got.asnumpy(), cases.zeros_ones(x), rtol=1e-13)
