@@ -635,10 +635,18 @@ class Dispatcher:
                 return x.reshape(*args)
             if stage.op == "ravel":
                 return x.reshape((x.size,))
-            if args and args != [None] and tuple(args[0] if len(args) == 1 else args) != \
-                    tuple(range(x.ndim))[::-1]:
-                raise NotImplementedError("only the full reversal of the axes is supported")
-            return x.T
+            if stage.op == "flip":
+                # numpy.flip (numpy/funcs.py:236-253): negative strides
+                if len(args) > 1 or (args and not (args[0] is None or
+                                                   isinstance(args[0], (int, np.integer)))):
+                    raise NotImplementedError("flip takes one integer axis or none")
+                axis = args[0] if args else None
+                if axis is not None and not -x.ndim <= axis < x.ndim:
+                    raise ValueError("axis out of range")
+                which = range(x.ndim) if axis is None else (axis % x.ndim,)
+                return x[tuple(slice(None, None, -1) if d in which else slice(None)
+                               for d in range(x.ndim))]
+            return x.transpose(*args)
         except (TypeError, ValueError, NotImplementedError) as exc:
             raise kernel_compiler.KernelCompileError(f"{where}: {stage.op}: {exc}") from exc
 

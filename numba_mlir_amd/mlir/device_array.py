@@ -178,6 +178,19 @@ class HipNdArray:
         return HipNdArray(self._buffer, self.shape[::-1], self.dtype,
                           self.strides[::-1], self._offset)
 
+    def transpose(self, *axes):
+        """numpy.transpose: a view with the dimensions permuted (reversed
+        when no permutation is given)."""
+        if len(axes) == 1 and (axes[0] is None or isinstance(axes[0], (tuple, list))):
+            axes = axes[0]
+        if not axes:
+            return self.T
+        axes = [int(a) + self.ndim if int(a) < 0 else int(a) for a in axes]
+        if sorted(axes) != list(range(self.ndim)):
+            raise ValueError("axes don't match array")
+        return HipNdArray(self._buffer, [self.shape[a] for a in axes], self.dtype,
+                          [self.strides[a] for a in axes], self._offset)
+
     def __len__(self):
         if not self.shape:
             raise TypeError("len() of a 0-d device array")

@@ -19,7 +19,7 @@ import ast
 
 REDUCTIONS = ("sum", "prod", "min", "max", "amin", "amax", "mean")
 CONTRACTIONS = ("dot",)
-VIEWS = ("reshape", "transpose", "ravel")    # no data moves
+VIEWS = ("reshape", "transpose", "ravel", "flip")    # no data moves
 ALLOCATIONS = ("empty", "zeros", "ones", "empty_like", "zeros_like", "ones_like")
 # NumPy functions that take an `out` array after this many operands
 # (reference: numpy/funcs.py registers them with out="out")
@@ -244,6 +244,11 @@ class Plan:
                 self.add(stage)
                 self.library_stages += 1
                 continue
+            if isinstance(stmt, ast.Expr):
+                # a call made for its effect: np.add(a, b, out)
+                if isinstance(splitter.visit(stmt.value), ast.Name):
+                    continue
+                raise NotStraightLine(f"line {stmt.lineno}: an expression without effect")
             if isinstance(stmt, ast.Assign) and len(stmt.targets) == 1:
                 target = stmt.targets[0]
                 value = splitter.visit(stmt.value)

@@ -386,3 +386,23 @@ def zeros_ones(x):
     e = np.empty_like(x)
     e[:] = x + o
     return e * 2 + z
+
+
+TRANSPOSES = [
+    ((0, 1, 2), lambda a: np.transpose(a, (0, 1, 2))),
+    ((0, 2, 1), lambda a: np.transpose(a, (0, 2, 1))),
+    ((1, 0, 2), lambda a: np.transpose(a, (1, 0, 2))),
+    ((1, 2, 0), lambda a: np.transpose(a, (1, 2, 0))),
+    ((2, 0, 1), lambda a: np.transpose(a, (2, 0, 1))),
+    ((2, 1, 0), lambda a: np.transpose(a, (2, 1, 0))),
+    ("T", lambda a: a.T),
+    ("method", lambda a: a.transpose(1, 0, 2) * 2),
+]
+
+FLIPS = [
+    ("all", lambda a: np.flip(a)),
+    ("axis0", lambda a: np.flip(a, 0)),
+    ("axis1", lambda a: np.flip(a, 1)),
+    ("axis-1", lambda a: np.flip(a, -1)),
+    ("flip+map", lambda a: np.flip(a, 1) + a),
+]

@@ -615,3 +615,31 @@ def test_clip_with_out_and_allocations(env):
     x = rng.uniform(-2, 2, (9, 11))
     got = njit(cases.zeros_ones)(hip.asarray(x))
     np.testing.assert_allclose(got.asnumpy(), cases.zeros_ones(x), rtol=1e-13)
+
+
+@pytest.mark.parametrize("name,func", cases.TRANSPOSES + cases.FLIPS,
+                         ids=[str(c[0]) for c in cases.TRANSPOSES + cases.FLIPS])
+def test_transpose_and_flip_are_views(env, name, func):
+    """test_transpose, test_flip1 (test_numpy.py): every permutation of the
+    axes, flips along each axis; no data moves."""
+    hip = env[0]
+    a = np.arange(3 * 4 * 5).reshape(3, 4, 5)
+    da = hip.asarray(a)
+    got = njit(func)(da)
+    np.testing.assert_array_equal(got.asnumpy(), func(a))
+    if "map" not in str(name) and name != "method":
+        assert got._buffer is da._buffer
+
+
+def test_affine_into_an_existing_array(env):
+    hip = env[0]
+    rng = np.random.default_rng(13)
+    a, b, c = rng.standard_normal((20, 30)), rng.standard_normal((30, 10)), \
+        rng.standard_normal(10)
+
+    def affine(a, b, c, out):
+        np.add(np.dot(a, b), c, out)
+
+    out = hip.asarray(np.zeros((20, 10)))
+    njit(affine)(hip.asarray(a), hip.asarray(b), hip.asarray(c), out)
+    np.testing.assert_allclose(out.asnumpy(), a @ b + c, rtol=1e-12)

@@ -442,6 +442,13 @@ def test_bodies_are_split_at_reductions_and_contractions():
     assert [s.kind for s in p.stages] == ["map", "lib", "map", "map", "store"]
     assert p.stages[3].target == "s" and ast.unparse(p.stages[3].expr) == "s + 1.0"
 
+    def affine(a, b, c, out):
+        np.add(np.dot(a, b), c, out)
+
+    p = plan(affine)
+    assert [repr(s) for s in p.stages] == ["_nmk_t1 = dot(a, b, {})",
+                                           "store out np.add(_nmk_t1, c)"]
+
     # nothing to split at, or not straight-line: left to the other paths
     assert plan(njit_cases.fused_map) is None
     assert plan(njit_cases.saxpy_loop) is None
