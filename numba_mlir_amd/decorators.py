@@ -707,10 +707,8 @@ class Dispatcher:
                      for v in views]
         else:
             run_shape, views = _collapse(shape, views)
-        if not 1 <= len(run_shape) <= 3:
-            raise kernel_compiler.KernelCompileError(
-                f"{self.py_func.__name__}: elementwise functions over strided arrays "
-                "support up to three dimensions")
+        if len(run_shape) > 3:
+            return self._elementwise_slices(ctx, args, shape, run_shape, views)
         compiled = self._compile("elementwise", views, len(run_shape), len(run_shape) > 1)
         for name, a, v in zip(self._params(), args, views):
             if isinstance(a, HipNdArray) and f"v_{name}" in compiled.written and \
@@ -736,6 +734,33 @@ class Dispatcher:
             entry["by_alias"][hip.disjoint(arrays)] = plan
         else:
             entry["plan"] = plan
+        return ret
+
+
+    def _elementwise_slices(self, ctx, args, shape, run_shape, views):
+        """More than three dimensions that do not merge: one launch of the 3-d
+        kernel per index of the leading ones."""
+        outer = run_shape[:-3]
+        plan = ret = ret_view = None
+        for index in np.ndindex(*outer):
+            part = [v[index] if isinstance(v, HipNdArray) else v for v in views]
+            if plan is None:
+                compiled = self._compile("elementwise", part, 3, True)
+                for name, a in zip(self._params(), args):
+                    if isinstance(a, HipNdArray) and f"v_{name}" in compiled.written and \
+                            a.shape != tuple(shape):
+                        raise ValueError(f"'{name}' is assigned but has shape {a.shape}, "
+                                         f"not the broadcast shape {tuple(shape)}")
+                if compiled.ret_dtype is not None:
+                    ret = HipNdArray.empty(shape, compiled.ret_dtype, device=ctx.device)
+                    ret_view = ret.reshape(run_shape)
+                plan = kernel_impl.plan_compiled(
+                    ctx, compiled, self.py_func.__name__, run_shape[-3:], part,
+                    None if ret_view is None else ret_view[index])
+                plan.run()
+            else:
+                plan.run(part, None if ret_view is None else ret_view[index])
+        self.last_launch = dict(plan.info, path="elementwise", launches=math.prod(outer))
         return ret
 
 

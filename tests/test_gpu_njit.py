@@ -575,10 +575,11 @@ def test_batchnorm(env):
 
 @pytest.mark.parametrize("a_shape, b_shape",
                          [((2, 3, 4), (2, 1, 4)), ((1, 2, 3), (1, 1)), ((2, 3, 4), (3, 4)),
-                          ((5, 6, 7, 8), (1, 7, 8)), ((3, 4, 5, 6, 7), (5, 6, 7))])
+                          ((5, 6, 7, 8), (1, 7, 8)), ((3, 4, 5, 6, 7), (5, 6, 7)),
+                          ((5, 6, 7, 8), (6, 1, 8)), ((2, 3, 4, 5, 6), (3, 1, 5, 1))])
 def test_broadcast_setitem(env, a_shape, b_shape):
     """test_broadcast_setitem (test_numpy.py), plus ranks above three whose
-    dimensions merge."""
+    dimensions merge, and ones that do not (one launch per leading index)."""
     import math
     hip = env[0]
     a = np.zeros(a_shape)
@@ -588,6 +589,9 @@ def test_broadcast_setitem(env, a_shape, b_shape):
     want = cases.broadcast_setitem(a.copy(), b)
     np.testing.assert_array_equal(got.asnumpy(), want)
     np.testing.assert_array_equal(da.asnumpy(), want)
+    # the same operands through a map that returns a new array
+    got = njit(cases.fused_map)(da, hip.asarray(b), hip.asarray(b), 0.5)
+    np.testing.assert_allclose(got.asnumpy(), cases.fused_map(want, b, b, 0.5), rtol=1e-13)
 
 
 @pytest.mark.parametrize("name,func", cases.OUT_FORMS, ids=[c[0] for c in cases.OUT_FORMS])
