@@ -330,8 +330,36 @@ class Dispatcher:
                         ok = False
                 if ok:
                     return self._served("library", _mean(x, axis), x.ctx)
-            # np.sqrt(np.sum(x * x))
+            # np.sqrt(np.square(a).sum(axis=1)), np.sqrt(np.sum(a * a, axis=1)): the
+            # fused row-norm kernel (test_l2_norm, test_gpu.py:2198-2223)
             call = np_call(expr, ("sqrt",))
+            if call and len(call[1]) == 1 and not call[2]:
+                inner = call[1][0]
+                x = None
+                if isinstance(inner, ast.Call) and isinstance(inner.func, ast.Attribute) and \
+                        inner.func.attr == "sum":
+                    base = inner.func.value
+                    if isinstance(base, ast.Name) and self._resolve(base.id) is np:
+                        operand, rest = (inner.args[0] if inner.args else None), inner.args[1:]
+                    else:
+                        operand, rest = base, inner.args
+                    axis = [a for a in rest] + [k.value for k in inner.keywords
+                                                if k.arg == "axis"]
+                    if operand is not None and len(axis) == 1 and \
+                            len(rest) + len(inner.keywords) == 1 and \
+                            isinstance(axis[0], ast.Constant) and axis[0].value in (1, -1):
+                        sq = np_call(operand, ("square",))
+                        if sq and len(sq[1]) == 1 and not sq[2]:
+                            x = array(sq[1][0])
+                        elif isinstance(operand, ast.BinOp) and \
+                                isinstance(operand.op, ast.Mult) and \
+                                isinstance(operand.left, ast.Name) and \
+                                isinstance(operand.right, ast.Name) and \
+                                operand.left.id == operand.right.id:
+                            x = array(operand.left)
+                if x is not None and x.dtype == np.float32 and x.ndim == 2:
+                    return self._served("library", ops.l2_norm_rows(x), x.ctx)
+            # np.sqrt(np.sum(x * x))
             if call and len(call[1]) == 1 and not call[2]:
                 inner = np_call(call[1][0], ("sum",))
                 if inner and len(inner[1]) == 1 and not inner[2]:

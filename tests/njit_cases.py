@@ -406,3 +406,7 @@ FLIPS = [
     ("axis-1", lambda a: np.flip(a, -1)),
     ("flip+map", lambda a: np.flip(a, 1) + a),
 ]
+
+
+def l2_norm_rows_product(a):
+    return np.sqrt(np.sum(a * a, axis=1))

@@ -474,10 +474,18 @@ def test_bodies_mixing_maps_reductions_and_products(env):
             assert np.asarray(got).shape == np.asarray(want).shape
         return f, dev
 
-    a32 = rng.standard_normal((65, 25)).astype(np.float32)
-    f, _ = run(cases.l2_norm_rows, a32, rtol=1e-5)
+    a64 = rng.standard_normal((65, 25))
+    f, _ = run(cases.l2_norm_rows, a64)
     assert [s["path"] for s in f.last_launch["stages"]] == ["elementwise", "library",
                                                             "elementwise"]
+    # float32 row-major input: the fused row-norm kernel serves the whole body
+    a32 = a64.astype(np.float32)
+    for func in (cases.l2_norm_rows, cases.l2_norm_rows_product):
+        g = njit(func)
+        got = g(hip.asarray(a32))
+        assert g.last_launch["path"] == "library"
+        assert g.last_launch["kernel"].startswith("nmk_norm2_axis1")
+        np.testing.assert_allclose(got.asnumpy(), func(a32), rtol=1e-5)
     x = rng.standard_normal(1000)
     run(cases.softmax, x)
     m = rng.standard_normal((200, 33))
