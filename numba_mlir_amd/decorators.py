@@ -184,6 +184,7 @@ class Dispatcher:
         self.boundscheck = bool(boundscheck)
         self.options = options
         self.last_launch = None          # what served the most recent call
+        self.last_plan = None            # its LaunchPlan, for a generated kernel
         self._compiled = {}
         self._plans = {}
         self._loop_plans = {}
@@ -526,6 +527,7 @@ class Dispatcher:
                     make_partials(math.prod(plan.grid))
                 plan.run(args, partials=partials)
             info = plan.info
+            self.last_plan = plan
         self.last_launch = dict(info, path="parallel loop")
         # fold the per-block partial results, in block order, onto the values
         # the reduction variables had before the loop
@@ -723,6 +725,7 @@ class Dispatcher:
                                            device=ctx.device)
                 plan.run(args, ret)
                 self.last_launch = dict(plan.info, path="elementwise")
+                self.last_plan = plan
                 return ret
 
         arrays = [a for a in args if isinstance(a, HipNdArray)]
@@ -751,6 +754,7 @@ class Dispatcher:
                                          run_shape, views, ret_view)
         plan.run()
         self.last_launch = dict(plan.info, path="elementwise")
+        self.last_plan = plan
 
         if len(self._plans) >= MAX_PLANS:
             self._plans.clear()

@@ -523,8 +523,10 @@ class FunctionTranslator:
         dst = f"{arr_code}.p[{' + '.join(terms)}]"
         if self.noalias and arr_code not in self.read_arrays:
             last = self.ndim - 1
+            # (the returned array is allocated dense by the caller)
+            unit = "true" if arr_code == "nmk_ret" else f"{arr_code}.stride[{last}] == 1"
             self.emit(f"NMK_STORE_ALONG{last}(&{dst}, ({elem.ctype})({value_code}), "
-                      f"{arr_code}.stride[{last}] == 1);")
+                      f"{unit});")
         else:
             self.emit(f"{dst} = {value_code};")
 

@@ -290,6 +290,7 @@ class Kernel(KernelBase):
         self.boundscheck = bool(kwargs.get(
             "boundscheck", readenv("NUMBA_MLIR_KERNEL_BOUNDSCHECK", int, 0)))
         self.last_launch = None
+        self.last_plan = None  # the LaunchPlan of the most recent compiled launch
         self._compiled = {}
         self._plans = {}       # stored launches (shared by configured copies)
 
@@ -349,7 +350,7 @@ class Kernel(KernelBase):
             plan = self._plans.get(key)
             if plan is not None:
                 plan.run(args)
-                self.last_launch = plan.info
+                self.last_launch, self.last_plan = plan.info, plan
                 return
             # With a runtime-chosen block a body that cannot observe its
             # grouping is laid out for coalescing (last dimension on x), unless
@@ -372,7 +373,7 @@ class Kernel(KernelBase):
             if len(self._plans) >= MAX_PLANS:
                 self._plans.clear()
             self._plans[key] = plan
-            self.last_launch = plan.info
+            self.last_launch, self.last_plan = plan.info, plan
             return
 
         params = _ParamList()
@@ -453,6 +454,17 @@ class LaunchPlan:
         self._descs = params.build()
         self._lock = threading.Lock()     # slots are rewritten per call
         self._launch = (ctx.queue, kern, *self.grid, *self.block, NO_DEPS, self._descs)
+
+    def enqueue(self):
+        """Launches with the slots as they are and returns the event without
+        waiting (the caller passes it to ``retire``): back-to-back launches
+        for timing."""
+        return runtime_lib.gpuxLaunchKernel(*self._launch)
+
+    def retire(self, event):
+        queue = self.ctx.queue
+        runtime_lib.gpuxWait(queue, event)
+        runtime_lib.gpuxDestroyEvent(queue, event)
 
     def run(self, args=None, ret=None, partials=()):
         """Launches; ``args`` (same types, shapes and strides as the plan was
