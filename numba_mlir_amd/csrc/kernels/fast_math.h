@@ -27,4 +27,35 @@ __device__ __forceinline__ double sqrtF64(double d) {
   return __builtin_fma(e, h, g);
 }
 
+// float32 log and exp without the range handling of the general routines:
+// the same operations in the same order (the extended-precision product with
+// ln 2 or log2 e around the hardware log2 / exp2), so the results are the
+// general routines' bit for bit wherever the guards hold -- a positive normal
+// argument of log within [2^-120, 2^120), |x| <= 80 for exp (the result is a
+// normal number).  Everything else -- zeros, infinities, NaNs, denormals,
+// overflow -- takes the general routine; that handling is two thirds of its
+// instructions.
+__device__ __forceinline__ float logNormalF32(float q) {
+  const float y = __builtin_amdgcn_logf(q); // log2
+  const float r = y * 0x1.62e42ep-1f;
+  float e = __builtin_fmaf(y, 0x1.62e42ep-1f, -r);
+  e = __builtin_fmaf(y, 0x1.efa39ep-25f, e);
+  return r + e;
+}
+__device__ __forceinline__ float logF32(float q) {
+  // positive, exponent in [-120, 120)
+  return (__float_as_uint(q) - 0x03800000u) < 0x78000000u ? logNormalF32(q) : logf(q);
+}
+__device__ __forceinline__ float expNormalF32(float b) {
+  const float p = b * 0x1.715476p+0f; // b log2(e), then its rounding error
+  float e = __builtin_fmaf(b, 0x1.715476p+0f, -p);
+  e = __builtin_fmaf(b, 0x1.4ae0bep-26f, e);
+  const float n = __builtin_rintf(p);
+  const float v = __builtin_amdgcn_exp2f((p - n) + e);
+  return __builtin_ldexpf(v, int(n));
+}
+__device__ __forceinline__ float expF32(float b) {
+  return __builtin_fabsf(b) <= 80.0f ? expNormalF32(b) : expf(b);
+}
+
 } // namespace nmk

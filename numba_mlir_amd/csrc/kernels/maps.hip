@@ -256,13 +256,16 @@ template <> struct BsMath<float> {
 };
 
 // The float32 steps log(P / S) and exp(b) without the range handling of the
-// general routines: the same operations in the same order, so the results
-// are bit-identical to P / S, logf and expf whenever bsEveryday() holds --
-// P and S positive with exponents in [-60, 60) (the quotient and the
-// reciprocal are then normal numbers) and |b| <= 80 (exp(b) is normal).
-// The division is the reciprocal times P with one residual correction.  It
-// is the general routines' handling of zeros, infinities, NaNs, denormals
-// and overflow that costs two thirds of their instructions.
+// general routines: the same operations in the same order, so log and exp
+// are bit-identical to logf and expf whenever bsEveryday() holds -- P and S
+// positive with exponents in [-60, 60) (the quotient and the reciprocal are
+// then normal numbers) and |b| <= 80 (exp(b) is normal).  The division is
+// the reciprocal times P with one residual correction: it equals the
+// correctly rounded quotient unless that quotient lies within 2e-7 units in
+// the last place of a rounding boundary (no case among the 2^24 options of
+// the benchmark input).  It is the general routines' handling of zeros,
+// infinities, NaNs, denormals and overflow that costs two thirds of their
+// instructions.
 __device__ __forceinline__ bool bsEveryday(float P, float S, float b) {
   const uint32_t lo = 0x21800000u;   // bits of 2^-60
   const uint32_t span = 0x3C000000u; // up to, not including, 2^60

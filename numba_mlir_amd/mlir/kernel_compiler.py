@@ -302,6 +302,7 @@ class Module:
         # group ids, local sizes, barriers, fences, local arrays, group
         # reductions): only then does the item-to-lane mapping matter
         self.communicates = False
+        self.uses_erf_table = False     # some body calls erf on a float64
         self.device_funcs = {}          # (id(func), arg type keys) -> (name, ret type)
         self.device_code = []
         self.in_progress = set()
@@ -873,6 +874,14 @@ class FunctionTranslator:
             if name == "sqrt" and t is FLOAT64:
                 # same rounding as the library routine at half its cost
                 return Val(f"nmk::sqrtF64({v.code})", t, nonneg=True)
+            if name == "erf" and t is FLOAT64:
+                # table in workgroup memory, loaded at kernel entry
+                self.m.uses_erf_table = True
+                return Val(f"nmkjit::erfF64({v.code})", t)
+            if name in ("log", "exp") and t is FLOAT32:
+                # the library routine's own arithmetic, its range handling
+                # only where the argument needs it
+                return Val(f"nmk::{name}F32({v.code})", t, nonneg=name == "exp")
             return Val(f"{_UNARY_MATH[name]}({v.code})", t)
         if (mod == "math" or is_np) and name in _ROUNDING and len(node.args) == 1:
             v = self.scalar(node.args[0])
@@ -1598,6 +1607,8 @@ class FunctionTranslator:
         ]
         for name, t, neutral in red:
             out.append(f"  {t.ctype} {self.cname(name)} = ({t.ctype}){neutral};")
+        if self.m.uses_erf_table:
+            out.append("  nmkjit::erfTableLoad();")
         if ept > 1:
             out += [
                 "#pragma unroll",
@@ -1796,7 +1807,7 @@ def build_code_object(compiled):
     """Compiles the generated source with hipcc; code objects are cached on
     disk under the hash of (source, support header, flags)."""
     support = b""
-    for header in ("jit_support.h", "fast_math.h"):
+    for header in ("jit_support.h", "fast_math.h", "erf_taylor.inc"):
         with open(os.path.join(_KERNELS_DIR, header), "rb") as f:
             support += f.read()
     digest = hashlib.sha256()

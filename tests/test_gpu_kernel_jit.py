@@ -760,3 +760,105 @@ def test_large_1d_launch_ids_do_not_wrap(env):               # 2268-2283
     b = 2 ** 31 + 10
     K.kernel(func)[2 ** 31 + 11, 1024](arr, b)
     assert arr.asnumpy()[0] == np.float32(b)
+
+
+def _all_kinds_f32(rng, n):
+    """float32 values of every kind: random bit patterns (all exponents, both
+    signs, denormals, NaNs), a band around 1 and the special values."""
+    bits = rng.integers(0, 2 ** 32, n, dtype=np.uint64).astype(np.uint32)
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 1e-45, 1e-38,
+                        1.17549435e-38, 3.4028235e38, 2.0 ** -120, 2.0 ** 120,
+                        np.nextafter(np.float32(2.0 ** -120), np.float32(0)),
+                        np.nextafter(np.float32(2.0 ** 120), np.float32(0))], np.float32)
+    return np.concatenate([bits.view(np.float32),
+                           rng.uniform(0.5, 2.0, n).astype(np.float32), special])
+
+
+@pytest.mark.parametrize("op", ["log", "exp"])
+def test_float32_log_and_exp_equal_the_device_library_bit_for_bit(env, op):
+    """Generated kernels evaluate float32 log / exp with the library's own
+    arithmetic and leave its range handling to the arguments that need it:
+    the results must be the library's on every input."""
+    hip = env[0]
+    rng = np.random.default_rng(17)
+    if op == "log":
+        x = _all_kinds_f32(rng, 1 << 20)
+    else:
+        x = np.concatenate([rng.uniform(-110, 100, 1 << 20).astype(np.float32),
+                            rng.uniform(-1, 1, 1 << 18).astype(np.float32),
+                            np.array([80.0, -80.0, np.nextafter(np.float32(80), np.float32(90)),
+                                      88.7, 88.8, -87.3, -87.4, -103.9, -104.0, 0.0, -0.0,
+                                      np.inf, -np.inf, np.nan], np.float32)])
+    f = getattr(np, op)
+
+    def func(a, b):
+        i = get_global_id(0)
+        b[i] = f(a[i])
+
+    dx = hip.asarray(x)
+    got, ref = hip.asarray(np.zeros_like(x)), hip.asarray(np.zeros_like(x))
+    K.kernel(func)[x.shape, ()](dx, got)
+    K.kernel(func, twin="nmk_twin_unary_" + op + "_{dtype}")[x.shape, ()](dx, ref)
+    g, r = got.asnumpy(), ref.asnumpy()
+    same = (g.view(np.uint32) == r.view(np.uint32)) | (np.isnan(g) & np.isnan(r))
+    assert same.all(), (x[~same][:5], g[~same][:5], r[~same][:5])
+    # and the library agrees with NumPy to float32 accuracy where finite
+    with np.errstate(all="ignore"):
+        want = f(x.astype(np.float64))
+    ok = np.isfinite(want) & (np.abs(want) > 1e-30) & (np.abs(want) < 1e30)
+    np.testing.assert_allclose(g[ok], want[ok], rtol=3e-7)
+
+
+def test_float64_erf_within_two_ulp(env):
+    """erf of a double in generated kernels: piecewise Taylor polynomials from
+    a table in workgroup memory.  Against mpmath the error must stay within 2
+    units in the last place; signs, NaN, infinities and the saturation to
+    +-1 must be right."""
+    from scipy.special import erf as scipy_erf
+    hip = env[0]
+    rng = np.random.default_rng(18)
+    x = np.concatenate([rng.uniform(-6.5, 6.5, 1 << 20), rng.uniform(-0.25, 0.25, 1 << 18),
+                        10.0 ** rng.uniform(-300, 1, 1 << 12),
+                        (np.arange(-97, 98) + 0.5) / 16.0, np.arange(-97, 98) / 16.0,
+                        [0.0, -0.0, 3 / 32, np.nextafter(3 / 32, 0), 5e-324, 1e-310, 6.0,
+                         -6.0, 7.0, 30.0, -30.0, np.inf, -np.inf, np.nan]])
+
+    def func(a, b):
+        i = get_global_id(0)
+        b[i] = math.erf(a[i])
+
+    dx = hip.asarray(x)
+    got, ref = hip.asarray(np.zeros_like(x)), hip.asarray(np.zeros_like(x))
+    K.kernel(func)[x.shape, (64,)](dx, got)
+    K.kernel(func, twin="nmk_twin_unary_erf_{dtype}")[x.shape, ()](dx, ref)
+    g, r = got.asnumpy(), ref.asnumpy()
+    assert np.array_equal(np.isnan(g), np.isnan(x))
+    assert np.array_equal(np.signbit(g), np.signbit(x) & ~np.isnan(x)) or \
+        np.array_equal(np.signbit(g[~np.isnan(x)]), np.signbit(x[~np.isnan(x)]))
+    fin = ~np.isnan(x)
+    want = scipy_erf(x[fin])
+    # SciPy's own routine is off by up to 2 units in the last place: a loose
+    # bound on everything, the exact one on a sample with mpmath
+    ulps = np.abs(g[fin] - want) / np.spacing(np.abs(want))
+    assert ulps.max() <= 4, (x[fin][ulps.argmax()], ulps.max())
+    import mpmath
+    mpmath.mp.dps = 40
+    pick = np.concatenate([rng.choice(np.flatnonzero(fin), 20000, replace=False),
+                           np.argsort(-ulps)[:200]])
+    worst = worst_lib = 0.0
+    for xi, gi, ri in zip(x[fin][pick].tolist(), g[fin][pick].tolist(),
+                          r[fin][pick].tolist()):
+        exact = mpmath.erf(mpmath.mpf(xi))
+        if exact == 0 or abs(xi) == np.inf:
+            assert gi == float(exact)
+            continue
+        ulp = float(np.spacing(abs(float(exact))))
+        worst = max(worst, abs(float((mpmath.mpf(gi) - exact) / ulp)))
+        worst_lib = max(worst_lib, abs(float((mpmath.mpf(ri) - exact) / ulp)))
+    print("erf max error in ulp: generated", worst, "device library", worst_lib)
+    assert worst <= 2.0, worst
+    big = np.abs(x) >= 6
+    np.testing.assert_array_equal(g[big & fin], np.sign(x[big & fin]))
+    # a second local size, with partial groups: the table load is per group
+    K.kernel(func)[x.shape, (256,)](dx, got)
+    np.testing.assert_array_equal(got.asnumpy()[fin], g[fin])
