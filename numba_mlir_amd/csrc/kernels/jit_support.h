@@ -25,6 +25,14 @@ template <typename T, int N> struct View {
   int64_t stride[N];
 };
 
+// Compile-time switches handed to a generic lambda.
+struct Yes {
+  static constexpr bool value = true;
+};
+struct No {
+  static constexpr bool value = false;
+};
+
 // Python index normalisation: a negative index counts from the end.
 __device__ __forceinline__ int64_t wrap(int64_t i, int64_t n) {
   return i < 0 ? i + n : i;

@@ -407,6 +407,7 @@ class FunctionTranslator:
         self.return_node = None      # parallel mode: the return after the loop
         self.allow_remap = False     # kernels only: see translate_kernel
         self.reversed = False
+        self.rows_per_lane = 1
         self.written_arrays = set()  # elementwise mode: arrays stored through [:]
         self.read_arrays = set()     # elementwise mode: arrays loaded as values
         self.noalias = False         # no two array arguments overlap (host-checked)
@@ -1600,57 +1601,97 @@ class FunctionTranslator:
         ept = self.elements_per_thread
         if self.m.communicates or self.ndim != 1 or self.mode == "kernel":
             ept = self.elements_per_thread = 1
+        # A remapped grid of two or three dimensions runs flat blocks (x only)
+        # and gives each lane ROWS_PER_LANE work-items along hardware y: what
+        # they load by the x index alone (a row vector against a matrix, the
+        # second operand of an outer product) is then loaded once, and the
+        # index on y is uniform over the wave.
+        rows = ROWS_PER_LANE if self.reversed else 1
+        self.rows_per_lane = rows
+        flat = self.reversed
         out += [
-            "  const int64_t " + ", ".join(f"nmk_lid{k} = threadIdx.{dim[k]}" for k in range(3)) + ";",
+            "  const int64_t " + ", ".join(
+                f"nmk_lid{k} = " + ("0" if flat and dim[k] != "x" else f"threadIdx.{dim[k]}")
+                for k in range(3)) + ";",
             "  const int64_t " + ", ".join(f"nmk_grp{k} = blockIdx.{dim[k]}" for k in range(3)) + ";",
-            "  const int64_t " + ", ".join(f"nmk_lsz{k} = blockDim.{dim[k]}" for k in range(3)) + ";",
+            "  const int64_t " + ", ".join(
+                f"nmk_lsz{k} = " + ("1" if flat and dim[k] != "x" else f"blockDim.{dim[k]}")
+                for k in range(3)) + ";",
+            "  (void)nmk_lid0; (void)nmk_lid1; (void)nmk_lid2; (void)nmk_grp0; (void)nmk_grp1;",
+            "  (void)nmk_grp2; (void)nmk_lsz0; (void)nmk_lsz1; (void)nmk_lsz2;",
         ]
         for name, t, neutral in red:
             out.append(f"  {t.ctype} {self.cname(name)} = ({t.ctype}){neutral};")
         if self.m.uses_erf_table:
             out.append("  nmkjit::erfTableLoad();")
-        if ept > 1:
+        body = ["    " + v for v in views]
+        body += ["    " + d for d in self.declarations() + self.private_decls]
+        body += lines
+        if rows > 1:
+            ky = dim.index("y")
+            others = [k for k in range(3) if k != ky]
+            out += [f"  const int64_t nmk_gid{k} = nmk_grp{k} * nmk_lsz{k} + nmk_lid{k};"
+                    for k in others]
             out += [
+                f"  const int64_t nmk_first = nmk_grp{ky} * {rows};",
+                f"  auto nmk_item = [&](const int64_t nmk_gid{ky}, auto nmk_guarded) {{",
+                f"    if (decltype(nmk_guarded)::value && !(nmk_gid{ky} < nmk_gsz{ky})) return;",
+            ] + body + [
+                "  };",
+                "  if (" + " && ".join(f"nmk_gid{k} < nmk_gsz{k}" for k in others) + ") {",
+                f"    if (nmk_first + {rows} <= nmk_gsz{ky}) {{",
                 "#pragma unroll",
-                f"  for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep) {{",
-                f"  const int64_t nmk_gid0 = (nmk_grp0 * {ept} + nmk_rep) * nmk_lsz0 + nmk_lid0;",
-                "  const int64_t nmk_gid1 = 0, nmk_gid2 = 0;",
+                f"      for (int nmk_row = 0; nmk_row < {rows}; ++nmk_row)",
+                "        nmk_item(nmk_first + nmk_row, nmkjit::No());",
+                "    } else {",
+                "#pragma unroll",
+                f"      for (int nmk_row = 0; nmk_row < {rows}; ++nmk_row)",
+                "        nmk_item(nmk_first + nmk_row, nmkjit::Yes());",
+                "    }",
+                "  }",
             ]
         else:
+            if ept > 1:
+                out += [
+                    "#pragma unroll",
+                    f"  for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep) {{",
+                    f"  const int64_t nmk_gid0 = (nmk_grp0 * {ept} + nmk_rep) * nmk_lsz0 + nmk_lid0;",
+                    "  const int64_t nmk_gid1 = 0, nmk_gid2 = 0;",
+                ]
+            else:
+                out += [
+                    "  const int64_t nmk_gid0 = nmk_grp0 * nmk_lsz0 + nmk_lid0;",
+                    "  const int64_t nmk_gid1 = nmk_grp1 * nmk_lsz1 + nmk_lid1;",
+                    "  const int64_t nmk_gid2 = nmk_grp2 * nmk_lsz2 + nmk_lid2;",
+                ]
             out += [
-                "  const int64_t nmk_gid0 = nmk_grp0 * nmk_lsz0 + nmk_lid0;",
-                "  const int64_t nmk_gid1 = nmk_grp1 * nmk_lsz1 + nmk_lid1;",
-                "  const int64_t nmk_gid2 = nmk_grp2 * nmk_lsz2 + nmk_lid2;",
+                "  const bool nmk_active = nmk_gid0 < nmk_gsz0 && nmk_gid1 < nmk_gsz1 && "
+                "nmk_gid2 < nmk_gsz2;",
             ]
-        out += [
-            "  const bool nmk_active = nmk_gid0 < nmk_gsz0 && nmk_gid1 < nmk_gsz1 && "
-            "nmk_gid2 < nmk_gsz2;",
-            "  (void)nmk_lid0; (void)nmk_lid1; (void)nmk_lid2; (void)nmk_grp0; (void)nmk_grp1;",
-            "  (void)nmk_grp2; (void)nmk_lsz0; (void)nmk_lsz1; (void)nmk_lsz2;",
-        ]
-        if self.group_sites:
-            out.append("  __shared__ int nmk_clipped;")
-            for slot, t, _ in self.group_sites:
-                out.append(f"  __shared__ {t.ctype} {slot}[nmkjit::kMaxGroup];")
-            out.append("  if (nmkjit::linearLocalId() == 0) nmk_clipped = 0;")
-            out.append("  __syncthreads();")
-            out.append("  if (!nmk_active) nmk_clipped = 1;")
-            for slot, t, neutral in self.group_sites:
-                out.append(f"  nmkjit::groupInit<{t.ctype}>({slot}, ({t.ctype}){neutral});")
-            out.append("  __syncthreads();")
-        out.append("  if (nmk_active) {")
-        out += ["    " + v for v in views]
-        out += ["    " + d for d in self.declarations() + self.private_decls]
-        out += lines
-        out.append("  }")
-        if ept > 1:
+            if self.group_sites:
+                out.append("  __shared__ int nmk_clipped;")
+                for slot, t, _ in self.group_sites:
+                    out.append(f"  __shared__ {t.ctype} {slot}[nmkjit::kMaxGroup];")
+                out.append("  if (nmkjit::linearLocalId() == 0) nmk_clipped = 0;")
+                out.append("  __syncthreads();")
+                out.append("  if (!nmk_active) nmk_clipped = 1;")
+                for slot, t, neutral in self.group_sites:
+                    out.append(f"  nmkjit::groupInit<{t.ctype}>({slot}, ({t.ctype}){neutral});")
+                out.append("  __syncthreads();")
+            out.append("  if (nmk_active) {")
+            out += body
             out.append("  }")
+            if ept > 1:
+                out.append("  }")
         for name, t, _ in red:
             op = "AddOp" if self.reductions[name] == "add" else "MulOp"
             out.append(f"  nmkjit::blockReduceStore<{t.ctype}>({self.cname(name)}, "
                        f"nmkjit::{op}(), nmk_part_{name});")
         out.append("}")
         return "\n".join(out)
+
+
+ROWS_PER_LANE = 4     # work-items per lane along hardware y of a remapped grid
 
 
 def _safe(name):
@@ -1710,6 +1751,10 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     compiled = CompiledKernel(name, source, tr.local_arrays)
     compiled.boundscheck = boundscheck
     compiled.reversed_dims = tr.reversed
+    # a remapped kernel runs blocks of shape (n, 1, 1) and gives each lane this
+    # many work-items along hardware y: the launcher divides that grid
+    # dimension by it
+    compiled.rows_per_lane = tr.rows_per_lane
     compiled.ret_dtype = tr.ret_type.dtype if (mode == "elementwise" and tr.ret_type) else None
     compiled.range_source = tr.range_source[1] if tr.range_source else None
     compiled.grid_sources = list(tr.grid_sources)   # per grid dimension

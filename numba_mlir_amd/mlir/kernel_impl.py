@@ -404,7 +404,14 @@ def _geometry(ctx, compiled, kern, global_size, local_size):
     if compiled.reversed_dims:
         order.reverse()
     sizes = [int(global_size[k]) for k in order]
-    if len(local_size) != 0:
+    rows = getattr(compiled, "rows_per_lane", 1)
+    if compiled.reversed_dims:
+        # flat blocks, several work-items per lane along y (see translate_kernel)
+        gsize = (ctypes.c_uint32 * 1)(min(sizes[0], 0xFFFFFFFF))
+        bsize = (ctypes.c_uint32 * 1)()
+        runtime_lib.gpuxSuggestBlockSize(ctx.queue, kern, gsize, bsize, 1)
+        block = [int(bsize[0])] + [1] * (ndim - 1)
+    elif len(local_size) != 0:
         block = [int(local_size[k]) for k in order]
     else:
         gsize = (ctypes.c_uint32 * ndim)(*[min(g, 0xFFFFFFFF) for g in sizes])
@@ -413,7 +420,10 @@ def _geometry(ctx, compiled, kern, global_size, local_size):
         block = list(bsize)
     sizes += [1] * (3 - ndim)
     block += [1] * (3 - ndim)
-    return block, [(g + b - 1) // b for g, b in zip(sizes, block)]
+    grid = [(g + b - 1) // b for g, b in zip(sizes, block)]
+    if rows > 1:
+        grid[1] = (grid[1] + rows - 1) // rows
+    return block, grid
 
 
 class LaunchPlan:

@@ -185,7 +185,8 @@ def test_reference_parfor_and_array_statement_tests(env):
     # the perfect nest is a 2-d grid with the inner loop on x ...
     big = hip.asarray(np.zeros((300, 1000), np.float32))
     f(big)
-    assert f.last_launch["grid"][1] == 300 and f.last_launch["block"][1] == 1
+    # (flat blocks, four rows of the outer loop per lane)
+    assert f.last_launch["grid"][1] == 75 and f.last_launch["block"][1] == 1
     np.testing.assert_array_equal(big.asnumpy(),
                                   np.arange(300000, dtype=np.float32).reshape(300, 1000))
     # ... unless the outer loop is too long for grid y: then it alone is the grid
