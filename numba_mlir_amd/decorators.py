@@ -560,6 +560,17 @@ class Dispatcher:
         scope = None
         launches = []
         for k, stage in enumerate(plan.stages):
+            if stage.kind == "map" and stage.deferred:
+                continue                  # evaluated inside the reduction that follows
+            if stage.kind == "lib" and stage.fused_map is not None:
+                if scope is None:
+                    scope = self._host_scope(())
+                value = self._stage_fused_reduction(k, stage, env, scope, launches)
+                if value is not NotImplemented:
+                    env[stage.target] = value
+                    continue
+                env[stage.fused_map.target] = self._stage_map(
+                    k - 1, stage.fused_map, env, scope, launches)
             if stage.kind == "lib":
                 env[stage.target] = self._stage_library(
                     stage, [env[n] for n in stage.operands], launches, env)
@@ -620,6 +631,65 @@ class Dispatcher:
         value = sub._run([env[p] for p in params])
         launches.append(sub.last_launch)
         return value
+
+    def _stage_fused_reduction(self, k, stage, env, scope, launches):
+        """np.sum / np.mean of a map over operands of one dense shape: the map
+        runs inside a parallel-loop reduction.  NotImplemented when the
+        operands do not fit (the caller then runs the two stages)."""
+        source = stage.fused_map
+        if any(n not in env for n in source.inputs):
+            return NotImplemented
+        values = [env[n] for n in source.inputs]
+        arrays = [n for n, v in zip(source.inputs, values) if isinstance(v, HipNdArray)]
+        if not arrays:
+            return NotImplemented
+        first = env[arrays[0]]
+        if first.size == 0 or not all(
+                env[n].shape == first.shape and env[n].is_c_contiguous() for n in arrays):
+            return NotImplemented
+        # NumPy's type of the expression, from one-element stand-ins
+        probe = {n: (np.ones(1, env[n].dtype) if n in arrays else env[n])
+                 for n in source.inputs}
+        try:
+            expr = ast.fix_missing_locations(ast.Expression(body=source.expr))
+            with np.errstate(all="ignore"):
+                dtype = np.asarray(eval(compile(expr, "<dtype probe>", "eval"),   # noqa: S307
+                                        scope, probe)).dtype
+        except Exception:                 # noqa: BLE001 -- not evaluable on the host
+            return NotImplemented
+        if dtype.kind not in "fiub":
+            return NotImplemented
+        integer = dtype.kind != "f"
+        key = ("sum", k, kernel_impl.captured_constants(self.py_func), tuple(arrays), integer)
+        entry = self._stage_funcs.get(key)
+        if entry is None:
+            namespace = dict(scope, _nmk_prange=prange)
+            try:
+                func, params = staging.reduction_function(
+                    source, f"{self.py_func.__name__}_stage{k}_sum", namespace, set(arrays),
+                    integer)
+                entry = (Dispatcher(func, parallel=True, boundscheck=self.boundscheck), params)
+            except kernel_compiler.KernelCompileError:
+                entry = False
+            self._stage_funcs[key] = entry
+        if entry is False:
+            return NotImplemented
+        sub, params = entry
+        flat = [first.size] + [env[n].reshape((first.size,)) if n in arrays else env[n]
+                               for n in source.inputs]
+        try:
+            total = sub._run(flat)
+        except kernel_compiler.KernelCompileError:
+            self._stage_funcs[key] = False        # not expressible per element
+            return NotImplemented
+        launches.append(dict(sub.last_launch, fused="map + sum"))
+        if stage.op == "sum":
+            # NumPy sums small integers in the platform integer
+            out = np.dtype(np.int64) if dtype.kind in "ib" else \
+                (np.dtype(np.uint64) if dtype.kind == "u" else dtype)
+            return out.type(total)
+        float_t = dtype.type if dtype.kind == "f" else np.float64
+        return float_t(float_t(total) / float_t(first.size))
 
     def _stage_alloc(self, stage, env, scope, call_args):
         """np.empty / zeros / ones (and *_like) on the device of the call's

@@ -50,6 +50,8 @@ class Stage:
         self.node = node            # the source node, for messages
         self.inputs = []            # local names the expression reads (map / store)
         self.args = []              # view / call stages: see above
+        self.deferred = False       # a map that the next stage evaluates itself
+        self.fused_map = None       # ... and that stage's link to it
 
     def __repr__(self):
         if self.kind == "lib":
@@ -273,6 +275,37 @@ class Plan:
                     if isinstance(n, ast.Name) and n.id in self.locals and n.id not in seen:
                         seen.append(n.id)
                 stage.inputs = seen
+        self._mark_fused_reductions()
+
+    def _mark_fused_reductions(self):
+        """np.sum / np.mean over everything of an expression materialised
+        just for it: the map can run inside the reduction (one pass over the
+        operands instead of a pass, a temporary and a second pass).  The map
+        stage is marked ``deferred`` and the library stage gets it as
+        ``fused_map``; the executor falls back to the two stages when the
+        operands do not all have one dense shape."""
+        uses = {}
+        for stage in self.stages:
+            for name in list(stage.inputs) + list(stage.operands) + \
+                    [a for a in stage.args if isinstance(a, str)] + \
+                    ([stage.kwargs["out"]] if "out" in stage.kwargs else []):
+                uses[name] = uses.get(name, 0) + 1
+            if stage.kind in ("view", "alloc"):
+                # their argument expressions may name anything
+                nodes = stage.args[0] + [k.value for k in stage.args[1]] \
+                    if stage.kind == "alloc" else stage.args
+                for node in nodes:
+                    for n in ast.walk(node):
+                        if isinstance(n, ast.Name):
+                            uses[n.id] = uses.get(n.id, 0) + 2
+        for before, stage in zip(self.stages, self.stages[1:]):
+            if stage.kind == "lib" and stage.op in ("sum", "mean") and \
+                    stage.kwargs.get("axis") is None and before.kind == "map" and \
+                    before.target == stage.operands[0] and \
+                    before.target.startswith("_nmk_t") and uses.get(before.target) == 1 and \
+                    not isinstance(before.expr, ast.Name):
+                before.deferred = True
+                stage.fused_map = before
 
     def fresh(self):
         self.counter += 1
@@ -313,6 +346,46 @@ def stage_function(stage, name, scope):
     fn = ast.FunctionDef(name=name, args=args, body=[body], decorator_list=[])
     ast.copy_location(fn, stage.node)
     ast.copy_location(body, stage.node)
+    module = ast.fix_missing_locations(ast.Module(body=[fn], type_ignores=[]))
+    namespace = dict(scope)
+    exec(compile(module, f"<stage of {name}>", "exec"), namespace)    # noqa: S102
+    func = namespace[name]
+    func.__nmk_ast__ = fn
+    return func, params
+
+
+def reduction_function(stage, name, scope, arrays, integer):
+    """A Python function summing one map stage's expression over dense 1-d
+    operands in a parallel loop: ``arrays`` are the inputs that are arrays
+    (indexed by the loop variable), the others stay scalars.  ``integer``
+    selects an integer accumulator."""
+    class Index(ast.NodeTransformer):
+        def visit_Name(self, node):
+            if node.id in arrays and isinstance(node.ctx, ast.Load):
+                return ast.copy_location(ast.Subscript(
+                    value=node, slice=ast.Name(id="_nmk_i", ctx=ast.Load()), ctx=ast.Load()),
+                    node)
+            return node
+
+    import copy
+    expr = Index().visit(copy.deepcopy(stage.expr))
+    params = ["_nmk_n"] + list(stage.inputs)
+    args = ast.arguments(posonlyargs=[], args=[ast.arg(arg=p) for p in params],
+                         kwonlyargs=[], kw_defaults=[], defaults=[])
+    body = [
+        ast.Assign(targets=[ast.Name(id="_nmk_acc", ctx=ast.Store())],
+                   value=ast.Constant(value=0 if integer else 0.0)),
+        ast.For(target=ast.Name(id="_nmk_i", ctx=ast.Store()),
+                iter=ast.Call(func=ast.Name(id="_nmk_prange", ctx=ast.Load()),
+                              args=[ast.Name(id="_nmk_n", ctx=ast.Load())], keywords=[]),
+                body=[ast.AugAssign(target=ast.Name(id="_nmk_acc", ctx=ast.Store()),
+                                    op=ast.Add(), value=expr)],
+                orelse=[]),
+        ast.Return(value=ast.Name(id="_nmk_acc", ctx=ast.Load())),
+    ]
+    fn = ast.FunctionDef(name=name, args=args, body=body, decorator_list=[])
+    for node in [fn] + body:
+        ast.copy_location(node, stage.node)
     module = ast.fix_missing_locations(ast.Module(body=[fn], type_ignores=[]))
     namespace = dict(scope)
     exec(compile(module, f"<stage of {name}>", "exec"), namespace)    # noqa: S102

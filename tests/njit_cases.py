@@ -410,3 +410,24 @@ FLIPS = [
 
 def l2_norm_rows_product(a):
     return np.sqrt(np.sum(a * a, axis=1))
+
+
+# reductions over everything of a map: one pass over the operands
+def frobenius(a, b):
+    return np.sqrt(np.sum((a - b) ** 2))
+
+
+def mean_abs_difference(a, b):
+    return np.mean(np.abs(a - b))
+
+
+def count_greater(a, b):
+    return np.sum(a > b)
+
+
+def sum_of_integer_squares(a):
+    return np.sum(a * a)
+
+
+def weighted_total(a, r):
+    return np.sum(a * r)          # broadcast operands: two stages

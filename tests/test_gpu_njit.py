@@ -656,3 +656,36 @@ def test_affine_into_an_existing_array(env):
     out = hip.asarray(np.zeros((20, 10)))
     njit(affine)(hip.asarray(a), hip.asarray(b), hip.asarray(c), out)
     np.testing.assert_allclose(out.asnumpy(), a @ b + c, rtol=1e-12)
+
+
+def test_maps_run_inside_full_reductions(env):
+    """np.sum / np.mean over everything of an expression of same-shaped dense
+    arrays is one kernel: the map is evaluated inside the reduction loop."""
+    hip = env[0]
+    rng = np.random.default_rng(31)
+    a, b = rng.standard_normal((257, 129)), rng.standard_normal((257, 129))
+
+    def run(func, *host, rtol=1e-12, fused=True):
+        f = njit(func)
+        got = f(*[hip.asarray(h) for h in host])
+        want = func(*host)
+        np.testing.assert_allclose(got, want, rtol=rtol)
+        assert np.asarray(got).dtype == np.asarray(want).dtype, func.__name__
+        marks = [s.get("fused") for s in f.last_launch["stages"]]
+        assert ("map + sum" in marks) == fused, f.last_launch
+        return f
+
+    run(cases.frobenius, a, b)
+    run(cases.mean_abs_difference, a, b)
+    run(cases.count_greater, a, b)
+    a32, b32 = a.astype(np.float32), b.astype(np.float32)
+    run(cases.frobenius, a32, b32, rtol=1e-5)
+    run(cases.mean_abs_difference, a32, b32, rtol=1e-5)
+    ai = rng.integers(-100, 100, (64, 33)).astype(np.int32)
+    run(cases.sum_of_integer_squares, ai)
+    # operands of different shapes take the map and the reduction separately
+    run(cases.weighted_total, a, rng.standard_normal(129), fused=False)
+    # views that are not dense, too
+    f = njit(cases.frobenius)
+    got = f(hip.asarray(a)[::2], hip.asarray(b)[::2])
+    np.testing.assert_allclose(got, cases.frobenius(a[::2], b[::2]), rtol=1e-12)
