@@ -405,18 +405,20 @@ class Dispatcher:
 
     def _compile(self, mode, args, ndim, remap):
         captured = kernel_impl.captured_constants(self.py_func)
-        noalias = hip.disjoint([a for a in args if isinstance(a, HipNdArray)])
+        arrays = [a for a in args if isinstance(a, HipNdArray)]
+        noalias = hip.disjoint(arrays)
+        stream = hip.streams(arrays)
         for specialize in (True, False):
             types = [kernel_compiler.type_of_argument(a, specialize) for a in args]
             key = (mode, ndim, tuple(kernel_compiler.type_key(t) for t in types),
-                   captured, remap, noalias)
+                   captured, remap, noalias, stream)
             compiled = self._compiled.get(key)
             if compiled is not None or len(self._compiled) < kernel_impl.MAX_SPECIALISATIONS:
                 break
         if compiled is None:
             compiled = kernel_compiler.translate(
                 self.py_func, types, ndim, kernel_impl, self.boundscheck, remap, mode,
-                noalias=noalias, elements_per_thread=ELEMENTS_PER_THREAD)
+                noalias=noalias, elements_per_thread=ELEMENTS_PER_THREAD, stream=stream)
             self._compiled[key] = compiled
         return compiled
 

@@ -354,3 +354,16 @@ def disjoint(arrays):
         spans.append((lo, hi + a.dtype.itemsize))
     spans.sort()
     return all(spans[k][1] <= spans[k + 1][0] for k in range(len(spans) - 1))
+
+
+STREAM_BYTES = 128 << 20
+
+
+def streams(arrays):
+    """True when the device arrays of a launch are too large to stay in the
+    256 MiB memory-side cache from one launch to the next: generated kernels
+    then read and write them with streaming accesses."""
+    total = 0
+    for a in arrays:
+        total += a.size * a.dtype.itemsize
+    return total >= STREAM_BYTES

@@ -408,6 +408,8 @@ class FunctionTranslator:
         self.allow_remap = False     # kernels only: see translate_kernel
         self.reversed = False
         self.rows_per_lane = 1
+        self.grid_stride = False
+        self.stream = True           # with noalias: arrays too big to stay cached
         self.written_arrays = set()  # elementwise mode: arrays stored through [:]
         self.read_arrays = set()     # elementwise mode: arrays loaded as values
         self.noalias = False         # no two array arguments overlap (host-checked)
@@ -515,7 +517,11 @@ class FunctionTranslator:
                            "in an elementwise function")
         self.read_arrays.add(arr.code)
         terms = [f"nmk_gid{d} * {arr.code}.stride[{d}]" for d in range(self.ndim)]
-        return Val(f"{arr.code}.p[{' + '.join(terms)}]", arr.type.elem)
+        ref = f"{arr.code}.p[{' + '.join(terms)}]"
+        if self.noalias and self.stream and arr.code not in self.written_arrays:
+            # read once, by this work-item only: no need to keep it cached
+            return Val(f"__builtin_nontemporal_load(&{ref})", arr.type.elem)
+        return Val(ref, arr.type.elem)
 
     def store_here(self, arr_code, elem, value_code):
         """Elementwise mode: the store of this work-item's element.  An array
@@ -523,7 +529,7 @@ class FunctionTranslator:
         past the caches."""
         terms = [f"nmk_gid{d} * {arr_code}.stride[{d}]" for d in range(self.ndim)]
         dst = f"{arr_code}.p[{' + '.join(terms)}]"
-        if self.noalias and arr_code not in self.read_arrays:
+        if self.noalias and self.stream and arr_code not in self.read_arrays:
             last = self.ndim - 1
             # (the returned array is allocated dense by the caller)
             unit = "true" if arr_code == "nmk_ret" else f"{arr_code}.stride[{last}] == 1"
@@ -1234,7 +1240,7 @@ class FunctionTranslator:
         code, elem = rest
         if not isinstance(v.type, Scalar):
             self.err(node, "Only scalars can be stored into an array element")
-        if self.noalias and self.last_elem_gid is not None and \
+        if self.noalias and self.stream and self.last_elem_gid is not None and \
                 isinstance(target.value, ast.Name) and \
                 target.value.id in self.store_only_params():
             # read by nobody in this launch: past the caches when adjacent
@@ -1561,9 +1567,14 @@ class FunctionTranslator:
             params.append(f"{self.ret_type.ctype} *{restrict}nmk_ret_p")
             params += [f"int64_t nmk_ret_s{k}" for k in range(n)]
             params += [f"int64_t nmk_ret_t{k}" for k in range(n)]
+            # (allocated dense by the caller: the strides follow from the
+            # extents, which lets adjacent stores of a lane merge)
+            dense = ["1"] * n
+            for k in range(n - 2, -1, -1):
+                dense[k] = f"{dense[k + 1]} * nmk_ret_s{k + 1}"
             views.append(f"nmkjit::View<{self.ret_type.ctype}, {n}> nmk_ret = {{nmk_ret_p, "
                          f"{{{', '.join(f'nmk_ret_s{k}' for k in range(n))}}}, "
-                         f"{{{', '.join(f'nmk_ret_t{k}' for k in range(n))}}}}};")
+                         f"{{{', '.join(dense)}}}}};")
         # one partial result per block and reduction variable, after the
         # function's own arguments (the host folds them in block order)
         red = []
@@ -1651,37 +1662,58 @@ class FunctionTranslator:
                 "  }",
             ]
         else:
-            if ept > 1:
+            # 1-d loops and maps stride over the iteration space by whole
+            # grids: the launcher may run fewer blocks than cover it (it does
+            # for reductions, whose per-block epilogue then runs once per many
+            # elements).  A lane takes `ept` elements a block apart (each
+            # access of the wave is contiguous on its own); a round that lies
+            # wholly inside the iteration space runs them unguarded, so a
+            # straight-line body has all its loads in flight together.
+            strided = self.ndim == 1 and not self.m.communicates and self.mode != "kernel"
+            self.grid_stride = strided
+            if strided:
                 out += [
-                    "#pragma unroll",
-                    f"  for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep) {{",
-                    f"  const int64_t nmk_gid0 = (nmk_grp0 * {ept} + nmk_rep) * nmk_lsz0 + nmk_lid0;",
                     "  const int64_t nmk_gid1 = 0, nmk_gid2 = 0;",
+                    "  (void)nmk_gid1; (void)nmk_gid2;",
+                    "  auto nmk_item = [&](const int64_t nmk_gid0, auto nmk_guarded) {",
+                    "    if (decltype(nmk_guarded)::value && !(nmk_gid0 < nmk_gsz0)) return;",
+                ] + body + [
+                    "  };",
+                    f"  for (int64_t nmk_round = nmk_grp0; nmk_round * {ept} * nmk_lsz0 < "
+                    "nmk_gsz0; nmk_round += gridDim.x) {",
+                    f"    const int64_t nmk_base = nmk_round * {ept} * nmk_lsz0 + nmk_lid0;",
+                    f"    if ((nmk_round + 1) * {ept} * nmk_lsz0 <= nmk_gsz0) {{",
+                    "#pragma unroll",
+                    f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep)",
+                    "        nmk_item(nmk_base + nmk_rep * nmk_lsz0, nmkjit::No());",
+                    "    } else {",
+                    "#pragma unroll 1",
+                    f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep)",
+                    "        nmk_item(nmk_base + nmk_rep * nmk_lsz0, nmkjit::Yes());",
+                    "    }",
+                    "  }",
                 ]
             else:
                 out += [
                     "  const int64_t nmk_gid0 = nmk_grp0 * nmk_lsz0 + nmk_lid0;",
                     "  const int64_t nmk_gid1 = nmk_grp1 * nmk_lsz1 + nmk_lid1;",
                     "  const int64_t nmk_gid2 = nmk_grp2 * nmk_lsz2 + nmk_lid2;",
+                    "  const bool nmk_active = nmk_gid0 < nmk_gsz0 && nmk_gid1 < nmk_gsz1 && "
+                    "nmk_gid2 < nmk_gsz2;",
                 ]
-            out += [
-                "  const bool nmk_active = nmk_gid0 < nmk_gsz0 && nmk_gid1 < nmk_gsz1 && "
-                "nmk_gid2 < nmk_gsz2;",
-            ]
-            if self.group_sites:
-                out.append("  __shared__ int nmk_clipped;")
-                for slot, t, _ in self.group_sites:
-                    out.append(f"  __shared__ {t.ctype} {slot}[nmkjit::kMaxGroup];")
-                out.append("  if (nmkjit::linearLocalId() == 0) nmk_clipped = 0;")
-                out.append("  __syncthreads();")
-                out.append("  if (!nmk_active) nmk_clipped = 1;")
-                for slot, t, neutral in self.group_sites:
-                    out.append(f"  nmkjit::groupInit<{t.ctype}>({slot}, ({t.ctype}){neutral});")
-                out.append("  __syncthreads();")
-            out.append("  if (nmk_active) {")
-            out += body
-            out.append("  }")
-            if ept > 1:
+                if self.group_sites:
+                    out.append("  __shared__ int nmk_clipped;")
+                    for slot, t, _ in self.group_sites:
+                        out.append(f"  __shared__ {t.ctype} {slot}[nmkjit::kMaxGroup];")
+                    out.append("  if (nmkjit::linearLocalId() == 0) nmk_clipped = 0;")
+                    out.append("  __syncthreads();")
+                    out.append("  if (!nmk_active) nmk_clipped = 1;")
+                    for slot, t, neutral in self.group_sites:
+                        out.append(f"  nmkjit::groupInit<{t.ctype}>({slot}, "
+                                   f"({t.ctype}){neutral});")
+                    out.append("  __syncthreads();")
+                out.append("  if (nmk_active) {")
+                out += body
                 out.append("  }")
         for name, t, _ in red:
             op = "AddOp" if self.reductions[name] == "add" else "MulOp"
@@ -1713,7 +1745,7 @@ class CompiledKernel:
 
 
 def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
-              mode="kernel", noalias=False, elements_per_thread=1):
+              mode="kernel", noalias=False, elements_per_thread=1, stream=True):
     """Python function + argument types -> CompiledKernel (source only).
 
     With ``boundscheck`` every index is tested against its dimension: an
@@ -1729,8 +1761,10 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     function whose top-level prange loop becomes a 1-d grid (``range_source``
     holds the source text of the prange arguments for the host to evaluate).
     ``noalias`` promises that no two array arguments overlap (pointers become
-    ``__restrict__``; arrays the body only stores into are written past the
-    caches).  For the last two modes ``elements_per_thread`` asks for that
+    ``__restrict__``); with ``stream`` as well -- the caller found the arrays
+    too large to stay in the memory-side cache between launches -- arrays the
+    body only stores into are written past the caches and a fused map reads
+    its operands with streaming loads.  For the last two modes ``elements_per_thread`` asks for that
     many elements per lane of a 1-d grid (the result says what it got: the launcher divides the grid
     by it)."""
     module = Module(stubs, boundscheck)
@@ -1738,6 +1772,7 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     tr.allow_remap = remap
     tr.mode = mode
     tr.noalias = noalias
+    tr.stream = stream
     if mode != "kernel":
         tr.elements_per_thread = max(1, int(elements_per_thread))
     if mode == "parallel":
@@ -1755,6 +1790,9 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     # many work-items along hardware y: the launcher divides that grid
     # dimension by it
     compiled.rows_per_lane = tr.rows_per_lane
+    # a 1-d loop or map that strides over its iteration space by whole grids:
+    # any number of blocks computes the same thing
+    compiled.grid_stride = tr.grid_stride
     compiled.ret_dtype = tr.ret_type.dtype if (mode == "elementwise" and tr.ret_type) else None
     compiled.range_source = tr.range_source[1] if tr.range_source else None
     compiled.grid_sources = list(tr.grid_sources)   # per grid dimension

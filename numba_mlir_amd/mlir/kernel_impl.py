@@ -29,7 +29,7 @@ import numpy as np
 from . import kernel_compiler, lowered
 from .gpu_runtime import runtime_lib
 from .utils import readenv
-from .device_array import HipNdArray, disjoint
+from .device_array import HipNdArray, disjoint, streams
 from .kernel_base import KernelBase
 from .lowered import GPUParamDesc, lib
 
@@ -223,6 +223,7 @@ class _ParamList:
 NO_DEPS = (ctypes.c_void_p * 1)(None)
 MAX_SPECIALISATIONS = 16   # per kernel, before new shapes get the general form
 MAX_PLANS = 64             # stored launches per kernel
+REDUCTION_BLOCKS = 2048    # of a generated 1-d reduction: eight per compute unit
 
 
 def _release_handles(handles):
@@ -299,10 +300,11 @@ class Kernel(KernelBase):
         tag = _DTYPE_TAGS.get(first.dtype) if first is not None else None
         return self.twin.format(dtype=tag, rank=len(self.global_size))
 
-    def compile(self, args, ndim, remap=False, noalias=False):
+    def compile(self, args, ndim, remap=False, noalias=False, stream=True):
         """The specialisation of the body for these arguments (translated on
         first use; constants captured by the body are part of the key).
-        ``noalias``: the caller found no two array arguments overlapping."""
+        ``noalias``: the caller found no two array arguments overlapping;
+        ``stream``: they are too large to stay cached between launches."""
         import sys
         # Specialised on dense layouts and short trailing extents; a kernel
         # that keeps meeting new ones gets the general form for the rest.
@@ -310,7 +312,7 @@ class Kernel(KernelBase):
         for specialize in (True, False):
             types = [kernel_compiler.type_of_argument(a, specialize) for a in args]
             key = (ndim, tuple(kernel_compiler.type_key(t) for t in types),
-                   captured, self.boundscheck, remap, noalias)
+                   captured, self.boundscheck, remap, noalias, stream)
             compiled = self._compiled.get(key)
             if compiled is not None or len(self._compiled) < MAX_SPECIALISATIONS:
                 break
@@ -318,7 +320,7 @@ class Kernel(KernelBase):
             compiled = kernel_compiler.translate(self.py_func, types, ndim,
                                                  sys.modules[__name__],
                                                  self.boundscheck, remap,
-                                                 noalias=noalias)
+                                                 noalias=noalias, stream=stream)
             self._compiled[key] = compiled
         return compiled
 
@@ -356,11 +358,12 @@ class Kernel(KernelBase):
             # grouping is laid out for coalescing (last dimension on x), unless
             # that pushes a long dimension past the y / z grid limit.
             remap = len(self.local_size) == 0 and ndim > 1
-            compiled = self.compile(args, ndim, remap, noalias)
+            stream = streams([a for a in args if isinstance(a, HipNdArray)])
+            compiled = self.compile(args, ndim, remap, noalias, stream)
             kern = _loaded_kernel(ctx, compiled)
             block, grid = _geometry(ctx, compiled, kern, gsize3[:ndim], self.local_size)
             if compiled.reversed_dims and max(grid[1:]) > 65535:
-                compiled = self.compile(args, ndim, False, noalias)
+                compiled = self.compile(args, ndim, False, noalias, stream)
                 kern = _loaded_kernel(ctx, compiled)
                 block, grid = _geometry(ctx, compiled, kern, gsize3[:ndim],
                                         self.local_size)
@@ -465,11 +468,29 @@ class LaunchPlan:
         self._lock = threading.Lock()     # slots are rewritten per call
         self._launch = (ctx.queue, kern, *self.grid, *self.block, NO_DEPS, self._descs)
 
-    def enqueue(self):
-        """Launches with the slots as they are and returns the event without
-        waiting (the caller passes it to ``retire``): back-to-back launches
-        for timing."""
-        return runtime_lib.gpuxLaunchKernel(*self._launch)
+    def _refresh(self, args, ret, partials):
+        """Rewrites the pointer and scalar slots (the lock is held)."""
+        for slot, a in zip(self._arg_slots, args):
+            if isinstance(a, HipNdArray):
+                slot.value = a.ptr
+            elif isinstance(a, slice):
+                for part_slot, part in zip(slot, (a.start, a.stop, a.step)):
+                    part_slot.value = (_ParamList.SLICE_NONE if part is None
+                                       else int(part))
+            else:
+                slot.value = a.item() if isinstance(a, np.generic) else a
+        if ret is not None:
+            self._ret_slot.value = ret.ptr
+        for slot, part in zip(self._partial_slots, partials):
+            slot.value = part.ptr
+
+    def enqueue(self, args=None, ret=None):
+        """Launches without waiting and returns the event (the caller passes
+        it to ``retire``): back-to-back launches for timing."""
+        with self._lock:                  # the launch call copies the values out
+            if args is not None:
+                self._refresh(args, ret, ())
+            return runtime_lib.gpuxLaunchKernel(*self._launch)
 
     def retire(self, event):
         queue = self.ctx.queue
@@ -484,19 +505,7 @@ class LaunchPlan:
         queue = self.ctx.queue
         with self._lock:                  # the launch call copies the values out
             if args is not None:
-                for slot, a in zip(self._arg_slots, args):
-                    if isinstance(a, HipNdArray):
-                        slot.value = a.ptr
-                    elif isinstance(a, slice):
-                        for part_slot, part in zip(slot, (a.start, a.stop, a.step)):
-                            part_slot.value = (_ParamList.SLICE_NONE if part is None
-                                               else int(part))
-                    else:
-                        slot.value = a.item() if isinstance(a, np.generic) else a
-                if ret is not None:
-                    self._ret_slot.value = ret.ptr
-                for slot, part in zip(self._partial_slots, partials):
-                    slot.value = part.ptr
+                self._refresh(args, ret, partials)
             event = runtime_lib.gpuxLaunchKernel(*self._launch)
         runtime_lib.gpuxWait(queue, event)
         runtime_lib.gpuxDestroyEvent(queue, event)
@@ -532,6 +541,9 @@ def plan_compiled(ctx, compiled, func_name, global_size, args, ret=None,
     per_lane = getattr(compiled, "elements_per_thread", 1)
     lanes = [-(-int(global_size[0]) // per_lane)] + [int(g) for g in global_size[1:]]
     block, grid = _geometry(ctx, compiled, kern, lanes, ())
+    if make_partials and getattr(compiled, "grid_stride", False):
+        # a reduction: few, long-running blocks (one partial result each)
+        grid[0] = min(grid[0], REDUCTION_BLOCKS)
     gsize3 = [int(g) for g in global_size] + [1] * (3 - len(global_size))
     partials = make_partials(grid[0] * grid[1] * grid[2]) if make_partials else ()
     return LaunchPlan(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret,

@@ -309,11 +309,17 @@ def test_fused_maps_take_several_elements_per_lane(K, tmp_path, monkeypatch):
                       noalias=True, elements_per_thread=4)
     assert ck.elements_per_thread == 4
     assert "for (int nmk_rep = 0; nmk_rep < 4; ++nmk_rep)" in ck.source
+    assert "nmk_item(nmk_base + nmk_rep * nmk_lsz0, nmkjit::No());" in ck.source
     assert "float *__restrict__ v_price_p" in ck.source
     # call and put are only written: streamed
     assert ck.source.count("NMK_STORE_ALONG0(&") == 2
     assert "#define NMK_STORE_ALONG0(p, v, unit) nmkjit::streamStore(p, v, unit)" in ck.source
     assert kc.build_code_object(ck)[:4] == b"\x7fELF"
+    # operands are read with streaming loads
+    assert "__builtin_nontemporal_load(&v_P.p[" in ck.source
+    small = kc.translate(njit_cases.black_scholes_arrays, types, ndim, K, mode=mode,
+                         noalias=True, elements_per_thread=4, stream=False)
+    assert "nontemporal" not in small.source and "NMK_STORE_ALONG0(&" not in small.source
     # overlapping arguments: plain pointers and stores
     ck = kc.translate(njit_cases.black_scholes_arrays, types, ndim, K, mode=mode,
                       noalias=False, elements_per_thread=4)
@@ -370,6 +376,10 @@ def test_kernels_stream_stores_nobody_reads_back(K):
     # as written (dimension 0 on x) lanes write a column apart: plain stores
     src = source_of(K, pairwise, [f64_2d] * 3, ndim=2, remap=False, noalias=True)
     assert "NMK_STORE_ALONG1(&v_D.p[" in src and stream(src) == [0]
+    # arrays small enough to stay cached between launches: ordinary stores
+    src = source_of(K, pairwise, [f64_2d] * 3, ndim=2, remap=True, noalias=True,
+                    stream=False)
+    assert "NMK_STORE_ALONG1(&" not in src and "double *__restrict__ v_D_p" in src
     # arguments that may overlap: nothing changes
     src = source_of(K, pairwise, [f64_2d] * 3, ndim=2, remap=True)
     assert "NMK_STORE_ALONG1(&" not in src and "__restrict__" not in src
