@@ -689,3 +689,41 @@ def test_maps_run_inside_full_reductions(env):
     f = njit(cases.frobenius)
     got = f(hip.asarray(a)[::2], hip.asarray(b)[::2])
     np.testing.assert_allclose(got, cases.frobenius(a[::2], b[::2]), rtol=1e-12)
+
+
+def test_concurrent_calls_from_python_threads(env):
+    """Compiled functions are called from Python threads holding no lock of
+    the runtime (GpuRuntime.cpp:275-300 pools events per queue): calls of one
+    function on different arrays from several threads must not mix up the
+    stored launch's pointer and scalar slots."""
+    import threading
+    hip = env[0]
+    f = njit(cases.fused_map)
+    g = njit(parallel=True)(cases.saxpy_loop)
+    rng = np.random.default_rng(41)
+    n, rounds, errors = 4096, 40, []
+    f(*(hip.asarray(rng.standard_normal(n)) for _ in range(3)), 1.0)       # compile once
+    g(1.0, hip.asarray(np.zeros(n)), hip.asarray(np.zeros(n)), hip.asarray(np.zeros(n)))
+
+    def worker(seed):
+        try:
+            local = np.random.default_rng(seed)
+            for k in range(rounds):
+                a, b, c = (local.standard_normal(n) for _ in range(3))
+                scale = float(seed + k)
+                got = f(hip.asarray(a), hip.asarray(b), hip.asarray(c), scale).asnumpy()
+                # (sin differs in the last place and t*t - t cancels)
+                np.testing.assert_allclose(got, cases.fused_map(a, b, c, scale), rtol=1e-9,
+                                           atol=1e-9)
+                out = hip.asarray(np.zeros(n))
+                g(scale, hip.asarray(a), hip.asarray(b), out)
+                np.testing.assert_array_equal(out.asnumpy(), scale * a + b)
+        except Exception as exc:          # noqa: BLE001 -- reported by the main thread
+            errors.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(s,)) for s in range(6)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors[0]
