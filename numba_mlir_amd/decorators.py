@@ -419,6 +419,8 @@ class Dispatcher:
             compiled = kernel_compiler.translate(
                 self.py_func, types, ndim, kernel_impl, self.boundscheck, remap, mode,
                 noalias=noalias, elements_per_thread=ELEMENTS_PER_THREAD, stream=stream)
+            # njit(fastmath=True): multiply-adds may fuse
+            compiled.fastmath = bool(self.options.get("fastmath", False))
             self._compiled[key] = compiled
         return compiled
 
@@ -628,7 +630,7 @@ class Dispatcher:
             func, params = staging.stage_function(
                 stage, f"{self.py_func.__name__}_stage{k}", scope)
             entry = self._stage_funcs[key] = (
-                Dispatcher(func, boundscheck=self.boundscheck), params)
+                Dispatcher(func, boundscheck=self.boundscheck, **self.options), params)
         sub, params = entry
         value = sub._run([env[p] for p in params])
         launches.append(sub.last_launch)
@@ -670,7 +672,8 @@ class Dispatcher:
                 func, params = staging.reduction_function(
                     source, f"{self.py_func.__name__}_stage{k}_sum", namespace, set(arrays),
                     integer)
-                entry = (Dispatcher(func, parallel=True, boundscheck=self.boundscheck), params)
+                entry = (Dispatcher(func, parallel=True, boundscheck=self.boundscheck,
+                                    **self.options), params)
             except kernel_compiler.KernelCompileError:
                 entry = False
             self._stage_funcs[key] = entry

@@ -1894,7 +1894,12 @@ def build_code_object(compiled):
         with open(os.path.join(_KERNELS_DIR, header), "rb") as f:
             support += f.read()
     digest = hashlib.sha256()
-    for part in (compiled.source.encode(), support, " ".join(_FLAGS).encode()):
+    flags = list(_FLAGS)
+    if getattr(compiled, "fastmath", False):
+        # fastmath=True (reference: test_gpu.py:980-1008 expects a * b + c to
+        # become one fma): contraction only, no value-changing shortcuts
+        flags[flags.index("-ffp-contract=off")] = "-ffp-contract=fast"
+    for part in (compiled.source.encode(), support, " ".join(flags).encode()):
         digest.update(part)
     key = digest.hexdigest()[:24]
     os.makedirs(CACHE_DIR, exist_ok=True)
@@ -1904,7 +1909,7 @@ def build_code_object(compiled):
         with open(src, "w") as f:
             f.write(compiled.source)
         tmp = obj + f".tmp{os.getpid()}"
-        proc = subprocess.run([_hipcc(), *_FLAGS, f"-I{_KERNELS_DIR}", "-o", tmp, src],
+        proc = subprocess.run([_hipcc(), *flags, f"-I{_KERNELS_DIR}", "-o", tmp, src],
                               capture_output=True, text=True)
         if proc.returncode != 0:
             raise KernelCompileError(

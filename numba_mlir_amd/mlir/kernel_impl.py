@@ -241,12 +241,13 @@ def _loaded_kernel(ctx, compiled):
         table = ctx._jit_kernels = {}
         ctx._jit_handles = []
         weakref.finalize(ctx, _release_handles, ctx._jit_handles)
-    kern = table.get(compiled.name)
+    key = (compiled.name, getattr(compiled, "fastmath", False))
+    kern = table.get(key)
     if kern is None:
         blob = kernel_compiler.build_code_object(compiled)
         module = runtime_lib.gpuxModuleLoad(ctx.queue, blob, len(blob))
         kern = runtime_lib.gpuxKernelGet(module, compiled.name.encode())
-        table[compiled.name] = kern
+        table[key] = kern
         ctx._jit_handles.append((kern, module))
     return kern
 
@@ -290,6 +291,9 @@ class Kernel(KernelBase):
         # launch instead of reading or writing foreign memory.
         self.boundscheck = bool(kwargs.get(
             "boundscheck", readenv("NUMBA_MLIR_KERNEL_BOUNDSCHECK", int, 0)))
+        # fastmath=True lets a * b + c contract into one fused multiply-add
+        # (the reference's kernel(fastmath=True), test_gpu.py:980-1008)
+        self.fastmath = bool(kwargs.get("fastmath", False))
         self.last_launch = None
         self.last_plan = None  # the LaunchPlan of the most recent compiled launch
         self._compiled = {}
@@ -321,6 +325,7 @@ class Kernel(KernelBase):
                                                  sys.modules[__name__],
                                                  self.boundscheck, remap,
                                                  noalias=noalias, stream=stream)
+            compiled.fastmath = self.fastmath
             self._compiled[key] = compiled
         return compiled
 

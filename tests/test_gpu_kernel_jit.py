@@ -363,6 +363,29 @@ def test_fastmath_off_keeps_two_roundings(env):              # 980-1008
         assert out[3].tobytes() == (a * b + c).tobytes()
 
 
+def test_fastmath_fuses_multiply_add(env):                   # 980-1008
+    """kernel(fastmath=True): the reference expects exactly one fma for
+    a * b + c.  A fused result is the exact product plus c rounded once."""
+    hip = env[0]
+
+    def func(a, b, c, res):
+        i = get_global_id(0)
+        res[i] = a[i] * b[i] + c[i]
+
+    rng = np.random.default_rng(3)
+    a = rng.uniform(1, 2, 4096).astype(np.float32)
+    b = rng.uniform(1, 2, 4096).astype(np.float32)
+    c = (-(a.astype(np.float64) * b)).astype(np.float32)       # cancels the leading bits
+    dev = [hip.asarray(x) for x in (a, b, c)]
+    fused, plain = hip.asarray(np.zeros_like(a)), hip.asarray(np.zeros_like(a))
+    K.kernel(func, fastmath=True)[a.shape, ()](*dev, fused)
+    K.kernel(func, fastmath=False)[a.shape, ()](*dev, plain)
+    exact = (a.astype(np.float64) * b + c).astype(np.float32)  # the product is exact in double
+    assert fused.asnumpy().tobytes() == exact.tobytes()
+    assert plain.asnumpy().tobytes() == (a * b + c).tobytes()
+    assert (fused.asnumpy() != plain.asnumpy()).any()
+
+
 def test_accumulation_in_float32(env):                       # 1011-1040
     def func(a, b, res):
         i = get_global_id(0)
