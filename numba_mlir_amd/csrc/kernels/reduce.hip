@@ -1,5 +1,5 @@
-// Reductions for gfx950: axis sums, full sum-of-squares norm, and a generic
-// strided fallback for sum/prod/min/max.
+// Reductions for gfx950: axis sums, full sum-of-squares norm, and generic
+// kernels for sum/prod/min/max of every type (strided, column-wise, chunked).
 //
 // They replace what the reference generates from a linalg.generic with
 // `reduction` iterators (reference: numba_mlir/numba_mlir/mlir/numpy/funcs.py:163-229).
@@ -322,12 +322,97 @@ reduceStrided(const IN *x, ACC *out, int64_t nKeep, int64_t nRed, int64_t sk,
     out[k * so] = acc;
 }
 
+// Generic reduction over the slow axis of a matrix whose kept index has unit
+// stride (column sums of a row-major matrix, row sums of a column-major one):
+// out[chunk * nKeep + k] = fold_{r in chunk} op(x[r * ld + k]).  A block owns
+// 256 consecutive kept indices (adjacent lanes read adjacent elements) and one
+// chunk of rowsPerChunk reduced indices, eight loads in flight per lane; with
+// more than one chunk the same kernel folds the partial results.
+template <typename IN, typename ACC, typename Op>
+__device__ __forceinline__ void
+reduceColumns(const IN *__restrict__ x, ACC *__restrict__ out, int64_t nRed,
+              int64_t nKeep, int64_t ld, int64_t rowsPerChunk, ACC init, Op op) {
+  const int64_t k = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (k >= nKeep)
+    return;
+  int64_t r = int64_t(blockIdx.y) * rowsPerChunk;
+  int64_t rEnd = r + rowsPerChunk;
+  if (rEnd > nRed)
+    rEnd = nRed;
+  const IN *p = x + r * ld + k;
+  ACC a[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u)
+    a[u] = init;
+  for (; r + 8 <= rEnd; r += 8) {
+    IN v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      v[u] = p[u * ld];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      a[u] = op(a[u], ACC(v[u]));
+    p += 8 * ld;
+  }
+  for (; r < rEnd; ++r) {
+    a[0] = op(a[0], ACC(*p));
+    p += ld;
+  }
+  out[int64_t(blockIdx.y) * nKeep + k] =
+      op(op(op(a[0], a[1]), op(a[2], a[3])), op(op(a[4], a[5]), op(a[6], a[7])));
+}
+
+// Generic reduction of a long contiguous run in chunks: out[c] = fold of
+// x[c * chunk .. min(n, (c + 1) * chunk)), one wave per chunk, four loads in
+// flight per lane.  A full reduction is this kernel followed by the strided
+// one over the partial results.
+template <typename IN, typename ACC, typename Op>
+__device__ __forceinline__ void
+reduceChunks(const IN *__restrict__ x, ACC *__restrict__ out, int64_t n,
+             int64_t chunk, int64_t nChunks, ACC init, Op op) {
+  const int lane = threadIdx.x % NMK_WAVE;
+  const int64_t c =
+      int64_t(blockIdx.x) * (blockDim.x / NMK_WAVE) + threadIdx.x / NMK_WAVE;
+  if (c >= nChunks)
+    return;
+  int64_t i = c * chunk + lane;
+  int64_t end = (c + 1) * chunk;
+  if (end > n)
+    end = n;
+  ACC a0 = init, a1 = init, a2 = init, a3 = init;
+  for (; i + 3 * NMK_WAVE < end; i += 4 * NMK_WAVE) {
+    const IN v0 = x[i], v1 = x[i + NMK_WAVE], v2 = x[i + 2 * NMK_WAVE],
+             v3 = x[i + 3 * NMK_WAVE];
+    a0 = op(a0, ACC(v0));
+    a1 = op(a1, ACC(v1));
+    a2 = op(a2, ACC(v2));
+    a3 = op(a3, ACC(v3));
+  }
+  for (; i < end; i += NMK_WAVE)
+    a0 = op(a0, ACC(x[i]));
+  ACC acc = waveAllReduce(op(op(a0, a1), op(a2, a3)), op);
+  if (lane == 0)
+    out[c] = acc;
+}
+
 #define NMK_DEFINE_REDUCE(OPNAME, OP, INIT, TNAME, IN, ACC)                    \
   NMK_KERNEL(256)                                                              \
   nmk_reduce_##OPNAME##_##TNAME(const IN *x, ACC *out, int64_t nKeep,          \
                                 int64_t nRed, int64_t sk, int64_t sr,          \
                                 int64_t so) {                                  \
     reduceStrided<IN, ACC>(x, out, nKeep, nRed, sk, sr, so, ACC(INIT), OP());  \
+  }                                                                            \
+  NMK_KERNEL(256)                                                              \
+  nmk_reducecols_##OPNAME##_##TNAME(const IN *x, ACC *out, int64_t nRed,       \
+                                    int64_t nKeep, int64_t ld,                 \
+                                    int64_t rowsPerChunk) {                    \
+    reduceColumns<IN, ACC>(x, out, nRed, nKeep, ld, rowsPerChunk, ACC(INIT),   \
+                           OP());                                              \
+  }                                                                            \
+  NMK_KERNEL(256)                                                              \
+  nmk_reducechunks_##OPNAME##_##TNAME(const IN *x, ACC *out, int64_t n,        \
+                                      int64_t chunk, int64_t nChunks) {        \
+    reduceChunks<IN, ACC>(x, out, n, chunk, nChunks, ACC(INIT), OP());         \
   }
 
 NMK_DEFINE_REDUCE(sum, AddOp, 0, i32, int32_t, int64_t)

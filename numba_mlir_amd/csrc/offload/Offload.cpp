@@ -192,14 +192,14 @@ const Blob *findBlob(const char *family) {
 
 // Kernel name -> family.  Names are prefixed by family:
 //   nmk_map2_*, nmk_black_scholes_*, nmk_fill_* : maps
-//   nmk_sum_*, nmk_norm2_*, nmk_reduce_*        : reduce
+//   nmk_sum_*, nmk_norm2_*, nmk_reduce*         : reduce
 //   nmk_twin_*                                  : twins
 const char *familyOf(const std::string &kernel) {
   auto starts = [&](const char *p) { return kernel.rfind(p, 0) == 0; };
   if (starts("nmk_map2_") || starts("nmk_black_scholes_") ||
       starts("nmk_fill_") || starts("nmk_copy_"))
     return "maps";
-  if (starts("nmk_sum_") || starts("nmk_norm2_") || starts("nmk_reduce_"))
+  if (starts("nmk_sum_") || starts("nmk_norm2_") || starts("nmk_reduce"))
     return "reduce";
   if (starts("nmk_twin_"))
     return "twins";
@@ -713,6 +713,60 @@ NMHIP_EXPORT void nmhipReduce(void *ctx, int op, int dtype, const void *x,
     }
     if (nKeep == 0)
       return;
+    const std::string opAndType = std::string(opNames[op]) + "_" + dtypeName(dtype);
+    // the accumulator type's own kernels fold partial results
+    const bool isInt = dtype == NMHIP_I32 || dtype == NMHIP_I64;
+    const std::string opAndAcc =
+        std::string(opNames[op]) + "_" + (isInt ? "i64" : dtypeName(dtype));
+    const size_t accSize = dtype == NMHIP_F32 ? 4 : 8;
+    // The kept index has unit stride (column sums of a row-major matrix):
+    // lanes along the kept index, row chunks over grid.y, partial results
+    // folded by the same kernel.
+    if (sk == 1 && nKeep > 1 && nRed >= 64 && sr >= nKeep) {
+      const int64_t strips = ceilDiv(nKeep, 256);
+      int64_t chunks = ceilDiv(2048, strips);
+      if (chunks > nRed / 32)
+        chunks = nRed / 32;
+      if (chunks < 1)
+        chunks = 1;
+      if (chunks > 65535)
+        chunks = 65535;
+      const int64_t rowsPerChunk = ceilDiv(nRed, chunks);
+      chunks = ceilDiv(nRed, rowsPerChunk);
+      if (chunks == 1) {
+        c->launch("nmk_reducecols_" + opAndType, size_t(strips), 1, 1, 256, 1, 1,
+                  {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(nRed), Arg::I64(nKeep),
+                   Arg::I64(sr), Arg::I64(nRed)});
+      } else {
+        void *partial = c->scratchFor(size_t(chunks) * size_t(nKeep) * accSize);
+        c->launch("nmk_reducecols_" + opAndType, size_t(strips), size_t(chunks), 1,
+                  256, 1, 1,
+                  {Arg::Ptr(x), Arg::Ptr(partial), Arg::I64(nRed), Arg::I64(nKeep),
+                   Arg::I64(sr), Arg::I64(rowsPerChunk)});
+        c->launch("nmk_reducecols_" + opAndAcc, size_t(strips), 1, 1, 256, 1, 1,
+                  {Arg::Ptr(partial), Arg::Ptr(out), Arg::I64(chunks),
+                   Arg::I64(nKeep), Arg::I64(nKeep), Arg::I64(chunks)});
+      }
+      return;
+    }
+    // A long contiguous run reduced to one value: a wave per chunk, then the
+    // chunks' results by one wave.
+    if (nKeep == 1 && sr == 1 && nRed >= 65536) {
+      int64_t nChunks = ceilDiv(nRed, 8192);
+      if (nChunks > 4096)
+        nChunks = 4096;
+      const int64_t chunk = ceilDiv(nRed, nChunks);
+      nChunks = ceilDiv(nRed, chunk);
+      void *partial = c->scratchFor(size_t(nChunks) * accSize);
+      c->launch("nmk_reducechunks_" + opAndType, size_t(ceilDiv(nChunks, 4)), 1, 1,
+                256, 1, 1,
+                {Arg::Ptr(x), Arg::Ptr(partial), Arg::I64(nRed), Arg::I64(chunk),
+                 Arg::I64(nChunks)});
+      c->launch("nmk_reduce_" + opAndAcc, 1, 1, 1, 256, 1, 1,
+                {Arg::Ptr(partial), Arg::Ptr(out), Arg::I64(1), Arg::I64(nChunks),
+                 Arg::I64(0), Arg::I64(1), Arg::I64(1)});
+      return;
+    }
     c->launch(std::string("nmk_reduce_") + opNames[op] + "_" + dtypeName(dtype),
               size_t(ceilDiv(nKeep, 4)), 1, 1, 256, 1, 1,
               {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(nKeep), Arg::I64(nRed),

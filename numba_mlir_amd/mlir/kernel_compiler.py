@@ -173,6 +173,7 @@ class Val:
         self.pyobj = pyobj            # a Python object known at compile time
         self.slice_parts = slice_parts  # (start, stop, step) Vals or None each
         self.gid = None               # k: the value is global id k plus a constant
+        self.arr = False              # elementwise mode: computed from array elements
 
 
 class _Deferred(Exception):
@@ -441,6 +442,10 @@ class FunctionTranslator:
         # ... and one bound once, at the top level, to a global id (plus a
         # constant) is known to run along that grid dimension
         self.gid_vars = {}
+        # elementwise mode: names that hold values computed from array
+        # elements (they follow the array typing rules, see arith_type)
+        self.array_valued = set()
+        self.array_reads = 0         # how many such values expressions have read so far
         self.top_level = {id(s) for s in body}
         return names - set(self.params)
 
@@ -464,6 +469,8 @@ class FunctionTranslator:
                     return constant(_convert_const(self.const_vars[name], t), t)
                 v = Val(self.cname(name), t, nonneg=name in self.nonneg_vars)
                 v.gid = self.gid_vars.get(name)
+                v.arr = name in self.array_valued
+                self.array_reads += v.arr
                 return v
             if isinstance(t, Array):
                 return Val(self.cname(name), t)
@@ -499,7 +506,11 @@ class FunctionTranslator:
         method = getattr(self, "expr_" + type(node).__name__, None)
         if method is None:
             self.err(node, f"Unsupported expression: {type(node).__name__}")
-        return method(node)
+        reads = self.array_reads
+        v = method(node)
+        if self.array_reads > reads and isinstance(v, Val) and isinstance(v.type, Scalar):
+            v.arr = True          # some operand was computed from array elements
+        return v
 
     def scalar(self, node):
         v = self.expr(node)
@@ -520,8 +531,11 @@ class FunctionTranslator:
         ref = f"{arr.code}.p[{' + '.join(terms)}]"
         if self.noalias and self.stream and arr.code not in self.written_arrays:
             # read once, by this work-item only: no need to keep it cached
-            return Val(f"__builtin_nontemporal_load(&{ref})", arr.type.elem)
-        return Val(ref, arr.type.elem)
+            ref = f"__builtin_nontemporal_load(&{ref})"
+        v = Val(ref, arr.type.elem)
+        v.arr = True
+        self.array_reads += 1
+        return v
 
     def store_here(self, arr_code, elem, value_code):
         """Elementwise mode: the store of this work-item's element.  An array
@@ -645,14 +659,34 @@ class FunctionTranslator:
             left = right
         return Val("(" + " && ".join(parts) + ")", BOOL)
 
-    def arith_type(self, a, b):
+    def arith_type(self, a, b, arrays=False):
+        """Result type of arithmetic on types ``a`` and ``b``.  Between values
+        computed from array elements (``arrays``) a float meeting an integer
+        keeps its own width, as the reference's array operators do
+        (_select_float_type, numpy/funcs.py:402-418: float32 array * 2 and
+        float32 array + int array are float32); scalars follow Numba's scalar
+        rules (numpy.promote_types)."""
+        if arrays and a is not b:
+            if a.is_float and not b.is_float:
+                return a
+            if b.is_float and not a.is_float:
+                return b
         t = promote(a, b)
         return INT64 if t.is_bool else t
+
+    def common_type(self, a, b):
+        """The type two alternatives (of a selection, a minimum ...) share."""
+        if (a.arr or b.arr) and a.type is not b.type:
+            if a.type.is_float and not b.type.is_float:
+                return a.type
+            if b.type.is_float and not a.type.is_float:
+                return b.type
+        return promote(a.type, b.type)
 
     def expr_IfExp(self, node):
         c = self.truth(self.scalar(node.test))
         a, b = self.scalar(node.body), self.scalar(node.orelse)
-        t = promote(a.type, b.type)
+        t = self.common_type(a, b)
         return Val(f"({c.code} ? {cast(a, t).code} : {cast(b, t).code})", t,
                    nonneg=a.nonneg and b.nonneg)
 
@@ -660,7 +694,12 @@ class FunctionTranslator:
         return self.binop(node.op, self.scalar(node.left), self.scalar(node.right), node)
 
     def binop(self, op, a, b, node):
-        t = self.arith_type(a.type, b.type)
+        v = self._binop(op, a, b, node)
+        v.arr = a.arr or b.arr
+        return v
+
+    def _binop(self, op, a, b, node):
+        t = self.arith_type(a.type, b.type, a.arr or b.arr)
         if isinstance(op, ast.Div):
             if not t.is_float:
                 t = FLOAT64
@@ -669,6 +708,15 @@ class FunctionTranslator:
         if isinstance(op, ast.Pow):
             if t.is_float:
                 x, y = cast(a, t), cast(b, t)
+                if b.const is not None and not isinstance(b.const, bool) and \
+                        b.const in (1, 2, 3, 4) and a.const is None:
+                    # a small whole power is a product (as NumPy evaluates x ** 2)
+                    self.m.counter += 1
+                    tmp = f"nmk_pw{self.m.counter}"
+                    chain = {1: "{0}", 2: "{0} * {0}", 3: "{0} * {0} * {0}",
+                             4: "({0} * {0}) * ({0} * {0})"}[int(b.const)].format(tmp)
+                    return Val(f"([&] {{ const {t.ctype} {tmp} = {x.code}; return {chain}; }}())",
+                               t, nonneg=int(b.const) % 2 == 0 or a.nonneg)
                 return Val(f"pow({x.code}, {y.code})", t)
             x, y = cast(a, t), cast(b, t)
             return Val(f"nmkjit::powInt<{t.ctype}>({x.code}, {y.code})", t,
@@ -854,7 +902,7 @@ class FunctionTranslator:
             is_min = obj is min or obj is np.minimum
             acc = vals[0]
             for v in vals[1:]:
-                t = promote(acc.type, v.type)
+                t = self.common_type(acc, v)
                 a, b = cast(acc, t), cast(v, t)
                 cmp = "<" if is_min else ">"
                 # Python keeps the first of equal arguments
@@ -916,7 +964,10 @@ class FunctionTranslator:
             # min(a_max, max(a, a_min)) in the operands' common type
             # (reference: numpy/funcs.py:571-578)
             a, lo, hi = (self.scalar(x) for x in node.args)
-            t = self.arith_type(promote(a.type, lo.type), hi.type)
+            t = self.common_type(a, lo)
+            t = self.common_type(Val("", t), hi) if not (a.arr or lo.arr) else \
+                self.arith_type(t, hi.type, True)
+            t = INT64 if t.is_bool else t
             a, lo, hi = cast(a, t), cast(lo, t), cast(hi, t)
             # (a NaN element stays NaN, as in NumPy)
             inner = f"({a.code} < {lo.code} ? {lo.code} : {a.code})"
@@ -924,7 +975,7 @@ class FunctionTranslator:
                        nonneg=hi.nonneg and (a.nonneg or lo.nonneg))
         if (mod == "math" or is_np) and name in _BINARY_MATH and len(node.args) == 2:
             a, b = self.scalar(node.args[0]), self.scalar(node.args[1])
-            t = promote(a.type, b.type)
+            t = self.common_type(a, b)
             t = t if t.is_float else FLOAT64
             return Val(f"{_BINARY_MATH[name]}({cast(a, t).code}, {cast(b, t).code})", t)
         if mod == "math" and name in ("isnan", "isinf", "isfinite") or \
@@ -936,7 +987,7 @@ class FunctionTranslator:
         if is_np and name == "where" and len(node.args) == 3:
             c = self.truth(self.scalar(node.args[0]))
             a, b = self.scalar(node.args[1]), self.scalar(node.args[2])
-            t = promote(a.type, b.type)
+            t = self.common_type(a, b)
             return Val(f"({c.code} ? {cast(a, t).code} : {cast(b, t).code})", t,
                        nonneg=a.nonneg and b.nonneg)
         if is_np and name == "square" and len(node.args) == 1:
@@ -1207,6 +1258,9 @@ class FunctionTranslator:
         if v.type is None:
             self.err(node, "This value cannot be assigned to a variable")
         self.bind(name, v.type, node)
+        if v.arr and name not in self.array_valued:
+            self.array_valued.add(name)
+            self.changed = True
         if isinstance(v.type, Scalar):
             if (v.const is not None and self.store_count.get(name) == 1 and
                     id(node) in self.top_level and name not in self.params):

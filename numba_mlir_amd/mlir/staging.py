@@ -278,9 +278,10 @@ class Plan:
         self._mark_fused_reductions()
 
     def _mark_fused_reductions(self):
-        """np.sum / np.mean over everything of an expression materialised
-        just for it: the map can run inside the reduction (one pass over the
-        operands instead of a pass, a temporary and a second pass).  The map
+        """np.sum / np.mean -- over everything, or along an axis of a matrix --
+        of an expression materialised just for it: the map can run inside the
+        reduction (one pass over the operands instead of a pass, a temporary
+        and a second pass).  The map
         stage is marked ``deferred`` and the library stage gets it as
         ``fused_map``; the executor falls back to the two stages when the
         operands do not all have one dense shape."""
@@ -300,7 +301,8 @@ class Plan:
                             uses[n.id] = uses.get(n.id, 0) + 2
         for before, stage in zip(self.stages, self.stages[1:]):
             if stage.kind == "lib" and stage.op in ("sum", "mean") and \
-                    stage.kwargs.get("axis") is None and before.kind == "map" and \
+                    stage.kwargs.get("axis") in (None, 0, 1, -1, -2) and \
+                    before.kind == "map" and \
                     before.target == stage.operands[0] and \
                     before.target.startswith("_nmk_t") and uses.get(before.target) == 1 and \
                     not isinstance(before.expr, ast.Name):
@@ -392,3 +394,117 @@ def reduction_function(stage, name, scope, arrays, integer):
     func = namespace[name]
     func.__nmk_ast__ = fn
     return func, params
+
+
+def _indexed(expr, arrays, index):
+    """``expr`` with every array name replaced by its element at ``index``
+    (a list of expression nodes)."""
+    import copy
+
+    class Index(ast.NodeTransformer):
+        def visit_Name(self, node):
+            if node.id in arrays and isinstance(node.ctx, ast.Load):
+                sub = ast.Tuple(elts=[copy.deepcopy(i) for i in index], ctx=ast.Load()) \
+                    if len(index) > 1 else copy.deepcopy(index[0])
+                return ast.copy_location(
+                    ast.Subscript(value=node, slice=sub, ctx=ast.Load()), node)
+            return node
+
+    return Index().visit(copy.deepcopy(expr))
+
+
+def _function(name, params, body_source, exprs, stage, scope):
+    """Parses ``body_source`` (with the placeholders NMK_EXPR0, NMK_EXPR1, ...
+    where the indexed expressions go) into a function and attaches its
+    tree."""
+    text = f"def {name}({', '.join(params)}):\n" + body_source
+    module = ast.parse(text)
+
+    class Put(ast.NodeTransformer):
+        def visit_Name(self, node):
+            if node.id.startswith("NMK_EXPR"):
+                return exprs[int(node.id[len("NMK_EXPR"):])]
+            return node
+
+    module = Put().visit(module)
+    fn = module.body[0]
+    for node in ast.walk(fn):
+        if not hasattr(node, "lineno"):
+            continue
+        node.lineno = node.end_lineno = stage.node.lineno
+    ast.fix_missing_locations(module)
+    namespace = dict(scope)
+    exec(compile(module, f"<stage of {name}>", "exec"), namespace)    # noqa: S102
+    func = namespace[name]
+    func.__nmk_ast__ = fn
+    return func
+
+
+def _offset(name, k):
+    node = ast.Name(id=name, ctx=ast.Load())
+    return node if k == 0 else ast.BinOp(left=node, op=ast.Add(), right=ast.Constant(value=k))
+
+
+ROW_LANES = 256       # work-group of the row-sum kernel
+
+
+def row_sum_function(stage, name, scope, arrays, integer):
+    """A @kernel body summing one map stage's expression along the rows of
+    dense matrices: one work-group per row, lanes stride over the columns
+    (four columns a work-group apart in flight), one work-group reduction.
+    Parameters: the column count, the stage's inputs, the output vector.
+    ``scope`` must bind _nmk_group_id, _nmk_local_id and _nmk_group (the
+    kernel API)."""
+    row = ast.Name(id="_nmk_row", ctx=ast.Load())
+    exprs = [_indexed(stage.expr, arrays, [row, _offset("_nmk_j", k * ROW_LANES)])
+             for k in range(4)]
+    params = ["_nmk_cols"] + list(stage.inputs) + ["_nmk_out"]
+    zero = "0" if integer else "0.0"
+    body = f"""    _nmk_row = _nmk_group_id(0)
+    _nmk_lid = _nmk_local_id(0)
+    _nmk_a0 = {zero}
+    _nmk_a1 = {zero}
+    _nmk_a2 = {zero}
+    _nmk_a3 = {zero}
+    _nmk_whole = _nmk_cols - _nmk_cols % {4 * ROW_LANES}
+    for _nmk_j in range(_nmk_lid, _nmk_whole, {4 * ROW_LANES}):
+        _nmk_a0 += NMK_EXPR0
+        _nmk_a1 += NMK_EXPR1
+        _nmk_a2 += NMK_EXPR2
+        _nmk_a3 += NMK_EXPR3
+    for _nmk_j in range(_nmk_whole + _nmk_lid, _nmk_cols, {ROW_LANES}):
+        _nmk_a0 += NMK_EXPR0
+    _nmk_total = _nmk_group.reduce_add((_nmk_a0 + _nmk_a1) + (_nmk_a2 + _nmk_a3))
+    if _nmk_lid == 0:
+        _nmk_out[_nmk_row] = _nmk_total
+"""
+    return _function(name, params, body, exprs, stage, scope), params
+
+
+COLUMNS_PER_ITEM = 4      # adjacent columns per work-item of the column-sum kernel
+
+
+def column_sum_function(stage, name, scope, arrays, integer):
+    """A @kernel body summing one map stage's expression down the columns of
+    dense matrices in chunks of rows: work-item (chunk, q) adds its chunk's
+    rows of columns 4q .. 4q + 3 (a wave reads 256 adjacent columns of a row,
+    two rows in flight) into partial[chunk, column]; the partial sums are
+    added by the column-sum kernel.  The column count must be a multiple of
+    four.  ``scope`` must bind _nmk_global_id."""
+    n = COLUMNS_PER_ITEM
+    exprs = [_indexed(stage.expr, arrays, [_offset("_nmk_i", r), _offset("_nmk_col", k)])
+             for r in range(2) for k in range(n)]
+    params = ["_nmk_rows", "_nmk_chunk"] + list(stage.inputs) + ["_nmk_part"]
+    zero = "0" if integer else "0.0"
+    lines = ["    _nmk_c = _nmk_global_id(0)", f"    _nmk_col = _nmk_global_id(1) * {n}"]
+    lines += [f"    _nmk_a{k} = {zero}" for k in range(2 * n)]
+    lines += ["    _nmk_first = _nmk_c * _nmk_chunk",
+              "    _nmk_last = min(_nmk_first + _nmk_chunk, _nmk_rows)",
+              "    _nmk_whole = _nmk_last - (_nmk_last - _nmk_first) % 2",
+              "    for _nmk_i in range(_nmk_first, _nmk_whole, 2):"]
+    lines += [f"        _nmk_a{k} += NMK_EXPR{k}" for k in range(2 * n)]
+    lines += ["    for _nmk_i in range(_nmk_whole, _nmk_last):"]
+    lines += [f"        _nmk_a{k} += NMK_EXPR{k}" for k in range(n)]
+    lines += [f"    _nmk_part[_nmk_c, _nmk_col + {k}] = _nmk_a{k} + _nmk_a{k + n}"
+              for k in range(n)]
+    return _function(name, params, "\n".join(lines) + "\n", exprs, stage, scope), params

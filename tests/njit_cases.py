@@ -431,3 +431,20 @@ def sum_of_integer_squares(a):
 
 def weighted_total(a, r):
     return np.sum(a * r)          # broadcast operands: two stages
+
+
+# reductions along an axis of a map over same-shaped matrices: one pass
+def row_dots(a, b):
+    return np.sum(a * b, axis=1)
+
+
+def column_variance(x, m):
+    return np.mean((x - m) ** 2, axis=0)
+
+
+def row_mean_abs(a, b, s):
+    return np.mean(np.abs(a - b) * s, axis=-1)
+
+
+def column_counts(a, b):
+    return np.sum(a > b, axis=0)

@@ -477,8 +477,8 @@ def test_bodies_mixing_maps_reductions_and_products(env):
 
     a64 = rng.standard_normal((65, 25))
     f, _ = run(cases.l2_norm_rows, a64)
-    assert [s["path"] for s in f.last_launch["stages"]] == ["elementwise", "library",
-                                                            "elementwise"]
+    # the square runs inside the row sums, the root is a map of its own
+    assert [s["path"] for s in f.last_launch["stages"]] == ["kernel", "elementwise"]
     # float32 row-major input: the fused row-norm kernel serves the whole body
     a32 = a64.astype(np.float32)
     for func in (cases.l2_norm_rows, cases.l2_norm_rows_product):
@@ -727,3 +727,38 @@ def test_concurrent_calls_from_python_threads(env):
     for t in threads:
         t.join()
     assert not errors, errors[0]
+
+
+@pytest.mark.parametrize("shape", [(257, 129), (1000, 36), (64, 2048), (5, 300)])
+def test_maps_run_inside_axis_reductions(env, shape):
+    """np.sum / np.mean along an axis of an expression of same-shaped dense
+    matrices is one generated kernel (plus the column-sum kernel over the
+    partial sums for axis 0)."""
+    hip = env[0]
+    rng = np.random.default_rng(51)
+    a, b = rng.standard_normal(shape), rng.standard_normal(shape)
+
+    def run(func, *host, rtol=1e-11, fused=True):
+        f = njit(func)
+        got = f(*[hip.asarray(h) if isinstance(h, np.ndarray) else h for h in host])
+        want = func(*host)
+        assert got.shape == want.shape and got.dtype == want.dtype, func.__name__
+        # (NumPy's own float32 sums carry an absolute error of this size)
+        np.testing.assert_allclose(got.asnumpy(), want, rtol=rtol,
+                                   atol=1e-12 if rtol < 1e-6 else 1e-5)
+        marks = [s.get("fused") for s in f.last_launch["stages"]]
+        assert ("map + axis sum" in marks) == fused, f.last_launch
+
+    rows_fused = shape[0] >= 64
+    run(cases.row_dots, a, b, fused=rows_fused)
+    run(cases.row_mean_abs, a, b, 0.5, fused=rows_fused)
+    columns_fused = shape[1] % 4 == 0
+    run(cases.column_variance, a, b, fused=columns_fused)
+    run(cases.column_counts, a, b, fused=columns_fused)
+    a32, b32 = a.astype(np.float32), b.astype(np.float32)
+    run(cases.row_dots, a32, b32, rtol=2e-5, fused=rows_fused)
+    run(cases.column_variance, a32, b32, rtol=2e-5, fused=columns_fused)
+    ai, bi = rng.integers(-9, 9, shape).astype(np.int32), rng.integers(-9, 9, shape).astype(np.int32)
+    run(cases.row_dots, ai, bi, fused=rows_fused)
+    # a broadcast operand: the map and the reduction run separately
+    run(cases.row_dots, a, rng.standard_normal(shape[1]), fused=False)

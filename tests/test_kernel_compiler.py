@@ -470,3 +470,33 @@ def test_bodies_are_split_at_reductions_and_contractions():
     assert params == ["x", "_nmk_t1"]
     assert kc._function_ast(func).name == "softmax_stage1"
     np.testing.assert_allclose(func(np.array([0.0, 1.0]), 1.0), np.exp([-1.0, 0.0]))
+
+
+def test_array_operands_follow_the_array_typing_rule(K):
+    """Between values computed from array elements a float meeting an integer
+    keeps its width (the reference's _select_float_type, numpy/funcs.py:
+    402-418); scalar arithmetic keeps Numba's scalar rules."""
+    f32 = kc.Array(kc.FLOAT32, 1, layout="C")
+    i32 = kc.Array(kc.INT32, 1, layout="C")
+
+    def ret(func, types):
+        return np.dtype(kc.translate(func, types, 1, K, mode="elementwise").ret_dtype)
+
+    assert ret(lambda a: a ** 2, [f32]) == np.float32
+    assert ret(lambda a: a * 2 + 1, [f32]) == np.float32
+    assert ret(lambda a, i: a + i, [f32, i32]) == np.float32
+    assert ret(lambda a, i: np.where(i > 0, a, i), [f32, i32]) == np.float32
+    assert ret(lambda a, i: np.maximum(a, i), [f32, i32]) == np.float32
+    assert ret(lambda a: a * 2.0, [f32]) == np.float64          # two floats promote
+    assert ret(lambda a: a / 3, [f32]) == np.float32
+    assert ret(lambda i: i / 3, [i32]) == np.float64
+    assert ret(lambda i: i * 2, [i32]) == np.int64
+    # a scalar argument times a literal is scalar arithmetic: float64
+    assert ret(lambda a, s: a + s * 2, [f32, kc.FLOAT32]) == np.float64
+
+    def through_names(a, i):
+        t = a - 1
+        u = t * i
+        return u ** 2
+
+    assert ret(through_names, [f32, i32]) == np.float32
