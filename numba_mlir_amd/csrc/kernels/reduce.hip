@@ -313,11 +313,20 @@ reduceStrided(const IN *x, ACC *out, int64_t nKeep, int64_t nRed, int64_t sk,
       int64_t(blockIdx.x) * (blockDim.x / NMK_WAVE) + threadIdx.x / NMK_WAVE;
   if (k >= nKeep)
     return;
-  ACC acc = init;
+  ACC acc = init, a1 = init, a2 = init, a3 = init;
   const IN *p = x + k * sk;
-  for (int64_t r = lane; r < nRed; r += NMK_WAVE)
+  int64_t r = lane;
+  for (; r + 3 * NMK_WAVE < nRed; r += 4 * NMK_WAVE) { // four loads in flight
+    const IN v0 = p[r * sr], v1 = p[(r + NMK_WAVE) * sr],
+             v2 = p[(r + 2 * NMK_WAVE) * sr], v3 = p[(r + 3 * NMK_WAVE) * sr];
+    acc = op(acc, ACC(v0));
+    a1 = op(a1, ACC(v1));
+    a2 = op(a2, ACC(v2));
+    a3 = op(a3, ACC(v3));
+  }
+  for (; r < nRed; r += NMK_WAVE)
     acc = op(acc, ACC(p[r * sr]));
-  acc = waveAllReduce(acc, op);
+  acc = waveAllReduce(op(op(acc, a1), op(a2, a3)), op);
   if (lane == 0)
     out[k * so] = acc;
 }
