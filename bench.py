@@ -39,15 +39,15 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 WAKE_SECONDS = 0.1
 
 MEASURED_TRAFFIC = {
-    "nmk_black_scholes_f32_w64": 335656763,
-    "nmk_black_scholes_f32_w32": 335619975,
-    "nmk_map2_rowbcast_add_f64": 268482394,
-    "nmk_sum_axis1_wide_f32": 537403513,
-    "nmk_norm2_f32": 536930306,
-    "nmk_sum_axis0_i32_i64": 538029894,
-    "nmk_twin_pairwise_f64_rows": 540384306,
+    "nmk_black_scholes_f32_w64": 335656913,
+    "nmk_black_scholes_f32_w32": 335620026,
+    "nmk_map2_rowbcast_add_f64": 268501361,
+    "nmk_sum_axis1_wide_f32": 537406686,
+    "nmk_norm2_f32": 536930307,
+    "nmk_sum_axis0_i32_i64": 538022729,
+    "nmk_twin_pairwise_f64_rows": 540384949,
     "nmk_copy_b128": 536870912,
-    "sgemm_mfma_256x256": 709183951,
+    "sgemm_mfma_256x256": 709712666,
 }
 
 
