@@ -10,6 +10,7 @@
 #include "numba_mlir_hip/MathRuntime.h"
 
 #include <hip/hip_runtime.h>
+#include <type_traits>
 
 #include <cstdarg>
 #include <cstdint>
@@ -76,11 +77,17 @@ thread_local const char *lastKernel = "";
 // K % BK == 0, leading dimensions multiples of the 128-bit vector, A and B
 // 16-byte aligned.
 template <typename T> struct Mfma;
+#ifndef NMHIP_SGEMM_BK
+#define NMHIP_SGEMM_BK 16
+#endif
 template <> struct Mfma<float> {
   typedef floatx4 Vec;   // 128-bit global access
   typedef floatx16 Acc;  // one MFMA tile per lane
-  static constexpr int TILE = 32, KSTEP = 2, BK = 16, VEC = 4, NACC = 16,
+  static constexpr int TILE = 32, KSTEP = 2, BK = NMHIP_SGEMM_BK, VEC = 4, NACC = 16,
                        PAD = 4;
+  // LDS reads after the compiler has paired them: one ds_read2_b32 for two
+  // fragments a tile apart.
+  static constexpr int fragmentReads(int fragments) { return fragments / 2; }
   __device__ static __forceinline__ Acc mma(float a, float b, Acc c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
   }
@@ -97,6 +104,7 @@ template <> struct Mfma<double> {
 #endif
   static constexpr int TILE = 16, KSTEP = 4, BK = NMHIP_DGEMM_BK, VEC = 2, NACC = 4,
                        PAD = 16;
+  static constexpr int fragmentReads(int fragments) { return fragments; }
   __device__ static __forceinline__ Acc mma(double a, double b, Acc c) {
     return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
   }
@@ -115,6 +123,7 @@ template <typename T, int X, bool K_CONTIG> struct SlabFetch {
   static constexpr int NV = X * M::BK / (M::VEC * 256);
   static constexpr int X_STEP = 256 * M::VEC / M::BK; // K_CONTIG: x rows per pass
   static constexpr int K_ROWS = 256 * M::VEC / X;     // else: k rows per pass
+  static constexpr int WRITES = K_CONTIG ? NV * M::VEC : NV; // LDS instructions
   int x, k;
   const T *base;
   int64_t ld;
@@ -140,9 +149,11 @@ template <typename T, int X, bool K_CONTIG> struct SlabFetch {
           K_CONTIG ? base + int64_t(X_STEP * i) * ld + k0
                    : base + int64_t(k0 + K_ROWS * i) * ld);
   }
-  __device__ __forceinline__ void stash(T (*lds)[X + M::PAD]) const {
+  // Words [i0, i1) of the slab to LDS.
+  __device__ __forceinline__ void stash(T (*lds)[X + M::PAD], int i0 = 0,
+                                        int i1 = NV) const {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
+    for (int i = i0; i < i1; ++i) {
       if (K_CONTIG) {
 #pragma unroll
         for (int q = 0; q < M::VEC; ++q)
@@ -153,6 +164,14 @@ template <typename T, int X, bool K_CONTIG> struct SlabFetch {
     }
   }
 };
+
+// n consecutive one-instruction groups of the instruction scheduler.
+template <int MASK> __device__ __forceinline__ void sched_groups(int n) {
+  if (n > 0) __builtin_amdgcn_sched_group_barrier(MASK, 1, 0);
+  if (n > 1) __builtin_amdgcn_sched_group_barrier(MASK, 1, 0);
+  if (n > 2) __builtin_amdgcn_sched_group_barrier(MASK, 1, 0);
+  if (n > 3) __builtin_amdgcn_sched_group_barrier(MASK, 1, 0);
+}
 
 template <typename T, int TM, int TN, bool A_KC, bool B_NC>
 __global__ __launch_bounds__(256) void
@@ -194,33 +213,90 @@ gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
 
   const int nSlabs = K / BK;
   const int kLane = lane / TILE, xLane = lane % TILE;
-  for (int s = 0; s < nSlabs; ++s) {
+  // One slab: BK / KSTEP steps of TM x TN MFMAs.  A wave is alone on its
+  // SIMD, so whatever it issues between two MFMAs beyond the ~60 cycles one
+  // MFMA runs leaves the matrix core idle: a clump of eight global loads or
+  // twelve LDS writes costs several hundred cycles a slab.  The directives at
+  // the end of the slab spread every memory instruction over the MFMAs, one
+  // behind each:
+  //   step 0            the global loads of the next slab (into registers),
+  //   every step        the LDS reads of the next step's operand fragments
+  //                     (double-buffered in registers),
+  //   the last steps    the LDS writes of the next slab to the other stage
+  //                     (the loads have had most of a slab to arrive).
+  auto slab = [&](int s, auto more) {
+    constexpr bool MORE = decltype(more)::value;
+    constexpr int STEPS = BK / MF::KSTEP, NMFMA = TM * TN;
     const int cur = s & 1;
-    if (s + 1 < nSlabs) {
+    if (MORE) {
       fa.fetch((s + 1) * BK);
       fb.fetch((s + 1) * BK);
     }
-#pragma unroll
-    for (int kk = 0; kk < BK; kk += MF::KSTEP) {
-      T a[TM], b[TN];
+    T a[2][TM], b[2][TN];
+    auto fragments = [&](int slot, int kk) {
 #pragma unroll
       for (int i = 0; i < TM; ++i)
-        a[i] = As[cur][kk + kLane][wm * (TM * TILE) + i * TILE + xLane];
+        a[slot][i] = As[cur][kk + kLane][wm * (TM * TILE) + i * TILE + xLane];
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        b[j] = Bs[cur][kk + kLane][wn * (TN * TILE) + j * TILE + xLane];
+        b[slot][j] = Bs[cur][kk + kLane][wn * (TN * TILE) + j * TILE + xLane];
+    };
+    fragments(0, 0);
+    // The LDS writes of the next slab sit in the second half of the steps,
+    // a share behind each step's MFMAs (the compiler cannot tell the two LDS
+    // stages apart, so reads and writes keep their program order).
+    constexpr int WRITE_STEPS = STEPS > 1 ? STEPS / 2 : 1;
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) {
+      if (st + 1 < STEPS)
+        fragments((st + 1) & 1, (st + 1) * MF::KSTEP);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = MF::mma(a[i], b[j], acc[i][j]);
+          acc[i][j] = MF::mma(a[st & 1][i], b[st & 1][j], acc[i][j]);
+      const int t = st - (STEPS - WRITE_STEPS);
+      if (MORE && t >= 0) {
+        fa.stash(As[cur ^ 1], t * fa.NV / WRITE_STEPS, (t + 1) * fa.NV / WRITE_STEPS);
+        fb.stash(Bs[cur ^ 1], t * fb.NV / WRITE_STEPS, (t + 1) * fb.NV / WRITE_STEPS);
+      }
     }
-    if (s + 1 < nSlabs) {
-      fa.stash(As[cur ^ 1]);
-      fb.stash(Bs[cur ^ 1]);
+    // Issue order (groups of the instruction scheduler; masks: 0x008 MFMA,
+    // 0x020 global load, 0x100 LDS read, 0x200 LDS write).  Counts are of
+    // instructions after the compiler has paired them; a group that finds
+    // no instruction stays empty.
+    constexpr int READS = MF::fragmentReads(TM + TN);
+    constexpr int LOADS = MORE ? fa.NV + fb.NV : 0;
+    constexpr int WRITES = MORE ? fa.WRITES + fb.WRITES : 0;
+    static_assert(READS + LOADS <= 4 * NMFMA && READS + WRITES <= 4 * NMFMA * WRITE_STEPS,
+                  "at most four memory instructions behind one MFMA");
+    sched_groups<0x100>(READS);
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) {
+      const int reads = st + 1 < STEPS ? READS : 0;
+      const int loads = st == 0 ? LOADS : 0;
+      const int t = st - (STEPS - WRITE_STEPS);
+      const int writes =
+          t < 0 ? 0
+                : ((t + 1) * fa.NV / WRITE_STEPS - t * fa.NV / WRITE_STEPS) * (fa.WRITES / fa.NV) +
+                      ((t + 1) * fb.NV / WRITE_STEPS - t * fb.NV / WRITE_STEPS) * (fb.WRITES / fb.NV);
+      // reads behind the first MFMAs of the step, writes behind the rest
+      const int head = reads < NMFMA / 2 ? reads : NMFMA / 2, tail = NMFMA - head;
+#pragma unroll
+      for (int m = 0; m < NMFMA; ++m) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (m < head)
+          sched_groups<0x100>((m + 1) * reads / head - m * reads / head);
+        else
+          sched_groups<0x200>((m - head + 1) * writes / tail - (m - head) * writes / tail);
+        sched_groups<0x020>((m + 1) * loads / NMFMA - m * loads / NMFMA);
+      }
     }
     __syncthreads();
-  }
+  };
+  for (int s = 0; s + 1 < nSlabs; ++s)
+    slab(s, std::true_type());
+  slab(nSlabs - 1, std::false_type());
 
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
