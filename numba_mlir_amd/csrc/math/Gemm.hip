@@ -55,7 +55,8 @@ thread_local const char *lastKernel = "";
 //
 // 256 threads = 4 waves in a 2 x 2 grid; each wave owns TM x TN MFMA tiles of
 // edge TILE (32 for float32, 16 for float64), so the block tile is
-// (2 TM TILE) x (2 TN TILE).  K advances in slabs of BK elements (64 bytes).
+// (2 TM TILE) x (2 TN TILE).  K advances in slabs of BK elements (16, or 32
+// for the large float32 tile).
 //
 // LDS holds both operands K-major ([k][m] and [k][n], rows padded so that the
 // rows one MFMA operand fetch touches fall on different banks): lane l needs
@@ -63,9 +64,10 @@ thread_local const char *lastKernel = "";
 // fetches are 128-bit along the operand's contiguous dimension: an operand
 // contiguous in m / n is written to LDS as one 128-bit word, one contiguous
 // in k is scattered over LDS rows.  Two LDS stages: the next K slab is
-// fetched from global memory into registers before the MFMAs of the current
-// slab are issued and written to the other stage after them, one barrier per
-// slab.
+// fetched from global memory into registers during the first step of the
+// current slab and written to the other stage during its later steps, one
+// barrier per slab; every memory instruction is issued behind an MFMA (see
+// the slab loop).
 //
 // MFMA operand layouts (64 lanes):
 //   f32 32x32x2: A[l % 32][l / 32], B[l / 32][l % 32],
@@ -77,13 +79,10 @@ thread_local const char *lastKernel = "";
 // K % BK == 0, leading dimensions multiples of the 128-bit vector, A and B
 // 16-byte aligned.
 template <typename T> struct Mfma;
-#ifndef NMHIP_SGEMM_BK
-#define NMHIP_SGEMM_BK 16
-#endif
 template <> struct Mfma<float> {
   typedef floatx4 Vec;   // 128-bit global access
   typedef floatx16 Acc;  // one MFMA tile per lane
-  static constexpr int TILE = 32, KSTEP = 2, BK = NMHIP_SGEMM_BK, VEC = 4, NACC = 16,
+  static constexpr int TILE = 32, KSTEP = 2, BK = 16, VEC = 4, NACC = 16,
                        PAD = 4;
   // LDS reads after the compiler has paired them: one ds_read2_b32 for two
   // fragments a tile apart.
@@ -99,12 +98,10 @@ template <> struct Mfma<double> {
   typedef doublex2 Vec;
   typedef doublex4 Acc;
   // PAD 16: consecutive k rows land 32 banks apart for a 128-wide tile
-#ifndef NMHIP_DGEMM_BK
-#define NMHIP_DGEMM_BK 16
-#endif
-  static constexpr int TILE = 16, KSTEP = 4, BK = NMHIP_DGEMM_BK, VEC = 2, NACC = 4,
+  static constexpr int TILE = 16, KSTEP = 4, BK = 16, VEC = 2, NACC = 4,
                        PAD = 16;
-  static constexpr int fragmentReads(int fragments) { return fragments; }
+  // one ds_read2_b64 for two fragments a tile apart
+  static constexpr int fragmentReads(int fragments) { return fragments / 2; }
   __device__ static __forceinline__ Acc mma(double a, double b, Acc c) {
     return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
   }
@@ -117,11 +114,11 @@ template <> struct Mfma<double> {
 // to LDS[k][x].  NV 128-bit words per thread.
 //   K_CONTIG: thread -> (x = tid / (BK/VEC) + X_STEP i, k = VEC (tid % (BK/VEC)) ..)
 //   else    : thread -> (k = tid / (X/VEC) + K_ROWS i, x = VEC (tid % (X/VEC)) ..)
-template <typename T, int X, bool K_CONTIG> struct SlabFetch {
+template <typename T, int X, int BK, bool K_CONTIG> struct SlabFetch {
   typedef Mfma<T> M;
   typedef typename M::Vec Vec;
-  static constexpr int NV = X * M::BK / (M::VEC * 256);
-  static constexpr int X_STEP = 256 * M::VEC / M::BK; // K_CONTIG: x rows per pass
+  static constexpr int NV = X * BK / (M::VEC * 256);
+  static constexpr int X_STEP = 256 * M::VEC / BK; // K_CONTIG: x rows per pass
   static constexpr int K_ROWS = 256 * M::VEC / X;     // else: k rows per pass
   static constexpr int WRITES = K_CONTIG ? NV * M::VEC : NV; // LDS instructions
   int x, k;
@@ -133,8 +130,8 @@ template <typename T, int X, bool K_CONTIG> struct SlabFetch {
                                        int tid) {
     ld = ld_;
     if (K_CONTIG) {
-      x = tid / (M::BK / M::VEC);
-      k = (tid % (M::BK / M::VEC)) * M::VEC;
+      x = tid / (BK / M::VEC);
+      k = (tid % (BK / M::VEC)) * M::VEC;
       base = p + int64_t(origin + x) * ld + k;
     } else {
       k = tid / (X / M::VEC);
@@ -173,13 +170,15 @@ template <int MASK> __device__ __forceinline__ void sched_groups(int n) {
   if (n > 3) __builtin_amdgcn_sched_group_barrier(MASK, 1, 0);
 }
 
-template <typename T, int TM, int TN, bool A_KC, bool B_NC>
-__global__ __launch_bounds__(256) void
+// float64 tiles need under 256 registers a lane: two blocks share a CU and
+// fill each other's stalls.  float32 256 x 256 tiles take a CU each.
+template <typename T, int BK, int TM, int TN, bool A_KC, bool B_NC>
+__global__ __launch_bounds__(256, sizeof(T) == 8 ? 2 : 1) void
 gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
           int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, T alpha,
           T beta) {
   typedef Mfma<T> MF;
-  constexpr int TILE = MF::TILE, BK = MF::BK;
+  constexpr int TILE = MF::TILE;
   constexpr int BM = 2 * TM * TILE, BN = 2 * TN * TILE;
   __shared__ __attribute__((aligned(16))) T As[2][BK][BM + MF::PAD];
   __shared__ __attribute__((aligned(16))) T Bs[2][BK][BN + MF::PAD];
@@ -191,8 +190,8 @@ gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
   const int bm = blockIdx.y * BM;
   const int bn = blockIdx.x * BN;
 
-  SlabFetch<T, BM, A_KC> fa;
-  SlabFetch<T, BN, !B_NC> fb;
+  SlabFetch<T, BM, BK, A_KC> fa;
+  SlabFetch<T, BN, BK, !B_NC> fb;
   fa.init(A, lda, bm, tid);
   fb.init(B, ldb, bn, tid);
 
@@ -205,81 +204,90 @@ gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
       for (int r = 0; r < MF::NACC; ++r)
         acc[i][j][r] = T(0);
 
+  const int nSlabs = K / BK;
+  const int kLane = lane / TILE, xLane = lane % TILE;
+  // Operand fragments of one step, double-buffered in registers.
+  T a[2][TM], b[2][TN];
+  auto fragments = [&](int stage, int slot, int kk) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      a[slot][i] = As[stage][kk + kLane][wm * (TM * TILE) + i * TILE + xLane];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      b[slot][j] = Bs[stage][kk + kLane][wn * (TN * TILE) + j * TILE + xLane];
+  };
+
   fa.fetch(0);
   fb.fetch(0);
   fa.stash(As[0]);
   fb.stash(Bs[0]);
   __syncthreads();
+  fragments(0, 0, 0);
 
-  const int nSlabs = K / BK;
-  const int kLane = lane / TILE, xLane = lane % TILE;
-  // One slab: BK / KSTEP steps of TM x TN MFMAs.  A wave is alone on its
-  // SIMD, so whatever it issues between two MFMAs beyond the ~60 cycles one
-  // MFMA runs leaves the matrix core idle: a clump of eight global loads or
-  // twelve LDS writes costs several hundred cycles a slab.  The directives at
-  // the end of the slab spread every memory instruction over the MFMAs, one
-  // behind each:
-  //   step 0            the global loads of the next slab (into registers),
-  //   every step        the LDS reads of the next step's operand fragments
-  //                     (double-buffered in registers),
-  //   the last steps    the LDS writes of the next slab to the other stage
-  //                     (the loads have had most of a slab to arrive).
+  // One slab: STEPS = BK / KSTEP steps of TM x TN MFMAs.  A wave is alone on
+  // its SIMD, so whatever it issues between two MFMAs beyond the ~60 cycles
+  // one MFMA runs leaves the matrix core idle: a clump of eight global loads
+  // or twelve LDS writes costs several hundred cycles a slab.  The
+  // directives at the end of the slab spread every memory instruction over
+  // the MFMAs, one or two behind each:
+  //   step 0          the global loads of the next slab (into registers),
+  //   every step      the LDS reads of the next step's fragments; in the last
+  //                   step, behind the slab's one barrier, those of the next
+  //                   slab's first step, so their latency runs under the last
+  //                   step's MFMAs,
+  //   the steps before the last, from the middle on
+  //                   the LDS writes of the next slab to the other stage (the
+  //                   loads have had a third of a slab or more to arrive).
+  // The compiler cannot tell the two LDS stages apart, so LDS reads and
+  // writes keep their program order: each sits in the step it is issued in.
   auto slab = [&](int s, auto more) {
     constexpr bool MORE = decltype(more)::value;
     constexpr int STEPS = BK / MF::KSTEP, NMFMA = TM * TN;
+    static_assert(STEPS >= 4 && STEPS % 2 == 0, "fragment slots alternate over a slab");
+    constexpr int WRITE_STEPS = STEPS / 2 - 1, WRITE_FROM = STEPS - 1 - WRITE_STEPS;
     const int cur = s & 1;
     if (MORE) {
       fa.fetch((s + 1) * BK);
       fb.fetch((s + 1) * BK);
     }
-    T a[2][TM], b[2][TN];
-    auto fragments = [&](int slot, int kk) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        a[slot][i] = As[cur][kk + kLane][wm * (TM * TILE) + i * TILE + xLane];
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        b[slot][j] = Bs[cur][kk + kLane][wn * (TN * TILE) + j * TILE + xLane];
-    };
-    fragments(0, 0);
-    // The LDS writes of the next slab sit in the second half of the steps,
-    // a share behind each step's MFMAs (the compiler cannot tell the two LDS
-    // stages apart, so reads and writes keep their program order).
-    constexpr int WRITE_STEPS = STEPS > 1 ? STEPS / 2 : 1;
 #pragma unroll
     for (int st = 0; st < STEPS; ++st) {
-      if (st + 1 < STEPS)
-        fragments((st + 1) & 1, (st + 1) * MF::KSTEP);
+      if (st + 1 < STEPS) {
+        fragments(cur, (st + 1) & 1, (st + 1) * MF::KSTEP);
+      } else if (MORE) {
+        __syncthreads();
+        fragments(cur ^ 1, 0, 0);
+      }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
           acc[i][j] = MF::mma(a[st & 1][i], b[st & 1][j], acc[i][j]);
-      const int t = st - (STEPS - WRITE_STEPS);
-      if (MORE && t >= 0) {
+      const int t = st - WRITE_FROM;
+      if (MORE && t >= 0 && t < WRITE_STEPS) {
         fa.stash(As[cur ^ 1], t * fa.NV / WRITE_STEPS, (t + 1) * fa.NV / WRITE_STEPS);
         fb.stash(Bs[cur ^ 1], t * fb.NV / WRITE_STEPS, (t + 1) * fb.NV / WRITE_STEPS);
       }
     }
     // Issue order (groups of the instruction scheduler; masks: 0x008 MFMA,
-    // 0x020 global load, 0x100 LDS read, 0x200 LDS write).  Counts are of
-    // instructions after the compiler has paired them; a group that finds
-    // no instruction stays empty.
+    // 0x020 global load, 0x100 LDS read, 0x200 LDS write).  Read counts are
+    // of instructions after the compiler has paired them, write counts
+    // before (it pairs some); a group that finds no instruction stays empty.
     constexpr int READS = MF::fragmentReads(TM + TN);
     constexpr int LOADS = MORE ? fa.NV + fb.NV : 0;
-    constexpr int WRITES = MORE ? fa.WRITES + fb.WRITES : 0;
-    static_assert(READS + LOADS <= 4 * NMFMA && READS + WRITES <= 4 * NMFMA * WRITE_STEPS,
+    static_assert(READS + LOADS <= 4 * NMFMA &&
+                      READS + fa.WRITES + fb.WRITES <= 4 * NMFMA * WRITE_STEPS,
                   "at most four memory instructions behind one MFMA");
-    sched_groups<0x100>(READS);
 #pragma unroll
     for (int st = 0; st < STEPS; ++st) {
-      const int reads = st + 1 < STEPS ? READS : 0;
+      const int reads = st + 1 < STEPS || MORE ? READS : 0;
       const int loads = st == 0 ? LOADS : 0;
-      const int t = st - (STEPS - WRITE_STEPS);
+      const int t = st - WRITE_FROM;
       const int writes =
-          t < 0 ? 0
-                : ((t + 1) * fa.NV / WRITE_STEPS - t * fa.NV / WRITE_STEPS) * (fa.WRITES / fa.NV) +
-                      ((t + 1) * fb.NV / WRITE_STEPS - t * fb.NV / WRITE_STEPS) * (fb.WRITES / fb.NV);
+          !MORE || t < 0 || t >= WRITE_STEPS
+              ? 0
+              : ((t + 1) * fa.NV / WRITE_STEPS - t * fa.NV / WRITE_STEPS) * (fa.WRITES / fa.NV) +
+                    ((t + 1) * fb.NV / WRITE_STEPS - t * fb.NV / WRITE_STEPS) * (fb.WRITES / fb.NV);
       // reads behind the first MFMAs of the step, writes behind the rest
       const int head = reads < NMFMA / 2 ? reads : NMFMA / 2, tail = NMFMA - head;
 #pragma unroll
@@ -292,7 +300,6 @@ gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
         sched_groups<0x020>((m + 1) * loads / NMFMA - m * loads / NMFMA);
       }
     }
-    __syncthreads();
   };
   for (int s = 0; s + 1 < nSlabs; ++s)
     slab(s, std::true_type());
@@ -445,7 +452,9 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       // float32: 256 x 256 block tiles (one block per CU on a 4096^2
       // problem) when the shape allows and there are enough tiles to fill the
       // 256 CUs, 128 x 128 otherwise (measured within 3 % of each other; the
-      // larger tile halves the operand traffic).  float64: 128 x 128.
+      // larger tile halves the operand traffic).  float64: 128 x 128.  The
+      // large tile advances K in slabs of 2 BK where K allows (half the
+      // barriers; 144 against 142 TFLOP/s on 4096^3).
       const bool big = sizeof(T) == 4 && Mz % 256 == 0 && Nz % 256 == 0 &&
                        (Mz / 256) * (Nz / 256) >= 192;
       const int BM = big ? 256 : 128, BN = BM;
@@ -455,31 +464,34 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           aligned16(X) && aligned16(Y) && M <= 0x7fffffff && N <= 0x7fffffff &&
           K <= 0x7fffffff && Mz / BM <= 65535) {
         dim3 grid(unsigned(Nz / BN), unsigned(Mz / BM), 1);
-#define NMHIP_GEMM_LAUNCH(TM, TN, XKC, YNC)                                    \
-  hipLaunchKernelGGL((gemm_mfma<T, TM, TN, XKC, YNC>), grid, dim3(256), 0,     \
-                     stream, X, Y, cData, int(Mz), int(Nz), int(K), ldx, ldy,  \
-                     ldz, alpha, beta)
-#define NMHIP_GEMM_LAYOUTS(TM, TN)                                             \
+#define NMHIP_GEMM_LAUNCH(SLAB, TM, TN, XKC, YNC)                              \
+  hipLaunchKernelGGL((gemm_mfma<T, SLAB, TM, TN, XKC, YNC>), grid, dim3(256),  \
+                     0, stream, X, Y, cData, int(Mz), int(Nz), int(K), ldx,    \
+                     ldy, ldz, alpha, beta)
+#define NMHIP_GEMM_LAYOUTS(SLAB, TM, TN)                                       \
   do {                                                                         \
     if (xKc && yNc)                                                            \
-      NMHIP_GEMM_LAUNCH(TM, TN, true, true);                                   \
+      NMHIP_GEMM_LAUNCH(SLAB, TM, TN, true, true);                             \
     else if (xKc)                                                              \
-      NMHIP_GEMM_LAUNCH(TM, TN, true, false);                                  \
+      NMHIP_GEMM_LAUNCH(SLAB, TM, TN, true, false);                            \
     else if (yNc)                                                              \
-      NMHIP_GEMM_LAUNCH(TM, TN, false, true);                                  \
+      NMHIP_GEMM_LAUNCH(SLAB, TM, TN, false, true);                            \
     else                                                                       \
-      NMHIP_GEMM_LAUNCH(TM, TN, false, false);                                 \
+      NMHIP_GEMM_LAUNCH(SLAB, TM, TN, false, false);                           \
   } while (0)
         if constexpr (sizeof(T) == 4) {
-          if (big) {
-            NMHIP_GEMM_LAYOUTS(4, 4);
+          if (big && K % (2 * BK) == 0) {
+            NMHIP_GEMM_LAYOUTS(2 * BK, 4, 4);
+            lastKernel = "sgemm_mfma_256x256";
+          } else if (big) {
+            NMHIP_GEMM_LAYOUTS(BK, 4, 4);
             lastKernel = "sgemm_mfma_256x256";
           } else {
-            NMHIP_GEMM_LAYOUTS(2, 2);
+            NMHIP_GEMM_LAYOUTS(BK, 2, 2);
             lastKernel = "sgemm_mfma_128x128";
           }
         } else {
-          NMHIP_GEMM_LAYOUTS(4, 4);
+          NMHIP_GEMM_LAYOUTS(BK, 4, 4);
           lastKernel = "dgemm_mfma_128x128";
         }
 #undef NMHIP_GEMM_LAYOUTS
