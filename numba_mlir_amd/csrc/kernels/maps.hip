@@ -344,10 +344,10 @@ __device__ __forceinline__ void bsTrip(const V &P, const V &S, const V &T,
   }
 }
 
-// VEC options per lane per iteration (float4 or float2 accesses).  The
-// float64 variant is ALU-bound and register-hungry: two options per lane at
-// five to six waves per SIMD measured fastest (no spills at five); the
-// float32 variant takes four.
+// VEC options per lane per iteration (float4 or float2 accesses).  Both
+// variants take four: the float64 one then needs 78 registers a lane, six
+// waves per SIMD without spills (60.6 us on 2^24 options against 63.1 us
+// with two options and 64-bit accesses; eight waves spill).
 template <int VEC> struct BsVec;
 template <> struct BsVec<4> {
   typedef float4_t type;
@@ -405,7 +405,7 @@ __attribute__((amdgpu_waves_per_eu(6, 6))) void
 nmk_black_scholes_f32_w64(const float *price, const float *strike,
                           const float *t, float rate, float volatility,
                           float *call, float *put, int64_t n) {
-  blackScholes<double, 2>(price, strike, t, rate, volatility, call, put, n);
+  blackScholes<double, 4>(price, strike, t, rate, volatility, call, put, n);
 }
 
 NMK_KERNEL(256)

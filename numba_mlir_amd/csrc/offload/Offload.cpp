@@ -613,9 +613,8 @@ NMHIP_EXPORT void nmhipBlackScholesF32(void *ctx, const float *price,
     if (n < 0)
       fail("nmhipBlackScholesF32: negative extent");
     int64_t blocks = tuning().bsBlocks ? tuning().bsBlocks : 256 * 16;
-    // The float64-literal kernel takes two options per lane, the float32 one
-    // four.
-    const int64_t need = ceilDiv(ceilDiv(n, wide ? 2 : 4), 256);
+    // Four options per lane and trip.
+    const int64_t need = ceilDiv(ceilDiv(n, 4), 256);
     if (blocks > need)
       blocks = need;
     c->launch(wide ? "nmk_black_scholes_f32_w64" : "nmk_black_scholes_f32_w32",
