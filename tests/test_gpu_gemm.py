@@ -80,7 +80,8 @@ def test_internal_gemm_fixture_grid(env):
 
 @pytest.mark.parametrize("ta,tb,tc", list(itertools.product([False, True], repeat=3)))
 @pytest.mark.parametrize("m,n,k", [(33, 29, 47), (128, 128, 16), (1, 1, 1), (64, 1, 300),
-                                   (256, 384, 64), (4096, 3072, 32)])
+                                   (256, 384, 64), (4096, 3072, 32), (4096, 3072, 48),
+                                   (3072, 4096, 96)])
 def test_layouts_against_float64(env, ta, tb, tc, m, n, k):
     """Every stride pattern the entry point accepts (row/column major A, B, C)."""
     hip, ops, orc, mrt = env
