@@ -174,6 +174,7 @@ class Val:
         self.slice_parts = slice_parts  # (start, stop, step) Vals or None each
         self.gid = None               # k: the value is global id k plus a constant
         self.arr = False              # elementwise mode: computed from array elements
+        self.origin = None            # an array: the parameter this is, under any name
 
 
 class _Deferred(Exception):
@@ -418,6 +419,10 @@ class FunctionTranslator:
         self.last_elem_gid = None    # of the element subscript() resolved last
         self.last_elem_unit = "false"
         self.elements_per_thread = 1
+        self.view_origin = {}        # array variable -> the parameter it is another name of
+        self.written_origins = set() # parameters assigned through [:] under any name
+        self.opaque_write = False    # [:] assignment to an array of unknown origin
+        self.prefetched = {}         # parameter -> Array type: loaded ahead of the body
         self._lambda_body = None
         self.reduction_types = []    # (name, Scalar) in parameter order
         self.site_names = {}         # ast node -> stable names
@@ -473,7 +478,12 @@ class FunctionTranslator:
                 self.array_reads += v.arr
                 return v
             if isinstance(t, Array):
-                return Val(self.cname(name), t)
+                v = Val(self.cname(name), t)
+                if name in self.params:
+                    v.origin = name if not self.store_count.get(name) else None
+                else:
+                    v.origin = self.view_origin.get(name)
+                return v
             if isinstance(t, SliceArg):
                 c = self.cname(name)
                 parts = tuple(Val(f"{c}_{k}", INT64) for k in ("start", "stop", "step"))
@@ -527,6 +537,13 @@ class FunctionTranslator:
             self.err(node, "Only whole arrays of the iteration space can be used "
                            "in an elementwise function")
         self.read_arrays.add(arr.code)
+        if self.prefetches(arr):
+            # loaded ahead of the body, for all of the lane's elements at once
+            self.prefetched[arr.origin] = arr.type
+            v = Val(f"nmk_pf_{arr.origin}", arr.type.elem)
+            v.arr = True
+            self.array_reads += 1
+            return v
         terms = [f"nmk_gid{d} * {arr.code}.stride[{d}]" for d in range(self.ndim)]
         ref = f"{arr.code}.p[{' + '.join(terms)}]"
         if self.noalias and self.stream and arr.code not in self.written_arrays:
@@ -536,6 +553,20 @@ class FunctionTranslator:
         v.arr = True
         self.array_reads += 1
         return v
+
+    _PREFETCH_CTYPES = ("float", "double", "int32_t", "int64_t", "uint32_t", "uint64_t")
+
+    def prefetches(self, arr):
+        """A 1-d map that gives a lane several elements loads the lane's
+        elements of its read-only array arguments before the first element's
+        arithmetic: a body with branches (the range checks of log, exp, erf)
+        would otherwise load, compute and store one element after the other,
+        one memory latency each.  Needs arguments that do not overlap, and a
+        parameter that no statement assigns through [:] under any name."""
+        return (self.mode == "elementwise" and self.ndim == 1 and self.noalias and
+                self.elements_per_thread > 1 and arr.origin is not None and
+                arr.origin not in self.written_origins and not self.opaque_write and
+                arr.type.elem.ctype in self._PREFETCH_CTYPES)
 
     def store_here(self, arr_code, elem, value_code):
         """Elementwise mode: the store of this work-item's element.  An array
@@ -1261,6 +1292,10 @@ class FunctionTranslator:
         if v.arr and name not in self.array_valued:
             self.array_valued.add(name)
             self.changed = True
+        if isinstance(v.type, Array) and v.origin is not None and \
+                self.store_count.get(name) == 1 and id(node) in self.top_level and \
+                name not in self.params:
+            self.view_origin[name] = v.origin      # P = price: P is price
         if isinstance(v.type, Scalar):
             if (v.const is not None and self.store_count.get(name) == 1 and
                     id(node) in self.top_level and name not in self.params):
@@ -1286,6 +1321,10 @@ class FunctionTranslator:
             if arr.type.ndim != self.ndim:
                 self.err(node, "Only whole arrays of the iteration space can be assigned")
             self.written_arrays.add(arr.code)
+            if arr.origin is not None:
+                self.written_origins.add(arr.origin)
+            else:
+                self.opaque_write = True
             self.store_here(arr.code, arr.type.elem, cast(v, arr.type.elem).code)
             return
         kind, *rest = self.subscript(target)
@@ -1553,6 +1592,7 @@ class FunctionTranslator:
 
     def run_emit(self, body):
         self.emitting = True
+        self.prefetched = {}        # (the passes before knew less of what is written)
         self.lines = []
         self.group_sites = []
         self.local_arrays = []
@@ -1726,10 +1766,22 @@ class FunctionTranslator:
             strided = self.ndim == 1 and not self.m.communicates and self.mode != "kernel"
             self.grid_stride = strided
             if strided:
+                # (name, element type, address of the element at index g)
+                pf = []
+                for name in [p for p in self.params if p in self.prefetched and ept > 1]:
+                    t, c = self.prefetched[name], self.cname(name)
+                    step = "" if t.layout == "C" else f" * {c}_t0"
+                    addr = f"&{c}_p[g{step}]"
+                    load = f"__builtin_nontemporal_load({addr})" if self.stream else f"*({addr})"
+                    pf.append((name, t.elem.ctype, load))
+                if self.prefetched and not pf:
+                    self.err(self.node, "internal: elements loaded ahead in a kernel that "
+                                        "takes one element per lane")
+                extra = "".join(f", const {ct} nmk_pf_{n}" for n, ct, _ in pf)
                 out += [
                     "  const int64_t nmk_gid1 = 0, nmk_gid2 = 0;",
                     "  (void)nmk_gid1; (void)nmk_gid2;",
-                    "  auto nmk_item = [&](const int64_t nmk_gid0, auto nmk_guarded) {",
+                    f"  auto nmk_item = [&](const int64_t nmk_gid0, auto nmk_guarded{extra}) {{",
                     "    if (decltype(nmk_guarded)::value && !(nmk_gid0 < nmk_gsz0)) return;",
                 ] + body + [
                     "  };",
@@ -1737,13 +1789,36 @@ class FunctionTranslator:
                     "nmk_gsz0; nmk_round += gridDim.x) {",
                     f"    const int64_t nmk_base = nmk_round * {ept} * nmk_lsz0 + nmk_lid0;",
                     f"    if ((nmk_round + 1) * {ept} * nmk_lsz0 <= nmk_gsz0) {{",
+                ]
+                if pf:
+                    # The empty asm statements keep the optimizer from moving
+                    # each load back down to its first use.
+                    out += [f"      {ct} nmk_ahead_{n}[{ept}];" for n, ct, _ in pf]
+                    out += [
+                        "#pragma unroll",
+                        f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep) {{",
+                        "        const int64_t g = nmk_base + nmk_rep * nmk_lsz0;",
+                    ] + [f"        nmk_ahead_{n}[nmk_rep] = {load};" for n, _, load in pf] + [
+                        "      }",
+                        "#pragma unroll",
+                        f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep) {{",
+                    ] + [f'        asm volatile("" : "+v"(nmk_ahead_{n}[nmk_rep]));'
+                         for n, _, _ in pf] + [
+                        "      }",
+                    ]
+                ahead = "".join(f", nmk_ahead_{n}[nmk_rep]" for n, _, _ in pf)
+                out += [
                     "#pragma unroll",
                     f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep)",
-                    "        nmk_item(nmk_base + nmk_rep * nmk_lsz0, nmkjit::No());",
+                    f"        nmk_item(nmk_base + nmk_rep * nmk_lsz0, nmkjit::No(){ahead});",
                     "    } else {",
                     "#pragma unroll 1",
-                    f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep)",
-                    "        nmk_item(nmk_base + nmk_rep * nmk_lsz0, nmkjit::Yes());",
+                    f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep) {{",
+                    "        const int64_t g = nmk_base + nmk_rep * nmk_lsz0;",
+                    "        if (g < nmk_gsz0)",
+                    "          nmk_item(g, nmkjit::No()" +
+                    "".join(f", {load}" for _, _, load in pf) + ");",
+                    "      }",
                     "    }",
                     "  }",
                 ]

@@ -189,6 +189,11 @@ def add_into(a, b, c):
     c[:] = a + b
 
 
+def scale_in_place(a, b):
+    x = a
+    x[:] = a * b + 1.0
+
+
 def fill(a):
     a[:] = 42
 

@@ -309,21 +309,34 @@ def test_fused_maps_take_several_elements_per_lane(K, tmp_path, monkeypatch):
                       noalias=True, elements_per_thread=4)
     assert ck.elements_per_thread == 4
     assert "for (int nmk_rep = 0; nmk_rep < 4; ++nmk_rep)" in ck.source
-    assert "nmk_item(nmk_base + nmk_rep * nmk_lsz0, nmkjit::No());" in ck.source
     assert "float *__restrict__ v_price_p" in ck.source
     # call and put are only written: streamed
     assert ck.source.count("NMK_STORE_ALONG0(&") == 2
     assert "#define NMK_STORE_ALONG0(p, v, unit) nmkjit::streamStore(p, v, unit)" in ck.source
     assert kc.build_code_object(ck)[:4] == b"\x7fELF"
-    # operands are read with streaming loads
-    assert "__builtin_nontemporal_load(&v_P.p[" in ck.source
+    # The read-only operands (P = price is price) are loaded for all four
+    # elements ahead of the first element's arithmetic, with streaming loads,
+    # and handed to the body as values.
+    assert "nmk_ahead_price[nmk_rep] = __builtin_nontemporal_load(&v_price_p[g]);" in ck.source
+    assert 'asm volatile("" : "+v"(nmk_ahead_t[nmk_rep]));' in ck.source
+    assert ("nmk_item(nmk_base + nmk_rep * nmk_lsz0, nmkjit::No(), nmk_ahead_price[nmk_rep], "
+            "nmk_ahead_strike[nmk_rep], nmk_ahead_t[nmk_rep]);") in ck.source
+    assert "v_a = nmk::logF32((nmk_pf_price / nmk_pf_strike));" in ck.source
+    assert "v_P.p[" not in ck.source
     small = kc.translate(njit_cases.black_scholes_arrays, types, ndim, K, mode=mode,
                          noalias=True, elements_per_thread=4, stream=False)
     assert "nontemporal" not in small.source and "NMK_STORE_ALONG0(&" not in small.source
-    # overlapping arguments: plain pointers and stores
+    assert "nmk_ahead_price[nmk_rep] = *(&v_price_p[g]);" in small.source
+    # overlapping arguments: plain pointers and stores, every load where it is used
     ck = kc.translate(njit_cases.black_scholes_arrays, types, ndim, K, mode=mode,
                       noalias=False, elements_per_thread=4)
     assert "__restrict__" not in ck.source and "nontemporal" not in ck.source
+    assert "nmk_ahead" not in ck.source and "v_P.p[" in ck.source
+    assert "nmk_item(nmk_base + nmk_rep * nmk_lsz0, nmkjit::No());" in ck.source
+    # an argument the body also assigns is not loaded ahead; the others are
+    ck = kc.translate(njit_cases.scale_in_place, [kc.Array(kc.FLOAT64, 1), kc.Array(kc.FLOAT64, 1)],
+                      1, K, mode="elementwise", noalias=True, elements_per_thread=4)
+    assert "nmk_ahead_b" in ck.source and "nmk_ahead_a" not in ck.source
     # more than one dimension, or an @kernel body: one element per lane
     mode, ndim, types = _njit_types("fused_map")
     ck = kc.translate(njit_cases.fused_map, types, ndim, K, mode=mode, noalias=True,
