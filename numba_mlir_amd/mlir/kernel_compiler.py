@@ -2045,10 +2045,5 @@ def build_code_object(compiled):
                 f"hipcc failed for {compiled.name}:\n{proc.stderr}\n--- source ---\n"
                 f"{compiled.source}")
         os.replace(tmp, obj)
-    else:
-        try:
-            os.utime(obj)           # last use, for whoever prunes the directory
-        except OSError:
-            pass
     with open(obj, "rb") as f:
         return f.read()
