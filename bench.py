@@ -377,9 +377,9 @@ def generated_kernels(b, workloads):
             k = turn[0] % len(arg_sets)
             turn[0] += 1
             events.append(plan.enqueue(arg_sets[k], None if ret_sets is None else ret_sets[k]))
-            # The context's synchronize() waits for the library's own launches
-            # only: bound the backlog of these by waiting for the launch 16
-            # back (the stream stays busy, the host stays just ahead).
+            # Bound the backlog (an enqueue takes 4 us, a kernel 60-100): wait
+            # for the launch 16 back; the stream stays busy, the host stays
+            # just ahead.
             if len(events) > 16:
                 plan.retire(events.pop(0))
 

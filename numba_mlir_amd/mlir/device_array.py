@@ -17,7 +17,7 @@ import weakref
 
 import numpy as np
 
-from . import lowered
+from . import gpu_runtime, lowered
 from .lowered import lib
 from .utils import readenv
 
@@ -44,6 +44,9 @@ class Context:
         self.handle = lib.nmhipContextCreate(device.encode() if device else None)
         self._finalizer = weakref.finalize(self, lib.nmhipContextDestroy,
                                            self.handle)
+        # events of launches enqueued from Python and not yet retired, oldest
+        # first (kernel_impl.LaunchPlan.enqueue / retire)
+        self.pending = []
 
     @property
     def queue(self):
@@ -53,7 +56,14 @@ class Context:
         lib.nmhipContextSetAsync(self.handle, 1 if flag else 0)
 
     def synchronize(self):
+        """Returns when everything submitted through this context is done:
+        the library's own launches and the launches enqueued from Python (the
+        queue is in order, so waiting for the youngest of those covers all;
+        their events stay the caller's to retire)."""
         lib.nmhipContextSynchronize(self.handle)
+        pending = self.pending
+        if pending:
+            gpu_runtime.runtime_lib.gpuxWait(self.queue, pending[-1])
 
     def last_kernel(self):
         return lib.nmhipLastKernelName(self.handle).decode()

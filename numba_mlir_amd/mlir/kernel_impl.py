@@ -495,11 +495,18 @@ class LaunchPlan:
         with self._lock:                  # the launch call copies the values out
             if args is not None:
                 self._refresh(args, ret, ())
-            return runtime_lib.gpuxLaunchKernel(*self._launch)
+            event = runtime_lib.gpuxLaunchKernel(*self._launch)
+            self.ctx.pending.append(event)    # the context's synchronize() waits for it
+            return event
 
     def retire(self, event):
         queue = self.ctx.queue
         runtime_lib.gpuxWait(queue, event)
+        with self._lock:
+            try:
+                self.ctx.pending.remove(event)
+            except ValueError:
+                pass
         runtime_lib.gpuxDestroyEvent(queue, event)
 
     def run(self, args=None, ret=None, partials=()):

@@ -311,6 +311,29 @@ def test_unsupported_functions_are_reported(env):
         njit(cases.add)(1.0, 2.0)
 
 
+def test_enqueued_launches_are_covered_by_synchronize(env):
+    """Launches put on the queue without waiting (the benchmark's timing path)
+    are finished when the context's synchronize() returns; their events stay
+    with the caller until retired."""
+    hip, ops, orc, workloads = env
+    from numba_mlir_amd.mlir import device_array as da
+    ctx = da.get_context()
+    a = np.arange(1 << 20, dtype=np.float64)
+    d_a = hip.asarray(a)
+    outs = [hip.asarray(np.zeros_like(a)) for _ in range(6)]
+    f = njit(cases.scale_into)
+    f(d_a, outs[0])
+    plan = f.last_plan
+    events = [plan.enqueue([d_a, o]) for o in outs]
+    assert ctx.pending[-len(events):] == events
+    ctx.synchronize()
+    for o in outs:
+        np.testing.assert_array_equal(o.asnumpy(), a * 2)
+    for e in events:
+        plan.retire(e)
+    assert not any(e in ctx.pending for e in events)
+
+
 def test_repeated_calls_replay_stored_launches(env):
     """A call whose argument types, shapes and strides were seen before reuses
     the prepared launch: new addresses, new scalar values and a change of
