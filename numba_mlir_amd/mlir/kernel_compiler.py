@@ -423,6 +423,8 @@ class FunctionTranslator:
         self.written_origins = set() # parameters assigned through [:] under any name
         self.opaque_write = False    # [:] assignment to an array of unknown origin
         self.prefetched = {}         # parameter -> Array type: loaded ahead of the body
+        self.ahead_nodes = {}        # parallel mode: id(p[i] node) -> parameter p
+        self.loop_kinds = []         # enclosing loops, outermost first: "grid" | "sequential"
         self._lambda_body = None
         self.reduction_types = []    # (name, Scalar) in parameter order
         self.site_names = {}         # ast node -> stable names
@@ -864,6 +866,11 @@ class FunctionTranslator:
     def expr_Subscript(self, node):
         if self.mode == "elementwise" and self.is_whole_slice(node.slice):
             return self.expr(node.value)          # a[:] is a itself
+        param = self.ahead_nodes.get(id(node))
+        if param is not None:
+            t = self.arg_types[self.params.index(param)]
+            self.prefetched[param] = t
+            return Val(f"nmk_pf_{param}", t.elem)
         kind, *rest = self.subscript(node)
         if kind == "elem":
             code, elem = rest
@@ -1446,10 +1453,18 @@ class FunctionTranslator:
                 self.maybe_negative.add(name)
             if step.const == 1 and self.store_count.get(name) == 1:
                 self.gid_vars[name] = depth
+            if depth == 0 and self.ndim == 1 and self.noalias and start.const == 0 and \
+                    step.const == 1 and self.elements_per_thread > 1 and \
+                    not self.m.boundscheck:
+                # what every iteration reads at its own index is loaded for
+                # all of a lane's iterations before the first one runs
+                self.ahead_nodes = self.loads_ahead_of(node)
             if self.emitting:
                 self.emit(f"{self.cname(name)} = {start.code} + nmk_gid{depth} * {step.code};")
             self.indent -= 1
+            self.loop_kinds.append("grid")
             self.block(node.body)
+            self.loop_kinds.pop()
             self.indent += 1
             return
         self.bind(name, INT64, node)
@@ -1472,10 +1487,70 @@ class FunctionTranslator:
             t = self.env[name]
             self.emit(f"{self.cname(name)} = ({t.ctype}){itv};")
         self.indent -= 1
+        self.loop_kinds.append("sequential")
         self.block(node.body)
+        self.loop_kinds.pop()
         self.emit("}")
         self.indent -= 1
         self.emit("}")
+
+    def loads_ahead_of(self, loop):
+        """prange loop of a 1-d launch, iterations 0, 1, 2 ...: the reads
+        ``p[i]`` of parameter arrays that every iteration performs, whatever
+        its data -- in a statement of the loop body itself, outside ``x if c
+        else y`` and ``and`` / ``or``, in a body without continue / break /
+        return.  ``p`` must be used for nothing but element reads and its
+        shape in the whole function.  Returns {id(subscript node): parameter}."""
+        var = loop.target.id
+        if self.store_count.get(var) != 1:
+            return {}
+        for n in ast.walk(ast.Module(body=loop.body, type_ignores=[])):
+            if isinstance(n, (ast.Continue, ast.Break, ast.Return)):
+                return {}
+        arrays = {p for p, t in zip(self.params, self.arg_types)
+                  if isinstance(t, Array) and t.space == "global" and t.ndim == 1 and
+                  t.elem.ctype in self._PREFETCH_CTYPES and not self.store_count.get(p)}
+        parents = {}
+        for parent in ast.walk(self.node):
+            for child in ast.iter_child_nodes(parent):
+                parents[id(child)] = parent
+        for n in ast.walk(self.node):
+            if isinstance(n, ast.Name) and n.id in arrays:
+                parent = parents.get(id(n))
+                if isinstance(parent, ast.Subscript) and parent.value is n and \
+                        isinstance(parent.ctx, ast.Load):
+                    continue
+                if isinstance(parent, ast.Attribute) and \
+                        parent.attr in ("shape", "size", "ndim", "dtype"):
+                    continue
+                if isinstance(parent, ast.Call) and isinstance(parent.func, ast.Name) and \
+                        parent.func.id == "len" and len(parent.args) == 1:
+                    continue
+                arrays.discard(n.id)
+        found = {}
+
+        def scan(n):
+            if isinstance(n, ast.IfExp):
+                scan(n.test)
+                return
+            if isinstance(n, ast.BoolOp):
+                scan(n.values[0])
+                return
+            if isinstance(n, (ast.Lambda, ast.ListComp, ast.GeneratorExp, ast.SetComp,
+                              ast.DictComp)):
+                return
+            if isinstance(n, ast.Subscript) and isinstance(n.ctx, ast.Load) and \
+                    isinstance(n.value, ast.Name) and n.value.id in arrays and \
+                    isinstance(n.slice, ast.Name) and n.slice.id == var:
+                found[id(n)] = n.value.id
+                return
+            for child in ast.iter_child_nodes(n):
+                scan(child)
+
+        for stmt in loop.body:
+            if isinstance(stmt, (ast.Assign, ast.AugAssign, ast.AnnAssign, ast.Expr)):
+                scan(stmt.value)
+        return found
 
     def grid_depth(self, node):
         """Which grid dimension a prange loop is, or None for a sequential one:
@@ -1494,14 +1569,20 @@ class FunctionTranslator:
             self.err(node, "while ... else is not supported")
         c = self.truth(self.scalar(node.test))
         self.emit(f"while ({c.code}) {{")
+        self.loop_kinds.append("sequential")
         self.block(node.body)
+        self.loop_kinds.pop()
         self.emit("}")
 
     def stmt_Break(self, node):
+        if self.loop_kinds and self.loop_kinds[-1] == "grid":
+            self.err(node, "A prange loop cannot be left with break")
         self.emit("break;")
 
     def stmt_Continue(self, node):
-        self.emit("continue;")
+        # an iteration of a prange loop is one call of the work-item body
+        grid = self.loop_kinds and self.loop_kinds[-1] == "grid"
+        self.emit("return;" if grid else "continue;")
 
     def stmt_Return(self, node):
         if node is self.return_node:
@@ -1772,7 +1853,9 @@ class FunctionTranslator:
                     t, c = self.prefetched[name], self.cname(name)
                     step = "" if t.layout == "C" else f" * {c}_t0"
                     addr = f"&{c}_p[g{step}]"
-                    load = f"__builtin_nontemporal_load({addr})" if self.stream else f"*({addr})"
+                    # (a loop's other iterations may read the element too)
+                    load = f"__builtin_nontemporal_load({addr})" \
+                        if self.stream and self.mode == "elementwise" else f"*({addr})"
                     pf.append((name, t.elem.ctype, load))
                 if self.prefetched and not pf:
                     self.err(self.node, "internal: elements loaded ahead in a kernel that "

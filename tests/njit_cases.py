@@ -189,6 +189,22 @@ def add_into(a, b, c):
     c[:] = a + b
 
 
+def loop_reads(n, a, b, c, out):
+    for i in prange(n):
+        x = a[i] + out[i]
+        y = b[i] if x > 0 else 0.0
+        if y > 1.0:
+            y = c[i]
+        out[i] = x + y
+
+
+def loop_leaves_early(n, a, out):
+    for i in prange(n):
+        if i % 2:
+            continue
+        out[i] = a[i]
+
+
 def scale_in_place(a, b):
     x = a
     x[:] = a * b + 1.0

@@ -311,6 +311,30 @@ def test_unsupported_functions_are_reported(env):
         njit(cases.add)(1.0, 2.0)
 
 
+@pytest.mark.parametrize("n", [1, 255, 1024, 4097, 100003])
+def test_prange_loops_with_reads_loaded_ahead(env, n):
+    """Loops whose unconditional reads are loaded ahead of the body, beside
+    conditional reads and a loop that skips iterations (which load nothing
+    ahead): results as the Python loops give them, at sizes with whole and
+    ragged rounds."""
+    hip, ops, orc, workloads = env
+    rng = np.random.default_rng(n)
+    a, b, c, out0 = (rng.standard_normal(n) for _ in range(4))
+    want = out0.copy()
+    x = a + want
+    y = np.where(x > 0, b, 0.0)
+    y = np.where(y > 1.0, c, y)
+    want = x + y
+    d_out = hip.asarray(out0.copy())
+    njit(parallel=True)(cases.loop_reads)(n, hip.asarray(a), hip.asarray(b), hip.asarray(c), d_out)
+    np.testing.assert_array_equal(d_out.asnumpy(), want)
+    d_out = hip.asarray(out0.copy())
+    njit(parallel=True)(cases.loop_leaves_early)(n, hip.asarray(a), d_out)
+    want = out0.copy()
+    want[::2] = a[::2]
+    np.testing.assert_array_equal(d_out.asnumpy(), want)
+
+
 def test_enqueued_launches_are_covered_by_synchronize(env):
     """Launches put on the queue without waiting (the benchmark's timing path)
     are finished when the context's synchronize() returns; their events stay

@@ -344,6 +344,34 @@ def test_fused_maps_take_several_elements_per_lane(K, tmp_path, monkeypatch):
     assert ck.elements_per_thread == 1 and "nmk_rep" not in ck.source
 
 
+def test_prange_loops_load_what_every_iteration_reads_ahead(K):
+    import njit_cases
+    f64, i64 = kc.Array(kc.FLOAT64, 1), kc.INT64
+    mode, ndim, types = _njit_types("black_scholes_loop")
+    ck = kc.translate(njit_cases.black_scholes_loop, types, ndim, K, mode=mode, noalias=True,
+                      elements_per_thread=4)
+    assert "nmk_ahead_price[nmk_rep] = *(&v_price_p[g]);" in ck.source
+    assert "v_P = nmk_pf_price;" in ck.source and "v_T = nmk_pf_t;" in ck.source
+    # overlapping arguments, or one element per lane: every load where it is written
+    for kw in ({"noalias": False, "elements_per_thread": 4},
+               {"noalias": True, "elements_per_thread": 1}):
+        ck = kc.translate(njit_cases.black_scholes_loop, types, ndim, K, mode=mode, **kw)
+        assert "nmk_ahead" not in ck.source and "v_P = v_price.p[" in ck.source
+    # Only reads that every iteration performs: not behind a condition, not
+    # in a loop that leaves early, not of an array the function also writes.
+    ck = kc.translate(njit_cases.loop_reads, [i64, f64, f64, f64, f64], 1, K, mode="parallel",
+                      noalias=True, elements_per_thread=4)
+    assert "nmk_ahead_a" in ck.source                  # x = a[i] + ...
+    assert "nmk_ahead_b" not in ck.source              # b[i] if x > 0 else 0.0
+    assert "nmk_ahead_c" not in ck.source              # c[i] inside an if statement
+    assert "nmk_ahead_out" not in ck.source            # written
+    ck = kc.translate(njit_cases.loop_leaves_early, [i64, f64, f64], 1, K, mode="parallel",
+                      noalias=True, elements_per_thread=4)
+    assert "nmk_ahead" not in ck.source
+    # (continue ends the iteration: the work-item body returns)
+    assert "return;" in ck.source and "continue;" not in ck.source
+
+
 def test_prange_reductions(K, tmp_path, monkeypatch):
     import njit_cases
     monkeypatch.setattr(kc, "CACHE_DIR", str(tmp_path))
