@@ -472,6 +472,10 @@ class LaunchPlan:
         self._descs = params.build()
         self._lock = threading.Lock()     # slots are rewritten per call
         self._launch = (ctx.queue, kern, *self.grid, *self.block, NO_DEPS, self._descs)
+        # what later arguments must look like (the kernel and its geometry
+        # were chosen for these types, shapes and strides)
+        self._key = plan_key(args)
+        self._ret_key = None if ret is None else (ret.dtype, ret.shape, ret.strides)
 
     def _refresh(self, args, ret, partials):
         """Rewrites the pointer and scalar slots (the lock is held)."""
@@ -492,6 +496,19 @@ class LaunchPlan:
     def enqueue(self, args=None, ret=None):
         """Launches without waiting and returns the event (the caller passes
         it to ``retire``): back-to-back launches for timing."""
+        if args is not None:
+            # (run() is called with arguments its caller has already matched
+            # to this plan; here they come from anywhere)
+            if plan_key(args) != self._key:
+                raise ValueError(
+                    f"{self.func_name}: arguments differ in type, shape or strides from "
+                    "those this launch was prepared for")
+            if (ret is None) != (self._ret_key is None) or (
+                    ret is not None and (ret.dtype, ret.shape, ret.strides) != self._ret_key):
+                raise ValueError(
+                    f"{self.func_name}: the result array must have dtype "
+                    f"{self._ret_key[0] if self._ret_key else None} and the shape and strides "
+                    "this launch was prepared for")
         with self._lock:                  # the launch call copies the values out
             if args is not None:
                 self._refresh(args, ret, ())

@@ -356,6 +356,18 @@ def test_enqueued_launches_are_covered_by_synchronize(env):
     for e in events:
         plan.retire(e)
     assert not any(e in ctx.pending for e in events)
+    # arguments that do not fit the prepared launch are refused, not launched
+    with pytest.raises(ValueError, match="differ in type, shape or strides"):
+        plan.enqueue([d_a, hip.asarray(np.zeros(a.size, np.float32))])
+    with pytest.raises(ValueError, match="differ in type, shape or strides"):
+        plan.enqueue([hip.asarray(a[:100]), outs[0]])
+    g = njit(lambda a, b: a * 2 + b)          # a generated kernel that returns an array
+    small = hip.asarray(np.arange(64, dtype=np.int32))
+    g(small, small)
+    with pytest.raises(ValueError, match="result array must have dtype"):
+        g.last_plan.enqueue([small, small], hip.asarray(np.zeros(64, np.int16)))
+    with pytest.raises(ValueError, match="result array must have dtype"):
+        g.last_plan.enqueue([small, small])
 
 
 def test_repeated_calls_replay_stored_launches(env):
