@@ -499,12 +499,14 @@ class LaunchPlan:
         if args is not None:
             # (run() is called with arguments its caller has already matched
             # to this plan; here they come from anywhere)
-            if plan_key(args) != self._key:
+            if len(args) != len(self._key) or not all(
+                    _fits(k, a) for k, a in zip(self._key, plan_key(args))):
                 raise ValueError(
                     f"{self.func_name}: arguments differ in type, shape or strides from "
                     "those this launch was prepared for")
             if (ret is None) != (self._ret_key is None) or (
-                    ret is not None and (ret.dtype, ret.shape, ret.strides) != self._ret_key):
+                    ret is not None and
+                    not _fits(self._ret_key, (ret.dtype, ret.shape, ret.strides))):
                 raise ValueError(
                     f"{self.func_name}: the result array must have dtype "
                     f"{self._ret_key[0] if self._ret_key else None} and the shape and strides "
@@ -544,6 +546,32 @@ class LaunchPlan:
             raise IndexError(
                 f"kernel '{self.func_name}' indexed an array out of bounds (the access "
                 "was redirected to element 0)")
+
+
+def _dense_size(shape, strides, itemsize):
+    """Element count of a C-contiguous array, None for any other layout."""
+    expect = itemsize
+    for n, st in zip(reversed(shape), reversed(strides)):
+        if n != 1 and st != expect:
+            return None
+        expect *= n
+    return expect // itemsize
+
+
+def _fits(planned, given):
+    """Whether an argument (its ``plan_key`` entry) can stand in for the one
+    a launch was prepared with: the same entry, or -- the dispatchers prepare
+    launches on arrays with their dimensions merged -- a dense array of the
+    same type and size as a dense planned one."""
+    if planned == given:
+        return True
+    if not (isinstance(planned, tuple) and isinstance(given, tuple)):
+        return False
+    (pd, ps, pst), (gd, gs, gst) = planned, given
+    if pd != gd:
+        return False
+    size = _dense_size(ps, pst, pd.itemsize)
+    return size is not None and size == _dense_size(gs, gst, gd.itemsize)
 
 
 def plan_key(args):

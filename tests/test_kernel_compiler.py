@@ -541,3 +541,24 @@ def test_array_operands_follow_the_array_typing_rule(K):
         return u ** 2
 
     assert ret(through_names, [f32, i32]) == np.float32
+
+
+def test_which_arguments_fit_a_prepared_launch():
+    """A stored launch accepts the arrays it was prepared with, or dense
+    arrays of the same type and size (launches are prepared on arrays with
+    their dimensions merged); anything else could be addressed out of bounds."""
+    from numba_mlir_amd.mlir import kernel_impl as ki
+    f8, f4 = np.dtype("f8"), np.dtype("f4")
+    assert ki._dense_size((4096, 4096), (32768, 8), 8) == 4096 * 4096
+    assert ki._dense_size((3, 1, 5), (40, 8, 8), 8) == 15          # a stride of a 1-extent is free
+    assert ki._dense_size((4, 4), (64, 8), 8) is None              # rows with gaps
+    assert ki._dense_size((4, 4), (8, 32), 8) is None              # column-major
+    merged = (f8, (16777216,), (8,))
+    assert ki._fits(merged, (f8, (4096, 4096), (32768, 8)))
+    assert ki._fits(merged, merged)
+    assert not ki._fits(merged, (f4, (4096, 4096), (16384, 4)))
+    assert not ki._fits(merged, (f8, (4096, 4095), (32760, 8)))
+    assert not ki._fits((f8, (16,), (8,)), (f8, (4, 4), (64, 8)))
+    assert ki._fits((f8, (4, 4), (64, 8)), (f8, (4, 4), (64, 8)))   # the same strided layout
+    assert ki._fits(float, float) and not ki._fits(float, int)
+    assert not ki._fits(np.dtype("f4"), merged)
