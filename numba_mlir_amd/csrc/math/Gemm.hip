@@ -449,24 +449,37 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       const bool xKc = xk == 1, yNc = yn == 1;
       const int64_t ldx = xKc ? xm : xk, ldy = yNc ? yk : yn;
       constexpr int VEC = Mfma<T>::VEC, BK = Mfma<T>::BK;
+      // The matrix-core kernel takes the part of the problem that is whole
+      // tiles, Z[0:Mt, 0:Nt] over k in [0, Kt); the strided kernel adds the
+      // rest of K to that block and computes the rows and columns beyond it
+      // (4000^3: 3968 x 3968 x 4000 on the matrix cores, 26 -> 65 TFLOP/s).
       // float32: 256 x 256 block tiles (one block per CU on a 4096^2
       // problem) when the shape allows and there are enough tiles to fill the
       // 256 CUs, 128 x 128 otherwise (measured within 3 % of each other; the
       // larger tile halves the operand traffic).  float64: 128 x 128.  The
       // large tile advances K in slabs of 2 BK where K allows (half the
       // barriers; 144 against 142 TFLOP/s on 4096^3).
-      const bool big = sizeof(T) == 4 && Mz % 256 == 0 && Nz % 256 == 0 &&
-                       (Mz / 256) * (Nz / 256) >= 192;
+      const int64_t Mt = Mz - Mz % 128, Nt = Nz - Nz % 128, Kt = K - K % BK;
+      const bool big = sizeof(T) == 4 && Mt % 256 == 0 && Nt % 256 == 0 &&
+                       (Mt / 256) * (Nt / 256) >= 192;
       const int BM = big ? 256 : 128, BN = BM;
       const bool unitOk = (xk == 1 || xm == 1) && (yk == 1 || yn == 1);
-      if (unitOk && K > 0 && Mz % BM == 0 && Nz % BN == 0 && K % BK == 0 &&
+      // worth it when the tiled part is most of the work and fills at least
+      // half the CUs (1000^3 is 49 tiles: the strided kernel alone, on 1024
+      // blocks, takes half the time of tiles plus three edge launches)
+      const bool whole = Mt == Mz && Nt == Nz && Kt == K;
+      const bool mostly = whole ||
+                          (double(Mt) * double(Nt) * double(Kt) >=
+                               0.5 * double(Mz) * double(Nz) * double(K) &&
+                           (Mt / 128) * (Nt / 128) >= 128);
+      if (unitOk && mostly && Mt > 0 && Nt > 0 && Kt > 0 &&
           ldx % VEC == 0 && ldy % VEC == 0 && ldx > 0 && ldy > 0 &&
           aligned16(X) && aligned16(Y) && M <= 0x7fffffff && N <= 0x7fffffff &&
-          K <= 0x7fffffff && Mz / BM <= 65535) {
-        dim3 grid(unsigned(Nz / BN), unsigned(Mz / BM), 1);
+          K <= 0x7fffffff && Mz <= 65535 * 32) {
+        dim3 grid(unsigned(Nt / BN), unsigned(Mt / BM), 1);
 #define NMHIP_GEMM_LAUNCH(SLAB, TM, TN, XKC, YNC)                              \
   hipLaunchKernelGGL((gemm_mfma<T, SLAB, TM, TN, XKC, YNC>), grid, dim3(256),  \
-                     0, stream, X, Y, cData, int(Mz), int(Nz), int(K), ldx,    \
+                     0, stream, X, Y, cData, int(Mt), int(Nt), int(Kt), ldx,   \
                      ldy, ldz, alpha, beta)
 #define NMHIP_GEMM_LAYOUTS(SLAB, TM, TN)                                       \
   do {                                                                         \
@@ -480,22 +493,37 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       NMHIP_GEMM_LAUNCH(SLAB, TM, TN, false, false);                           \
   } while (0)
         if constexpr (sizeof(T) == 4) {
-          if (big && K % (2 * BK) == 0) {
+          if (big && Kt % (2 * BK) == 0) {
             NMHIP_GEMM_LAYOUTS(2 * BK, 4, 4);
-            lastKernel = "sgemm_mfma_256x256";
+            lastKernel = whole ? "sgemm_mfma_256x256" : "sgemm_mfma_256x256+edges";
           } else if (big) {
             NMHIP_GEMM_LAYOUTS(BK, 4, 4);
-            lastKernel = "sgemm_mfma_256x256";
+            lastKernel = whole ? "sgemm_mfma_256x256" : "sgemm_mfma_256x256+edges";
           } else {
             NMHIP_GEMM_LAYOUTS(BK, 2, 2);
-            lastKernel = "sgemm_mfma_128x128";
+            lastKernel = whole ? "sgemm_mfma_128x128" : "sgemm_mfma_128x128+edges";
           }
         } else {
           NMHIP_GEMM_LAYOUTS(BK, 4, 4);
-          lastKernel = "dgemm_mfma_128x128";
+          lastKernel = whole ? "dgemm_mfma_128x128" : "dgemm_mfma_128x128+edges";
         }
 #undef NMHIP_GEMM_LAYOUTS
 #undef NMHIP_GEMM_LAUNCH
+        // Z[m0:m0+m, n0:n0+n] = alpha X[m0.., k0:k0+k] Y[k0.., n0..] + bz Z
+        auto edge = [&](int64_t m0, int64_t m, int64_t n0, int64_t n, int64_t k0,
+                        int64_t k, T bz) {
+          if (m <= 0 || n <= 0)
+            return;
+          dim3 g{unsigned((n + 31) / 32), unsigned((m + 31) / 32), 1};
+          hipLaunchKernelGGL(gemm_generic<T>, g, dim3(256), 0, stream,
+                             X + m0 * xm + k0 * xk, Y + k0 * yk + n0 * yn,
+                             cData + m0 * ldz + n0, m, n, k, xm, xk, yk, yn, ldz,
+                             int64_t(1), alpha, bz);
+        };
+        if (Kt < K)
+          edge(0, Mt, 0, Nt, Kt, K - Kt, T(1)); // the rest of K, on top
+        edge(Mt, Mz - Mt, 0, Nz, 0, K, beta);   // rows below the tiles
+        edge(0, Mt, Nt, Nz - Nt, 0, K, beta);   // columns right of them
         launched = true;
       }
     }

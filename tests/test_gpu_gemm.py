@@ -81,7 +81,8 @@ def test_internal_gemm_fixture_grid(env):
 @pytest.mark.parametrize("ta,tb,tc", list(itertools.product([False, True], repeat=3)))
 @pytest.mark.parametrize("m,n,k", [(33, 29, 47), (128, 128, 16), (1, 1, 1), (64, 1, 300),
                                    (256, 384, 64), (4096, 3072, 32), (4096, 3072, 48),
-                                   (3072, 4096, 96)])
+                                   (3072, 4096, 96), (300, 260, 100), (257, 129, 17),
+                                   (1000, 1000, 1000), (131, 4100, 40), (1500, 2000, 52)])
 def test_layouts_against_float64(env, ta, tb, tc, m, n, k):
     """Every stride pattern the entry point accepts (row/column major A, B, C)."""
     hip, ops, orc, mrt = env
@@ -93,14 +94,41 @@ def test_layouts_against_float64(env, ta, tb, tc, m, n, k):
     d_c = _to_dev(hip, lay(c0, tc))
     ops.gemm(_to_dev(hip, lay(a, ta)), _to_dev(hip, lay(b, tb)), d_c, 0.5, 2.0)
     got = d_c.asnumpy()
-    if m % 128 == 0 and n % 128 == 0 and k % 16 == 0:
+    mt, nt, kt = m - m % 128, n - n % 128, k - k % 16
+    if (mt, nt, kt) == (m, n, k):
         # every layout of a tile-aligned problem runs on the matrix cores
-        assert mrt.last_kernel().startswith("sgemm_mfma")
-    else:
+        assert mrt.last_kernel() in ("sgemm_mfma_128x128", "sgemm_mfma_256x256")
+    elif 2 * mt * nt * kt < m * n * k or (mt // 128) * (nt // 128) < 128:
         assert mrt.last_kernel() == "sgemm_generic"
+    else:
+        # whole tiles on the matrix cores, the edges on the strided kernel
+        # (when the leading dimensions allow 128-bit loads)
+        assert mrt.last_kernel() in ("sgemm_generic", "sgemm_mfma_128x128+edges",
+                                     "sgemm_mfma_256x256+edges")
     truth = 2.0 * c0 + 0.5 * (a.astype(np.float64) @ b.astype(np.float64))
     bound = 1e-5 * (2.0 * np.abs(c0) + 0.5 * (np.abs(a).astype(np.float64) @ np.abs(b))) + 1e-30
     assert (np.abs(got - truth) <= bound).all()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("m,n,k", [(2000, 1500, 1000), (1540, 1420, 2004), (1409, 1536, 16),
+                                   (4100, 4200, 36)])
+def test_ragged_shapes_split_into_tiles_and_edges(env, dtype, m, n, k):
+    """Shapes that are not whole tiles: the tiled part runs on the matrix
+    cores, the rest of K, the last rows and the last columns on the strided
+    kernel -- with alpha and beta applied once to every element."""
+    hip, ops, orc, mrt = env
+    rng = np.random.default_rng(m + n + k)
+    a = rng.standard_normal((m, k)).astype(dtype)
+    b = rng.standard_normal((k, n)).astype(dtype)
+    c0 = rng.standard_normal((m, n)).astype(dtype)
+    d_c = _to_dev(hip, c0)
+    ops.gemm(_to_dev(hip, a), _to_dev(hip, b), d_c, 1.5, -0.5)
+    assert mrt.last_kernel().endswith("+edges")
+    truth = -0.5 * c0.astype(np.float64) + 1.5 * (a.astype(np.float64) @ b.astype(np.float64))
+    scale = 0.5 * np.abs(c0) + 1.5 * (np.abs(a).astype(np.float64) @ np.abs(b))
+    rel = 1e-5 if dtype == np.float32 else 1e-13
+    assert (np.abs(d_c.asnumpy() - truth) <= rel * scale + 1e-30).all()
 
 
 # Tolerance for float32 matmul: |gpu - truth| <= 1e-4 * (|a| @ |b|) elementwise
