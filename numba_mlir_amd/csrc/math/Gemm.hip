@@ -75,9 +75,10 @@ thread_local const char *lastKernel = "";
 //   f64 16x16x4: A[l % 16][l / 16], B[l / 16][l % 16],
 //                D reg r = D[4*r + l/16][l % 16]                  (4 regs)
 //
-// Requirements (checked by the host): M and N multiples of the block tile,
-// K % BK == 0, leading dimensions multiples of the 128-bit vector, A and B
-// 16-byte aligned.
+// Requirements (checked by the host): leading dimensions multiples of the
+// 128-bit vector, A and B 16-byte aligned; M and N multiples of the block
+// tile and K % BK == 0, or (GUARD) extents along each operand's contiguous
+// dimension multiples of the vector.
 template <typename T> struct Mfma;
 template <> struct Mfma<float> {
   typedef floatx4 Vec;   // 128-bit global access
@@ -114,7 +115,11 @@ template <> struct Mfma<double> {
 // to LDS[k][x].  NV 128-bit words per thread.
 //   K_CONTIG: thread -> (x = tid / (BK/VEC) + X_STEP i, k = VEC (tid % (BK/VEC)) ..)
 //   else    : thread -> (k = tid / (X/VEC) + K_ROWS i, x = VEC (tid % (X/VEC)) ..)
-template <typename T, int X, int BK, bool K_CONTIG> struct SlabFetch {
+// GUARD: the operand need not fill the tile or the last slab; a word that
+// lies outside it (words are whole: the host checks that the extents along
+// the contiguous dimension are multiples of the word) is read from the
+// operand's first word instead and replaced by zeros.
+template <typename T, int X, int BK, bool K_CONTIG, bool GUARD> struct SlabFetch {
   typedef Mfma<T> M;
   typedef typename M::Vec Vec;
   static constexpr int NV = X * BK / (M::VEC * 256);
@@ -125,10 +130,15 @@ template <typename T, int X, int BK, bool K_CONTIG> struct SlabFetch {
   const T *base;
   int64_t ld;
   Vec reg[NV];
+  const T *first; // GUARD: the operand's first word
+  int xLeft;      // GUARD: extent - origin - x: how many x from this thread's on
+  int kEnd;       // GUARD: K
 
   __device__ __forceinline__ void init(const T *p, int64_t ld_, int origin,
-                                       int tid) {
+                                       int tid, int extent = 0, int K = 0) {
     ld = ld_;
+    first = p;
+    kEnd = K;
     if (K_CONTIG) {
       x = tid / (BK / M::VEC);
       k = (tid % (BK / M::VEC)) * M::VEC;
@@ -138,13 +148,24 @@ template <typename T, int X, int BK, bool K_CONTIG> struct SlabFetch {
       x = (tid % (X / M::VEC)) * M::VEC;
       base = p + int64_t(k) * ld + origin + x;
     }
+    xLeft = extent - origin - x;
   }
   __device__ __forceinline__ void fetch(int k0) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i)
-      reg[i] = *reinterpret_cast<const Vec *>(
-          K_CONTIG ? base + int64_t(X_STEP * i) * ld + k0
-                   : base + int64_t(k0 + K_ROWS * i) * ld);
+    for (int i = 0; i < NV; ++i) {
+      const T *src = K_CONTIG ? base + int64_t(X_STEP * i) * ld + k0
+                              : base + int64_t(k0 + K_ROWS * i) * ld;
+      if (GUARD) {
+        const bool inside = K_CONTIG ? (X_STEP * i < xLeft && k0 + k < kEnd)
+                                     : (0 < xLeft && k0 + k + K_ROWS * i < kEnd);
+        const Vec v = *reinterpret_cast<const Vec *>(inside ? src : first);
+#pragma unroll
+        for (int q = 0; q < M::VEC; ++q)
+          reg[i][q] = inside ? v[q] : T(0);
+      } else {
+        reg[i] = *reinterpret_cast<const Vec *>(src);
+      }
+    }
   }
   // Words [i0, i1) of the slab to LDS.
   __device__ __forceinline__ void stash(T (*lds)[X + M::PAD], int i0 = 0,
@@ -172,7 +193,7 @@ template <int MASK> __device__ __forceinline__ void sched_groups(int n) {
 
 // float64 tiles need under 256 registers a lane: two blocks share a CU and
 // fill each other's stalls.  float32 256 x 256 tiles take a CU each.
-template <typename T, int BK, int TM, int TN, bool A_KC, bool B_NC>
+template <typename T, int BK, int TM, int TN, bool A_KC, bool B_NC, bool GUARD = false>
 __global__ __launch_bounds__(256, sizeof(T) == 8 ? 2 : 1) void
 gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
           int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, T alpha,
@@ -190,10 +211,10 @@ gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
   const int bm = blockIdx.y * BM;
   const int bn = blockIdx.x * BN;
 
-  SlabFetch<T, BM, BK, A_KC> fa;
-  SlabFetch<T, BN, BK, !B_NC> fb;
-  fa.init(A, lda, bm, tid);
-  fb.init(B, ldb, bn, tid);
+  SlabFetch<T, BM, BK, A_KC, GUARD> fa;
+  SlabFetch<T, BN, BK, !B_NC, GUARD> fb;
+  fa.init(A, lda, bm, tid, M, K);
+  fb.init(B, ldb, bn, tid, N, K);
 
   typename MF::Acc acc[TM][TN];
 #pragma unroll
@@ -204,7 +225,7 @@ gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
       for (int r = 0; r < MF::NACC; ++r)
         acc[i][j][r] = T(0);
 
-  const int nSlabs = K / BK;
+  const int nSlabs = (K + BK - 1) / BK; // (a multiple of BK unless GUARD)
   const int kLane = lane / TILE, xLane = lane % TILE;
   // Operand fragments of one step, double-buffered in registers.
   T a[2][TM], b[2][TN];
@@ -314,6 +335,8 @@ gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
       for (int r = 0; r < MF::NACC; ++r) {
         const int row =
             bm + wm * (TM * TILE) + i * TILE + MF::accRow(r, lane);
+        if (GUARD && !(row < M && col < N))
+          continue;
         T *dst = C + int64_t(row) * ldc + col;
         T v = alpha * acc[i][j][r];
         if (beta != T(0))
@@ -472,7 +495,46 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
                           (double(Mt) * double(Nt) * double(Kt) >=
                                0.5 * double(Mz) * double(Nz) * double(K) &&
                            (Mt / 128) * (Nt / 128) >= 128);
-      if (unitOk && mostly && Mt > 0 && Nt > 0 && Kt > 0 &&
+      // Ragged shapes whose 128-bit words are whole (the extent along each
+      // operand's contiguous dimension a multiple of the word): one launch
+      // of 128 x 128 tiles that read zeros beyond the operands and store
+      // only inside Z.
+      const bool wordsWhole = (xKc ? K : Mz) % VEC == 0 && (yNc ? Nz : K) % VEC == 0;
+      const int64_t tilesM = (Mz + 127) / 128, tilesN = (Nz + 127) / 128;
+      // (only K ragged: the tiles as they are plus the rest of K on the
+      // strided kernel is faster, 116 against 106 TFLOP/s on 4096 x 4096 x 4100)
+      const bool onlyK = Mt == Mz && Nt == Nz && mostly;
+      if (!whole && !onlyK && unitOk && wordsWhole && K > 0 && ldx % VEC == 0 && ldy % VEC == 0 &&
+          ldx > 0 && ldy > 0 && aligned16(X) && aligned16(Y) && M <= 0x7fffffff &&
+          N <= 0x7fffffff && K <= 0x7fffffff - 64 && tilesM <= 65535 &&
+          tilesM * tilesN >= 16) {
+        dim3 grid(unsigned(tilesN), unsigned(tilesM), 1);
+#define NMHIP_GEMM_RAGGED(TM, TN, XKC, YNC)                                    \
+  hipLaunchKernelGGL((gemm_mfma<T, BK, TM, TN, XKC, YNC, true>), grid,         \
+                     dim3(256), 0, stream, X, Y, cData, int(Mz), int(Nz),      \
+                     int(K), ldx, ldy, ldz, alpha, beta)
+#define NMHIP_GEMM_RAGGED_LAYOUTS(TM, TN)                                      \
+  do {                                                                         \
+    if (xKc && yNc)                                                            \
+      NMHIP_GEMM_RAGGED(TM, TN, true, true);                                   \
+    else if (xKc)                                                              \
+      NMHIP_GEMM_RAGGED(TM, TN, true, false);                                  \
+    else if (yNc)                                                              \
+      NMHIP_GEMM_RAGGED(TM, TN, false, true);                                  \
+    else                                                                       \
+      NMHIP_GEMM_RAGGED(TM, TN, false, false);                                 \
+  } while (0)
+        if constexpr (sizeof(T) == 4) {
+          NMHIP_GEMM_RAGGED_LAYOUTS(2, 2);
+          lastKernel = "sgemm_mfma_128x128_ragged";
+        } else {
+          NMHIP_GEMM_RAGGED_LAYOUTS(4, 4);
+          lastKernel = "dgemm_mfma_128x128_ragged";
+        }
+#undef NMHIP_GEMM_RAGGED_LAYOUTS
+#undef NMHIP_GEMM_RAGGED
+        launched = true;
+      } else if (unitOk && mostly && Mt > 0 && Nt > 0 && Kt > 0 &&
           ldx % VEC == 0 && ldy % VEC == 0 && ldx > 0 && ldy > 0 &&
           aligned16(X) && aligned16(Y) && M <= 0x7fffffff && N <= 0x7fffffff &&
           K <= 0x7fffffff && Mz <= 65535 * 32) {

@@ -98,37 +98,77 @@ def test_layouts_against_float64(env, ta, tb, tc, m, n, k):
     if (mt, nt, kt) == (m, n, k):
         # every layout of a tile-aligned problem runs on the matrix cores
         assert mrt.last_kernel() in ("sgemm_mfma_128x128", "sgemm_mfma_256x256")
-    elif 2 * mt * nt * kt < m * n * k or (mt // 128) * (nt // 128) < 128:
+    elif -(-m // 128) * -(-n // 128) < 16:
         assert mrt.last_kernel() == "sgemm_generic"
     else:
         # whole tiles on the matrix cores, the edges on the strided kernel
         # (when the leading dimensions allow 128-bit loads)
         assert mrt.last_kernel() in ("sgemm_generic", "sgemm_mfma_128x128+edges",
-                                     "sgemm_mfma_256x256+edges")
+                                     "sgemm_mfma_256x256+edges", "sgemm_mfma_128x128_ragged")
     truth = 2.0 * c0 + 0.5 * (a.astype(np.float64) @ b.astype(np.float64))
     bound = 1e-5 * (2.0 * np.abs(c0) + 0.5 * (np.abs(a).astype(np.float64) @ np.abs(b))) + 1e-30
     assert (np.abs(got - truth) <= bound).all()
 
 
+def _check_scaled(got, a, b, c0, alpha, beta, rel):
+    truth = beta * c0.astype(np.float64) + alpha * (a.astype(np.float64) @ b.astype(np.float64))
+    scale = abs(beta) * np.abs(c0) + abs(alpha) * (np.abs(a).astype(np.float64) @ np.abs(b))
+    assert (np.abs(got - truth) <= rel * scale + 1e-30).all()
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-@pytest.mark.parametrize("m,n,k", [(2000, 1500, 1000), (1540, 1420, 2004), (1409, 1536, 16),
-                                   (4100, 4200, 36)])
-def test_ragged_shapes_split_into_tiles_and_edges(env, dtype, m, n, k):
-    """Shapes that are not whole tiles: the tiled part runs on the matrix
-    cores, the rest of K, the last rows and the last columns on the strided
-    kernel -- with alpha and beta applied once to every element."""
+@pytest.mark.parametrize("m,n,k", [(2000, 1500, 1000), (1540, 1420, 2004), (1412, 1536, 20),
+                                   (4100, 4200, 36), (516, 520, 4)])
+def test_ragged_shapes_on_tiles_that_read_zeros_outside(env, dtype, m, n, k, ta, tb):
+    """Shapes that are not whole tiles but whose 128-bit words are whole run
+    in one launch of tiles that read zeros beyond the operands and store only
+    inside C: every layout, alpha and beta applied once to every element."""
     hip, ops, orc, mrt = env
     rng = np.random.default_rng(m + n + k)
     a = rng.standard_normal((m, k)).astype(dtype)
     b = rng.standard_normal((k, n)).astype(dtype)
     c0 = rng.standard_normal((m, n)).astype(dtype)
+    lay = lambda x, t: np.asfortranarray(x) if t else x
     d_c = _to_dev(hip, c0)
-    ops.gemm(_to_dev(hip, a), _to_dev(hip, b), d_c, 1.5, -0.5)
-    assert mrt.last_kernel().endswith("+edges")
-    truth = -0.5 * c0.astype(np.float64) + 1.5 * (a.astype(np.float64) @ b.astype(np.float64))
-    scale = 0.5 * np.abs(c0) + 1.5 * (np.abs(a).astype(np.float64) @ np.abs(b))
-    rel = 1e-5 if dtype == np.float32 else 1e-13
-    assert (np.abs(d_c.asnumpy() - truth) <= rel * scale + 1e-30).all()
+    ops.gemm(_to_dev(hip, lay(a, ta)), _to_dev(hip, lay(b, tb)), d_c, 1.5, -0.5)
+    assert mrt.last_kernel().endswith("_mfma_128x128_ragged")
+    _check_scaled(d_c.asnumpy(), a, b, c0, 1.5, -0.5, 1e-5 if dtype == np.float32 else 1e-13)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_ragged_k_alone_keeps_the_tiles(env, dtype):
+    """Whole tiles in M and N, a K that is not whole slabs: the tiles as they
+    are, the rest of K added by the strided kernel."""
+    hip, ops, orc, mrt = env
+    m, n, k = 1536, 2048, 100
+    rng = np.random.default_rng(6)
+    a = rng.standard_normal((m, k)).astype(dtype)
+    b = rng.standard_normal((k, n)).astype(dtype)
+    c0 = rng.standard_normal((m, n)).astype(dtype)
+    d_c = hip.asarray(c0)
+    ops.gemm(hip.asarray(a), hip.asarray(b), d_c, 1.5, -0.5)
+    assert mrt.last_kernel().endswith("_mfma_128x128+edges")
+    _check_scaled(d_c.asnumpy(), a, b, c0, 1.5, -0.5, 1e-5 if dtype == np.float32 else 1e-13)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_ragged_shapes_split_into_tiles_and_edges(env, dtype):
+    """Operands whose rows do not end on a 128-bit word (views of wider
+    arrays): the tiled part runs on the matrix cores, the rest of K, the last
+    rows and the last columns on the strided kernel."""
+    hip, ops, orc, mrt = env
+    m, n, k = 1540, 2052, 1001
+    rng = np.random.default_rng(5)
+    a_wide = rng.standard_normal((m, k + 3)).astype(dtype)
+    b = rng.standard_normal((k, n)).astype(dtype)
+    c0 = rng.standard_normal((m, n)).astype(dtype)
+    d_a = hip.asarray(a_wide)[:, :k]
+    d_c = hip.asarray(c0)
+    ops.gemm(d_a, hip.asarray(b), d_c, 1.5, -0.5)
+    assert mrt.last_kernel().endswith("_mfma_128x128+edges")
+    _check_scaled(d_c.asnumpy(), a_wide[:, :k], b, c0, 1.5, -0.5,
+                  1e-5 if dtype == np.float32 else 1e-13)
 
 
 # Tolerance for float32 matmul: |gpu - truth| <= 1e-4 * (|a| @ |b|) elementwise
