@@ -98,7 +98,7 @@ def test_missing_library_fails_loudly(tmp_path):
     """No fallback: if the runtime library is absent the import raises."""
     code = (
         "import numba_mlir_amd.mlir.utils as u\n"
-        f"u._PACKAGE_DIR = {str(tmp_path)!r}\n"
+        f"import pathlib; u.PACKAGE_DIR = pathlib.Path({str(tmp_path)!r})\n"
         "import os; os.environ.pop('PYTHONPATH', None)\n"
         "import numba_mlir_amd.mlir.gpu_runtime\n")
     proc = _run_child(code)
