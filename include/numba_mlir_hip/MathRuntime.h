@@ -59,9 +59,9 @@ void nmrtMathRuntimeFinalize(void);
 /* Name of the device kernel the most recent gemm call on this thread ran
  * ("sgemm_mfma_256x256", "sgemm_mfma_128x128", "dgemm_mfma_128x128",
  * "sgemm_generic", "dgemm_generic"; "<tile kernel>_ragged" for the guarded
- * instance that takes shapes which are not whole tiles, "<tile kernel>+edges"
- * when the strided kernel completed what the tiles left); for tests and
- * profiling. */
+ * instance that takes shapes which are not whole tiles, "_splitk" after
+ * either when K was cut into slices, "<tile kernel>+edges" when the strided
+ * kernel completed what the tiles left); for tests and profiling. */
 const char *nmhipMathLastKernel(void);
 
 #ifdef __cplusplus

@@ -181,7 +181,7 @@ nmk_sum_axis0_i32_i64(const int32_t *__restrict__ x, int64_t *__restrict__ out,
   awaitStores();
   __syncthreads();
   if (threadIdx.x == 0)
-    isLast = (takeTicket(&tickets[strip]) == gridDim.y - 1) ? 1u : 0u;
+    isLast = drawLastTicket(&tickets[strip], gridDim.y) ? 1u : 0u;
   __syncthreads();
   if (!isLast)
     return;
@@ -271,7 +271,7 @@ fullSumF32(const float *__restrict__ x, float *__restrict__ out, int64_t n,
   if (threadIdx.x == 0) {
     publish(partial + blockIdx.x, total);
     awaitStores();
-    isLast = (takeTicket(ticket) == gridDim.x - 1) ? 1u : 0u;
+    isLast = drawLastTicket(ticket, gridDim.x) ? 1u : 0u;
   }
   __syncthreads();
   if (!isLast)

@@ -16,6 +16,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <mutex>
 
 namespace {
 
@@ -193,16 +194,31 @@ template <int MASK> __device__ __forceinline__ void sched_groups(int n) {
 
 // float64 tiles need under 256 registers a lane: two blocks share a CU and
 // fill each other's stalls.  float32 256 x 256 tiles take a CU each.
+//
+// Split K (sliceK > 0): grid.z slices of sliceK elements of K (a multiple of
+// BK) each; slice z leaves its unscaled partial product in the workspace,
+// W[z][M][N] with row stride ldw, and gemm_splitk_fold adds the slices in
+// index order.  Used when the tiles alone would leave most CUs idle.
 template <typename T, int BK, int TM, int TN, bool A_KC, bool B_NC, bool GUARD = false>
 __global__ __launch_bounds__(256, sizeof(T) == 8 ? 2 : 1) void
 gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
           int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, T alpha,
-          T beta) {
+          T beta, int sliceK, T *__restrict__ W, int64_t ldw) {
   typedef Mfma<T> MF;
   constexpr int TILE = MF::TILE;
   constexpr int BM = 2 * TM * TILE, BN = 2 * TN * TILE;
   __shared__ __attribute__((aligned(16))) T As[2][BK][BM + MF::PAD];
   __shared__ __attribute__((aligned(16))) T Bs[2][BK][BN + MF::PAD];
+  if (sliceK > 0) {
+    const int k0 = blockIdx.z * sliceK;
+    A += A_KC ? int64_t(k0) : int64_t(k0) * lda;
+    B += B_NC ? int64_t(k0) * ldb : int64_t(k0);
+    K = K - k0 < sliceK ? K - k0 : sliceK;
+    C = W + int64_t(blockIdx.z) * int64_t(M) * ldw;
+    ldc = ldw;
+    alpha = T(1);
+    beta = T(0);
+  }
 
   const int tid = threadIdx.x;
   const int lane = tid % 64;
@@ -348,6 +364,41 @@ gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
 }
 
 // ---------------------------------------------------------------------------
+// C[m][n] = alpha * (W[0][m][n] + W[1][m][n] + ...) + beta * C[m][n]: the
+// slices of a split-K product added in index order (a fixed order, so the
+// result does not depend on which block finished first).  One thread per
+// 128-bit word of a row of W (ldw and the slice stride are multiples of the
+// word); stores to C are per element, C may end inside the last word.
+template <typename T>
+__global__ __launch_bounds__(256) void
+gemm_splitk_fold(const T *__restrict__ W, int slices, int64_t sliceStride,
+                 int64_t ldw, T *__restrict__ C, int M, int N, int64_t ldc,
+                 T alpha, T beta) {
+  typedef typename Mfma<T>::Vec Vec;
+  constexpr int VEC = Mfma<T>::VEC;
+  const int wordsPerRow = (N + VEC - 1) / VEC;
+  const int64_t word = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (word >= int64_t(M) * wordsPerRow)
+    return;
+  const int m = int(word / wordsPerRow);
+  const int n = int(word % wordsPerRow) * VEC;
+  const T *src = W + int64_t(m) * ldw + n;
+  Vec sum = *reinterpret_cast<const Vec *>(src);
+  for (int z = 1; z < slices; ++z)
+    sum += *reinterpret_cast<const Vec *>(src + z * sliceStride);
+  T *dst = C + int64_t(m) * ldc + n;
+#pragma unroll
+  for (int q = 0; q < VEC; ++q) {
+    if (n + q < N) {
+      T v = alpha * sum[q];
+      if (beta != T(0))
+        v += beta * dst[q];
+      dst[q] = v;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Any shape, any strides (element strides per dimension), float or double:
 // classic 32 x 32 LDS tiling, one output per thread x 4 rows, bounds checked.
 // Used for the transposed / column-major / ragged cases the MFMA kernel does
@@ -397,6 +448,92 @@ gemm_generic(const T *A, const T *B, T *C, int64_t M, int64_t N, int64_t K,
   }
 }
 
+// ---------------------------------------------------------------------------
+// Workspace of the split-K path: one hipMalloc'ed block per device, grown on
+// demand and released by nmrtMathRuntimeFinalize.
+constexpr int kMaxDevices = 64;
+struct DeviceWorkspace {
+  void *heap = nullptr;
+  size_t heapBytes = 0;
+};
+DeviceWorkspace workspaces[kMaxDevices];
+std::mutex workspaceMutex;
+
+DeviceWorkspace &workspaceOf(int device) {
+  if (device < 0 || device >= kMaxDevices)
+    fatal("mkl_gemm_device: device ordinal %d out of range\n", device);
+  return workspaces[device];
+}
+
+// Grown on demand; nullptr when the device has no memory left (the caller
+// then runs without splitting K).  The device must be current.
+void *heapWorkspace(int device, size_t bytes) {
+  std::lock_guard<std::mutex> lock(workspaceMutex);
+  DeviceWorkspace &w = workspaceOf(device);
+  if (bytes <= w.heapBytes)
+    return w.heap;
+  if (w.heap) {
+    checkHip(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    checkHip(hipFree(w.heap), "hipFree");
+    w.heap = nullptr;
+    w.heapBytes = 0;
+  }
+  const size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : bytes;
+  void *p = nullptr;
+  if (hipMalloc(&p, want) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  w.heap = p;
+  w.heapBytes = want;
+  return p;
+}
+
+void releaseHeapWorkspaces() {
+  std::lock_guard<std::mutex> lock(workspaceMutex);
+  for (int d = 0; d < kMaxDevices; ++d) {
+    DeviceWorkspace &w = workspaces[d];
+    if (!w.heap)
+      continue;
+    if (hipSetDevice(d) == hipSuccess)
+      (void)hipFree(w.heap);
+    w.heap = nullptr;
+    w.heapBytes = 0;
+  }
+}
+
+// How K is cut for a launch of `tiles` block tiles: 1 slice when the tiles
+// fill the GPU by themselves or K is short.
+struct SplitPlan {
+  int slices = 1;
+  int sliceK = 0;
+};
+SplitPlan planSplit(int64_t tiles, int64_t K, int BK, int blocksPerCu) {
+  SplitPlan plan;
+  const int64_t slots = int64_t(256) * blocksPerCu; // resident blocks
+  if (tiles <= 0 || tiles * 2 > slots)
+    return plan;
+  int64_t slices = slots / tiles;
+  if (slices > 16)
+    slices = 16;
+  const int64_t minSlice = int64_t(8) * BK; // at least eight slabs a slice
+  if (slices > K / minSlice)
+    slices = K / minSlice;
+  if (slices < 2)
+    return plan;
+  int64_t sliceK = (K + slices - 1) / slices;
+  sliceK = (sliceK + BK - 1) / BK * BK;
+  plan.sliceK = int(sliceK);
+  plan.slices = int((K + sliceK - 1) / sliceK);
+  if (plan.slices < 2) {
+    plan.slices = 1;
+    plan.sliceK = 0;
+  }
+  return plan;
+}
+
+enum WorkspaceKind { WORKSPACE_HEAP };
+
 template <typename T> struct MemrefOf;
 template <> struct MemrefOf<float> {
   typedef NmhipMemref2F32 type;
@@ -419,9 +556,10 @@ bool aligned16(const void *p) {
 }
 
 template <typename T>
-void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
-                const typename MemrefOf<T>::type *b,
-                typename MemrefOf<T>::type *c, T alpha, T beta) {
+int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
+               const typename MemrefOf<T>::type *b,
+               typename MemrefOf<T>::type *c, T alpha, T beta,
+               WorkspaceKind workspaceKind) {
   if (!queueObj || !a || !b || !c)
     fatal("mkl_gemm_device: null argument\n");
   auto *base = static_cast<numba::GPUQueueInterface *>(queueObj);
@@ -449,8 +587,32 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
   const T *bData = b->data + b->offset;
   T *cData = c->data + c->offset;
 
-  checkHip(hipSetDevice(queue->hipDevice()), "hipSetDevice");
+  const int device = queue->hipDevice();
+  checkHip(hipSetDevice(device), "hipSetDevice");
   auto stream = static_cast<hipStream_t>(queue->hipStream());
+
+  // Split-K workspace for `plan` over an [m, ldw] partial product per slice;
+  // leaves plan unsplit when the heap has no room.
+  bool tooLarge = false;
+  auto workspaceFor = [&](SplitPlan &plan, int64_t m, int64_t ldw) -> T * {
+    if (plan.slices < 2)
+      return nullptr;
+    const size_t bytes = size_t(plan.slices) * size_t(m) * size_t(ldw) * sizeof(T);
+    void *p = nullptr;
+    {
+      p = heapWorkspace(device, bytes);
+      if (!p)
+        plan = SplitPlan();
+    }
+    return static_cast<T *>(p);
+  };
+  auto fold = [&](const SplitPlan &plan, const T *W, int64_t m, int64_t n,
+                  int64_t ldw, int64_t ldz, T *Z) {
+    const int64_t words = m * ((n + Mfma<T>::VEC - 1) / Mfma<T>::VEC);
+    hipLaunchKernelGGL(gemm_splitk_fold<T>, dim3(unsigned((words + 255) / 256)),
+                       dim3(256), 0, stream, W, plan.slices, m * ldw, ldw, Z,
+                       int(m), int(n), ldz, alpha, beta);
+  };
 
   if (M > 0 && N > 0) {
     bool launched = false;
@@ -508,11 +670,16 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           ldx > 0 && ldy > 0 && aligned16(X) && aligned16(Y) && M <= 0x7fffffff &&
           N <= 0x7fffffff && K <= 0x7fffffff - 64 && tilesM <= 65535 &&
           tilesM * tilesN >= 16) {
-        dim3 grid(unsigned(tilesN), unsigned(tilesM), 1);
+        SplitPlan plan = planSplit(tilesM * tilesN, K, BK, sizeof(T) == 8 ? 2 : 1);
+        const int64_t ldw = (Nz + VEC - 1) / VEC * VEC;
+        T *W = workspaceFor(plan, Mz, ldw);
+        if (tooLarge)
+          return 1;
+        dim3 grid(unsigned(tilesN), unsigned(tilesM), unsigned(plan.slices));
 #define NMHIP_GEMM_RAGGED(TM, TN, XKC, YNC)                                    \
   hipLaunchKernelGGL((gemm_mfma<T, BK, TM, TN, XKC, YNC, true>), grid,         \
                      dim3(256), 0, stream, X, Y, cData, int(Mz), int(Nz),      \
-                     int(K), ldx, ldy, ldz, alpha, beta)
+                     int(K), ldx, ldy, ldz, alpha, beta, plan.sliceK, W, ldw)
 #define NMHIP_GEMM_RAGGED_LAYOUTS(TM, TN)                                      \
   do {                                                                         \
     if (xKc && yNc)                                                            \
@@ -526,11 +693,15 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
   } while (0)
         if constexpr (sizeof(T) == 4) {
           NMHIP_GEMM_RAGGED_LAYOUTS(2, 2);
-          lastKernel = "sgemm_mfma_128x128_ragged";
+          lastKernel = plan.slices > 1 ? "sgemm_mfma_128x128_ragged_splitk"
+                                       : "sgemm_mfma_128x128_ragged";
         } else {
           NMHIP_GEMM_RAGGED_LAYOUTS(4, 4);
-          lastKernel = "dgemm_mfma_128x128_ragged";
+          lastKernel = plan.slices > 1 ? "dgemm_mfma_128x128_ragged_splitk"
+                                       : "dgemm_mfma_128x128_ragged";
         }
+        if (plan.slices > 1)
+          fold(plan, W, Mz, Nz, ldw, ldz, cData);
 #undef NMHIP_GEMM_RAGGED_LAYOUTS
 #undef NMHIP_GEMM_RAGGED
         launched = true;
@@ -538,11 +709,17 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           ldx % VEC == 0 && ldy % VEC == 0 && ldx > 0 && ldy > 0 &&
           aligned16(X) && aligned16(Y) && M <= 0x7fffffff && N <= 0x7fffffff &&
           K <= 0x7fffffff && Mz <= 65535 * 32) {
-        dim3 grid(unsigned(Nt / BN), unsigned(Mt / BM), 1);
+        SplitPlan plan;
+        if (!big)
+          plan = planSplit((Mt / BM) * (Nt / BN), Kt, BK, sizeof(T) == 8 ? 2 : 1);
+        T *W = workspaceFor(plan, Mt, Nt);
+        if (tooLarge)
+          return 1;
+        dim3 grid(unsigned(Nt / BN), unsigned(Mt / BM), unsigned(plan.slices));
 #define NMHIP_GEMM_LAUNCH(SLAB, TM, TN, XKC, YNC)                              \
   hipLaunchKernelGGL((gemm_mfma<T, SLAB, TM, TN, XKC, YNC>), grid, dim3(256),  \
                      0, stream, X, Y, cData, int(Mt), int(Nt), int(Kt), ldx,   \
-                     ldy, ldz, alpha, beta)
+                     ldy, ldz, alpha, beta, plan.sliceK, W, int64_t(Nt))
 #define NMHIP_GEMM_LAYOUTS(SLAB, TM, TN)                                       \
   do {                                                                         \
     if (xKc && yNc)                                                            \
@@ -563,12 +740,22 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
             lastKernel = whole ? "sgemm_mfma_256x256" : "sgemm_mfma_256x256+edges";
           } else {
             NMHIP_GEMM_LAYOUTS(BK, 2, 2);
-            lastKernel = whole ? "sgemm_mfma_128x128" : "sgemm_mfma_128x128+edges";
+            lastKernel = plan.slices > 1
+                             ? (whole ? "sgemm_mfma_128x128_splitk"
+                                      : "sgemm_mfma_128x128_splitk+edges")
+                             : (whole ? "sgemm_mfma_128x128"
+                                      : "sgemm_mfma_128x128+edges");
           }
         } else {
           NMHIP_GEMM_LAYOUTS(BK, 4, 4);
-          lastKernel = whole ? "dgemm_mfma_128x128" : "dgemm_mfma_128x128+edges";
+          lastKernel = plan.slices > 1
+                           ? (whole ? "dgemm_mfma_128x128_splitk"
+                                    : "dgemm_mfma_128x128_splitk+edges")
+                           : (whole ? "dgemm_mfma_128x128"
+                                    : "dgemm_mfma_128x128+edges");
         }
+        if (plan.slices > 1)
+          fold(plan, W, Mt, Nt, Nt, ldz, cData);
 #undef NMHIP_GEMM_LAYOUTS
 #undef NMHIP_GEMM_LAUNCH
         // Z[m0:m0+m, n0:n0+n] = alpha X[m0.., k0:k0+k] Y[k0.., n0..] + bz Z
@@ -607,6 +794,7 @@ void deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
   }
   // The reference call returns only when C is complete (.wait(), 127/145).
   checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
+  return 0;
 }
 
 } // namespace
@@ -618,7 +806,7 @@ NMHIP_MATH_EXPORT void mkl_gemm_float32_device(void *queue,
                                                const NmhipMemref2F32 *b,
                                                float alpha, float beta,
                                                NmhipMemref2F32 *c) {
-  deviceGemm<float>(queue, a, b, c, alpha, beta);
+  (void)deviceGemm<float>(queue, a, b, c, alpha, beta, WORKSPACE_HEAP);
 }
 
 NMHIP_MATH_EXPORT void mkl_gemm_float64_device(void *queue,
@@ -626,10 +814,12 @@ NMHIP_MATH_EXPORT void mkl_gemm_float64_device(void *queue,
                                                const NmhipMemref2F64 *b,
                                                double alpha, double beta,
                                                NmhipMemref2F64 *c) {
-  deviceGemm<double>(queue, a, b, c, alpha, beta);
+  (void)deviceGemm<double>(queue, a, b, c, alpha, beta, WORKSPACE_HEAP);
 }
 
 NMHIP_MATH_EXPORT void nmrtMathRuntimeInit(void) {}
-NMHIP_MATH_EXPORT void nmrtMathRuntimeFinalize(void) {}
+NMHIP_MATH_EXPORT void nmrtMathRuntimeFinalize(void) {
+  releaseHeapWorkspaces();
+}
 
 NMHIP_MATH_EXPORT const char *nmhipMathLastKernel(void) { return lastKernel; }

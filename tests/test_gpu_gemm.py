@@ -21,6 +21,12 @@ def env(hip):
     return hip, ops, orc, math_runtime
 
 
+def _kernel(mrt):
+    """Name of the last gemm kernel without the split-K marker (whether K is
+    cut into slices depends only on how many tiles the shape has)."""
+    return mrt.last_kernel().replace("_splitk", "")
+
+
 def _printed(x):
     return np.array([float("%.6g" % v) for v in np.ravel(x)]).reshape(np.shape(x))
 
@@ -97,13 +103,13 @@ def test_layouts_against_float64(env, ta, tb, tc, m, n, k):
     mt, nt, kt = m - m % 128, n - n % 128, k - k % 16
     if (mt, nt, kt) == (m, n, k):
         # every layout of a tile-aligned problem runs on the matrix cores
-        assert mrt.last_kernel() in ("sgemm_mfma_128x128", "sgemm_mfma_256x256")
+        assert _kernel(mrt) in ("sgemm_mfma_128x128", "sgemm_mfma_256x256")
     elif -(-m // 128) * -(-n // 128) < 16:
         assert mrt.last_kernel() == "sgemm_generic"
     else:
         # whole tiles on the matrix cores, the edges on the strided kernel
         # (when the leading dimensions allow 128-bit loads)
-        assert mrt.last_kernel() in ("sgemm_generic", "sgemm_mfma_128x128+edges",
+        assert _kernel(mrt) in ("sgemm_generic", "sgemm_mfma_128x128+edges",
                                      "sgemm_mfma_256x256+edges", "sgemm_mfma_128x128_ragged")
     truth = 2.0 * c0 + 0.5 * (a.astype(np.float64) @ b.astype(np.float64))
     bound = 1e-5 * (2.0 * np.abs(c0) + 0.5 * (np.abs(a).astype(np.float64) @ np.abs(b))) + 1e-30
@@ -132,7 +138,7 @@ def test_ragged_shapes_on_tiles_that_read_zeros_outside(env, dtype, m, n, k, ta,
     lay = lambda x, t: np.asfortranarray(x) if t else x
     d_c = _to_dev(hip, c0)
     ops.gemm(_to_dev(hip, lay(a, ta)), _to_dev(hip, lay(b, tb)), d_c, 1.5, -0.5)
-    assert mrt.last_kernel().endswith("_mfma_128x128_ragged")
+    assert _kernel(mrt).endswith("_mfma_128x128_ragged")
     _check_scaled(d_c.asnumpy(), a, b, c0, 1.5, -0.5, 1e-5 if dtype == np.float32 else 1e-13)
 
 
@@ -148,7 +154,7 @@ def test_ragged_k_alone_keeps_the_tiles(env, dtype):
     c0 = rng.standard_normal((m, n)).astype(dtype)
     d_c = hip.asarray(c0)
     ops.gemm(hip.asarray(a), hip.asarray(b), d_c, 1.5, -0.5)
-    assert mrt.last_kernel().endswith("_mfma_128x128+edges")
+    assert _kernel(mrt).endswith("_mfma_128x128+edges")
     _check_scaled(d_c.asnumpy(), a, b, c0, 1.5, -0.5, 1e-5 if dtype == np.float32 else 1e-13)
 
 
@@ -166,7 +172,7 @@ def test_ragged_shapes_split_into_tiles_and_edges(env, dtype):
     d_a = hip.asarray(a_wide)[:, :k]
     d_c = hip.asarray(c0)
     ops.gemm(d_a, hip.asarray(b), d_c, 1.5, -0.5)
-    assert mrt.last_kernel().endswith("_mfma_128x128+edges")
+    assert _kernel(mrt).endswith("_mfma_128x128+edges")
     _check_scaled(d_c.asnumpy(), a_wide[:, :k], b, c0, 1.5, -0.5,
                   1e-5 if dtype == np.float32 else 1e-13)
 
@@ -192,7 +198,7 @@ def test_mfma_kernel(env, m, n, k):
     expect_kernel = "sgemm_mfma_256x256" if (m % 256 == 0 and n % 256 == 0 and
                                              (m // 256) * (n // 256) >= 192) \
         else "sgemm_mfma_128x128"
-    assert mrt.last_kernel() == expect_kernel
+    assert _kernel(mrt) == expect_kernel
     _check(got, a, b)
     if m * n * k <= 1 << 27:
         # against the oracle's float32 contraction (k innermost)
@@ -225,21 +231,23 @@ def test_identity_and_linearity_full_size(env):
     d_A, d_B = hip.asarray(A), hip.asarray(B)
     C = ops.dot(d_A, d_B).asnumpy()
     assert mrt.last_kernel().startswith("sgemm_mfma")
-    rows = np.array([0, 1, 63, 64, 127, 128, 2047, 2048, 4032, 4095])
-    truth = A[rows].astype(np.float64) @ B.astype(np.float64)
-    bound = 1e-4 * (np.abs(A[rows]).astype(np.float64) @ np.abs(B).astype(np.float64))
-    assert (np.abs(C[rows] - truth) <= bound).all()
-    assert np.linalg.norm(C[rows] - truth) <= 1e-4 * np.linalg.norm(truth)
-    # column checks too (catches a transposed tile)
-    cols = np.array([0, 31, 32, 100, 4095])
-    truth_c = A.astype(np.float64) @ B[:, cols].astype(np.float64)
-    assert np.linalg.norm(C[:, cols] - truth_c) <= 1e-4 * np.linalg.norm(truth_c)
+    # every element against the float64 product, in blocks of 512 rows
+    B64, absB = B.astype(np.float64), np.abs(B).astype(np.float64)
+    err2 = ref2 = 0.0
+    for r0 in range(0, 4096, 512):
+        rows = slice(r0, r0 + 512)
+        truth = A[rows].astype(np.float64) @ B64
+        bound = 1e-4 * (np.abs(A[rows]).astype(np.float64) @ absB)
+        diff = C[rows] - truth
+        assert (np.abs(diff) <= bound).all(), r0
+        err2 += float((diff * diff).sum())
+        ref2 += float((truth * truth).sum())
+    assert err2 <= (1e-4) ** 2 * ref2
     eye = hip.asarray(np.eye(4096, dtype=np.float32))
     assert np.array_equal(ops.dot(d_A, eye).asnumpy(), A)
     assert np.array_equal(ops.dot(eye, d_B).asnumpy(), B)
-    # numpy's own float32 sgemm as a second reference
-    np.testing.assert_allclose(C[::97, ::89], np.dot(A, B)[::97, ::89], rtol=0,
-                               atol=1e-4 * 64 * 3)
+    # numpy's own float32 sgemm as a second reference, every element
+    np.testing.assert_allclose(C, np.dot(A, B), rtol=0, atol=1e-4 * 64 * 3)
 
 
 @pytest.mark.parametrize("ta,tb,tc", list(itertools.product([False, True], repeat=3)))
@@ -254,7 +262,7 @@ def test_float64_mfma(env, ta, tb, tc, m, n, k):
     lay = lambda x, t: np.asfortranarray(x) if t else x
     d_c = _to_dev(hip, lay(c0, tc))
     ops.gemm(_to_dev(hip, lay(a, ta)), _to_dev(hip, lay(b, tb)), d_c, 1.25, -0.5)
-    assert mrt.last_kernel() == "dgemm_mfma_128x128"
+    assert _kernel(mrt) == "dgemm_mfma_128x128"
     got = d_c.asnumpy()
     truth = -0.5 * c0 + 1.25 * (a @ b)
     bound = 1e-13 * (0.5 * np.abs(c0) + 1.25 * (np.abs(a) @ np.abs(b)))
@@ -268,3 +276,42 @@ def test_float64_gemm(env):
     a, b = rng.standard_normal((70, 90)), rng.standard_normal((90, 50))
     got = ops.dot(hip.asarray(a), hip.asarray(b)).asnumpy()
     np.testing.assert_allclose(got, a @ b, rtol=1e-12, atol=1e-12)
+
+
+# ---- split K: few tiles, long K ------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("ta,tb,tc", [(False, False, False), (True, False, False),
+                                      (False, True, True), (True, True, False)])
+@pytest.mark.parametrize("m,n,k", [(1024, 1024, 1024), (128, 256, 4096), (512, 384, 2000),
+                                   (1000, 1000, 1000), (640, 516, 1028), (1280, 1280, 272)])
+def test_split_k(env, dtype, ta, tb, tc, m, n, k):
+    """Shapes with too few tiles to fill the GPU cut K into slices whose
+    partial products are added in slice order: every layout, alpha and beta
+    applied once, K that is not a whole number of slices or slabs, and the
+    same bits on a second run."""
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(m + 3 * n + 7 * k)
+    a = rng.standard_normal((m, k)).astype(dtype)
+    b = rng.standard_normal((k, n)).astype(dtype)
+    c0 = rng.standard_normal((m, n)).astype(dtype)
+    lay = lambda x, t: np.asfortranarray(x) if t else x
+    d_a, d_b = _to_dev(hip, lay(a, ta)), _to_dev(hip, lay(b, tb))
+    runs = []
+    for _ in range(2):
+        d_c = _to_dev(hip, lay(c0, tc))
+        ops.gemm(d_a, d_b, d_c, 1.5, -0.5)
+        assert "_splitk" in mrt.last_kernel(), mrt.last_kernel()
+        runs.append(d_c.asnumpy())
+    assert np.array_equal(runs[0], runs[1])
+    _check_scaled(runs[0], a, b, c0, 1.5, -0.5, 1e-5 if dtype == np.float32 else 1e-13)
+
+
+def test_split_k_beta_zero_ignores_c(env):
+    hip, ops, _, mrt = env
+    a = np.ones((256, 2048), np.float32)
+    b = np.ones((2048, 256), np.float32)
+    c = hip.asarray(np.full((256, 256), np.nan, np.float32))
+    ops.gemm(hip.asarray(a), hip.asarray(b), c, 1.0, 0.0)
+    assert "_splitk" in mrt.last_kernel()
+    assert (c.asnumpy() == 2048).all()
