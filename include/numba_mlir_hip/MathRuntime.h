@@ -52,6 +52,29 @@ void mkl_gemm_float64_device(void *queue, const NmhipMemref2F64 *a,
                              const NmhipMemref2F64 *b, double alpha,
                              double beta, NmhipMemref2F64 *c);
 
+/*
+ * mkl_gemm_float32_device for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  Same arguments, same
+ * kernels, same results as mkl_gemm_float32_device bit for bit; it calls no
+ * hipMalloc / hipFree.  Where that entry point takes split-K workspace from
+ * a heap block it grows on demand, this one uses a fixed 16 MiB array that
+ * lives in the library's device image on every GPU it runs on.  The first
+ * call on a device looks the array's address up (no allocation).  Returns 0,
+ * or 1 -- with a message on stderr and nothing launched -- when the product
+ * would need more split-K workspace than the array holds.  Only shapes with
+ * fewer than 128 tiles of 128 x 128 split K, into slices x tiles <= 256
+ * partial tiles of 64 KiB: 16 MiB is the most a float32 product asks for
+ * (1024 x 1024 with k >= 512 does), so the limit is a guard, not a case a
+ * float32 caller meets.  The array is shared by every call on a GPU and
+ * keeps the last call's partial products; nothing in it needs clearing,
+ * each slice is written before it is read.  Calls that overlap on one GPU
+ * race on it.
+ */
+int mkl_gemm_float32_device_noalloc(void *queue, const NmhipMemref2F32 *a,
+                                    const NmhipMemref2F32 *b, float alpha,
+                                    float beta, NmhipMemref2F32 *c);
+
 /* NumpyLinalg.cpp:178-183.  Not thread safe, as in the reference. */
 void nmrtMathRuntimeInit(void);
 void nmrtMathRuntimeFinalize(void);

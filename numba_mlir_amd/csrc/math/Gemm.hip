@@ -449,10 +449,22 @@ gemm_generic(const T *A, const T *B, T *C, int64_t M, int64_t N, int64_t K,
 }
 
 // ---------------------------------------------------------------------------
-// Workspace of the split-K path: one hipMalloc'ed block per device, grown on
-// demand and released by nmrtMathRuntimeFinalize.
+// Workspace of the split-K path, per device.
+//
+// mkl_gemm_<dtype>_device keeps one hipMalloc'ed block per device, grown on
+// demand and released by nmrtMathRuntimeFinalize.  The *_noalloc entry point
+// may not allocate: it uses `scratch`, a fixed array in the code object's own
+// device memory (every GPU the library runs on holds a copy until the process
+// ends).  In host code the array's name is only a handle; its device address
+// is looked up once per device with hipGetSymbolAddress and kept.
+// 16 MiB: planSplit never asks for more in float32 (slices x tiles <= 256
+// resident blocks, 64 KiB of partial product per 128 x 128 tile).
+constexpr size_t kScratchBytes = size_t(16) << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
 constexpr int kMaxDevices = 64;
 struct DeviceWorkspace {
+  void *fixed = nullptr; // device address of `scratch` on this device
   void *heap = nullptr;
   size_t heapBytes = 0;
 };
@@ -487,6 +499,20 @@ void *heapWorkspace(int device, size_t bytes) {
   w.heap = p;
   w.heapBytes = want;
   return p;
+}
+
+// Device address of the fixed array on the current device (set up on the
+// first call per device; allocates nothing).
+void *fixedWorkspace(int device) {
+  std::lock_guard<std::mutex> lock(workspaceMutex);
+  DeviceWorkspace &w = workspaceOf(device);
+  if (!w.fixed) {
+    void *p = nullptr;
+    checkHip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)),
+             "hipGetSymbolAddress(scratch)");
+    w.fixed = p;
+  }
+  return w.fixed;
 }
 
 void releaseHeapWorkspaces() {
@@ -532,7 +558,7 @@ SplitPlan planSplit(int64_t tiles, int64_t K, int BK, int blocksPerCu) {
   return plan;
 }
 
-enum WorkspaceKind { WORKSPACE_HEAP };
+enum WorkspaceKind { WORKSPACE_HEAP, WORKSPACE_FIXED };
 
 template <typename T> struct MemrefOf;
 template <> struct MemrefOf<float> {
@@ -555,6 +581,8 @@ bool aligned16(const void *p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }
 
+// Returns 0, or (WORKSPACE_FIXED only) 1 when the product would need more
+// workspace than the fixed array holds; nothing has been launched then.
 template <typename T>
 int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
                const typename MemrefOf<T>::type *b,
@@ -592,14 +620,28 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
   auto stream = static_cast<hipStream_t>(queue->hipStream());
 
   // Split-K workspace for `plan` over an [m, ldw] partial product per slice;
-  // leaves plan unsplit when the heap has no room.
+  // leaves plan unsplit when the heap has no room, reports the fixed array
+  // as too small through tooLarge.
   bool tooLarge = false;
   auto workspaceFor = [&](SplitPlan &plan, int64_t m, int64_t ldw) -> T * {
     if (plan.slices < 2)
       return nullptr;
     const size_t bytes = size_t(plan.slices) * size_t(m) * size_t(ldw) * sizeof(T);
     void *p = nullptr;
-    {
+    if (workspaceKind == WORKSPACE_FIXED) {
+      if (bytes > kScratchBytes) {
+        std::fprintf(stderr,
+                     "mkl_gemm_device_noalloc: [%lld,%lld] x [%lld,%lld] needs "
+                     "%zu bytes of split-K workspace, the fixed workspace "
+                     "holds %zu\n",
+                     (long long)a->dims[0], (long long)a->dims[1],
+                     (long long)b->dims[0], (long long)b->dims[1], bytes,
+                     kScratchBytes);
+        tooLarge = true;
+        return nullptr;
+      }
+      p = fixedWorkspace(device);
+    } else {
       p = heapWorkspace(device, bytes);
       if (!p)
         plan = SplitPlan();
@@ -815,6 +857,12 @@ NMHIP_MATH_EXPORT void mkl_gemm_float64_device(void *queue,
                                                double alpha, double beta,
                                                NmhipMemref2F64 *c) {
   (void)deviceGemm<double>(queue, a, b, c, alpha, beta, WORKSPACE_HEAP);
+}
+
+NMHIP_MATH_EXPORT int mkl_gemm_float32_device_noalloc(
+    void *queue, const NmhipMemref2F32 *a, const NmhipMemref2F32 *b,
+    float alpha, float beta, NmhipMemref2F32 *c) {
+  return deviceGemm<float>(queue, a, b, c, alpha, beta, WORKSPACE_FIXED);
 }
 
 NMHIP_MATH_EXPORT void nmrtMathRuntimeInit(void) {}

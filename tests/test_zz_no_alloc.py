@@ -1,0 +1,83 @@
+"""GPU parity of mkl_gemm_float32_device_noalloc, the gemm entry point that
+allocates no device memory, against mkl_gemm_float32_device through the raw
+C-ABI: two calls in a row on one GPU, the second on a smaller problem, so the
+fixed workspace still holds the first call's partial products."""
+
+import ctypes
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+class Memref2F32(ctypes.Structure):
+    """Memref<2, float> (numba_mlir/numba_mlir/math_runtime/include/Common.hpp:17-28)."""
+    _fields_ = [("userData", ctypes.c_void_p), ("data", ctypes.c_void_p),
+                ("offset", ctypes.c_size_t), ("dims", ctypes.c_size_t * 2),
+                ("strides", ctypes.c_size_t * 2)]
+
+
+def _memref(arr):
+    ref = Memref2F32()
+    ref.userData = None
+    ref.data = arr.ptr
+    ref.offset = 0
+    ref.dims[0], ref.dims[1] = arr.shape
+    ref.strides[0], ref.strides[1] = arr.elem_strides
+    return ref
+
+
+@pytest.fixture(scope="module")
+def gemm_entry_points(hip):
+    from numba_mlir_amd.mlir import math_runtime
+
+    lib = math_runtime.runtime_hip_lib
+    sig = [ctypes.c_void_p, ctypes.POINTER(Memref2F32), ctypes.POINTER(Memref2F32),
+           ctypes.c_float, ctypes.c_float, ctypes.POINTER(Memref2F32)]
+    lib.mkl_gemm_float32_device.argtypes = sig
+    lib.mkl_gemm_float32_device.restype = None
+    lib.mkl_gemm_float32_device_noalloc.argtypes = sig
+    lib.mkl_gemm_float32_device_noalloc.restype = ctypes.c_int
+    return hip, lib, math_runtime
+
+
+def _both(hip, lib, mrt, m, n, k, alpha, beta, seed):
+    rng = np.random.default_rng(seed)
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    b = rng.standard_normal((k, n), dtype=np.float32)
+    c0 = rng.standard_normal((m, n), dtype=np.float32)
+    d_a, d_b = hip.asarray(a), hip.asarray(b)
+    queue = d_a.ctx.queue
+    ra, rb = _memref(d_a), _memref(d_b)
+
+    d_ref = hip.asarray(c0)
+    rc = _memref(d_ref)
+    lib.mkl_gemm_float32_device(queue, ra, rb, alpha, beta, rc)
+    ref_kernel = mrt.last_kernel()
+
+    d_got = hip.asarray(c0)
+    rc = _memref(d_got)
+    status = lib.mkl_gemm_float32_device_noalloc(queue, ra, rb, alpha, beta, rc)
+    return status, d_got.asnumpy(), d_ref.asnumpy(), ref_kernel, mrt.last_kernel(), (a, b, c0)
+
+
+def test_two_calls_in_a_row_match_the_allocating_entry_point(gemm_entry_points):
+    hip, lib, mrt = gemm_entry_points
+    # 1024^3 cuts K into four slices (16 MiB of workspace), 640 x 516 x 1028
+    # is ragged and cuts it into eight (10 MiB), 4096 x 3072 x 64 does not split
+    for m, n, k, alpha, beta in ((1024, 1024, 1024, 1.0, 0.0),
+                                 (640, 516, 1028, 1.5, -0.5),
+                                 (256, 384, 2048, 0.5, 2.0),
+                                 (4096, 3072, 64, 1.0, 0.0)):
+        status, got, ref, k_ref, k_got, (a, b, c0) = _both(
+            hip, lib, mrt, m, n, k, alpha, beta, seed=m + n + k)
+        assert status == 0
+        assert k_got == k_ref
+        assert ("_splitk" in k_got) == (k > 64)
+        assert np.array_equal(got, ref), (m, n, k)
+        truth = beta * c0.astype(np.float64) + alpha * (
+            a.astype(np.float64) @ b.astype(np.float64))
+        scale = abs(beta) * np.abs(c0) + abs(alpha) * (
+            np.abs(a).astype(np.float64) @ np.abs(b))
+        assert (np.abs(got - truth) <= 1e-4 * scale + 1e-30).all()
