@@ -61,12 +61,53 @@ def parse_args():
                          "sum0,pairwise,matmul,generated (plus copy, only on "
                          "request)")
     ap.add_argument("--no-cpu", action="store_true",
-                    help="skip the CPU baseline leg")
+                    help="skip the CPU baseline legs")
+    ap.add_argument("--no-rotate", action="store_true",
+                    help="launch every step on the same arrays instead of "
+                         "rotating over several sets (shows what the 256 MiB "
+                         "memory-side cache contributes)")
     return ap.parse_args()
 
 
+# Launches rotate over this many sets of arrays, so that no step finds its
+# inputs (or the lines it is about to overwrite) in the 256 MiB memory-side
+# cache: every configuration's sets together exceed 256 MiB several times.
+ROTATE_SETS = 3
+
+
+class StreamTimer:
+    """HIP events on the gpux queue's own stream (libnmhip-bench-timer.so, a
+    helper of this benchmark; the offloaded path itself has no timers)."""
+
+    def __init__(self, queue):
+        from numba_mlir_amd import build as native_build
+
+        lib = ctypes.CDLL(os.path.join(native_build.HERE, native_build.BENCH_TIMER_LIB))
+        lib.benchTimerCreate.restype = ctypes.c_void_p
+        lib.benchTimerCreate.argtypes = [ctypes.c_void_p]
+        for name in ("benchTimerStart", "benchTimerStop", "benchTimerDestroy"):
+            getattr(lib, name).restype = None
+            getattr(lib, name).argtypes = [ctypes.c_void_p]
+        lib.benchTimerElapsedMs.restype = ctypes.c_double
+        lib.benchTimerElapsedMs.argtypes = [ctypes.c_void_p]
+        self.lib = lib
+        self.handle = lib.benchTimerCreate(queue)
+
+    def start(self):
+        self.lib.benchTimerStart(self.handle)
+
+    def stop(self):
+        self.lib.benchTimerStop(self.handle)
+
+    def elapsed_ms(self):
+        return self.lib.benchTimerElapsedMs(self.handle)
+
+    def close(self):
+        self.lib.benchTimerDestroy(self.handle)
+
+
 class Bench:
-    def __init__(self, steps, warmup):
+    def __init__(self, steps, warmup, rotate=True):
         from numba_mlir_amd import build as native_build
 
         if not native_build.libraries_present():
@@ -78,10 +119,21 @@ class Bench:
         self.lib = da.lib
         self.ctx = da.get_context()
         self.steps, self.warmup = steps, warmup
+        self.sets = ROTATE_SETS if rotate else 1
 
-    def measure(self, launch, blocking=False):
-        """Returns (wall ms/step, HIP-event ms/step, kernel name)."""
-        ctx, lib = self.ctx, self.lib
+    def measure(self, launches, blocking=False):
+        """``launches``: one callable per set of arrays (or a single callable);
+        step k runs launches[k % len].  Returns (wall ms/step, HIP-event
+        ms/step, kernel name)."""
+        ctx = self.ctx
+        if callable(launches):
+            launches = [launches]
+        turn = [0]
+
+        def launch():
+            launches[turn[0] % len(launches)]()
+            turn[0] += 1
+
         ctx.set_async(not blocking)
         # The GPU leaves its idle clocks only after some tens of milliseconds
         # of work (the first kernel of a process measured 75 us cold, 63 us
@@ -95,16 +147,16 @@ class Bench:
         for _ in range(self.warmup):
             launch()
         ctx.synchronize()
-        timer = lib.nmhipTimerCreate(ctx.handle)
-        lib.nmhipTimerStart(timer)
+        timer = StreamTimer(ctx.queue)
+        timer.start()
         t0 = time.perf_counter()
         for _ in range(self.steps):
             launch()
-        lib.nmhipTimerStop(timer)
+        timer.stop()
         ctx.synchronize()
-        ev_ms = lib.nmhipTimerElapsedMs(timer)
+        ev_ms = timer.elapsed_ms()
         t1 = time.perf_counter()
-        lib.nmhipTimerDestroy(timer)
+        timer.close()
         ctx.set_async(False)
         return ((t1 - t0) * 1e3 / self.steps, ev_ms / self.steps,
                 ctx.last_kernel())
@@ -175,126 +227,179 @@ def hbm_entry(name, workload, alg_bytes, wall_ms, ev_ms, kernel, extra=None):
     return e
 
 
+def cpu_leg(fn, units, unit, threads, sample, kind="port"):
+    """Times ``fn`` on the host outside every GPU-timed region: one untimed
+    call, then repeats for about a second (at most five)."""
+    fn()
+    reps, t0 = 0, time.perf_counter()
+    while reps < 5 and (reps == 0 or time.perf_counter() - t0 < 1.0):
+        fn()
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": units / dt, "unit": unit, "cores": threads, "kind": kind,
+            "sample": f"{sample}, {reps} passes"}
+
+
 def run(args):
     import numpy as np
 
     from numba_mlir_amd import workloads
     from numba_mlir_amd.mlir import math_runtime
 
-    b = Bench(args.steps, args.warmup)
+    b = Bench(args.steps, args.warmup, rotate=not args.no_rotate)
     da, ops = b.da, b.ops
     only = set(x for x in args.only.split(",") if x)
     want = lambda n: not only or n in only
     per_config = []
     headline = None
+    nsets = b.sets
+    orc = threads = None
+    if not args.no_cpu:
+        from oracle import oracle as orc
+
+        threads = min(orc.max_threads(), os.cpu_count() or 1)
+    omp = "C restatement of the reference's CPU path (OpenMP threads)"
 
     # -- config 2: Black-Scholes (headline) ---------------------------------
     if want("bs") or want("bs32"):
         nopt = 2 ** 24
         price, strike, t, rate, vol, call, put = workloads.black_scholes(nopt)
-        d = [da.asarray(x) for x in (price, strike, t, call, put)]
+        sets = [[da.asarray(x) for x in (price, strike, t, call, put)]
+                for _ in range(nsets)]
         alg = 20 * nopt
         for key, wide in (("bs", True), ("bs32", False)):
             if not want(key):
                 continue
-            launch = c_call(b.lib.nmhipBlackScholesF32, b.ctx.handle, d[0].ptr,
-                            d[1].ptr, d[2].ptr, float(rate), float(vol),
-                            d[3].ptr, d[4].ptr, nopt, 1 if wide else 0)
-            wall, ev, kern = b.measure(launch)
+            launches = [c_call(b.lib.nmhipBlackScholesF32, b.ctx.handle, d[0].ptr,
+                               d[1].ptr, d[2].ptr, float(rate), float(vol),
+                               d[3].ptr, d[4].ptr, nopt, 1 if wide else 0)
+                        for d in sets]
+            wall, ev, kern = b.measure(launches)
             e = hbm_entry(
                 key, f"Black-Scholes, 2^24 float32 options, literals typed "
                      f"{'float64 (reference typing)' if wide else 'float32'}",
                 alg, wall, ev, kern,
                 {"options_per_s": nopt / (wall * 1e-3)})
+            if orc:
+                e["cpu_baseline"] = cpu_leg(
+                    lambda: orc.black_scholes(price, strike, t, rate, vol, wide, threads),
+                    nopt, "options/s", threads, f"all 2^24 options, {omp}")
             per_config.append(e)
             if wide:
-                headline = (e, nopt, (price, strike, t, rate, vol))
-        del d
+                headline = (e, nopt)
+        del sets
 
     # -- yardstick: plain copy of known size (scales the HBM counters) -------
     if "copy" in only:
         nbytes = 1 << 28
-        src, dst = da.empty((nbytes,), np.uint8), da.empty((nbytes,), np.uint8)
-        wall, ev, kern = b.measure(c_call(b.lib.nmhipCopy, b.ctx.handle, dst.ptr,
-                                          src.ptr, nbytes))
+        pairs = [(da.empty((nbytes,), np.uint8), da.empty((nbytes,), np.uint8))
+                 for _ in range(nsets)]
+        wall, ev, kern = b.measure([c_call(b.lib.nmhipCopy, b.ctx.handle, dst.ptr,
+                                           src.ptr, nbytes) for src, dst in pairs])
         per_config.append(hbm_entry("copy", "device copy of 256 MiB",
                                     2 * nbytes, wall, ev, kern))
-        del src, dst
+        del pairs
 
     # -- config 1: broadcast add --------------------------------------------
     if want("add"):
         a, bb = workloads.broadcast_add()
-        d_a, d_b = da.asarray(a), da.asarray(bb)
-        d_o = da.empty(a.shape, a.dtype)
+        sets = [(da.asarray(a), da.asarray(bb), da.empty(a.shape, a.dtype))
+                for _ in range(nsets)]
         i64x2 = ctypes.c_int64 * 2
-        launch = c_call(b.lib.nmhipMapBinary, b.ctx.handle, 0, 3, d_a.ptr,
-                        i64x2(a.shape[1], 1), d_b.ptr, i64x2(0, 1), d_o.ptr,
-                        i64x2(a.shape[1], 1), a.shape[0], a.shape[1])
-        wall, ev, kern = b.measure(launch)
-        per_config.append(hbm_entry(
-            "add", "a[4096,4096] + b[1,4096], float64",
-            2 * a.nbytes + bb.nbytes, wall, ev, kern))
-        del d_a, d_b, d_o, a, bb
+        launches = [c_call(b.lib.nmhipMapBinary, b.ctx.handle, 0, 3, d_a.ptr,
+                           i64x2(a.shape[1], 1), d_b.ptr, i64x2(0, 1), d_o.ptr,
+                           i64x2(a.shape[1], 1), a.shape[0], a.shape[1])
+                    for d_a, d_b, d_o in sets]
+        wall, ev, kern = b.measure(launches)
+        alg = 2 * a.nbytes + bb.nbytes
+        e = hbm_entry("add", "a[4096,4096] + b[1,4096], float64", alg, wall, ev, kern)
+        if orc:
+            e["cpu_baseline"] = cpu_leg(lambda: orc.add(a, bb, threads), alg / 1e9,
+                                        "GB/s", threads, f"the whole array, {omp}")
+        per_config.append(e)
+        del sets, a, bb
 
     # -- config 3: reductions ------------------------------------------------
     if want("sum1") or want("norm2"):
         x = workloads.reduce_f32()
-        d_x = da.asarray(x)
+        d_xs = [da.asarray(x) for _ in range(nsets)]
         if want("sum1"):
             d_o = da.empty((x.shape[0],), np.float32)
-            launch = c_call(b.lib.nmhipReduce, b.ctx.handle, 0, 2, d_x.ptr,
-                            x.shape[0], x.shape[1], x.shape[1], 1, 1, d_o.ptr)
-            wall, ev, kern = b.measure(launch)
-            per_config.append(hbm_entry(
-                "sum1", "np.sum(x, axis=1), float32 [16384,8192]",
-                x.nbytes + 4 * x.shape[0], wall, ev, kern))
+            launches = [c_call(b.lib.nmhipReduce, b.ctx.handle, 0, 2, d_x.ptr,
+                               x.shape[0], x.shape[1], x.shape[1], 1, 1, d_o.ptr)
+                        for d_x in d_xs]
+            wall, ev, kern = b.measure(launches)
+            alg = x.nbytes + 4 * x.shape[0]
+            e = hbm_entry("sum1", "np.sum(x, axis=1), float32 [16384,8192]",
+                          alg, wall, ev, kern)
+            if orc:
+                e["cpu_baseline"] = cpu_leg(lambda: orc.sum_axis1_f32(x, threads),
+                                            alg / 1e9, "GB/s", threads,
+                                            f"the whole array, {omp}")
+            per_config.append(e)
         if want("norm2"):
             d_o = da.empty((1,), np.float32)
-            wall, ev, kern = b.measure(c_call(
-                b.lib.nmhipNorm2F32, b.ctx.handle, d_x.ptr, x.size, d_o.ptr))
-            per_config.append(hbm_entry(
-                "norm2", "np.sqrt(np.sum(x*x)), float32 [16384,8192]",
-                x.nbytes + 4, wall, ev, kern))
-        del d_x, x
+            wall, ev, kern = b.measure([c_call(
+                b.lib.nmhipNorm2F32, b.ctx.handle, d_x.ptr, x.size, d_o.ptr)
+                for d_x in d_xs])
+            alg = x.nbytes + 4
+            e = hbm_entry("norm2", "np.sqrt(np.sum(x*x)), float32 [16384,8192]",
+                          alg, wall, ev, kern)
+            if orc:
+                e["cpu_baseline"] = cpu_leg(lambda: orc.norm2_f32(x, threads),
+                                            alg / 1e9, "GB/s", threads,
+                                            f"the whole array, {omp}")
+            per_config.append(e)
+        del d_xs, x
     if want("sum0"):
         xi = workloads.reduce_i32()
-        d_x = da.asarray(xi)
+        d_xs = [da.asarray(xi) for _ in range(nsets)]
         d_o = da.empty((xi.shape[1],), np.int64)
-        launch = c_call(b.lib.nmhipReduce, b.ctx.handle, 0, 0, d_x.ptr,
-                        xi.shape[0], xi.shape[1], xi.shape[1], 1, 0, d_o.ptr)
-        wall, ev, kern = b.measure(launch)
-        per_config.append(hbm_entry(
-            "sum0", "np.sum(x, axis=0), int32 [16384,8192] -> int64",
-            xi.nbytes + 8 * xi.shape[1], wall, ev, kern))
-        del d_x, xi
+        launches = [c_call(b.lib.nmhipReduce, b.ctx.handle, 0, 0, d_x.ptr,
+                           xi.shape[0], xi.shape[1], xi.shape[1], 1, 0, d_o.ptr)
+                    for d_x in d_xs]
+        wall, ev, kern = b.measure(launches)
+        alg = xi.nbytes + 8 * xi.shape[1]
+        e = hbm_entry("sum0", "np.sum(x, axis=0), int32 [16384,8192] -> int64",
+                      alg, wall, ev, kern)
+        if orc:
+            e["cpu_baseline"] = cpu_leg(lambda: orc.sum_axis0_i32(xi, threads),
+                                        alg / 1e9, "GB/s", threads,
+                                        f"the whole array, {omp}")
+        per_config.append(e)
+        del d_xs, xi
 
     # -- config 4: pairwise distance @kernel ---------------------------------
     if want("pairwise"):
         X, Y = workloads.pairwise()
         d_X, d_Y = da.asarray(X), da.asarray(Y)
-        d_D = da.empty((X.shape[0], Y.shape[0]), np.float64)
-        wall, ev, kern = b.measure(c_call(
+        outs = [da.empty((X.shape[0], Y.shape[0]), np.float64) for _ in range(nsets)]
+        wall, ev, kern = b.measure([c_call(
             b.lib.nmhipPairwiseF64, b.ctx.handle, d_X.ptr, d_Y.ptr, d_D.ptr,
-            X.shape[0], Y.shape[0]))
-        per_config.append(hbm_entry(
-            "pairwise", "pairwise distance @kernel, float64 [8192,3]^2",
-            X.nbytes + Y.nbytes + 8 * X.shape[0] * Y.shape[0], wall, ev, kern))
-        del d_X, d_Y, d_D
+            X.shape[0], Y.shape[0]) for d_D in outs])
+        alg = X.nbytes + Y.nbytes + 8 * X.shape[0] * Y.shape[0]
+        e = hbm_entry("pairwise", "pairwise distance @kernel, float64 [8192,3]^2",
+                      alg, wall, ev, kern)
+        if orc:
+            e["cpu_baseline"] = cpu_leg(lambda: orc.pairwise(X, Y, threads), alg / 1e9,
+                                        "GB/s", threads, f"all 8192^2 distances, {omp}")
+        per_config.append(e)
+        del d_X, d_Y, outs
 
     # -- config 5: matmul ----------------------------------------------------
     if want("matmul"):
         n = 4096
         A, B = workloads.matmul(n)
         d_A, d_B = da.asarray(A), da.asarray(B)
-        d_C = da.empty((n, n), np.float32)
+        d_Cs = [da.empty((n, n), np.float32) for _ in range(nsets)]
         saved = b.steps
         b.steps = max(5, min(saved, 20))
-        wall, ev, _ = b.measure(lambda: ops.dot(d_A, d_B, out=d_C),
-                                blocking=True)
+        wall, ev, _ = b.measure([lambda d_C=d_C: ops.dot(d_A, d_B, out=d_C)
+                                 for d_C in d_Cs], blocking=True)
         b.steps = saved
         flops = 2.0 * n ** 3
         tf = flops / (ev * 1e-3) / 1e12
-        per_config.append({
+        e = {
             "name": "matmul", "workload": "np.dot float32 [4096,4096]^2",
             "kernel": math_runtime.last_kernel(),
             "ms_per_step": round(wall, 5), "kernel_ms": round(ev, 5),
@@ -304,38 +409,36 @@ def run(args):
                          "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4),
                          "traffic": MEASURED_TRAFFIC.get(
                              math_runtime.last_kernel())},
-        })
-        del d_A, d_B, d_C
+        }
+        if orc:
+            # The reference's CPU np.dot is MKL cblas_sgemm on all cores
+            # (math_runtime/lib/NumpyLinalg.cpp:61-107); MKL is not in this
+            # image, NumPy's OpenBLAS sgemm stands in for it.
+            blas_threads = os.cpu_count() or 1
+            try:
+                from threadpoolctl import threadpool_info
+
+                blas_threads = max([p.get("num_threads", 1) for p in threadpool_info()
+                                    if p.get("user_api") == "blas"] or [blas_threads])
+            except Exception:     # noqa: BLE001 -- the count is informational
+                pass
+            e["cpu_baseline"] = cpu_leg(lambda: np.dot(A, B), flops / 1e12, "TFLOP/s",
+                                        blas_threads, "the whole 4096^3 product, "
+                                        "NumPy/OpenBLAS sgemm standing in for MKL",
+                                        kind="port")
+        per_config.append(e)
+        del d_A, d_B, d_Cs
 
     # -- kernels generated from Python bodies behind @njit / @kernel ---------
     if want("generated"):
         per_config += generated_kernels(b, workloads)
-
-    # -- CPU baseline for the headline (oracle, all host cores) --------------
-    cpu = None
-    if headline is not None and not args.no_cpu:
-        from oracle import oracle as orc
-
-        price, strike, t, rate, vol = headline[2]
-        threads = min(orc.max_threads(), os.cpu_count() or 1)
-        orc.black_scholes(price[:1 << 16], strike[:1 << 16], t[:1 << 16], rate,
-                          vol, True, threads)
-        reps = 3
-        t0 = time.perf_counter()
-        for _ in range(reps):
-            orc.black_scholes(price, strike, t, rate, vol, True, threads)
-        dt = (time.perf_counter() - t0) / reps
-        cpu = {"value": headline[1] / dt, "unit": "options/s", "cores": threads,
-               "kind": "port",
-               "sample": f"all 2^24 options, {reps} passes, C restatement of "
-                         "the reference CPU path with OpenMP threads"}
 
     if headline is None:
         e = per_config[0]
         line = {"metric": e["name"], "value": None, "unit": "",
                 "per_config": per_config}
     else:
-        e, nopt, _ = headline
+        e, nopt = headline
         line = {
             "metric": "black_scholes_options_per_sec",
             "value": nopt / (e["ms_per_step"] * 1e-3),
@@ -348,9 +451,12 @@ def run(args):
             "data": "synthetic",
             "config": {"workload": "Black-Scholes, 2^24 float32 options, "
                                    "price/strike~U(10,50), t~U(1,2), rate=0.1, "
-                                   "vol=0.2, seed 777777"},
+                                   "vol=0.2, seed 777777",
+                       "path": "hand-written kernel " + e["kernel"] +
+                               " through nmhipBlackScholesF32",
+                       "array_sets_rotated": nsets},
             "roofline": e["roofline"],
-            "cpu_baseline": cpu,
+            "cpu_baseline": e.get("cpu_baseline"),
             "per_config": per_config,
         }
     print(json.dumps(line))

@@ -21,8 +21,8 @@
  * the GPU only through function pointers registered with
  * nmhipRegisterSymbol, the counterpart of the reference's symbol registration
  * for JIT'd code (numba_mlir/numba_mlir/mlir/gpu_runtime.py:34-79,
- * mlir_compiler/lib/Lowering.cpp:1554-1561); the only direct HIP calls are
- * host<->device copies and event timers.
+ * mlir_compiler/lib/Lowering.cpp:1554-1561) and makes no HIP call of its own:
+ * the library does not link the HIP runtime.
  *
  * Every pointer named `dev` / a / b / out / x ... is a device-accessible
  * pointer obtained from nmhipAlloc (or gpuxAlloc).  Sizes and strides are in
@@ -92,8 +92,10 @@ const char *nmhipLastKernelName(void *ctx);
 /* gpuxAlloc + gpuxWait + gpuxDestroyEvent (GpuRuntimeToLlvm.cpp:630-754). */
 void *nmhipAlloc(void *ctx, size_t bytes, int gpuxAllocType);
 void nmhipFree(void *ctx, void *dev);
-/* Blocking copies on the context's stream (counterpart of the USM copies
- * dpctl performs for the reference's device arrays). */
+/* Blocking host <-> device copies (counterpart of the USM copies dpctl
+ * performs for the reference's device arrays), done without leaving the gpux
+ * C-ABI: a pinned staging block from gpuxAlloc(Host) and a byte-copy kernel
+ * launched with gpuxLaunchKernel. */
 void nmhipMemcpyHtoD(void *ctx, void *dev, const void *host, size_t bytes);
 void nmhipMemcpyDtoH(void *ctx, void *host, const void *dev, size_t bytes);
 
@@ -190,14 +192,6 @@ const void *nmhipKernelBlob(const char *family, size_t *size);
 /* Overrides a launch-shape knob ("rowbcast_rows", "map_blocks", "bs_blocks",
  * "reduce_blocks", "axis0_rows", "pairwise_rows"); 0 restores the default. */
 void nmhipSetTuning(const char *knob, int64_t value);
-
-/* ---- timers (HIP events on the context's stream) ------------------------ */
-
-void *nmhipTimerCreate(void *ctx);
-void nmhipTimerStart(void *timer);
-void nmhipTimerStop(void *timer);
-double nmhipTimerElapsedMs(void *timer); /* waits for the stop event */
-void nmhipTimerDestroy(void *timer);
 
 #ifdef __cplusplus
 } /* extern "C" */

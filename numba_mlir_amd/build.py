@@ -8,6 +8,8 @@ reference: numba_mlir/numba_mlir/mlir/utils.py:17-42):
   libnumba-mlir-math-hip-runtime.so   mkl_gemm_<dtype>_device
   libnumba-mlir-hip-offload.so        lowered host code, dispatcher and the
                                       embedded code objects of the kernels
+                                      (plain C++, does not link HIP)
+  libnmhip-bench-timer.so             HIP-event stopwatch used by bench.py
 
 The HIP runtime is built by its own hipcc step, separate from everything
 else, as the reference builds its SYCL runtime with its own compiler
@@ -50,6 +52,7 @@ KERNEL_FAMILIES = ["maps", "reduce", "twins"]
 RUNTIME_LIB = "libnumba-mlir-gpu-runtime-hip.so"
 MATH_LIB = "libnumba-mlir-math-hip-runtime.so"
 OFFLOAD_LIB = "libnumba-mlir-hip-offload.so"
+BENCH_TIMER_LIB = "libnmhip-bench-timer.so"
 
 
 def _run(cmd):
@@ -95,12 +98,21 @@ def build_math():
 
 
 def build_offload():
-    _run([CXX, *HOST_FLAGS, *HIP_HOST_FLAGS, "-shared",
+    """Plain C++: the lowered host code reaches the GPU only through the
+    registered gpux* pointers, so neither HIP headers nor libamdhip64."""
+    _run([CXX, *HOST_FLAGS, "-shared",
           os.path.join(CSRC, "offload", "Offload.cpp"),
           os.path.join(CSRC, "offload", "Blobs.S"),
           "-Wa,-I" + BUILD,
           "-Wl,--version-script=" + os.path.join(CSRC, "offload", "export.map"),
-          "-o", os.path.join(HERE, OFFLOAD_LIB), *HIP_LINK_FLAGS, "-lpthread"])
+          "-o", os.path.join(HERE, OFFLOAD_LIB), "-lpthread"])
+
+
+def build_bench_timer():
+    """HIP-event stopwatch on a gpux queue's stream, for bench.py only."""
+    _run([CXX, *HOST_FLAGS, *HIP_HOST_FLAGS, "-shared",
+          os.path.join(CSRC, "bench", "StreamTimer.cpp"),
+          "-o", os.path.join(HERE, BENCH_TIMER_LIB), *HIP_LINK_FLAGS])
 
 
 def build_all(jobs=4):
@@ -109,6 +121,7 @@ def build_all(jobs=4):
         futures = [pool.submit(build_code_object, f) for f in KERNEL_FAMILIES]
         futures.append(pool.submit(build_runtime))
         futures.append(pool.submit(build_math))
+        futures.append(pool.submit(build_bench_timer))
         for f in futures:
             f.result()
     build_offload()  # embeds the code objects built above
@@ -116,7 +129,7 @@ def build_all(jobs=4):
 
 def libraries_present():
     return all(os.path.exists(os.path.join(HERE, n))
-               for n in (RUNTIME_LIB, MATH_LIB, OFFLOAD_LIB))
+               for n in (RUNTIME_LIB, MATH_LIB, OFFLOAD_LIB, BENCH_TIMER_LIB))
 
 
 if __name__ == "__main__":

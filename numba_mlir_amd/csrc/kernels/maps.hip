@@ -191,29 +191,67 @@ NMK_DEFINE_MAP2_ALL_T(mul, OpMul)
 // NumPy computes for the same source, and what the reference computes when
 // the literals are written as np.float32).
 //
-// Cost.  Arithmetic and HBM traffic take about the same time here (about
-// 40 us of vector-ALU issue against 52 us for the five streams of 2^24
-// options), so every instruction counts:
-//   0.5 + 0.5 erf(x)  is a degree-7 polynomial for erf / 2 around the nearest
-//        of 97 nodes 1/16 apart on [0, 6] (erf_table.inc, absolute error of
-//        erf below 1e-15; erf(|x| >= 5.97) = 1 in double), coefficients
-//        staged in LDS; halving is exact, so the sum rounds as
-//        0.5 + 0.5 * erf(x) would;
-//   1 / sqrt(z)  is v_rsq_f64 with one third-order correction (below one unit
-//        in the last place);
-//   log(P / S) and exp(b)  are the float32 library routines' own operation
-//        sequences without their range handling wherever every lane of the
-//        wave has everyday operands (bit-identical results), and the library
-//        routines otherwise.
+// The float64 kernel moves 20 bytes per option and, done naively, spends more
+// time in the vector ALU than in memory.  It therefore has two bodies:
+//
+//  * the plain body, taken by a wave whose 256 options all have everyday
+//    operands (bsWaveIsPlain): about 60 vector instructions per option,
+//      0.5 + 0.5 erf(x)   a degree-5 polynomial for erf / 2 around the nearest
+//          of 97 nodes 1/16 apart on [0, 6] (erf_table.inc; absolute error of
+//          erf 1.5e-12, far below what a float32 price can show), three
+//          128-bit LDS reads of the node's 48-byte row per erf;
+//      1 / sqrt(z)        v_rsq_f64 (relative error e about 2^-24) with one
+//          second-order step y (1 + e / 2): 3/8 e^2, below 1e-14;
+//      P / S, log, exp    the hardware reciprocal, log2 and exp2 with one
+//          multiply each: within 2 units in the last place of the float32
+//          library results (|rate T| <= 1 keeps exp2's argument small enough
+//          for that);
+//      P d1 - Se d2       one fused multiply-add in float64: it differs from
+//          two roundings by 1e-16 relative, invisible after the result is
+//          rounded to float32;
+//    none of it can produce or lose a NaN: the operands are positive normal
+//    numbers, so z > 0 and w1, w2 are finite;
+//
+//  * the careful body for any other wave: the float32 library routines, the
+//    rsq special cases (z = 0, inf), NaN propagation.  It is kept out of line
+//    and rolled up so that it does not cost the plain body registers (54
+//    instead of 78 a lane with both inlined).
+//
+// A wave that contains one odd option computes all its options with the
+// careful body, so a price can differ in the last places of float32 from what
+// the same option gets inside an all-plain wave; both are within the stated
+// tolerance of the reference (rel 1e-4), by orders of magnitude.
 #include "erf_table.inc"
+
+typedef double double2_lds __attribute__((ext_vector_type(2)));
+
+// 0.5 + 0.5 * erf(x) for a non-NaN x on the LDS copy of the table.
+__device__ __forceinline__ double bsCdfTerm(double x, const double2_lds *tab) {
+  static_assert(NMK_ERF_COEFFS == 6 && NMK_ERF_ROW == 6, "three 128-bit words a row");
+  const double ax = __builtin_fmin(__builtin_fabs(x), 6.0);
+  // Adding 1.5 * 2^48 rounds ax to the nearest sixteenth and leaves that
+  // count, 0..96, in the low word of the sum.
+  const double magic = 0x1.8p48;
+  const double t = ax + magic;
+  const int node = __double2loint(t);
+  const double u = ax - (t - magic); // exact, |u| <= 1/32
+  const double2_lds *row = tab + __mul24(node, 3);
+  const double2_lds c01 = row[0], c23 = row[1], c45 = row[2];
+  double p = c45[1];
+  p = __builtin_fma(p, u, c45[0]);
+  p = __builtin_fma(p, u, c23[1]);
+  p = __builtin_fma(p, u, c23[0]);
+  p = __builtin_fma(p, u, c01[1]);
+  p = __builtin_fma(p, u, c01[0]);
+  return 0.5 + __builtin_copysign(p, x);
+}
 
 template <typename W> struct BsMath;
 template <> struct BsMath<double> {
   // 1 / sqrt(z) for z = T * sigSigTwo: the product of a float and of the
   // double of a float, so z is 0, inf, NaN, negative or a normal double far
   // from the ends of the range, and neither y * y nor z * y * y can overflow.
-  // The hardware seed (relative error e below 2^-20) gets one third-order
-  // step y (1 + e/2 + 3 e^2 / 8), leaving 5/16 e^3: below 2^-60.
+  // The hardware seed gets one third-order step y (1 + e/2 + 3 e^2 / 8).
   __device__ static __forceinline__ double rsqrt_(double z) {
     const double y = __builtin_amdgcn_rsq(z);
     const double e = __builtin_fma(-z, y * y, 1.0); // 1 - z y^2
@@ -222,32 +260,18 @@ template <> struct BsMath<double> {
     // a negative or NaN z gives NaN either way.
     return __builtin_amdgcn_class(z, 0x260 /* -0 | +0 | +inf */) ? y : step;
   }
-  // 0.5 + 0.5 * erf(x) for a non-NaN x (a NaN x gives a finite value: the
-  // caller tests for it).
-  __device__ static __forceinline__ double cdfTerm(double x, const double *tab) {
-    const double ax = __builtin_fmin(__builtin_fabs(x), 6.0);
-    // Adding 1.5 * 2^48 rounds ax to the nearest sixteenth and leaves that
-    // count, 0..96, in the low word of the sum.
-    const double magic = 0x1.8p48;
-    const double t = ax + magic;
-    const int node = __double2loint(t);
-    const double u = ax - (t - magic); // exact, |u| <= 1/32
-    const double *c = tab + __mul24(node, NMK_ERF_ROW);
-    double p = c[NMK_ERF_COEFFS - 1];
-#pragma unroll
-    for (int k = NMK_ERF_COEFFS - 2; k >= 0; --k)
-      p = __builtin_fma(p, u, c[k]);
-    return 0.5 + __builtin_copysign(p, x);
+  __device__ static __forceinline__ double cdfTerm(double x, const double2_lds *tab) {
+    return bsCdfTerm(x, tab);
   }
   __device__ static __forceinline__ bool eitherNaN(double a, double b) {
-    return __builtin_isunordered(a, b);
+    return __builtin_isunordered(a, b); // bsCdfTerm maps NaN to a number
   }
 };
 template <> struct BsMath<float> {
   __device__ static __forceinline__ float rsqrt_(float z) {
     return 1.0f / sqrtf(z);
   }
-  __device__ static __forceinline__ float cdfTerm(float x, const double *) {
+  __device__ static __forceinline__ float cdfTerm(float x, const double2_lds *) {
     return 0.5f + 0.5f * erff(x);
   }
   __device__ static __forceinline__ bool eitherNaN(float, float) {
@@ -262,10 +286,7 @@ template <> struct BsMath<float> {
 // then normal numbers) and |b| <= 80 (exp(b) is normal).  The division is
 // the reciprocal times P with one residual correction: it equals the
 // correctly rounded quotient unless that quotient lies within 2e-7 units in
-// the last place of a rounding boundary (no case among the 2^24 options of
-// the benchmark input).  It is the general routines' handling of zeros,
-// infinities, NaNs, denormals and overflow that costs two thirds of their
-// instructions.
+// the last place of a rounding boundary.  Used by the all-float32 kernel.
 __device__ __forceinline__ bool bsEveryday(float P, float S, float b) {
   const uint32_t lo = 0x21800000u;   // bits of 2^-60
   const uint32_t span = 0x3C000000u; // up to, not including, 2^60
@@ -278,28 +299,13 @@ __device__ __forceinline__ float bsDivEveryday(float P, float S) {
   const float e = __builtin_fmaf(-q, S, P);
   return __builtin_fmaf(e, y, q);
 }
-__device__ __forceinline__ float bsLogEveryday(float q) {
-  const float y = __builtin_amdgcn_logf(q); // log2
-  const float r = y * 0x1.62e42ep-1f;
-  float e = __builtin_fmaf(y, 0x1.62e42ep-1f, -r);
-  e = __builtin_fmaf(y, 0x1.efa39ep-25f, e);
-  return r + e;
-}
-__device__ __forceinline__ float bsExpEveryday(float b) {
-  const float p = b * 0x1.715476p+0f; // b log2(e), then its rounding error
-  float e = __builtin_fmaf(b, 0x1.715476p+0f, -p);
-  e = __builtin_fmaf(b, 0x1.4ae0bep-26f, e);
-  const float n = __builtin_rintf(p);
-  const float v = __builtin_amdgcn_exp2f((p - n) + e);
-  return __builtin_ldexpf(v, int(n));
-}
 
 template <typename W, bool EVERYDAY>
 __device__ __forceinline__ void
 blackScholesOne(float P, float S, float T, float mr, W sigSigTwo,
-                const double *erfTab, float &call, float &put) {
+                const double2_lds *erfTab, float &call, float &put) {
   const float b = T * mr;
-  const float a = EVERYDAY ? bsLogEveryday(bsDivEveryday(P, S)) : logf(P / S);
+  const float a = EVERYDAY ? logNormalF32(bsDivEveryday(P, S)) : logf(P / S);
   const W z = W(T) * sigSigTwo;
   const W c = W(0.25) * z;
   const W y = BsMath<W>::rsqrt_(z);
@@ -308,111 +314,234 @@ blackScholesOne(float P, float S, float T, float mr, W sigSigTwo,
   const W w2 = (W(amb) - c) * y;
   const W d1 = BsMath<W>::cdfTerm(w1, erfTab); // 0.5 + 0.5 * erf(w1)
   const W d2 = BsMath<W>::cdfTerm(w2, erfTab);
-  const float Se = (EVERYDAY ? bsExpEveryday(b) : expf(b)) * S;
+  const float Se = (EVERYDAY ? expNormalF32(b) : expf(b)) * S;
   const W r = W(P) * d1 - W(Se) * d2;
   const bool nan = BsMath<W>::eitherNaN(w1, w2);
   call = nan ? __builtin_nanf("") : float(r);
   put = nan ? __builtin_nanf("") : float(r - W(P) + W(Se));
 }
 
-// One trip of VEC options per lane.  The everyday forms are taken when every
-// lane of the wave qualifies, so each version stays one straight-line block.
-template <typename W, int VEC, typename V>
-__device__ __forceinline__ void bsTrip(const V &P, const V &S, const V &T,
-                                       float mr, W sigSigTwo,
-                                       const double *erfTab, V &c, V &u) {
-  bool everyday = true;
-#pragma unroll
-  for (int k = 0; k < VEC; ++k)
-    everyday = everyday && bsEveryday(P[k], S[k], T[k] * mr);
-  if (__builtin_amdgcn_ballot_w64(!everyday) == 0) {
-#pragma unroll
-    for (int k = 0; k < VEC; ++k) {
-      float ck, uk;
-      blackScholesOne<W, true>(P[k], S[k], T[k], mr, sigSigTwo, erfTab, ck, uk);
-      c[k] = ck;
-      u[k] = uk;
-    }
-  } else {
-#pragma unroll
-    for (int k = 0; k < VEC; ++k) {
-      float ck, uk;
-      blackScholesOne<W, false>(P[k], S[k], T[k], mr, sigSigTwo, erfTab, ck, uk);
-      c[k] = ck;
-      u[k] = uk;
-    }
-  }
+// ---- float64 typing: plain and careful bodies ------------------------------
+
+struct BsPrices {
+  float call, put;
+};
+
+__device__ __attribute__((noinline)) BsPrices
+bsCareful(float P, float S, float T, float mr, double sigSigTwo,
+          const double2_lds *erfTab) {
+  BsPrices out;
+  blackScholesOne<double, false>(P, S, T, mr, sigSigTwo, erfTab, out.call, out.put);
+  return out;
 }
 
-// VEC options per lane per iteration (float4 or float2 accesses).  Both
-// variants take four: the float64 one then needs 78 registers a lane, six
-// waves per SIMD without spills (60.6 us on 2^24 options against 63.1 us
-// with two options and 64-bit accesses; eight waves spill).
-template <int VEC> struct BsVec;
-template <> struct BsVec<4> {
-  typedef float4_t type;
-};
-template <> struct BsVec<2> {
-  typedef float type __attribute__((ext_vector_type(2)));
+#ifndef NMK_BS_EXACT_F32_STEPS
+#define NMK_BS_EXACT_F32_STEPS 0 // 1: library-identical division, log and exp
+#endif
+
+__device__ __forceinline__ void
+bsPlain(float P, float S, float T, float mr, double sigSigTwo,
+        const double2_lds *erfTab, float &call, float &put) {
+  const float b = T * mr;
+#if NMK_BS_EXACT_F32_STEPS
+  const float a = logNormalF32(bsDivEveryday(P, S));
+  const float eb = expNormalF32(b);
+#else
+  const float a =
+      __builtin_amdgcn_logf(P * __builtin_amdgcn_rcpf(S)) * 0x1.62e430p-1f;
+  const float eb = __builtin_amdgcn_exp2f(b * 0x1.715476p+0f);
+#endif
+  const double z = double(T) * sigSigTwo;
+  const double c = 0.25 * z;
+  double y = __builtin_amdgcn_rsq(z);
+  const double e = __builtin_fma(-z, y * y, 1.0);
+  y = __builtin_fma(y * e, 0.5, y);
+  const float amb = a - b;
+  const double w1 = (double(amb) + c) * y;
+  const double w2 = (double(amb) - c) * y;
+  const double d1 = bsCdfTerm(w1, erfTab);
+  const double d2 = bsCdfTerm(w2, erfTab);
+  const float Se = eb * S;
+  const double Pd = double(P), Sed = double(Se);
+  const double r = __builtin_fma(Pd, d1, -(Sed * d2));
+  call = float(r);
+  put = float(r - Pd + Sed);
+}
+
+// Wave-uniform constants of the plain-body test: a lane's four options
+// qualify when P and S are positive with exponents in [-60, 60) and T lies
+// in [2^-60, tLimit), where tLimit keeps |rate T| <= 1 (80 with the exact
+// float32 steps); rate must be finite and |volatility| in [2^-50, 2^50], or
+// no option qualifies (tLimitBits == 0).
+struct BsPlainTest {
+  uint32_t tLimitBits;
+  __device__ __forceinline__ BsPlainTest(float rate, float volatility) {
+    const float av = __builtin_fabsf(volatility);
+    const bool scalarsOk =
+        __builtin_fabsf(rate) < 0x1p60f && av >= 0x1p-50f && av <= 0x1p50f;
+    const float bMax = NMK_BS_EXACT_F32_STEPS ? 80.0f : 1.0f;
+    float tLimit =
+        __builtin_fminf(0x1p60f, bMax * 0.999f / __builtin_fabsf(rate));
+    if (!(tLimit > 0x1p-59f))
+      tLimit = 0.f;
+    tLimitBits = scalarsOk ? __float_as_uint(tLimit) : 0u;
+  }
+  // The bit patterns of positive floats order like the floats; negative
+  // numbers, infinities and NaNs are above every finite positive pattern, zero
+  // and denormals below 2^-60's: three unsigned compares settle twelve values.
+  __device__ __forceinline__ bool operator()(const float4_t &P, const float4_t &S,
+                                             const float4_t &T) const {
+    uint32_t p[4], s[4], t[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      p[k] = __float_as_uint(P[k]);
+      s[k] = __float_as_uint(S[k]);
+      t[k] = __float_as_uint(T[k]);
+    }
+    auto lo3 = [](uint32_t a, uint32_t b, uint32_t c) { return min(min(a, b), c); };
+    auto hi3 = [](uint32_t a, uint32_t b, uint32_t c) { return max(max(a, b), c); };
+    const uint32_t least = lo3(lo3(lo3(p[0], p[1], p[2]), p[3], s[0]),
+                               lo3(s[1], s[2], s[3]),
+                               lo3(lo3(t[0], t[1], t[2]), t[3], t[3]));
+    const uint32_t mostPS = hi3(hi3(p[0], p[1], p[2]), hi3(p[3], s[0], s[1]),
+                                max(s[2], s[3]));
+    const uint32_t mostT = max(hi3(t[0], t[1], t[2]), t[3]);
+    return least >= 0x21800000u /* 2^-60 */ && mostPS < 0x5D800000u /* 2^60 */ &&
+           mostT < tLimitBits;
+  }
 };
 
-template <typename W, int VEC>
+// Copies the erf table into LDS (97 rows of three 128-bit words).
+__device__ __forceinline__ void bsStageTable(double2_lds *tab) {
+  const double2_lds *src = reinterpret_cast<const double2_lds *>(kHalfErfTable);
+  for (int i = threadIdx.x; i < NMK_ERF_NODES * 3; i += blockDim.x)
+    tab[i] = src[i];
+  __syncthreads();
+}
+
+// Four options per lane per trip: 128-bit non-temporal loads of price, strike
+// and t, stores of call and put.  The launch uses many short blocks (two
+// trips a lane at 2^24 options): they stream better than a few long ones.
 __device__ __forceinline__ void
-blackScholes(const float *__restrict__ price, const float *__restrict__ strike,
-             const float *__restrict__ t, float rate, float volatility,
-             float *__restrict__ call, float *__restrict__ put, int64_t n) {
-  typedef typename BsVec<VEC>::type V;
-  __shared__ __attribute__((aligned(16))) double
-      erfTab[sizeof(W) == 8 ? NMK_ERF_NODES * NMK_ERF_ROW : 1];
-  if (sizeof(W) == 8) {
-    for (int i = threadIdx.x; i < NMK_ERF_NODES * NMK_ERF_ROW;
-         i += blockDim.x)
-      erfTab[i] = kHalfErfTable[i];
-    __syncthreads();
-  }
+blackScholesWide(const float *__restrict__ price, const float *__restrict__ strike,
+                 const float *__restrict__ t, float rate, float volatility,
+                 float *__restrict__ call, float *__restrict__ put, int64_t n) {
+  __shared__ __attribute__((aligned(16))) double2_lds erfTab[NMK_ERF_NODES * 3];
+  bsStageTable(erfTab);
   const float mr = -rate;
-  const W sigSigTwo = W(volatility * volatility) * W(2);
-  const int64_t nvec = n / VEC;
+  const double sigSigTwo = double(volatility * volatility) * 2.0;
+  const BsPlainTest isPlain(rate, volatility);
+  const int64_t nvec = n / 4;
   const int64_t stride = int64_t(gridDim.x) * blockDim.x;
-  const V *pv = reinterpret_cast<const V *>(price);
-  const V *sv = reinterpret_cast<const V *>(strike);
-  const V *tv = reinterpret_cast<const V *>(t);
-  V *cv = reinterpret_cast<V *>(call);
-  V *uv = reinterpret_cast<V *>(put);
+  const float4_t *pv = reinterpret_cast<const float4_t *>(price);
+  const float4_t *sv = reinterpret_cast<const float4_t *>(strike);
+  const float4_t *tv = reinterpret_cast<const float4_t *>(t);
+  float4_t *cv = reinterpret_cast<float4_t *>(call);
+  float4_t *uv = reinterpret_cast<float4_t *>(put);
   for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec;
        i += stride) {
-    const V P = streamLoad(pv + i);
-    const V S = streamLoad(sv + i);
-    const V T = streamLoad(tv + i);
-    V c, u;
-    bsTrip<W, VEC>(P, S, T, mr, sigSigTwo, erfTab, c, u);
+    const float4_t P = streamLoad(pv + i);
+    const float4_t S = streamLoad(sv + i);
+    const float4_t T = streamLoad(tv + i);
+    float4_t c, u;
+    if (__builtin_amdgcn_ballot_w64(!isPlain(P, S, T)) == 0) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float ck, uk;
+        bsPlain(P[k], S[k], T[k], mr, sigSigTwo, erfTab, ck, uk);
+        c[k] = ck;
+        u[k] = uk;
+      }
+    } else {
+#pragma unroll 1
+      for (int k = 0; k < 4; ++k) {
+        const BsPrices o = bsCareful(P[k], S[k], T[k], mr, sigSigTwo, erfTab);
+        c[k] = o.call;
+        u[k] = o.put;
+      }
+    }
     streamStore(c, cv + i);
     streamStore(u, uv + i);
   }
-  // n % VEC trailing options, one per lane of the first block.
-  const int64_t tail = nvec * VEC + threadIdx.x;
+  // n % 4 trailing options, one per lane of the first block.
+  const int64_t tail = nvec * 4 + threadIdx.x;
+  if (blockIdx.x == 0 && tail < n) {
+    const BsPrices o =
+        bsCareful(price[tail], strike[tail], t[tail], mr, sigSigTwo, erfTab);
+    call[tail] = o.call;
+    put[tail] = o.put;
+  }
+}
+
+// ---- float32 typing ---------------------------------------------------------
+// One trip of four options per lane.  The everyday forms are taken when every
+// lane of the wave qualifies, so each version stays one straight-line block.
+__device__ __forceinline__ void
+blackScholesNarrow(const float *__restrict__ price, const float *__restrict__ strike,
+                   const float *__restrict__ t, float rate, float volatility,
+                   float *__restrict__ call, float *__restrict__ put, int64_t n) {
+  const float mr = -rate;
+  const float sigSigTwo = (volatility * volatility) * 2.0f;
+  const int64_t nvec = n / 4;
+  const int64_t stride = int64_t(gridDim.x) * blockDim.x;
+  const float4_t *pv = reinterpret_cast<const float4_t *>(price);
+  const float4_t *sv = reinterpret_cast<const float4_t *>(strike);
+  const float4_t *tv = reinterpret_cast<const float4_t *>(t);
+  float4_t *cv = reinterpret_cast<float4_t *>(call);
+  float4_t *uv = reinterpret_cast<float4_t *>(put);
+  for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec;
+       i += stride) {
+    const float4_t P = streamLoad(pv + i);
+    const float4_t S = streamLoad(sv + i);
+    const float4_t T = streamLoad(tv + i);
+    float4_t c, u;
+    bool everyday = true;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      everyday = everyday && bsEveryday(P[k], S[k], T[k] * mr);
+    if (__builtin_amdgcn_ballot_w64(!everyday) == 0) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float ck, uk;
+        blackScholesOne<float, true>(P[k], S[k], T[k], mr, sigSigTwo, nullptr, ck, uk);
+        c[k] = ck;
+        u[k] = uk;
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float ck, uk;
+        blackScholesOne<float, false>(P[k], S[k], T[k], mr, sigSigTwo, nullptr, ck, uk);
+        c[k] = ck;
+        u[k] = uk;
+      }
+    }
+    streamStore(c, cv + i);
+    streamStore(u, uv + i);
+  }
+  const int64_t tail = nvec * 4 + threadIdx.x;
   if (blockIdx.x == 0 && tail < n) {
     float ck, uk;
-    blackScholesOne<W, false>(price[tail], strike[tail], t[tail], mr, sigSigTwo,
-                       erfTab, ck, uk);
+    blackScholesOne<float, false>(price[tail], strike[tail], t[tail], mr, sigSigTwo,
+                                  nullptr, ck, uk);
     call[tail] = ck;
     put[tail] = uk;
   }
 }
 
 extern "C" __global__ __launch_bounds__(256)
-__attribute__((amdgpu_waves_per_eu(6, 6))) void
+__attribute__((amdgpu_waves_per_eu(6, 8))) void
 nmk_black_scholes_f32_w64(const float *price, const float *strike,
                           const float *t, float rate, float volatility,
                           float *call, float *put, int64_t n) {
-  blackScholes<double, 4>(price, strike, t, rate, volatility, call, put, n);
+  blackScholesWide(price, strike, t, rate, volatility, call, put, n);
 }
 
 NMK_KERNEL(256)
 nmk_black_scholes_f32_w32(const float *price, const float *strike,
                           const float *t, float rate, float volatility,
                           float *call, float *put, int64_t n) {
-  blackScholes<float, 4>(price, strike, t, rate, volatility, call, put, n);
+  blackScholesNarrow(price, strike, t, rate, volatility, call, put, n);
 }
 
 // Plain copy of nvec 128-bit words (force_copy of a contiguous operand; also
@@ -425,6 +554,29 @@ nmk_copy_b128(const int4_t *__restrict__ src, int4_t *__restrict__ dst,
   for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec;
        i += stride)
     streamStore(streamLoad(src + i), dst + i);
+}
+
+// Copy of nbytes bytes between any two device-visible buffers (host <-> device
+// staging: one side is pinned host memory).  128-bit words when both ends are
+// 16-byte aligned, single bytes otherwise and for the tail.
+NMK_KERNEL(256)
+nmk_copy_bytes(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+               int64_t nbytes) {
+  const int64_t stride = int64_t(gridDim.x) * blockDim.x;
+  const int64_t first = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  const bool wide =
+      ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0;
+  int64_t done = 0;
+  if (wide) {
+    const int64_t nvec = nbytes / 16;
+    const int4_t *s = reinterpret_cast<const int4_t *>(src);
+    int4_t *d = reinterpret_cast<int4_t *>(dst);
+    for (int64_t i = first; i < nvec; i += stride)
+      d[i] = s[i];
+    done = nvec * 16;
+  }
+  for (int64_t i = done + first; i < nbytes; i += stride)
+    dst[i] = src[i];
 }
 
 // Fills n 32-bit words with a value (used to zero ticket counters: a

@@ -10,8 +10,6 @@
 #include "numba_mlir_hip/GpuQueueInterface.hpp"
 #include "numba_mlir_hip/MathRuntime.h"
 
-#include <hip/hip_runtime_api.h>
-
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -51,12 +49,6 @@ template <typename F> auto guarded(F &&body) noexcept {
     std::fflush(stdout);
     std::abort();
   }
-}
-
-void checkHip(hipError_t err, const char *what) {
-  if (err != hipSuccess)
-    fail("%s failed: %s (%d)", what, hipGetErrorString(err),
-         static_cast<int>(err));
 }
 
 // ---- the symbol table the lowered code calls through ----------------------
@@ -219,6 +211,8 @@ public:
     // (LowerToGpu.cpp:698-715, 832-858).
     if (lastEvent)
       retireEvent(lastEvent, true);
+    if (staging)
+      symbols().DeAlloc(queue, staging);
     if (scratch)
       symbols().DeAlloc(queue, scratch);
     if (tickets)
@@ -324,12 +318,81 @@ public:
 
   uint32_t *tickets = nullptr;
 
-  hipStream_t stream() {
-    auto *iface = static_cast<numba::HipQueueInterface *>(queue);
-    if (iface->hipMagic() != numba::HipQueueInterface::kMagic)
-      fail("Queue was not created by the HIP GPU runtime");
-    checkHip(hipSetDevice(iface->hipDevice()), "hipSetDevice");
-    return static_cast<hipStream_t>(iface->hipStream());
+  // Host <-> device transfers without leaving the C-ABI: a pinned, device-
+  // visible staging block from gpuxAlloc(Host), filled or drained by memcpy
+  // on the host side and by the byte-copy kernel (launched and waited for
+  // through gpuxLaunchKernel / gpuxWait) on the device side.  Two halves
+  // alternate, so the host copies one while the kernel moves the other.
+  static constexpr size_t kStagingHalf = size_t(16) << 20;
+
+  char *stagingHalf(int which) {
+    if (!staging)
+      staging = static_cast<char *>(alloc(2 * kStagingHalf, GPUX_ALLOC_HOST));
+    return staging + size_t(which) * kStagingHalf;
+  }
+
+  void *copyBytesAsync(const void *src, void *dst, size_t bytes) {
+    Arg slots[3] = {Arg::Ptr(src), Arg::Ptr(dst), Arg::I64(int64_t(bytes))};
+    GpuxParamDesc descs[4];
+    for (int i = 0; i < 3; ++i) {
+      descs[i].data = &slots[i].v;
+      descs[i].size = slots[i].size;
+      descs[i].type = slots[i].type;
+    }
+    descs[3] = GpuxParamDesc{nullptr, 0, GPUX_PARAM_NULL};
+    size_t blocks = (bytes / 16 + 255) / 256;
+    if (blocks < 1)
+      blocks = 1;
+    if (blocks > 4096)
+      blocks = 4096;
+    void *deps[1] = {nullptr};
+    return SYM(LaunchKernel, "gpuxLaunchKernel")(
+        queue, kernel("nmk_copy_bytes"), blocks, 1, 1, 256, 1, 1, deps, descs);
+  }
+
+  void hostToDevice(void *dev, const void *host, size_t bytes) {
+    synchronize();
+    void *pending[2] = {nullptr, nullptr};
+    int half = 0;
+    for (size_t off = 0; off < bytes; off += kStagingHalf, half ^= 1) {
+      const size_t n = bytes - off < kStagingHalf ? bytes - off : kStagingHalf;
+      if (pending[half]) { // the kernel that last read this half
+        retireEvent(pending[half], true);
+        pending[half] = nullptr;
+      }
+      char *stage = stagingHalf(half);
+      std::memcpy(stage, static_cast<const char *>(host) + off, n);
+      pending[half] = copyBytesAsync(stage, static_cast<char *>(dev) + off, n);
+    }
+    for (void *ev : pending)
+      if (ev)
+        retireEvent(ev, true);
+  }
+
+  void deviceToHost(void *host, const void *dev, size_t bytes) {
+    synchronize();
+    void *pending[2] = {nullptr, nullptr};
+    size_t pendingOff[2] = {0, 0}, pendingBytes[2] = {0, 0};
+    auto drain = [&](int half) {
+      if (!pending[half])
+        return;
+      retireEvent(pending[half], true);
+      pending[half] = nullptr;
+      std::memcpy(static_cast<char *>(host) + pendingOff[half], stagingHalf(half),
+                  pendingBytes[half]);
+    };
+    int half = 0;
+    for (size_t off = 0; off < bytes; off += kStagingHalf, half ^= 1) {
+      const size_t n = bytes - off < kStagingHalf ? bytes - off : kStagingHalf;
+      drain(half);
+      pending[half] = copyBytesAsync(static_cast<const char *>(dev) + off,
+                                     stagingHalf(half), n);
+      pendingOff[half] = off;
+      pendingBytes[half] = n;
+      drain(half ^ 1); // the other half's kernel ran while this one was queued
+    }
+    drain(0);
+    drain(1);
   }
 
 private:
@@ -338,6 +401,7 @@ private:
   void *lastEvent = nullptr;
   void *scratch = nullptr;
   size_t scratchBytes = 0;
+  char *staging = nullptr;
 
   void retireEvent(void *ev, bool wait) {
     if (wait)
@@ -369,12 +433,6 @@ const char *dtypeName(int dtype) {
 size_t dtypeSize(int dtype) {
   return (dtype == NMHIP_I32 || dtype == NMHIP_F32) ? 4 : 8;
 }
-
-struct Timer {
-  Context *ctx;
-  hipEvent_t start;
-  hipEvent_t stop;
-};
 
 } // namespace
 
@@ -474,24 +532,20 @@ NMHIP_EXPORT void nmhipFree(void *ctx, void *dev) {
 NMHIP_EXPORT void nmhipMemcpyHtoD(void *ctx, void *dev, const void *host,
                                   size_t bytes) {
   guarded([&]() {
-    if (bytes == 0)
-      return;
-    hipStream_t s = toCtx(ctx)->stream();
-    checkHip(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, s),
-             "hipMemcpyAsync(HtoD)");
-    checkHip(hipStreamSynchronize(s), "hipStreamSynchronize");
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    if (bytes != 0)
+      c->hostToDevice(dev, host, bytes);
   });
 }
 
 NMHIP_EXPORT void nmhipMemcpyDtoH(void *ctx, void *host, const void *dev,
                                   size_t bytes) {
   guarded([&]() {
-    if (bytes == 0)
-      return;
-    hipStream_t s = toCtx(ctx)->stream();
-    checkHip(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, s),
-             "hipMemcpyAsync(DtoH)");
-    checkHip(hipStreamSynchronize(s), "hipStreamSynchronize");
+    Context *c = toCtx(ctx);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    if (bytes != 0)
+      c->deviceToHost(host, dev, bytes);
   });
 }
 
@@ -612,11 +666,18 @@ NMHIP_EXPORT void nmhipBlackScholesF32(void *ctx, const float *price,
       fail("nmhipBlackScholesF32: arrays must be 16-byte aligned");
     if (n < 0)
       fail("nmhipBlackScholesF32: negative extent");
-    int64_t blocks = tuning().bsBlocks ? tuning().bsBlocks : 256 * 16;
-    // Four options per lane and trip.
+    // Four options per lane and trip.  The float64-typed kernel streams best
+    // from many short blocks, two trips a lane (8192 blocks at 2^24 options:
+    // 56.5 us against 59 us for 4096 blocks and for 16384); the float32 one
+    // is bound by its arithmetic and keeps 4096 long-running blocks.
     const int64_t need = ceilDiv(ceilDiv(n, 4), 256);
+    int64_t blocks = tuning().bsBlocks ? tuning().bsBlocks
+                     : wide            ? ceilDiv(need, 2)
+                                       : 256 * 16;
     if (blocks > need)
       blocks = need;
+    if (blocks > 0x7fffffff)
+      blocks = 0x7fffffff;
     c->launch(wide ? "nmk_black_scholes_f32_w64" : "nmk_black_scholes_f32_w32",
               size_t(blocks), 1, 1, 256, 1, 1,
               {Arg::Ptr(price), Arg::Ptr(strike), Arg::Ptr(t), Arg::F32(rate),
@@ -939,52 +1000,5 @@ NMHIP_EXPORT void nmhipSetTuning(const char *knob, int64_t value) {
       t.bsBlocks = value;
     else
       fail("Unknown tuning knob '%s'", knob);
-  });
-}
-
-NMHIP_EXPORT void *nmhipTimerCreate(void *ctx) {
-  return guarded([&]() -> void * {
-    Context *c = toCtx(ctx);
-    (void)c->stream(); // selects the device
-    auto *t = new Timer{c, nullptr, nullptr};
-    checkHip(hipEventCreate(&t->start), "hipEventCreate");
-    checkHip(hipEventCreate(&t->stop), "hipEventCreate");
-    return t;
-  });
-}
-
-NMHIP_EXPORT void nmhipTimerStart(void *timer) {
-  guarded([&]() {
-    auto *t = static_cast<Timer *>(timer);
-    checkHip(hipEventRecord(t->start, t->ctx->stream()), "hipEventRecord");
-  });
-}
-
-NMHIP_EXPORT void nmhipTimerStop(void *timer) {
-  guarded([&]() {
-    auto *t = static_cast<Timer *>(timer);
-    checkHip(hipEventRecord(t->stop, t->ctx->stream()), "hipEventRecord");
-  });
-}
-
-NMHIP_EXPORT double nmhipTimerElapsedMs(void *timer) {
-  return guarded([&]() -> double {
-    auto *t = static_cast<Timer *>(timer);
-    checkHip(hipEventSynchronize(t->stop), "hipEventSynchronize");
-    float ms = 0.f;
-    checkHip(hipEventElapsedTime(&ms, t->start, t->stop),
-             "hipEventElapsedTime");
-    return ms;
-  });
-}
-
-NMHIP_EXPORT void nmhipTimerDestroy(void *timer) {
-  guarded([&]() {
-    auto *t = static_cast<Timer *>(timer);
-    if (!t)
-      return;
-    (void)hipEventDestroy(t->start);
-    (void)hipEventDestroy(t->stop);
-    delete t;
   });
 }

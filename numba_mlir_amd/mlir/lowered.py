@@ -51,11 +51,6 @@ _SIGNATURES = {
     "nmhipPairwiseF64": (None, [_vp, _vp, _vp, _vp, _i64, _i64]),
     "nmhipKernelBlob": (_vp, [ctypes.c_char_p, ctypes.POINTER(_sz)]),
     "nmhipSetTuning": (None, [ctypes.c_char_p, _i64]),
-    "nmhipTimerCreate": (_vp, [_vp]),
-    "nmhipTimerStart": (None, [_vp]),
-    "nmhipTimerStop": (None, [_vp]),
-    "nmhipTimerElapsedMs": (ctypes.c_double, [_vp]),
-    "nmhipTimerDestroy": (None, [_vp]),
 }
 
 for _name, (_res, _args) in _SIGNATURES.items():

@@ -51,6 +51,21 @@ def test_offload_exports(native_libs):
         assert hasattr(native_libs.lib, name)
 
 
+def test_offload_library_reaches_the_gpu_only_through_registered_symbols(native_libs):
+    """The lowered host code makes no HIP call of its own: it imports no hip*
+    symbol and does not link libamdhip64 (the reference's JIT'd host code sees
+    the device only through the gpux* functions, export.txt:1-4,
+    GpuRuntimeToLlvm.cpp:95-194)."""
+    path = os.path.join(PKG, "libnumba-mlir-hip-offload.so")
+    undefined = subprocess.run(["nm", "-D", "--undefined-only", path], check=True,
+                               capture_output=True, text=True).stdout
+    names = [line.split()[-1] for line in undefined.splitlines() if line.strip()]
+    assert not [n for n in names if n.lower().startswith(("hip", "hsa", "gpux"))], names
+    needed = subprocess.run(["readelf", "-d", path], check=True, capture_output=True,
+                            text=True).stdout
+    assert "amdhip64" not in needed and "hsa-runtime" not in needed
+
+
 def test_wire_struct_layouts(native_libs):
     from numba_mlir_amd.mlir.gpu_runtime import GPUAllocResult, GPUParamDesc
     # {ptr, i32, i32} and {ptr, ptr}: mlir/lib/Conversion/GpuRuntimeToLlvm.cpp:87-93

@@ -194,10 +194,15 @@ def test_black_scholes_out_of_range_operands(env):
         assert np.array_equal(put[~ok & ~np.isnan(rp)], rp[~ok & ~np.isnan(rp)])
 
 
-def test_black_scholes_general_and_everyday_forms_agree(env):
-    """One odd lane sends its whole wave through the general routines; every
-    other option of that wave must come out bit-identical to the run without
-    the odd lane."""
+def test_black_scholes_plain_and_careful_bodies_agree(env):
+    """One odd lane sends its whole wave through the careful body (library
+    routines, NaN care).  float32 typing: the everyday forms repeat the library
+    routines' operations, so every other option of the wave comes out
+    bit-identical to the run without the odd lane.  float64 typing: the plain
+    body takes the hardware reciprocal, log2 and exp2 directly (within 2 units
+    in the last place of the library's float32 results), so the two runs may
+    differ by what a relative change of 3e-7 in exp(b) S moves a price: under
+    2e-5 absolute on prices up to 40, far inside the tolerance."""
     hip, ops, orc = env
     n = 1 << 16
     (price, strike, t, rate, vol), call0, put0 = _run_bs(hip, ops, n, True)
@@ -217,12 +222,48 @@ def test_black_scholes_general_and_everyday_forms_agree(env):
         c2, u2 = d[3].asnumpy(), d[4].asnumpy()
         keep = np.ones(n, bool)
         keep[odd] = False
-        assert np.array_equal(c2[keep], base_c[keep])
-        assert np.array_equal(u2[keep], base_p[keep])
+        if wide:
+            np.testing.assert_allclose(c2[keep], base_c[keep], rtol=1e-6, atol=2e-5)
+            np.testing.assert_allclose(u2[keep], base_p[keep], rtol=1e-6, atol=2e-5)
+            # and both runs meet the bar against the oracle
+            rc, rp = orc.black_scholes(price, strike, t, rate, vol, wide=True)
+            for got_c, got_p in ((base_c, base_p), (c2, u2)):
+                np.testing.assert_allclose(got_c[keep], rc[keep], rtol=BS_RTOL, atol=BS_ATOL)
+                np.testing.assert_allclose(got_p[keep], rp[keep], rtol=BS_RTOL, atol=BS_ATOL)
+        else:
+            assert np.array_equal(c2[keep], base_c[keep])
+            assert np.array_equal(u2[keep], base_p[keep])
         with np.errstate(all="ignore"):
             rc, rp = orc.black_scholes(p2[odd], s2[odd], t2[odd], rate, vol, wide=wide)
         np.testing.assert_allclose(c2[odd], rc, rtol=1e-4, atol=2e-5)
         np.testing.assert_allclose(u2[odd], rp, rtol=1e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("rate,vol", [
+    (0.1, 0.2), (0.49, 0.2), (0.51, 0.2), (0.7, 0.3), (-0.3, 0.2), (-0.6, 0.2),
+    (0.0, 0.2), (40.0, 0.2), (0.1, 1e-20), (0.1, 1e18), (0.1, 0.0), (0.1, -0.2),
+    (np.nan, 0.2), (0.1, np.nan), (np.inf, 0.2), (0.1, np.inf), (1e30, 0.2)])
+def test_black_scholes_scalar_ranges(env, rate, vol):
+    """The plain body is taken only while |rate t| <= 1 and the scalars are
+    ordinary; rates around that limit, zero, negative, huge, infinite and NaN
+    scalars all match the oracle (same NaN pattern, same prices)."""
+    hip, ops, orc = env
+    from numba_mlir_amd import workloads
+    n = 4096
+    price, strike, t, _, _, call, put = workloads.black_scholes(n)
+    rate, vol = np.float32(rate), np.float32(vol)
+    d = [hip.asarray(x) for x in (price, strike, t, call, put)]
+    ops.black_scholes(d[0], d[1], d[2], rate, vol, d[3], d[4])
+    with np.errstate(all="ignore"):
+        rc, rp = orc.black_scholes(price, strike, t, rate, vol, wide=True)
+    got_c, got_p = d[3].asnumpy(), d[4].asnumpy()
+    for got, ref in ((got_c, rc), (got_p, rp)):
+        assert np.array_equal(np.isnan(got), np.isnan(ref)), (rate, vol)
+        fin = np.isfinite(ref)
+        np.testing.assert_allclose(got[fin], ref[fin], rtol=BS_RTOL,
+                                   atol=BS_ATOL + 4e-6 * float(np.abs(ref[fin]).max(initial=0)))
+        rest = ~fin & ~np.isnan(ref)
+        assert np.array_equal(got[rest], ref[rest])
 
 
 def test_black_scholes_float32_typing(env):
