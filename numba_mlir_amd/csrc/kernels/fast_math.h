@@ -58,4 +58,42 @@ __device__ __forceinline__ float expF32(float b) {
   return __builtin_fabsf(b) <= 80.0f ? expNormalF32(b) : expf(b);
 }
 
+// 1 / sqrt(z) of a double: the hardware seed (relative error e about 2^-24)
+// with one third-order step y (1 + e/2 + 3 e^2 / 8), below one unit in the
+// last place.  z = 0 -> inf and z = inf -> 0 come from the seed (e is NaN
+// there); a negative or NaN z gives NaN either way.  z must be far enough
+// from the ends of the range that z y^2 cannot overflow or underflow:
+// [1e-300, 1e300] is; other finite positive z take the division.
+__device__ __forceinline__ double rsqrtF64Core(double z) {
+  const double y = __builtin_amdgcn_rsq(z);
+  const double e = __builtin_fma(-z, y * y, 1.0); // 1 - z y^2
+  const double step = __builtin_fma(y * e, __builtin_fma(0.375, e, 0.5), y);
+  return __builtin_amdgcn_class(z, 0x260 /* -0 | +0 | +inf */) ? y : step;
+}
+__device__ __forceinline__ double rsqrtF64(double z) {
+  if (z > 0.0 && !(z >= 1e-300 && z <= 1e300))
+    return 1.0 / sqrt(z);
+  return rsqrtF64Core(z);
+}
+
+// log(a / b) in float32 for positive a, b with exponents in [-60, 60) (the
+// reciprocal and the quotient are then normal numbers): reciprocal times a
+// with one residual correction -- the correctly rounded quotient unless that
+// lies within 2e-7 units in the last place of a rounding boundary -- then the
+// library's own log arithmetic.
+__device__ __forceinline__ bool quotientIsPlainF32(float a, float b) {
+  const uint32_t lo = 0x21800000u;   // bits of 2^-60
+  const uint32_t span = 0x3C000000u; // up to, not including, 2^60
+  return ((__float_as_uint(a) - lo) < span) & ((__float_as_uint(b) - lo) < span);
+}
+__device__ __forceinline__ float divNormalF32(float a, float b) {
+  const float y = __builtin_amdgcn_rcpf(b);
+  const float q = a * y;
+  const float e = __builtin_fmaf(-q, b, a);
+  return __builtin_fmaf(e, y, q);
+}
+__device__ __forceinline__ float logQuotientF32(float a, float b) {
+  return quotientIsPlainF32(a, b) ? logNormalF32(divNormalF32(a, b)) : logf(a / b);
+}
+
 } // namespace nmk

@@ -11,6 +11,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "erf_table.inc"
 #include "erf_taylor.inc"
 #include "fast_math.h"
 
@@ -305,6 +306,99 @@ __device__ __forceinline__ double erfF64(double x) {
     r = __builtin_copysign(p, x);
   }
   return x != x ? x : r;
+}
+
+// ---- 0.5 + 0.5 * erf(x) of a double ----------------------------------------
+// The normal distribution's cdf term as one operation: a degree-5 polynomial
+// for erf / 2 around the nearest of 97 nodes 1/16 apart (absolute error of
+// erf 1.5e-12), the node's 48-byte row read from workgroup memory in three
+// 128-bit words (cdfTableLoad at kernel entry).  Halving is exact, so the sum
+// rounds as 0.5 + 0.5 * erf(x) would.  NaN stays NaN.
+typedef double cdf_word __attribute__((ext_vector_type(2)));
+__shared__ __attribute__((aligned(16))) cdf_word cdfLds[NMK_ERF_NODES * 3];
+
+__device__ __forceinline__ void cdfTableLoad() {
+  static_assert(NMK_ERF_COEFFS == 6 && NMK_ERF_ROW == 6, "three 128-bit words a row");
+  const cdf_word *src = reinterpret_cast<const cdf_word *>(kHalfErfTable);
+  for (int k = linearLocalId(); k < NMK_ERF_NODES * 3; k += localCount())
+    cdfLds[k] = src[k];
+  __syncthreads();
+}
+
+__device__ __forceinline__ double cdfTermF64(double x) {
+  const double ax = __builtin_fmin(__builtin_fabs(x), 6.0);
+  const double t = ax + 0x1.8p48; // low word: the nearest sixteenth, 0..96
+  const int node = __double2loint(t);
+  const double u = ax - (t - 0x1.8p48);
+  const cdf_word *row = cdfLds + __mul24(node, 3);
+  const cdf_word c01 = row[0], c23 = row[1], c45 = row[2];
+  double p = c45[1];
+  p = __builtin_fma(p, u, c45[0]);
+  p = __builtin_fma(p, u, c23[1]);
+  p = __builtin_fma(p, u, c23[0]);
+  p = __builtin_fma(p, u, c01[1]);
+  p = __builtin_fma(p, u, c01[0]);
+  const double r = 0.5 + __builtin_copysign(p, x);
+  return x != x ? x : r;
+}
+
+// ---- speculation on everyday operands ---------------------------------------
+// A fused map that gives a lane four adjacent elements computes them first
+// with the routines' plain forms -- the library's own arithmetic without its
+// range handling, bit-identical wherever the operand is in range -- while
+// each such call clears `ok` if its operand is out of range.  The stores come
+// last, so a wave in which any lane saw such an operand simply computes its
+// elements again with the general routines (CAREFUL) before anything is
+// written.  One wave-uniform branch per four elements replaces a divergent
+// branch per call.
+// Whether a double is positive with an exponent in [-900, 900): one unsigned
+// comparison of its high word (negative numbers, NaNs, infinities, zero and
+// denormals all fall outside).
+__device__ __forceinline__ bool midRangeF64(double z) {
+  return (uint32_t(__double2hiint(z)) - (123u << 20)) < (1800u << 20);
+}
+
+// (The tests are combined with & so that the plain form stays one basic
+// block.)
+template <bool CAREFUL> __device__ __forceinline__ float logF32m(float q, bool &ok) {
+  if (CAREFUL)
+    return logf(q);
+  ok = ok & ((__float_as_uint(q) - 0x03800000u) < 0x78000000u); // normal, positive
+  return nmk::logNormalF32(q);
+}
+template <bool CAREFUL> __device__ __forceinline__ float expF32m(float b, bool &ok) {
+  if (CAREFUL)
+    return expf(b);
+  ok = ok & (__builtin_fabsf(b) <= 80.0f);
+  return nmk::expNormalF32(b);
+}
+template <bool CAREFUL>
+__device__ __forceinline__ float logQuotientF32m(float a, float b, bool &ok) {
+  if (CAREFUL)
+    return logf(a / b);
+  ok = ok & nmk::quotientIsPlainF32(a, b);
+  return nmk::logNormalF32(nmk::divNormalF32(a, b));
+}
+template <bool CAREFUL> __device__ __forceinline__ double rsqrtF64m(double z, bool &ok) {
+  if (CAREFUL)
+    return nmk::rsqrtF64(z);
+  ok = ok & midRangeF64(z);
+  const double y = __builtin_amdgcn_rsq(z);
+  const double e = __builtin_fma(-z, y * y, 1.0); // 1 - z y^2
+  return __builtin_fma(y * e, __builtin_fma(0.375, e, 0.5), y);
+}
+template <bool CAREFUL> __device__ __forceinline__ double sqrtF64m(double d, bool &ok) {
+  if (CAREFUL)
+    return sqrt(d);
+  ok = ok & midRangeF64(d);
+  const double y = __builtin_amdgcn_rsq(d);
+  double g = d * y;
+  double h = 0.5 * y;
+  const double r = __builtin_fma(-h, g, 0.5);
+  g = __builtin_fma(g, r, g);
+  h = __builtin_fma(h, r, h);
+  const double e = __builtin_fma(-g, g, d);
+  return __builtin_fma(e, h, g);
 }
 
 } // namespace nmkjit

@@ -175,6 +175,10 @@ class Val:
         self.gid = None               # k: the value is global id k plus a constant
         self.arr = False              # elementwise mode: computed from array elements
         self.origin = None            # an array: the parameter this is, under any name
+        # what the value was computed from, for the fused forms of
+        # log(a / b), 1.0 / sqrt(x) and 0.5 + 0.5 * erf(x):
+        # ("quot", a, b) | ("sqrt", x) | ("erf", x) | ("halferf", x)
+        self.tag = None
 
 
 class _Deferred(Exception):
@@ -304,7 +308,6 @@ class Module:
         # group ids, local sizes, barriers, fences, local arrays, group
         # reductions): only then does the item-to-lane mapping matter
         self.communicates = False
-        self.uses_erf_table = False     # some body calls erf on a float64
         self.device_funcs = {}          # (id(func), arg type keys) -> (name, ret type)
         self.device_code = []
         self.in_progress = set()
@@ -364,6 +367,55 @@ def _function_ast(func):
         if isinstance(n, (ast.FunctionDef,)) and n.name == name:
             return n
     raise KernelCompileError(f"Cannot find the definition of {name}")
+
+
+def _unwrapped_unary(obj):
+    """``def f(x): return g(x)`` (or the lambda, or the vectorize()d form of
+    either) with ``g`` a function of the math or numpy module: ``g``.
+    Anything else: ``obj`` itself."""
+    func = getattr(obj, "_nmk_vectorized", None) or obj
+    if not inspect.isfunction(func):
+        return obj
+    try:
+        node = _function_ast(func)
+    except KernelCompileError:
+        return obj
+    params = [a.arg for a in node.args.args]
+    if len(params) != 1 or node.args.vararg or node.args.kwarg or node.args.kwonlyargs:
+        return obj
+    if isinstance(node, ast.Lambda):
+        value = node.body
+    else:
+        body = [st for st in node.body
+                if not (isinstance(st, ast.Expr) and isinstance(st.value, ast.Constant))]
+        if len(body) != 1 or not isinstance(body[0], ast.Return):
+            return obj
+        value = body[0].value
+    if not (isinstance(value, ast.Call) and len(value.args) == 1 and not value.keywords and
+            isinstance(value.args[0], ast.Name) and value.args[0].id == params[0]):
+        return obj
+    target, scope = value.func, dict(getattr(func, "__globals__", {}))
+    try:
+        scope.update(inspect.getclosurevars(func).nonlocals)
+    except (TypeError, ValueError):
+        pass
+    if isinstance(target, ast.Name):
+        inner = scope.get(target.id)
+    elif isinstance(target, ast.Attribute) and isinstance(target.value, ast.Name):
+        inner = getattr(scope.get(target.value.id), target.attr, None)
+    else:
+        inner = None
+    if inner is None:
+        return obj
+    mod = getattr(inner, "__module__", None)
+    if (mod == "math" or mod == "numpy" or isinstance(inner, np.ufunc)) and \
+            getattr(inner, "__name__", None) in _UNARY_MATH:
+        return inner
+    return obj
+
+
+class _NotAdjacent(Exception):
+    """The body does not fit the adjacent-elements form of a fused map."""
 
 
 class FunctionTranslator:
@@ -429,6 +481,11 @@ class FunctionTranslator:
         self.reduction_types = []    # (name, Scalar) in parameter order
         self.site_names = {}         # ast node -> stable names
         self.array_info = {}         # variable name -> Array type (views)
+        # elementwise 1-d maps over dense arrays: a lane takes ADJACENT
+        # elements, 128-bit loads and stores (see translate_kernel)
+        self.adjacent = False
+        self.adjacent_outs = {}      # output array (code) -> (element ctype, pointer)
+        self.speculates = False      # some call of the body has a plain and a careful form
 
     # -- helpers -----------------------------------------------------------
     def err(self, node, msg):
@@ -546,6 +603,8 @@ class FunctionTranslator:
             v.arr = True
             self.array_reads += 1
             return v
+        if self.adjacent and self.emitting:
+            raise _NotAdjacent(f"'{arr.code}' cannot be loaded ahead of the body")
         terms = [f"nmk_gid{d} * {arr.code}.stride[{d}]" for d in range(self.ndim)]
         ref = f"{arr.code}.p[{' + '.join(terms)}]"
         if self.noalias and self.stream and arr.code not in self.written_arrays:
@@ -570,10 +629,150 @@ class FunctionTranslator:
                 arr.origin not in self.written_origins and not self.opaque_write and
                 arr.type.elem.ctype in self._PREFETCH_CTYPES)
 
-    def store_here(self, arr_code, elem, value_code):
+    def speculation(self):
+        """Template argument of the routines that come in a plain and a
+        careful form, where the body is computed under speculation (a fused
+        map over adjacent elements), else the empty string."""
+        if self.adjacent and self.mode == "elementwise" and self.is_kernel:
+            self.speculates = True
+            return "<decltype(nmk_careful)::value>"
+        return ""
+
+    def outputs_are_float32(self):
+        """A fused map all of whose results are float32 arrays: its float64
+        intermediates need float32's accuracy and a margin, not their own."""
+        if not (self.is_kernel and self.mode == "elementwise") or self.opaque_write:
+            return False
+        outs = [t.elem for p, t in zip(self.params, self.arg_types)
+                if isinstance(t, Array) and p in self.written_origins]
+        if self.ret_type is not None:
+            outs.append(self.ret_type)
+        return bool(outs) and all(e is FLOAT32 for e in outs)
+
+    _WORD_CTYPES = ("float", "int32_t", "uint32_t")
+
+    def may_be_adjacent(self):
+        """Whether the fused map can give each lane four ADJACENT elements:
+        one dimension, dense arrays of 4-byte elements that do not overlap.
+        (What the body does with them is found out while its statements are
+        written: _NotAdjacent.  Maps over 8-byte elements measured faster with
+        a lane's elements a block apart.)"""
+        if not (self.is_kernel and self.mode == "elementwise" and self.ndim == 1 and
+                self.noalias and self.elements_per_thread == 4) or \
+                self.m.communicates or self.m.boundscheck or self.reductions or \
+                self.opaque_write:
+            return False
+        elems = [t.elem for t in self.arg_types if isinstance(t, Array)]
+        if any(isinstance(t, Array) and (t.layout != "C" or t.ndim != 1)
+               for t in self.arg_types):
+            return False
+        if self.ret_type is not None:
+            elems.append(self.ret_type)
+        return all(e.ctype in self._WORD_CTYPES for e in elems)
+
+    def adjacent_rounds(self, pf, body):
+        """The rounds of a fused map over adjacent elements.  A lane loads its
+        four elements of every operand in one 128-bit word, computes the four
+        results and stores them the same way.  Calls with a plain and a
+        careful form run plain first (``nmk_ok`` records whether every operand
+        was in range); a wave in which some lane's was not computes its
+        elements again the careful way before anything is stored.  Words need
+        16-byte aligned arrays: otherwise, and for the last n % 4 elements,
+        lanes take single elements."""
+        nt = self.stream
+        outs = sorted(self.adjacent_outs.items())
+        ins = [(n, ct, self.cname(n)) for n, ct, _ in pf]
+        pointers = [f"{c}_p" for _, _, c in ins] + [ptr for _, (_, ptr) in outs]
+        out = [
+            "  const int64_t nmk_gid1 = 0, nmk_gid2 = 0;",
+            "  (void)nmk_gid1; (void)nmk_gid2;",
+            "  struct nmk_results {",
+        ] + [f"    {ct} {code};" for code, (ct, _) in outs] + [
+            "  };",
+        ]
+        for n, ct, _ in ins:
+            out.append(f"  typedef {ct} nmk_in_t_{n} __attribute__((ext_vector_type(4)));")
+        for code, (ct, _) in outs:
+            out.append(f"  typedef {ct} nmk_out_t_{code} __attribute__((ext_vector_type(4)));")
+        extra = "".join(f", const {ct} nmk_pf_{n}" for n, ct, _ in ins)
+        names = "".join(f", nmk_pf_{n}" for n, _, _ in ins)
+        # The careful form is kept out of line (and the closures hold copies,
+        # not addresses): inlined, it would cost the plain form registers.
+        out += [
+            "  auto nmk_item = [=](const int64_t nmk_gid0, auto nmk_careful, bool &nmk_ok"
+            f"{extra}) -> nmk_results {{",
+            "    (void)nmk_gid0; (void)nmk_ok;",
+            "    nmk_results nmk_out = {};",
+        ] + body + [
+            "    return nmk_out;",
+            "  };",
+            f"  auto nmk_item_careful = [=](const int64_t nmk_gid0{extra}) "
+            "__attribute__((noinline)) -> nmk_results {",
+            "    bool nmk_unused = true;",
+            f"    return nmk_item(nmk_gid0, nmkjit::Yes(), nmk_unused{names});",
+            "  };",
+            "  const bool nmk_words = ((" + " | ".join(
+                f"reinterpret_cast<uintptr_t>({p})" for p in pointers) + ") & 15u) == 0;",
+            "  const int64_t nmk_nvec = nmk_words ? nmk_gsz0 / 4 : 0;",
+            "  const int64_t nmk_lane = nmk_grp0 * nmk_lsz0 + nmk_lid0;",
+            "  const int64_t nmk_lanes = int64_t(gridDim.x) * nmk_lsz0;",
+            "  for (int64_t nmk_i = nmk_lane; nmk_i < nmk_nvec; nmk_i += nmk_lanes) {",
+        ]
+        for n, ct, c in ins:
+            src = f"reinterpret_cast<const nmk_in_t_{n} *>({c}_p) + nmk_i"
+            load = f"__builtin_nontemporal_load({src})" if nt else f"*({src})"
+            out.append(f"    const nmk_in_t_{n} nmk_in_{n} = {load};")
+        out += [f"    nmk_out_t_{code} nmk_vec_{code};" for code, _ in outs]
+        args = "".join(f", nmk_in_{n}[nmk_k]" for n, _, _ in ins)
+        keep = [f"      nmk_vec_{code}[nmk_k] = nmk_r.{code};" for code, _ in outs]
+        out += [
+            "    bool nmk_ok = true;",
+            "#pragma unroll",
+            "    for (int nmk_k = 0; nmk_k < 4; ++nmk_k) {",
+            f"      const nmk_results nmk_r = nmk_item(nmk_i * 4 + nmk_k, nmkjit::No(), nmk_ok"
+            f"{args});",
+        ] + keep + [
+            "    }",
+        ]
+        if self.speculates:
+            out += [
+                "    if (__builtin_amdgcn_ballot_w64(!nmk_ok) != 0) {",
+                "#pragma unroll 1",
+                "      for (int nmk_k = 0; nmk_k < 4; ++nmk_k) {",
+                f"        const nmk_results nmk_r = nmk_item_careful(nmk_i * 4 + nmk_k{args});",
+            ] + ["  " + line for line in keep] + [
+                "      }",
+                "    }",
+            ]
+        for code, (_, ptr) in outs:
+            dst = f"reinterpret_cast<nmk_out_t_{code} *>({ptr}) + nmk_i"
+            out.append(f"    __builtin_nontemporal_store(nmk_vec_{code}, {dst});" if nt else
+                       f"    *({dst}) = nmk_vec_{code};")
+        scalars = "".join(f", {c}_p[g]" for _, _, c in ins)
+        out += [
+            "  }",
+            "  for (int64_t g = nmk_nvec * 4 + nmk_lane; g < nmk_gsz0; g += nmk_lanes) {",
+            f"    const nmk_results nmk_r = nmk_item_careful(g{scalars});",
+        ] + [f"    {ptr}[g] = nmk_r.{code};" for code, (_, ptr) in outs] + [
+            "  }",
+        ]
+        return out
+
+    def store_here(self, arr_code, elem, value_code, origin=None):
         """Elementwise mode: the store of this work-item's element.  An array
         that is only written, and that no other argument overlaps, is streamed
         past the caches."""
+        if self.adjacent and self.emitting:
+            # the lane's four values of an output array leave in one store,
+            # after the last of them is computed
+            if arr_code in self.read_arrays or origin is None:
+                raise _NotAdjacent(f"'{arr_code}' is read as well as assigned")
+            if self.indent != 2:
+                raise _NotAdjacent(f"'{arr_code}' is assigned under a condition")
+            pointer = "nmk_ret_p" if origin == "nmk_ret" else f"{self.cname(origin)}_p"
+            self.adjacent_outs[arr_code] = (elem.ctype, pointer)
+            self.emit(f"nmk_out.{arr_code} = ({elem.ctype})({value_code});")
+            return
         terms = [f"nmk_gid{d} * {arr_code}.stride[{d}]" for d in range(self.ndim)]
         dst = f"{arr_code}.p[{' + '.join(terms)}]"
         if self.noalias and self.stream and arr_code not in self.read_arrays:
@@ -737,7 +936,17 @@ class FunctionTranslator:
             if not t.is_float:
                 t = FLOAT64
             x, y = cast(a, t), cast(b, t)
-            return Val(f"({x.code} / {y.code})", t, nonneg=a.nonneg and b.nonneg)
+            if t is FLOAT64 and x.const == 1.0 and b.type is FLOAT64 and b.tag and \
+                    b.tag[0] == "sqrt":
+                # 1.0 / sqrt(z): the reciprocal square root and one correction
+                # instead of a square root and a division
+                spec = self.speculation()
+                return Val(f"nmkjit::rsqrtF64m{spec}({b.tag[1]}, nmk_ok)" if spec else
+                           f"nmk::rsqrtF64({b.tag[1]})", t, nonneg=True)
+            v = Val(f"({x.code} / {y.code})", t, nonneg=a.nonneg and b.nonneg)
+            if t is FLOAT32:
+                v.tag = ("quot", x.code, y.code)
+            return v
         if isinstance(op, ast.Pow):
             if t.is_float:
                 x, y = cast(a, t), cast(b, t)
@@ -774,6 +983,17 @@ class FunctionTranslator:
                     return constant(r, t)
             nonneg = a.nonneg and b.nonneg and sym != "-"
             code = f"({x.code} {sym} {y.code})"
+            if t is FLOAT64 and sym in "+*":
+                # 0.5 + 0.5 * erf(x): one table lookup for the whole term
+                for half, other in ((x, b), (y, a)):
+                    if half.const == 0.5 and other.type is FLOAT64 and other.tag:
+                        if sym == "*" and other.tag[0] == "erf":
+                            v = Val(code, t)
+                            v.tag = ("halferf", other.tag[1])
+                            return v
+                        if sym == "+" and other.tag[0] == "halferf" and \
+                                self.emitting and self.outputs_are_float32():
+                            return Val(f"nmkjit::cdfTermF64({other.tag[1]})", t, nonneg=True)
             gid = None
             if t is INT64:                # id + constant still runs along the id
                 if sym in "+-" and a.gid is not None and y.const is not None:
@@ -957,6 +1177,10 @@ class FunctionTranslator:
             self.err(node, "len() needs an array or a tuple")
         if obj is range:
             self.err(node, "range() is only supported as the iterable of a for loop")
+        if len(node.args) == 1 and not kwargs:
+            # def f(x): return math.erf(x) -- and its vectorize()d form -- is
+            # the function it wraps
+            obj = _unwrapped_unary(obj)
         name = getattr(obj, "__name__", None)
         mod = getattr(obj, "__module__", None)
         is_np = isinstance(obj, np.ufunc) or mod == "numpy"
@@ -964,17 +1188,28 @@ class FunctionTranslator:
             v = self.scalar(node.args[0])
             t = FLOAT32 if v.type is FLOAT32 else FLOAT64
             v = cast(v, t)
+            spec = self.speculation()
             if name == "sqrt" and t is FLOAT64:
                 # same rounding as the library routine at half its cost
-                return Val(f"nmk::sqrtF64({v.code})", t, nonneg=True)
+                r = Val(f"nmkjit::sqrtF64m{spec}({v.code}, nmk_ok)" if spec else
+                        f"nmk::sqrtF64({v.code})", t, nonneg=True)
+                r.tag = ("sqrt", v.code)
+                return r
             if name == "erf" and t is FLOAT64:
                 # table in workgroup memory, loaded at kernel entry
-                self.m.uses_erf_table = True
-                return Val(f"nmkjit::erfF64({v.code})", t)
+                r = Val(f"nmkjit::erfF64({v.code})", t)
+                r.tag = ("erf", v.code)
+                return r
+            if name == "log" and t is FLOAT32 and v.tag and v.tag[0] == "quot":
+                # log(a / b): the quotient feeds nothing else
+                _, qa, qb = v.tag
+                return Val(f"nmkjit::logQuotientF32m{spec}({qa}, {qb}, nmk_ok)" if spec else
+                           f"nmk::logQuotientF32({qa}, {qb})", t)
             if name in ("log", "exp") and t is FLOAT32:
                 # the library routine's own arithmetic, its range handling
                 # only where the argument needs it
-                return Val(f"nmk::{name}F32({v.code})", t, nonneg=name == "exp")
+                return Val(f"nmkjit::{name}F32m{spec}({v.code}, nmk_ok)" if spec else
+                           f"nmk::{name}F32({v.code})", t, nonneg=name == "exp")
             return Val(f"{_UNARY_MATH[name]}({v.code})", t)
         if (mod == "math" or is_np) and name in _ROUNDING and len(node.args) == 1:
             v = self.scalar(node.args[0])
@@ -1332,7 +1567,8 @@ class FunctionTranslator:
                 self.written_origins.add(arr.origin)
             else:
                 self.opaque_write = True
-            self.store_here(arr.code, arr.type.elem, cast(v, arr.type.elem).code)
+            self.store_here(arr.code, arr.type.elem, cast(v, arr.type.elem).code,
+                            origin=arr.origin)
             return
         kind, *rest = self.subscript(target)
         if kind != "elem":
@@ -1340,6 +1576,8 @@ class FunctionTranslator:
         code, elem = rest
         if not isinstance(v.type, Scalar):
             self.err(node, "Only scalars can be stored into an array element")
+        if self.adjacent and self.emitting:
+            raise _NotAdjacent("the body stores single elements")
         if self.noalias and self.stream and self.last_elem_gid is not None and \
                 isinstance(target.value, ast.Name) and \
                 target.value.id in self.store_only_params():
@@ -1602,7 +1840,7 @@ class FunctionTranslator:
                 self.changed = True
             elif self.ret_type is not v.type:
                 self.err(node, "An elementwise function has one return statement")
-            self.store_here("nmk_ret", self.ret_type, v.code)
+            self.store_here("nmk_ret", self.ret_type, v.code, origin="nmk_ret")
             return
         if self.is_kernel:
             self.err(node, "A kernel cannot return a value")
@@ -1674,6 +1912,8 @@ class FunctionTranslator:
     def run_emit(self, body):
         self.emitting = True
         self.prefetched = {}        # (the passes before knew less of what is written)
+        self.adjacent_outs = {}
+        self.speculates = False
         self.lines = []
         self.group_sites = []
         self.local_arrays = []
@@ -1702,7 +1942,16 @@ class FunctionTranslator:
     def translate_kernel(self, cname):
         body = self.body_stmts()
         self.infer(body)
-        lines = self.run_emit(body)
+        self.adjacent = self.may_be_adjacent()
+        if self.adjacent:
+            try:
+                lines = self.run_emit(body)
+                if not self.adjacent_outs:
+                    raise _NotAdjacent("no array is assigned as a whole")
+            except _NotAdjacent:
+                self.adjacent = False
+        if not self.adjacent:
+            lines = self.run_emit(body)
         params, views = [], []
         # (a kernel whose work-items exchange data through memory keeps plain
         # pointers)
@@ -1766,7 +2015,10 @@ class FunctionTranslator:
         params += ["int64_t nmk_gsz0", "int64_t nmk_gsz1", "int64_t nmk_gsz2"]
         if self.m.boundscheck:
             params.append("int *nmk_oob")
-        out = [f'extern "C" __global__ __launch_bounds__(1024) void {cname}(',
+        # (the launcher picks the block of a fused map: never above 256 lanes,
+        # and a tighter bound wins)
+        bound = 256 if self.adjacent else 1024
+        out = [f'extern "C" __global__ __launch_bounds__({bound}) void {cname}(',
                "    " + ", ".join(params) + ") {"]
         # Work-items that cannot tell how they are grouped may be laid out on
         # the lanes in any order: put the LAST global dimension on x, so that
@@ -1808,8 +2060,12 @@ class FunctionTranslator:
         ]
         for name, t, neutral in red:
             out.append(f"  {t.ctype} {self.cname(name)} = ({t.ctype}){neutral};")
-        if self.m.uses_erf_table:
+        # tables in workgroup memory, staged by the routines' users
+        text = "\n".join(self.m.device_code + lines)
+        if "nmkjit::erfF64(" in text:
             out.append("  nmkjit::erfTableLoad();")
+        if "nmkjit::cdfTermF64(" in text:
+            out.append("  nmkjit::cdfTableLoad();")
         body = ["    " + v for v in views]
         body += ["    " + d for d in self.declarations() + self.private_decls]
         body += lines
@@ -1861,50 +2117,54 @@ class FunctionTranslator:
                     self.err(self.node, "internal: elements loaded ahead in a kernel that "
                                         "takes one element per lane")
                 extra = "".join(f", const {ct} nmk_pf_{n}" for n, ct, _ in pf)
-                out += [
-                    "  const int64_t nmk_gid1 = 0, nmk_gid2 = 0;",
-                    "  (void)nmk_gid1; (void)nmk_gid2;",
-                    f"  auto nmk_item = [&](const int64_t nmk_gid0, auto nmk_guarded{extra}) {{",
-                    "    if (decltype(nmk_guarded)::value && !(nmk_gid0 < nmk_gsz0)) return;",
-                ] + body + [
-                    "  };",
-                    f"  for (int64_t nmk_round = nmk_grp0; nmk_round * {ept} * nmk_lsz0 < "
-                    "nmk_gsz0; nmk_round += gridDim.x) {",
-                    f"    const int64_t nmk_base = nmk_round * {ept} * nmk_lsz0 + nmk_lid0;",
-                    f"    if ((nmk_round + 1) * {ept} * nmk_lsz0 <= nmk_gsz0) {{",
-                ]
-                if pf:
-                    # The empty asm statements keep the optimizer from moving
-                    # each load back down to its first use.
-                    out += [f"      {ct} nmk_ahead_{n}[{ept}];" for n, ct, _ in pf]
-                    out += [
-                        "#pragma unroll",
-                        f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep) {{",
-                        "        const int64_t g = nmk_base + nmk_rep * nmk_lsz0;",
-                    ] + [f"        nmk_ahead_{n}[nmk_rep] = {load};" for n, _, load in pf] + [
-                        "      }",
-                        "#pragma unroll",
-                        f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep) {{",
-                    ] + [f'        asm volatile("" : "+v"(nmk_ahead_{n}[nmk_rep]));'
-                         for n, _, _ in pf] + [
-                        "      }",
-                    ]
-                ahead = "".join(f", nmk_ahead_{n}[nmk_rep]" for n, _, _ in pf)
-                out += [
-                    "#pragma unroll",
-                    f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep)",
-                    f"        nmk_item(nmk_base + nmk_rep * nmk_lsz0, nmkjit::No(){ahead});",
-                    "    } else {",
-                    "#pragma unroll 1",
-                    f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep) {{",
-                    "        const int64_t g = nmk_base + nmk_rep * nmk_lsz0;",
-                    "        if (g < nmk_gsz0)",
-                    "          nmk_item(g, nmkjit::No()" +
-                    "".join(f", {load}" for _, _, load in pf) + ");",
-                    "      }",
-                    "    }",
-                    "  }",
-                ]
+                if self.adjacent:
+                    out += self.adjacent_rounds(pf, body)
+                    strided = False       # (the rounds are written)
+                if strided:
+                  out += [
+                      "  const int64_t nmk_gid1 = 0, nmk_gid2 = 0;",
+                      "  (void)nmk_gid1; (void)nmk_gid2;",
+                      f"  auto nmk_item = [&](const int64_t nmk_gid0, auto nmk_guarded{extra}) {{",
+                      "    if (decltype(nmk_guarded)::value && !(nmk_gid0 < nmk_gsz0)) return;",
+                  ] + body + [
+                      "  };",
+                      f"  for (int64_t nmk_round = nmk_grp0; nmk_round * {ept} * nmk_lsz0 < "
+                      "nmk_gsz0; nmk_round += gridDim.x) {",
+                      f"    const int64_t nmk_base = nmk_round * {ept} * nmk_lsz0 + nmk_lid0;",
+                      f"    if ((nmk_round + 1) * {ept} * nmk_lsz0 <= nmk_gsz0) {{",
+                  ]
+                  if pf:
+                      # The empty asm statements keep the optimizer from moving
+                      # each load back down to its first use.
+                      out += [f"      {ct} nmk_ahead_{n}[{ept}];" for n, ct, _ in pf]
+                      out += [
+                          "#pragma unroll",
+                          f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep) {{",
+                          "        const int64_t g = nmk_base + nmk_rep * nmk_lsz0;",
+                      ] + [f"        nmk_ahead_{n}[nmk_rep] = {load};" for n, _, load in pf] + [
+                          "      }",
+                          "#pragma unroll",
+                          f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep) {{",
+                      ] + [f'        asm volatile("" : "+v"(nmk_ahead_{n}[nmk_rep]));'
+                           for n, _, _ in pf] + [
+                          "      }",
+                      ]
+                  ahead = "".join(f", nmk_ahead_{n}[nmk_rep]" for n, _, _ in pf)
+                  out += [
+                      "#pragma unroll",
+                      f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep)",
+                      f"        nmk_item(nmk_base + nmk_rep * nmk_lsz0, nmkjit::No(){ahead});",
+                      "    } else {",
+                      "#pragma unroll 1",
+                      f"      for (int nmk_rep = 0; nmk_rep < {ept}; ++nmk_rep) {{",
+                      "        const int64_t g = nmk_base + nmk_rep * nmk_lsz0;",
+                      "        if (g < nmk_gsz0)",
+                      "          nmk_item(g, nmkjit::No()" +
+                      "".join(f", {load}" for _, _, load in pf) + ");",
+                      "      }",
+                      "    }",
+                      "  }",
+                  ]
             else:
                 out += [
                     "  const int64_t nmk_gid0 = nmk_grp0 * nmk_lsz0 + nmk_lid0;",
@@ -2102,7 +2362,7 @@ def build_code_object(compiled):
     """Compiles the generated source with hipcc; code objects are cached on
     disk under the hash of (source, support header, flags)."""
     support = b""
-    for header in ("jit_support.h", "fast_math.h", "erf_taylor.inc"):
+    for header in ("jit_support.h", "fast_math.h", "erf_taylor.inc", "erf_table.inc"):
         with open(os.path.join(_KERNELS_DIR, header), "rb") as f:
             support += f.read()
     digest = hashlib.sha256()

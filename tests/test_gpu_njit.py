@@ -44,6 +44,85 @@ def test_black_scholes_whole_array_body(env, n):
     np.testing.assert_allclose(put.asnumpy(), p2.asnumpy(), rtol=2e-6, atol=2e-6)
 
 
+def test_black_scholes_body_unaligned_views_and_ragged_ends(env):
+    """The fused map gives a lane four adjacent options in 128-bit words when
+    every array starts on a 16-byte boundary; a view that starts one element
+    further on, and the last n % 4 options, are computed one option a lane.
+    Both orders of evaluation give every option the same price."""
+    hip, ops, orc, workloads = env
+    n = 4099
+    price, strike, t, rate, vol, _, _ = workloads.black_scholes(n + 1)
+    f = njit(cases.black_scholes_arrays)
+    got = []
+    for first in (0, 1):
+        dev = [hip.asarray(x)[first:first + n] for x in (price, strike, t)]
+        call = hip.asarray(np.zeros(n + 1, np.float32))[first:first + n]
+        put = hip.asarray(np.zeros(n + 1, np.float32))[first:first + n]
+        f(dev[0], dev[1], dev[2], rate, vol, call, put)
+        assert f.last_launch["path"] == "elementwise"
+        rc, rp = orc.black_scholes(price[first:first + n], strike[first:first + n],
+                                   t[first:first + n], rate, vol, wide=True)
+        np.testing.assert_allclose(call.asnumpy(), rc, rtol=1e-4, atol=1e-7)
+        np.testing.assert_allclose(put.asnumpy(), rp, rtol=1e-4, atol=1e-7)
+        got.append((call.asnumpy(), put.asnumpy()))
+    # options 1 .. n-1 of the first run are options 0 .. n-2 of the second
+    np.testing.assert_allclose(got[0][0][1:], got[1][0][:-1], rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(got[0][1][1:], got[1][1][:-1], rtol=1e-6, atol=1e-6)
+
+
+def test_black_scholes_body_odd_operands(env):
+    """Zeros, infinities, NaNs, negative, huge, tiny and denormal operands and
+    a discount factor that underflows: the wave computes its options again
+    with the general routines and matches the oracle; the everyday options
+    that share a wave with an odd one keep their prices."""
+    hip, ops, orc, workloads = env
+    inf, nan = np.inf, np.nan
+    price = np.array([30, 0, 30, 0, inf, 30, nan, 30, 30, 1e-30, 50, 10, 1e38, 1e-38, 1e-42,
+                      30, 30, -30, 30, 2.0 ** 60, 2.0 ** -61, 30, 1e20], np.float32)
+    strike = np.array([30, 30, 0, 0, 30, inf, 30, nan, 30, 30, 10, 50, 1e38, 1e-38, 1e-42,
+                       1e38, 1e-38, 30, -30, 2.0 ** 59, 2.0 ** -60, 30, 1e-20], np.float32)
+    t = np.array([1.5, 1, 1, 1, 1, 1, 1, 1, 0, 1, 2, 1, 1, 1, 1, 1, 1, 1, 1, 1.5, 1.5, 1000, 1],
+                 np.float32)
+    f = njit(cases.black_scholes_arrays)
+    n = len(price)
+    d = [hip.asarray(x) for x in (price, strike, t, np.zeros(n, np.float32),
+                                  np.zeros(n, np.float32))]
+    f(d[0], d[1], d[2], np.float32(0.1), np.float32(0.2), d[3], d[4])
+    with np.errstate(all="ignore"):
+        rc, rp = orc.black_scholes(price, strike, t, 0.1, 0.2, wide=True)
+    call, put = d[3].asnumpy(), d[4].asnumpy()
+    for got, ref in ((call, rc), (put, rp)):
+        assert np.array_equal(np.isnan(got), np.isnan(ref)), (got, ref)
+        ok = np.isfinite(ref)
+        np.testing.assert_allclose(got[ok], ref[ok], rtol=1e-4, atol=1e-7)
+        assert np.array_equal(got[~ok & ~np.isnan(ref)], ref[~ok & ~np.isnan(ref)])
+    # one odd option in every wave
+    n = 1 << 16
+    price, strike, t, rate, vol, _, _ = workloads.black_scholes(n)
+    runs = []
+    p2, s2, t2 = price.copy(), strike.copy(), t.copy()
+    odd = np.arange(7, n, 97)
+    p2[odd[0::3]] = 0.0
+    s2[odd[1::3]] = np.inf
+    t2[odd[2::3]] = 900.0
+    for p, s, tt in ((price, strike, t), (p2, s2, t2)):
+        d = [hip.asarray(x) for x in (p, s, tt, np.zeros(n, np.float32),
+                                      np.zeros(n, np.float32))]
+        f(d[0], d[1], d[2], rate, vol, d[3], d[4])
+        runs.append((d[3].asnumpy(), d[4].asnumpy()))
+    keep = np.ones(n, bool)
+    keep[odd] = False
+    # (the two forms repeat the same operations but for the quotient, which
+    # the plain form rounds differently in about one case in 10^7)
+    np.testing.assert_allclose(runs[1][0][keep], runs[0][0][keep], rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(runs[1][1][keep], runs[0][1][keep], rtol=1e-6, atol=1e-6)
+    assert np.mean(runs[1][0][keep] == runs[0][0][keep]) > 0.999
+    with np.errstate(all="ignore"):
+        rc, rp = orc.black_scholes(p2[odd], s2[odd], t2[odd], rate, vol, wide=True)
+    np.testing.assert_allclose(runs[1][0][odd], rc, rtol=1e-4, atol=2e-5)
+    np.testing.assert_allclose(runs[1][1][odd], rp, rtol=1e-4, atol=2e-5)
+
+
 def test_black_scholes_prange_body(env):
     hip, ops, orc, workloads = env
     n = 100003

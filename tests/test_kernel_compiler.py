@@ -308,25 +308,59 @@ def test_fused_maps_take_several_elements_per_lane(K, tmp_path, monkeypatch):
     ck = kc.translate(njit_cases.black_scholes_arrays, types, ndim, K, mode=mode,
                       noalias=True, elements_per_thread=4)
     assert ck.elements_per_thread == 4
-    assert "for (int nmk_rep = 0; nmk_rep < 4; ++nmk_rep)" in ck.source
     assert "float *__restrict__ v_price_p" in ck.source
-    # call and put are only written: streamed
-    assert ck.source.count("NMK_STORE_ALONG0(&") == 2
-    assert "#define NMK_STORE_ALONG0(p, v, unit) nmkjit::streamStore(p, v, unit)" in ck.source
+    # Dense arrays that do not overlap: a lane takes four ADJACENT options,
+    # one 128-bit streaming load per operand, one 128-bit streaming store per
+    # result, the operands handed to the body as values.
+    assert "__launch_bounds__(256)" in ck.source
+    assert ("const nmk_in_t_price nmk_in_price = __builtin_nontemporal_load("
+            "reinterpret_cast<const nmk_in_t_price *>(v_price_p) + nmk_i);") in ck.source
+    assert ("__builtin_nontemporal_store(nmk_vec_v_call, "
+            "reinterpret_cast<nmk_out_t_v_call *>(v_call_p) + nmk_i);") in ck.source
+    assert "NMK_STORE_ALONG0(&" not in ck.source and "v_P.p[" not in ck.source
+    # words need 16-byte aligned arrays; single elements otherwise and at the end
+    assert "const int64_t nmk_nvec = nmk_words ? nmk_gsz0 / 4 : 0;" in ck.source
+    assert "for (int64_t g = nmk_nvec * 4 + nmk_lane; g < nmk_gsz0; g += nmk_lanes)" in ck.source
+    # log(P / S), 1.0 / sqrt(z), exp: the plain forms first, the careful ones
+    # (out of line) for a wave with an operand out of range
+    assert ("v_a = nmkjit::logQuotientF32m<decltype(nmk_careful)::value>(nmk_pf_price, "
+            "nmk_pf_strike, nmk_ok);") in ck.source
+    assert "v_y = nmkjit::rsqrtF64m<decltype(nmk_careful)::value>(v_z, nmk_ok);" in ck.source
+    assert "if (__builtin_amdgcn_ballot_w64(!nmk_ok) != 0) {" in ck.source
+    assert "__attribute__((noinline)) -> nmk_results {" in ck.source
+    # 0.5 + 0.5 * erf(w) with float32 results only: one table term, its own table
+    assert "v_d1 = nmkjit::cdfTermF64(v_w1);" in ck.source
+    assert "nmkjit::cdfTableLoad();" in ck.source and "erfTableLoad" not in ck.source
     assert kc.build_code_object(ck)[:4] == b"\x7fELF"
-    # The read-only operands (P = price is price) are loaded for all four
-    # elements ahead of the first element's arithmetic, with streaming loads,
-    # and handed to the body as values.
-    assert "nmk_ahead_price[nmk_rep] = __builtin_nontemporal_load(&v_price_p[g]);" in ck.source
-    assert 'asm volatile("" : "+v"(nmk_ahead_t[nmk_rep]));' in ck.source
-    assert ("nmk_item(nmk_base + nmk_rep * nmk_lsz0, nmkjit::No(), nmk_ahead_price[nmk_rep], "
-            "nmk_ahead_strike[nmk_rep], nmk_ahead_t[nmk_rep]);") in ck.source
-    assert "v_a = nmk::logF32((nmk_pf_price / nmk_pf_strike));" in ck.source
-    assert "v_P.p[" not in ck.source
     small = kc.translate(njit_cases.black_scholes_arrays, types, ndim, K, mode=mode,
                          noalias=True, elements_per_thread=4, stream=False)
     assert "nontemporal" not in small.source and "NMK_STORE_ALONG0(&" not in small.source
-    assert "nmk_ahead_price[nmk_rep] = *(&v_price_p[g]);" in small.source
+    assert ("const nmk_in_t_price nmk_in_price = *(reinterpret_cast<const nmk_in_t_price *>"
+            "(v_price_p) + nmk_i);") in small.source
+    # arrays with a stride: elements a block apart, loaded ahead of the body
+    strided = [kc.Array(t.elem, 1) if isinstance(t, kc.Array) else t for t in types]
+    ck = kc.translate(njit_cases.black_scholes_arrays, strided, ndim, K, mode=mode,
+                      noalias=True, elements_per_thread=4)
+    assert "for (int nmk_rep = 0; nmk_rep < 4; ++nmk_rep)" in ck.source
+    assert ck.source.count("NMK_STORE_ALONG0(&") == 2
+    assert "#define NMK_STORE_ALONG0(p, v, unit) nmkjit::streamStore(p, v, unit)" in ck.source
+    assert ("nmk_ahead_price[nmk_rep] = __builtin_nontemporal_load(&v_price_p[g * v_price_t0]);"
+            in ck.source)
+    assert 'asm volatile("" : "+v"(nmk_ahead_t[nmk_rep]));' in ck.source
+    assert ("nmk_item(nmk_base + nmk_rep * nmk_lsz0, nmkjit::No(), nmk_ahead_price[nmk_rep], "
+            "nmk_ahead_strike[nmk_rep], nmk_ahead_t[nmk_rep]);") in ck.source
+    assert "v_a = nmk::logQuotientF32(nmk_pf_price, nmk_pf_strike);" in ck.source
+    assert "nmkjit::cdfTableLoad();" in ck.source and "__launch_bounds__(1024)" in ck.source
+    assert kc.build_code_object(ck)[:4] == b"\x7fELF"
+    # a body that stores single elements keeps one element per lane and trip
+    def by_index(a, b, c):
+        for i in range(len(a)):
+            c[i] = a[i] + b[i]
+
+    f32c = kc.Array(kc.FLOAT32, 1, layout="C")
+    ck = kc.translate(by_index, [f32c, f32c, f32c], 1, K, mode="elementwise", noalias=True,
+                      elements_per_thread=4)
+    assert "nmk_words" not in ck.source and "__launch_bounds__(1024)" in ck.source
     # overlapping arguments: plain pointers and stores, every load where it is used
     ck = kc.translate(njit_cases.black_scholes_arrays, types, ndim, K, mode=mode,
                       noalias=False, elements_per_thread=4)
