@@ -162,6 +162,48 @@ class Bench:
                 ctx.last_kernel())
 
 
+class Yardsticks:
+    """The benchmark's own memory-only kernels (csrc/bench/yardsticks.hip),
+    loaded and launched through the gpux* C-ABI like any other code object."""
+
+    def __init__(self, ctx):
+        from numba_mlir_amd import build as native_build
+        from numba_mlir_amd.mlir import gpu_runtime
+
+        self.rt, self.lib, self.queue = gpu_runtime, gpu_runtime.runtime_lib, ctx.queue
+        with open(native_build.BENCH_YARDSTICKS, "rb") as f:
+            blob = f.read()
+        self.module = self.lib.gpuxModuleLoad(self.queue, blob, len(blob))
+        self.no_deps = (ctypes.c_void_p * 1)(None)
+        self.events, self.keep, self.kernels = [], [], []
+
+    def launcher(self, name, blocks, threads, pointers, n):
+        """A callable that enqueues kernel(pointers..., int64 n)."""
+        kern = self.lib.gpuxKernelGet(self.module, name.encode())
+        self.kernels.append(kern)
+        values = [ctypes.c_void_p(p) for p in pointers] + [ctypes.c_int64(n)]
+        descs = (self.rt.GPUParamDesc * (len(values) + 1))()
+        for i, v in enumerate(values):
+            descs[i].data = ctypes.cast(ctypes.pointer(v), ctypes.c_void_p)
+            descs[i].size = ctypes.sizeof(v)
+            descs[i].type = 8 if i < len(pointers) else 5
+        self.keep.append((values, descs))
+
+        def launch():
+            self.events.append(self.lib.gpuxLaunchKernel(
+                self.queue, kern, blocks, 1, 1, threads, 1, 1, self.no_deps, descs))
+        return launch
+
+    def close(self):
+        for ev in self.events:
+            self.lib.gpuxWait(self.queue, ev)
+            self.lib.gpuxDestroyEvent(self.queue, ev)
+        for kern in self.kernels:
+            self.lib.gpuxKernelDestroy(kern)
+        self.lib.gpuxModuleDestroy(self.module)
+        self.events, self.kernels = [], []
+
+
 # Bodies written against the decorators, as a user of the reference writes
 # them (Black-Scholes: numba_mlir/mlir/tests/test_numpy.py:2827-2852;
 # pairwise: test_gpu.py:1397-1408): translated to HIP at the first call and
@@ -287,6 +329,19 @@ def run(args):
             per_config.append(e)
             if wide:
                 headline = (e, nopt)
+                # The same five streams (three arrays read, two written) with
+                # next to no arithmetic, on the same arrays and grid: the time
+                # the memory system needs for this access pattern.
+                yard = Yardsticks(b.ctx)
+                blocks = -(-(nopt // 4) // 256) // 2
+                wall_y, ev_y, _ = b.measure([yard.launcher(
+                    "bench_streams_3r2w_f32", blocks, 256, [x.ptr for x in d], nopt)
+                    for d in sets])
+                yard.close()
+                e["memory_floor"] = {
+                    "kernel": "bench_streams_3r2w_f32", "kernel_ms": round(ev_y, 5),
+                    "frac_of_peak": round(alg / (ev_y * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                    "kernel_over_floor": round(ev / ev_y, 4)}
         del sets
 
     # -- yardstick: plain copy of known size (scales the HBM counters) -------

@@ -10,6 +10,8 @@ reference: numba_mlir/numba_mlir/mlir/utils.py:17-42):
                                       embedded code objects of the kernels
                                       (plain C++, does not link HIP)
   libnmhip-bench-timer.so             HIP-event stopwatch used by bench.py
+  csrc/build/bench_yardsticks.hsaco   memory-only kernels bench.py times beside
+                                      the real ones (loaded by bench.py alone)
 
 The HIP runtime is built by its own hipcc step, separate from everything
 else, as the reference builds its SYCL runtime with its own compiler
@@ -115,6 +117,14 @@ def build_bench_timer():
           "-o", os.path.join(HERE, BENCH_TIMER_LIB), *HIP_LINK_FLAGS])
 
 
+BENCH_YARDSTICKS = os.path.join(BUILD, "bench_yardsticks.hsaco")
+
+
+def build_bench_yardsticks():
+    _run([HIPCC, "--genco", "--no-gpu-bundle-output", *DEVICE_FLAGS,
+          "-o", BENCH_YARDSTICKS, os.path.join(CSRC, "bench", "yardsticks.hip")])
+
+
 def build_all(jobs=4):
     os.makedirs(BUILD, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as pool:
@@ -122,6 +132,7 @@ def build_all(jobs=4):
         futures.append(pool.submit(build_runtime))
         futures.append(pool.submit(build_math))
         futures.append(pool.submit(build_bench_timer))
+        futures.append(pool.submit(build_bench_yardsticks))
         for f in futures:
             f.result()
     build_offload()  # embeds the code objects built above
