@@ -10,6 +10,9 @@ reference: numba_mlir/numba_mlir/mlir/utils.py:17-42):
                                       embedded code objects of the kernels
                                       (plain C++, does not link HIP)
   libnmhip-bench-timer.so             HIP-event stopwatch used by bench.py
+  hip-runner                          standalone runner of the reference's
+                                      mlir/test/L0_RUNNER cases against a gpux*
+                                      runtime named by -shared-libs
   csrc/build/bench_yardsticks.hsaco   memory-only kernels bench.py times beside
                                       the real ones (loaded by bench.py alone)
 
@@ -125,6 +128,21 @@ def build_bench_yardsticks():
           "-o", BENCH_YARDSTICKS, os.path.join(CSRC, "bench", "yardsticks.hip")])
 
 
+RUNNER = "hip-runner"
+
+
+def build_runner():
+    """Plain C++ with the code object of its kernels embedded; reaches the
+    runtime only through dlopen of the -shared-libs it is given."""
+    runner = os.path.join(CSRC, "runner")
+    _run([HIPCC, "--genco", "--no-gpu-bundle-output", *DEVICE_FLAGS,
+          "-ffp-contract=off", "-o", os.path.join(BUILD, "runner_kernels.hsaco"),
+          os.path.join(runner, "runner_kernels.hip")])
+    _run([CXX, "-O2", "-std=c++17", f"-I{INCLUDE}", "-Wall",
+          os.path.join(runner, "HipRunner.cpp"), os.path.join(runner, "RunnerBlob.S"),
+          "-Wa,-I" + BUILD, "-o", os.path.join(HERE, RUNNER), "-ldl"])
+
+
 def build_all(jobs=4):
     os.makedirs(BUILD, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as pool:
@@ -133,6 +151,7 @@ def build_all(jobs=4):
         futures.append(pool.submit(build_math))
         futures.append(pool.submit(build_bench_timer))
         futures.append(pool.submit(build_bench_yardsticks))
+        futures.append(pool.submit(build_runner))
         for f in futures:
             f.result()
     build_offload()  # embeds the code objects built above
@@ -140,7 +159,8 @@ def build_all(jobs=4):
 
 def libraries_present():
     return all(os.path.exists(os.path.join(HERE, n))
-               for n in (RUNTIME_LIB, MATH_LIB, OFFLOAD_LIB, BENCH_TIMER_LIB))
+               for n in (RUNTIME_LIB, MATH_LIB, OFFLOAD_LIB, BENCH_TIMER_LIB, RUNNER)) \
+        and os.path.exists(BENCH_YARDSTICKS)
 
 
 if __name__ == "__main__":

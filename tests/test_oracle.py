@@ -38,6 +38,25 @@ def test_add_golden_linalg_addf():
     assert np.array_equal(out, np.array(g["out"], np.float32))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_fused_map_golden_linalg_test(dtype):
+    """linalg_test_f32.mlir / _f64.mlir: the nineteen one-op linalg.generic
+    steps of @foo, each rounded in the tensor's type, print 500 x 1.00002."""
+    g = GOLD["linalg_test"]
+    a = np.full(g["n"], g["a"], dtype)
+    s = [dtype(v) for v in g["s"]]
+    v11, v13, v15 = s[0] + s[1], s[4] - s[3], -s[2]
+    t19 = a - s[0]
+    t27 = np.exp(v15 * t19) + a
+    t35 = s[3] + v13 / t27
+    out = v11 + t35 * (a - s[0])
+    assert out.dtype == dtype
+    assert np.array_equal(_printed(out), np.full(g["n"], g["printed"]))
+    # the correction term is what the print shows: 4 / (e^12 + 1)
+    # (t35 * -4 is near -8, where float32 numbers are 1e-6 apart)
+    assert abs(float(out[0]) - (1 + 4 / (np.exp(12.0) + 1))) < (2e-6 if dtype is np.float32 else 1e-14)
+
+
 @pytest.mark.parametrize("i", range(6))
 @pytest.mark.parametrize("j", range(6))
 def test_add_broadcast_fixtures(i, j):
