@@ -58,7 +58,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", type=str, default="",
                     help="comma-separated subset of: add,bs,bs32,sum1,norm2,"
-                         "sum0,pairwise,matmul,generated (plus copy, only on "
+                         "sum0,pairwise,matmul,dispatch,generated (plus copy, only on "
                          "request)")
     ap.add_argument("--no-cpu", action="store_true",
                     help="skip the CPU baseline legs")
@@ -193,6 +193,25 @@ class Yardsticks:
             self.events.append(self.lib.gpuxLaunchKernel(
                 self.queue, kern, blocks, 1, 1, threads, 1, 1, self.no_deps, descs))
         return launch
+
+    def triple(self, name, blocks, threads, pointers):
+        """A callable that runs the compiled host code's sequence for one
+        kernel: gpuxLaunchKernel, gpuxWait, gpuxDestroyEvent."""
+        kern = self.lib.gpuxKernelGet(self.module, name.encode())
+        self.kernels.append(kern)
+        values = [ctypes.c_void_p(p) for p in pointers]
+        descs = (self.rt.GPUParamDesc * (len(values) + 1))()
+        for i, v in enumerate(values):
+            descs[i].data = ctypes.cast(ctypes.pointer(v), ctypes.c_void_p)
+            descs[i].size, descs[i].type = 8, 8
+        self.keep.append((values, descs))
+        lib, queue, no_deps = self.lib, self.queue, self.no_deps
+
+        def call():
+            ev = lib.gpuxLaunchKernel(queue, kern, blocks, 1, 1, threads, 1, 1, no_deps, descs)
+            lib.gpuxWait(queue, ev)
+            lib.gpuxDestroyEvent(queue, ev)
+        return call
 
     def close(self):
         for ev in self.events:
@@ -484,6 +503,10 @@ def run(args):
         per_config.append(e)
         del d_A, d_B, d_Cs
 
+    # -- per-call overhead of a launch (no roofline: eight elements) --------
+    if want("dispatch"):
+        per_config.append(dispatch_overhead(b))
+
     # -- kernels generated from Python bodies behind @njit / @kernel ---------
     if want("generated"):
         per_config += generated_kernels(b, workloads)
@@ -515,6 +538,76 @@ def run(args):
             "per_config": per_config,
         }
     print(json.dumps(line))
+
+
+# The kernels of the reference's dispatch microbenchmark: 1, 2, 6 and 12 array
+# arguments, the first one written (written out: the translator reads source).
+def _touch1(arg1):
+    i = get_global_id(0)          # noqa: F821 -- bound in dispatch_overhead()
+    arg1[i] = i
+
+
+def _touch2(arg1, arg2):
+    i = get_global_id(0)          # noqa: F821
+    arg1[i] = i
+
+
+def _touch6(arg1, arg2, arg3, arg4, arg5, arg6):
+    i = get_global_id(0)          # noqa: F821
+    arg1[i] = i
+
+
+def _touch12(arg1, arg2, arg3, arg4, arg5, arg6, arg7, arg8, arg9, arg10, arg11, arg12):
+    i = get_global_id(0)          # noqa: F821
+    arg1[i] = i
+
+
+_TOUCH = {1: _touch1, 2: _touch2, 6: _touch6, 12: _touch12}
+
+
+def dispatch_overhead(b, calls=2000):
+    """Microseconds per call of a kernel over an 8-element int32 array taking
+    1, 2, 6 and 12 array arguments (the reference's kernel_dispatcher
+    microbenchmark, benchmarks/benchmarks/microbenchmarks/kernel_dispatcher/
+    numba_mlir.py:52-75): through the raw C-ABI -- gpuxLaunchKernel, gpuxWait,
+    gpuxDestroyEvent per call, as compiled host code does it -- and through
+    the Python front, kern[8, DEFAULT_LOCAL_SIZE](*args)."""
+    import numpy as np
+
+    from numba_mlir_amd import kernel as kapi
+
+    globals()["get_global_id"] = kapi.get_global_id
+    yard = Yardsticks(b.ctx)
+    array = b.da.asarray(np.zeros(8, np.int32))
+    raw, front = {}, {}
+
+    def per_call(fn):
+        for _ in range(200):
+            fn()
+        best = None
+        for _ in range(3):
+            t0 = time.perf_counter()
+            for _ in range(calls):
+                fn()
+            dt = (time.perf_counter() - t0) / calls * 1e6
+            best = dt if best is None else min(best, dt)
+        return round(best, 2)
+
+    for count in (1, 2, 6, 12):
+        raw[str(count)] = per_call(yard.triple(f"bench_touch_{count}", 1, 8,
+                                               [array.ptr] * count))
+        try:
+            launch = kapi.kernel(_TOUCH[count])[8, kapi.DEFAULT_LOCAL_SIZE]
+            args = (array,) * count
+            launch(*args)
+            front[str(count)] = per_call(lambda: launch(*args))
+        except Exception as exc:      # noqa: BLE001 -- e.g. no hipcc on this machine
+            front[str(count)] = f"{type(exc).__name__}: {exc}"
+    assert list(array.asnumpy()) == list(range(8))
+    yard.close()
+    return {"name": "dispatch", "path": "launch -> wait -> destroy event, 8 int32 elements",
+            "workload": "kernel over 8 elements with 1 / 2 / 6 / 12 array arguments",
+            "us_per_call_c_abi": raw, "us_per_call_python_kernel": front, "calls": calls}
 
 
 def generated_kernels(b, workloads):

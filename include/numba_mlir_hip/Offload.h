@@ -47,7 +47,8 @@ enum NmhipDType {
   NMHIP_F64 = 3
 };
 
-enum NmhipBinaryOp { NMHIP_ADD = 0, NMHIP_SUB = 1, NMHIP_MUL = 2 };
+/* NMHIP_DIV: float32 and float64 only (true division). */
+enum NmhipBinaryOp { NMHIP_ADD = 0, NMHIP_SUB = 1, NMHIP_MUL = 2, NMHIP_DIV = 3 };
 
 enum NmhipReduceOp {
   NMHIP_SUM = 0,

@@ -31,3 +31,25 @@ bench_streams_3r2w_f32(const float *__restrict__ a, const float *__restrict__ b,
     __builtin_nontemporal_store(C * B, yv + i);
   }
 }
+
+// Dispatch-overhead yardsticks: eight work-items write their index into the
+// first of 1, 2, 6 or 12 int32 array arguments (the kernels of the
+// reference's kernel_dispatcher microbenchmark,
+// benchmarks/benchmarks/microbenchmarks/kernel_dispatcher/numba_mlir.py:16-48);
+// bench.py times launch -> wait -> destroy event around them.
+#define TOUCH_BODY                                                             \
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;                         \
+  if (i < 8)                                                                   \
+    a1[i] = i;
+extern "C" __global__ void bench_touch_1(int *a1) { TOUCH_BODY }
+extern "C" __global__ void bench_touch_2(int *a1, int *a2) { TOUCH_BODY }
+extern "C" __global__ void bench_touch_6(int *a1, int *a2, int *a3, int *a4,
+                                         int *a5, int *a6) {
+  TOUCH_BODY
+}
+extern "C" __global__ void bench_touch_12(int *a1, int *a2, int *a3, int *a4,
+                                          int *a5, int *a6, int *a7, int *a8,
+                                          int *a9, int *a10, int *a11,
+                                          int *a12) {
+  TOUCH_BODY
+}

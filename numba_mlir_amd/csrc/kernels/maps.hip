@@ -175,6 +175,13 @@ mapStrided2(const T *a, int64_t sa0, int64_t sa1, const T *b, int64_t sb0,
 NMK_DEFINE_MAP2_ALL_T(add, OpAdd)
 NMK_DEFINE_MAP2_ALL_T(sub, OpSub)
 NMK_DEFINE_MAP2_ALL_T(mul, OpMul)
+// True division of floats (numpy/funcs.py:457ff: the result type of an
+// integer division is float64, which is not a same-type map: the generated
+// kernels take it).  The quotient is the correctly rounded one.
+NMK_DEFINE_MAP2(div, OpDiv, f32, float)
+NMK_DEFINE_MAP2(div, OpDiv, f64, double)
+NMK_DEFINE_MAP2_FAST(div, OpDiv, f32, float)
+NMK_DEFINE_MAP2_FAST(div, OpDiv, f64, double)
 
 // ---------------------------------------------------------------------------
 // Fused Black-Scholes map (formula: reference

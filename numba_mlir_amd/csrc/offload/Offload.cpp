@@ -578,9 +578,11 @@ NMHIP_EXPORT void nmhipMapBinary(void *ctx, int op, int dtype, const void *a,
       fail("nmhipMapBinary: negative extent");
     if (n0 == 0 || n1 == 0)
       return;
-    static const char *const opNames[] = {"add", "sub", "mul"};
-    if (op < 0 || op > NMHIP_MUL)
+    static const char *const opNames[] = {"add", "sub", "mul", "div"};
+    if (op < 0 || op > NMHIP_DIV)
       fail("Unsupported binary op %d", op);
+    if (op == NMHIP_DIV && dtype != NMHIP_F32 && dtype != NMHIP_F64)
+      fail("nmhipMapBinary: division is implemented for float32 and float64");
     const std::string suffix =
         std::string(opNames[op]) + "_" + dtypeName(dtype);
     const bool isFloat = dtype == NMHIP_F32 || dtype == NMHIP_F64;
@@ -608,7 +610,8 @@ NMHIP_EXPORT void nmhipMapBinary(void *ctx, int op, int dtype, const void *a,
     const void *full = a;
     const void *row = b;
     bool rowCase = dense(aS) && rowBroadcast(bS);
-    if (!rowCase && op != NMHIP_SUB && dense(bS) && rowBroadcast(aS)) {
+    if (!rowCase && op != NMHIP_SUB && op != NMHIP_DIV && dense(bS) &&
+        rowBroadcast(aS)) {
       full = b;
       row = a;
       rowCase = true;

@@ -69,7 +69,8 @@ ELEMENTS_PER_THREAD = 4     # of a fused 1-d map or prange loop
 MAX_PLANS = kernel_impl.MAX_PLANS   # stored launches per compiled function
 
 
-_BINARY = {ast.Add: ops.add, ast.Sub: ops.subtract, ast.Mult: ops.multiply}
+_BINARY = {ast.Add: ops.add, ast.Sub: ops.subtract, ast.Mult: ops.multiply,
+           ast.Div: ops.divide}
 _REDUCE = {"sum": ops.sum, "prod": ops.prod, "min": ops.amin, "max": ops.amax,
            "amin": ops.amin, "amax": ops.amax}
 

@@ -72,7 +72,7 @@ math_runtime.register_funcs(register_cfunc)
 
 # dtype / op codes of include/numba_mlir_hip/Offload.h
 I32, I64, F32, F64 = 0, 1, 2, 3
-ADD, SUB, MUL = 0, 1, 2
+ADD, SUB, MUL, DIV = 0, 1, 2, 3
 SUM, PROD, MIN, MAX = 0, 1, 2, 3
 ALLOC_DEVICE, ALLOC_SHARED, ALLOC_LOCAL, ALLOC_HOST = 0, 1, 2, 3
 

@@ -86,6 +86,14 @@ def multiply(a, b, out=None):
     return _binary(lowered.MUL, a, b, out)
 
 
+def divide(a, b, out=None):
+    """numpy.divide of two float32 or two float64 arrays (integer operands
+    give float64: not a same-type map)."""
+    if np.dtype(asarray(a).dtype).kind != "f":
+        raise NotImplementedError("true division of integers yields float64")
+    return _binary(lowered.DIV, a, b, out)
+
+
 def black_scholes(price, strike, t, rate, volatility, call, put,
                   float64_literals=True):
     """The fused Black-Scholes body of the reference's test

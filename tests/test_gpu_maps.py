@@ -90,7 +90,7 @@ def test_contiguous_maps(env, dtype, n):
     b = rng.standard_normal(n).astype(dtype)
     d_a, d_b = hip.asarray(a), hip.asarray(b)
     for fn, ref in ((ops.add, np.add), (ops.subtract, np.subtract),
-                    (ops.multiply, np.multiply)):
+                    (ops.divide, np.divide), (ops.multiply, np.multiply)):
         got = fn(d_a, d_b).asnumpy()
         assert _bits(got) == _bits(ref(a, b))
     kern = hip.get_context().last_kernel()
@@ -109,6 +109,28 @@ def test_column_broadcast_and_transposed_operands(env):
     at = hip.asarray(np.ascontiguousarray(a.T)).T      # strided view of a
     assert at.shape == a.shape and not at.is_c_contiguous()
     assert _bits(ops.multiply(at, d_a).asnumpy()) == _bits(a * a)
+
+
+def test_division_of_floats_is_correctly_rounded(env):
+    """Row-broadcast (either side), strided and special operands of the
+    hand-written division; integers are left to the generated kernels."""
+    hip, ops, _ = env
+    rng = np.random.default_rng(3)
+    for dtype in (np.float32, np.float64):
+        a = rng.standard_normal((64, 1024)).astype(dtype)
+        row = (rng.standard_normal((1, 1024)) + 3).astype(dtype)
+        d_a, d_row = hip.asarray(a), hip.asarray(row)
+        assert _bits(ops.divide(d_a, d_row).asnumpy()) == _bits(a / row)
+        assert "rowbcast_div" in hip.get_context().last_kernel()
+        assert _bits(ops.divide(d_row, d_a).asnumpy()) == _bits(row / a)   # does not commute
+        assert "strided_div" in hip.get_context().last_kernel()
+        odd = np.array([0, -0.0, 1, np.inf, -np.inf, np.nan, 1e-40, 3], dtype)
+        with np.errstate(all="ignore"):
+            expect = odd[:, None] / odd[None, :]
+        got = ops.divide(hip.asarray(odd.reshape(8, 1)), hip.asarray(odd.reshape(1, 8))).asnumpy()
+        assert _bits(got) == _bits(expect)
+    with pytest.raises(NotImplementedError):
+        ops.divide(hip.asarray(np.arange(4)), hip.asarray(np.arange(4)))
 
 
 def test_empty_inputs(env):
