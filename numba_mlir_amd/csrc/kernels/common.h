@@ -68,14 +68,21 @@ struct MulOp {
     return a * b;
   }
 };
+// min / max as the reference folds them: select(x < acc, x, acc) starting from
+// +inf (select(x > acc, ...) from -inf), numba_mlir/mlir/builtin/funcs.py:
+// 145-146, 176-177 and numpy/funcs.py:283-303 -- a NaN element never wins a
+// comparison, so NaNs are skipped (NumPy's amin / amax would propagate them)
+// and an all-NaN or empty input gives the starting value.  Here partial
+// results meet in any order: a NaN on either side loses.  (a != a is false
+// for integers and folds away.)
 struct MinOp {
   template <typename T> __device__ __forceinline__ T operator()(T a, T b) const {
-    return b < a ? b : a;
+    return (b < a || a != a) ? b : a;
   }
 };
 struct MaxOp {
   template <typename T> __device__ __forceinline__ T operator()(T a, T b) const {
-    return a < b ? b : a;
+    return (a < b || a != a) ? b : a;
   }
 };
 

@@ -186,11 +186,17 @@ struct AddOp {
 struct MulOp {
   template <typename T> __device__ T operator()(T a, T b) const { return a * b; }
 };
+// (a NaN on either side loses, as in the group minimum / maximum of the
+// reference's target, which skip NaNs)
 struct MinOp {
-  template <typename T> __device__ T operator()(T a, T b) const { return b < a ? b : a; }
+  template <typename T> __device__ T operator()(T a, T b) const {
+    return (b < a || a != a) ? b : a;
+  }
 };
 struct MaxOp {
-  template <typename T> __device__ T operator()(T a, T b) const { return a < b ? b : a; }
+  template <typename T> __device__ T operator()(T a, T b) const {
+    return (a < b || a != a) ? b : a;
+  }
 };
 
 constexpr int kMaxGroup = 1024;

@@ -228,36 +228,55 @@ AllocRegistry &allocRegistry() {
 // Device blocks given back by gpuxDeAlloc are kept for the next gpuxAlloc of
 // the same size on the same device: hipMalloc / hipFree of the arrays a
 // compiled function returns cost several kernel times each (hipFree also
-// synchronises the device).  As with hipFree in the reference's sequence, the
-// caller has waited for the work that used a block before giving it back.
-// Blocks below 64 KiB are not worth keeping; the total kept is capped
-// (NUMBA_MLIR_GPU_ALLOC_CACHE_MB, default 16384, 0 = off) and everything is
-// released when an allocation fails.
+// synchronises the device, which the cache does not).  A kept block therefore
+// goes back only to the queue that released it -- work of that queue which
+// may still touch the block is ahead of any new use on the same in-order
+// stream -- or to any queue once the releasing queue's stream has been
+// drained and destroyed.  Blocks below 64 KiB are not worth keeping; the
+// total kept is capped (NUMBA_MLIR_GPU_ALLOC_CACHE_MB, default 16384, 0 =
+// off) and everything is released when an allocation fails.
 class DeviceBlockCache {
 public:
   static constexpr size_t kMinBytes = 64 * 1024;
 
-  void *take(int device, size_t bytes) {
+  // A block of `bytes` on `device` that `stream` may use at once.
+  void *take(int device, size_t bytes, hipStream_t stream) {
     std::lock_guard<std::mutex> lock(mutex);
     auto it = blocks.find(key(device, bytes));
-    if (it == blocks.end() || it->second.empty())
+    if (it == blocks.end())
       return nullptr;
-    void *ptr = it->second.back();
-    it->second.pop_back();
-    kept -= bytes;
-    return ptr;
+    std::vector<Block> &kept_ = it->second;
+    for (size_t k = kept_.size(); k-- > 0;) {
+      if (kept_[k].stream != stream && kept_[k].stream != nullptr)
+        continue;
+      void *ptr = kept_[k].ptr;
+      kept_.erase(kept_.begin() + long(k));
+      kept -= bytes;
+      return ptr;
+    }
+    return nullptr;
   }
 
   // False when the block should be freed for real.
-  bool put(int device, void *ptr, size_t bytes) {
+  bool put(int device, void *ptr, size_t bytes, hipStream_t stream) {
     if (bytes < kMinBytes)
       return false;
     std::lock_guard<std::mutex> lock(mutex);
     if (kept + bytes > limit())
       return false;
-    blocks[key(device, bytes)].push_back(ptr);
+    blocks[key(device, bytes)].push_back(Block{ptr, stream});
     kept += bytes;
     return true;
+  }
+
+  // `stream` has finished all its work and is gone: what it released is
+  // anybody's.
+  void streamRetired(hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(mutex);
+    for (auto &entry : blocks)
+      for (Block &b : entry.second)
+        if (b.stream == stream)
+          b.stream = nullptr;
   }
 
   // Hands every kept block of `device` to `release`.
@@ -269,7 +288,8 @@ public:
         if (int(entry.first >> 48) != device)
           continue;
         kept -= (entry.first & ((uint64_t(1) << 48) - 1)) * entry.second.size();
-        all.insert(all.end(), entry.second.begin(), entry.second.end());
+        for (const Block &b : entry.second)
+          all.push_back(b.ptr);
         entry.second.clear();
       }
     }
@@ -278,6 +298,10 @@ public:
   }
 
 private:
+  struct Block {
+    void *ptr;
+    hipStream_t stream; // the releasing queue's; nullptr: idle for everybody
+  };
   static uint64_t key(int device, size_t bytes) {
     return (uint64_t(device) << 48) | uint64_t(bytes);
   }
@@ -290,7 +314,7 @@ private:
     return value;
   }
   std::mutex mutex;
-  std::unordered_map<uint64_t, std::vector<void *>> blocks;
+  std::unordered_map<uint64_t, std::vector<Block>> blocks;
   size_t kept = 0;
 };
 
@@ -337,8 +361,12 @@ public:
         (void)hipApi().eventDestroy(ev->event);
       delete ev;
     }
-    if (stream)
+    if (stream) {
+      // Drained first: the blocks this queue released become anybody's.
+      (void)hipApi().streamSynchronize(stream);
       (void)hipApi().streamDestroy(stream);
+      deviceBlockCache().streamRetired(stream);
+    }
   }
 
   std::string_view getDeviceName() override { return deviceName; }
@@ -526,7 +554,7 @@ public:
                                   : (size ? size : 1);
     switch (type) {
     case GPUX_ALLOC_DEVICE:
-      ptr = deviceBlockCache().take(device, bytes);
+      ptr = deviceBlockCache().take(device, bytes, stream);
       if (!ptr && (hipApi().malloc_(&ptr, bytes) != hipSuccess || !ptr)) {
         // give back what is kept and try once more
         ptr = nullptr;
@@ -573,7 +601,7 @@ public:
       if (info.kind == GPUX_ALLOC_HOST)
         check(hipApi().hostFree(ptr), "hipHostFree");
       else if (info.kind != GPUX_ALLOC_DEVICE ||
-               !deviceBlockCache().put(info.device, ptr, info.bytes))
+               !deviceBlockCache().put(info.device, ptr, info.bytes, stream))
         check(hipApi().free_(ptr), "hipFree");
     }
     release(); // taken in alloc()
@@ -757,7 +785,13 @@ GPUX_EXPORT void gpuxWait(void *queue, void *event) {
 
 GPUX_EXPORT void gpuxDestroyEvent(void *queue, void *event) {
   CallLog log(__func__);
-  guarded([&]() { toQueue(queue)->destroyEvent(static_cast<Event *>(event)); });
+  guarded([&]() {
+    // The event goes back to the pool of the queue that handed it out (and
+    // drops that queue's reference), whichever queue the caller names.
+    Queue *named = toQueue(queue);
+    Event *ev = static_cast<Event *>(event);
+    (ev && ev->owner ? ev->owner : named)->destroyEvent(ev);
+  });
 }
 
 GPUX_EXPORT void gpuxAlloc(void *queue, size_t size, size_t alignment, int type,

@@ -2257,6 +2257,9 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     source = HEADER.format(name=func.__name__) + "\n" + text.replace("NMK_KERNEL_NAME", name) + "\n"
     compiled = CompiledKernel(name, source, tr.local_arrays)
     compiled.boundscheck = boundscheck
+    # translated for arguments that do not overlap (__restrict__ pointers,
+    # streaming stores, loads ahead of the body): launches must keep to that
+    compiled.noalias = bool(noalias)
     compiled.reversed_dims = tr.reversed
     # a remapped kernel runs blocks of shape (n, 1, 1) and gives each lane this
     # many work-items along hardware y: the launcher divides that grid

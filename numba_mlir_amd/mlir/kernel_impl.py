@@ -511,6 +511,13 @@ class LaunchPlan:
                     f"{self.func_name}: the result array must have dtype "
                     f"{self._ret_key[0] if self._ret_key else None} and the shape and strides "
                     "this launch was prepared for")
+            arrays = [a for a in args if isinstance(a, HipNdArray)]
+            if ret is not None:
+                arrays.append(ret)
+            if getattr(self.compiled, "noalias", False) and not disjoint(arrays):
+                raise ValueError(
+                    f"{self.func_name}: this launch was translated for arrays that do not "
+                    "overlap; the arguments given do")
         with self._lock:                  # the launch call copies the values out
             if args is not None:
                 self._refresh(args, ret, ())

@@ -440,6 +440,10 @@ def test_enqueued_launches_are_covered_by_synchronize(env):
         plan.enqueue([d_a, hip.asarray(np.zeros(a.size, np.float32))])
     with pytest.raises(ValueError, match="differ in type, shape or strides"):
         plan.enqueue([hip.asarray(a[:100]), outs[0]])
+    # a launch translated for arrays that do not overlap refuses ones that do
+    assert plan.compiled.noalias
+    with pytest.raises(ValueError, match="do not\\s+overlap"):
+        plan.enqueue([d_a, d_a])
     g = njit(lambda a, b: a * 2 + b)          # a generated kernel that returns an array
     small = hip.asarray(np.arange(64, dtype=np.int32))
     g(small, small)

@@ -65,6 +65,40 @@ def test_reference_reduce_1d(env, size):
     np.testing.assert_allclose(got, a.astype(np.float64).sum(), rtol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_min_max_skip_nans_as_the_reference_fold_does(env, dtype):
+    """The reference folds select(x < acc, x, acc) from +inf (builtin/funcs.py:
+    145-146, numpy/funcs.py:283-303): a NaN never wins, whatever its position;
+    all-NaN and empty inputs give the starting value.  numpy.fmin / fmax
+    reduced from the same starting value are that fold's closed form."""
+    hip, ops, _ = env
+    rng = np.random.default_rng(11)
+    for shape in ((7,), (300,), (70000,), (5, 9), (129, 1000), (2000, 33)):
+        a = rng.standard_normal(shape).astype(dtype)
+        flat = a.reshape(-1)
+        for where in (0, flat.size // 2, flat.size - 1):     # first, middle, last
+            b = flat.copy()
+            b[where] = np.nan
+            b = b.reshape(shape)
+            d = hip.asarray(b)
+            assert ops.amin(d) == np.fmin.reduce(b, axis=None, initial=np.inf)
+            assert ops.amax(d) == np.fmax.reduce(b, axis=None, initial=-np.inf)
+            if b.ndim == 2:
+                for axis in (0, 1):
+                    np.testing.assert_array_equal(
+                        ops.amin(d, axis=axis).asnumpy(),
+                        np.fmin.reduce(b, axis=axis, initial=np.inf))
+                    np.testing.assert_array_equal(
+                        ops.amax(d, axis=axis).asnumpy(),
+                        np.fmax.reduce(b, axis=axis, initial=-np.inf))
+    every = hip.asarray(np.full((4, 6), np.nan, dtype))
+    assert ops.amin(every) == np.inf and ops.amax(every) == -np.inf
+    np.testing.assert_array_equal(ops.amin(every, axis=1).asnumpy(), np.full(4, np.inf, dtype))
+    none = hip.asarray(np.zeros((0, 3), dtype))
+    assert ops.amin(none) == np.inf and ops.amax(none) == -np.inf
+    np.testing.assert_array_equal(ops.amax(none, axis=0).asnumpy(), np.full(3, -np.inf, dtype))
+
+
 def test_int_dtype_promotion(env):
     hip, ops, _ = env
     a = np.full((70000, 8), 2 ** 31 - 1, np.int32)

@@ -328,6 +328,57 @@ def test_large_device_blocks_are_kept_for_reuse(rt, qk):
         rt.gpuxDeAlloc(q, p)
 
 
+def test_kept_blocks_go_back_to_the_queue_that_released_them(rt, qk):
+    """A released block may still be in use by work of the releasing queue's
+    stream: only that queue (same in-order stream) gets it back at once;
+    another queue on the device gets it once the first one's stream has been
+    drained and destroyed."""
+    q, _, _ = qk
+    res = AllocResult()
+
+    def alloc(queue, nbytes):
+        rt.gpuxAlloc(queue, nbytes, 64, 0, NO_DEPS, ctypes.byref(res))
+        rt.gpuxDestroyEvent(queue, res.event)
+        return res.ptr
+
+    size = 3 << 20                                           # a size no other test keeps
+    q2 = rt.gpuxQueueCreate(None)                            # same device, its own stream
+    a = alloc(q2, size)
+    rt.gpuxDeAlloc(q2, a)
+    mallocs = counter(rt, "mallocs_device")
+    b = alloc(q, size)                                       # q must not see q2's block
+    assert b != a and counter(rt, "mallocs_device") == mallocs + 1
+    c = alloc(q2, size)                                      # q2 itself does
+    assert c == a and counter(rt, "mallocs_device") == mallocs + 1
+    rt.gpuxDeAlloc(q2, c)
+    syncs = counter(rt, "stream_syncs")
+    rt.gpuxQueueDestroy(q2)                                  # last reference: drained, destroyed
+    assert counter(rt, "stream_syncs") == syncs + 1
+    d = alloc(q, size)                                       # now anybody's
+    assert d == a and counter(rt, "mallocs_device") == mallocs + 1
+    rt.gpuxDeAlloc(q, b)
+    rt.gpuxDeAlloc(q, d)
+
+
+def test_an_event_returns_to_the_queue_that_handed_it_out(rt, qk):
+    """gpuxDestroyEvent names a queue, but the event belongs to its owner's
+    pool and holds a reference to the owner: both go back there."""
+    q, _, k = qk
+    q2 = rt.gpuxQueueCreate(None)
+    descs, _ = make_params([])
+    rt.mockExpectParams(0)
+    streams = counter(rt, "streams_live")
+    ev = rt.gpuxLaunchKernel(q, k, 1, 1, 1, 1, 1, 1, NO_DEPS, descs)
+    rt.gpuxWait(q, ev)
+    rt.gpuxDestroyEvent(q2, ev)                              # the wrong queue is named
+    rt.gpuxQueueDestroy(q2)                                  # q2 held no event: it goes
+    assert counter(rt, "streams_live") == streams - 1
+    ev2 = rt.gpuxLaunchKernel(q, k, 1, 1, 1, 1, 1, 1, NO_DEPS, descs)
+    assert ev2 == ev                                         # reused from q's own pool
+    rt.gpuxWait(q, ev2)
+    rt.gpuxDestroyEvent(q, ev2)
+
+
 def test_event_pool_reuses_events(rt, qk):
     """Cross-queue use creates a device event once per pooled slot."""
     q, _, k = qk
