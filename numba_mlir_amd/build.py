@@ -9,6 +9,8 @@ reference: numba_mlir/numba_mlir/mlir/utils.py:17-42):
   libnumba-mlir-hip-offload.so        lowered host code, dispatcher and the
                                       embedded code objects of the kernels
                                       (plain C++, does not link HIP)
+  libnumba-mlir-python-runtime-hip.so the unboxer of HIP device arrays and the
+                                      MemInfo helpers (CPython API, no HIP)
   libnmhip-bench-timer.so             HIP-event stopwatch used by bench.py
   hip-runner                          standalone runner of the reference's
                                       mlir/test/L0_RUNNER cases against a gpux*
@@ -120,6 +122,16 @@ def build_bench_timer():
           "-o", os.path.join(HERE, BENCH_TIMER_LIB), *HIP_LINK_FLAGS])
 
 
+PYTHON_RT_LIB = "libnumba-mlir-python-runtime-hip.so"
+
+
+def build_python_runtime():
+    import sysconfig
+    _run([CXX, *HOST_FLAGS, "-I" + sysconfig.get_paths()["include"], "-shared",
+          os.path.join(CSRC, "python_runtime", "HipBoxing.cpp"),
+          "-o", os.path.join(HERE, PYTHON_RT_LIB)])
+
+
 BENCH_YARDSTICKS = os.path.join(BUILD, "bench_yardsticks.hsaco")
 
 
@@ -152,6 +164,7 @@ def build_all(jobs=4):
         futures.append(pool.submit(build_bench_timer))
         futures.append(pool.submit(build_bench_yardsticks))
         futures.append(pool.submit(build_runner))
+        futures.append(pool.submit(build_python_runtime))
         for f in futures:
             f.result()
     build_offload()  # embeds the code objects built above
@@ -159,7 +172,8 @@ def build_all(jobs=4):
 
 def libraries_present():
     return all(os.path.exists(os.path.join(HERE, n))
-               for n in (RUNTIME_LIB, MATH_LIB, OFFLOAD_LIB, BENCH_TIMER_LIB, RUNNER)) \
+               for n in (RUNTIME_LIB, MATH_LIB, OFFLOAD_LIB, BENCH_TIMER_LIB, RUNNER,
+                         PYTHON_RT_LIB)) \
         and os.path.exists(BENCH_YARDSTICKS)
 
 

@@ -255,7 +255,9 @@ class HipNdArray:
         return {
             "data": (self.ptr, False),
             "shape": self.shape,
-            "strides": self.strides,
+            # in elements, None for a dense row-major array: the convention
+            # of __sycl_usm_array_interface__, which the unboxer follows
+            "strides": None if self.is_c_contiguous() else self.elem_strides,
             "typestr": self.dtype.str,
             "version": 1,
             "queue": self.ctx.queue,

@@ -44,6 +44,17 @@ def test_math_runtime_exports(native_libs):
     assert _exported("libnumba-mlir-math-hip-runtime.so") == declared
 
 
+def test_python_runtime_exports(native_libs):
+    declared = _declared("PythonRuntime.h")
+    assert declared == ["nmrtAllocMemInfo", "nmrtSetMemInfoAllocFunc", "nmrtUnboxHipInterface"]
+    assert _exported("libnumba-mlir-python-runtime-hip.so") == declared
+    # CPython API only: no HIP and no libpython of its own
+    needed = subprocess.run(["readelf", "-d", os.path.join(
+        PKG, "libnumba-mlir-python-runtime-hip.so")], check=True, capture_output=True,
+        text=True).stdout
+    assert "amdhip64" not in needed and "libpython" not in needed
+
+
 def test_offload_exports(native_libs):
     declared = _declared("Offload.h")
     assert _exported("libnumba-mlir-hip-offload.so") == declared

@@ -24,7 +24,12 @@ def test_round_trip_and_interface(env, usm_type, order):
     np.testing.assert_array_equal(d.asnumpy(), a)
     iface = d.__hip_array_interface__
     assert iface["data"] == (d.ptr, False) and iface["shape"] == a.shape
-    assert iface["strides"] == a.strides and iface["typestr"] == a.dtype.str
+    assert iface["strides"] == (None if order == "C" else (1, 4))     # in elements
+    assert iface["typestr"] == a.dtype.str
+    from numba_mlir_amd.mlir import python_rt
+    rec = python_rt.unbox(d)               # what compiled code would receive
+    assert rec.data == d.ptr and rec.nitems == 24 and rec.itemsize == 8
+    assert tuple(rec.shape) == a.shape and tuple(rec.strides) == a.strides
     assert iface["queue"] == hip.get_context().queue
     np.testing.assert_array_equal(d.T.asnumpy(), a.T)
     if usm_type != "device":
