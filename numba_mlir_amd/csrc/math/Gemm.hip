@@ -199,11 +199,32 @@ template <int MASK> __device__ __forceinline__ void sched_groups(int n) {
 // BK) each; slice z leaves its unscaled partial product in the workspace,
 // W[z][M][N] with row stride ldw, and gemm_splitk_fold adds the slices in
 // index order.  Used when the tiles alone would leave most CUs idle.
+//
+// Even shares (streamSlabs > 0): the work is counted in units of one K slab of
+// one block tile, tiles in row-major order, streamSlabs units a tile; the
+// launch runs just as many blocks as are resident at once (grid.x of them,
+// grid.y = grid.z = 1) and block g takes the units [g U / G, (g + 1) U / G):
+// the end of one tile, whole tiles, the beginning of another.  A whole tile
+// goes to C as usual; a piece of one is left, unscaled, in the workspace --
+// a dense BM x BN tile at W[(2 g + j) BM BN], j = 0 for the block's first
+// segment, 1 for a later one (which can only be its last) -- and
+// gemm_even_fold adds a tile's pieces in K order.  Used when whole tiles
+// would leave the last round of blocks mostly empty (576 tiles on 256 CUs:
+// 2.25 rounds) or would not fill the first.
+struct EvenShares {
+  int slabs;  // K slabs a tile (0: not in use)
+  int tilesN; // block tiles along N
+};
+__host__ __device__ inline int64_t evenSharesStart(int64_t g, int64_t units,
+                                                   int64_t blocks) {
+  return g * units / blocks; // (units * blocks stays far below 2^63)
+}
+
 template <typename T, int BK, int TM, int TN, bool A_KC, bool B_NC, bool GUARD = false>
 __global__ __launch_bounds__(256, sizeof(T) == 8 ? 2 : 1) void
 gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
           int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, T alpha,
-          T beta, int sliceK, T *__restrict__ W, int64_t ldw) {
+          T beta, int sliceK, T *__restrict__ W, int64_t ldw, EvenShares even) {
   typedef Mfma<T> MF;
   constexpr int TILE = MF::TILE;
   constexpr int BM = 2 * TM * TILE, BN = 2 * TN * TILE;
@@ -224,8 +245,34 @@ gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
   const int lane = tid % 64;
   const int wave = tid / 64;
   const int wm = wave / 2, wn = wave % 2;
-  const int bm = blockIdx.y * BM;
-  const int bn = blockIdx.x * BN;
+  const int kLane = lane / TILE, xLane = lane % TILE;
+
+  // This block's units (one segment, the whole of K of one tile, without
+  // even shares).
+  int64_t unit = 0, unitEnd = 0;
+  const int slabsPerTile = even.slabs > 0 ? even.slabs : (K + BK - 1) / BK;
+  if (even.slabs > 0) {
+    const int64_t units = int64_t((M + BM - 1) / BM) * even.tilesN * even.slabs;
+    unit = evenSharesStart(blockIdx.x, units, gridDim.x);
+    unitEnd = evenSharesStart(int64_t(blockIdx.x) + 1, units, gridDim.x);
+  } else {
+    unitEnd = slabsPerTile;
+  }
+#pragma nounroll
+  for (int segment = 0; unit < unitEnd; ++segment) {
+  int bm = blockIdx.y * BM, bn = blockIdx.x * BN;
+  int slab0 = 0, slab1 = slabsPerTile; // the K slabs of this segment
+  if (even.slabs > 0) {
+    const int64_t tile = unit / even.slabs;
+    slab0 = int(unit - tile * even.slabs);
+    slab1 = unitEnd - unit < even.slabs - slab0 ? slab0 + int(unitEnd - unit) : even.slabs;
+    bm = int(tile / even.tilesN) * BM;
+    bn = int(tile % even.tilesN) * BN;
+    if (segment > 0)
+      __syncthreads(); // every wave is done with the last segment's LDS slabs
+  }
+  unit += slab1 - slab0;
+  const bool piece = even.slabs > 0 && !(slab0 == 0 && slab1 == even.slabs);
 
   SlabFetch<T, BM, BK, A_KC, GUARD> fa;
   SlabFetch<T, BN, BK, !B_NC, GUARD> fb;
@@ -241,8 +288,6 @@ gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
       for (int r = 0; r < MF::NACC; ++r)
         acc[i][j][r] = T(0);
 
-  const int nSlabs = (K + BK - 1) / BK; // (a multiple of BK unless GUARD)
-  const int kLane = lane / TILE, xLane = lane % TILE;
   // Operand fragments of one step, double-buffered in registers.
   T a[2][TM], b[2][TN];
   auto fragments = [&](int stage, int slot, int kk) {
@@ -254,8 +299,8 @@ gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
       b[slot][j] = Bs[stage][kk + kLane][wn * (TN * TILE) + j * TILE + xLane];
   };
 
-  fa.fetch(0);
-  fb.fetch(0);
+  fa.fetch(slab0 * BK);
+  fb.fetch(slab0 * BK);
   fa.stash(As[0]);
   fb.stash(Bs[0]);
   __syncthreads();
@@ -282,7 +327,7 @@ gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
     constexpr int STEPS = BK / MF::KSTEP, NMFMA = TM * TN;
     static_assert(STEPS >= 4 && STEPS % 2 == 0, "fragment slots alternate over a slab");
     constexpr int WRITE_STEPS = STEPS / 2 - 1, WRITE_FROM = STEPS - 1 - WRITE_STEPS;
-    const int cur = s & 1;
+    const int cur = (s - slab0) & 1;
     if (MORE) {
       fa.fetch((s + 1) * BK);
       fb.fetch((s + 1) * BK);
@@ -338,27 +383,96 @@ gemm_mfma(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
       }
     }
   };
-  for (int s = 0; s + 1 < nSlabs; ++s)
+  for (int s = slab0; s + 1 < slab1; ++s)
     slab(s, std::true_type());
-  slab(nSlabs - 1, std::false_type());
+  slab(slab1 - 1, std::false_type());
 
+  // A whole tile goes to C, scaled; a piece of one goes to its workspace
+  // slot as a dense BM x BN block, unscaled.
+  T *out = C + int64_t(bm) * ldc + bn;
+  int64_t ldo = ldc;
+  T scale = alpha, keep = beta;
+  int rowsLeft = GUARD ? M - bm : BM, colsLeft = GUARD ? N - bn : BN;
+  if (piece) {
+    out = W + (int64_t(blockIdx.x) * 2 + (segment > 0 ? 1 : 0)) * (BM * BN);
+    ldo = BN;
+    scale = T(1);
+    keep = T(0);
+    rowsLeft = BM;
+    colsLeft = BN;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      const int col = bn + wn * (TN * TILE) + j * TILE + xLane;
+      const int col = wn * (TN * TILE) + j * TILE + xLane;
 #pragma unroll
       for (int r = 0; r < MF::NACC; ++r) {
-        const int row =
-            bm + wm * (TM * TILE) + i * TILE + MF::accRow(r, lane);
-        if (GUARD && !(row < M && col < N))
+        const int row = wm * (TM * TILE) + i * TILE + MF::accRow(r, lane);
+        if (GUARD && !(row < rowsLeft && col < colsLeft))
           continue;
-        T *dst = C + int64_t(row) * ldc + col;
-        T v = alpha * acc[i][j][r];
-        if (beta != T(0))
-          v += beta * *dst;
+        T *dst = out + int64_t(row) * ldo + col;
+        T v = scale * acc[i][j][r];
+        if (keep != T(0))
+          v += keep * *dst;
         *dst = v;
       }
+    }
+  }
+  } // segments
+}
+
+// ---------------------------------------------------------------------------
+// The tiles that gemm_mfma's even shares cut into pieces: C[tile] = alpha *
+// (piece + piece + ...) + beta * C[tile], pieces in K order (the order of the
+// blocks that computed them: a fixed order).  One block per tile row-chunk:
+// grid (tiles, BM * BN / (256 * VEC * ROWS))...  A thread owns one 128-bit
+// word of the tile; stores to C are per element and stay inside C.
+template <typename T, int BM, int BN>
+__global__ __launch_bounds__(256) void
+gemm_even_fold(const T *__restrict__ W, int64_t blocks, int slabs, int tilesN,
+               int64_t units, T *__restrict__ C, int M, int N, int64_t ldc,
+               T alpha, T beta) {
+  typedef typename Mfma<T>::Vec Vec;
+  constexpr int VEC = Mfma<T>::VEC;
+  const int64_t tile = blockIdx.x;
+  const int64_t u0 = tile * slabs, u1 = u0 + slabs;
+  // the block whose share holds the tile's first unit
+  int64_t g = u0 * blocks / units;
+  while (g > 0 && evenSharesStart(g, units, blocks) > u0)
+    --g;
+  while (g + 1 < blocks && evenSharesStart(g + 1, units, blocks) <= u0)
+    ++g;
+  {
+    const int64_t b = evenSharesStart(g, units, blocks);
+    const int64_t e = evenSharesStart(g + 1, units, blocks);
+    if (b <= u0 && e >= u1)
+      return; // one block computed the whole tile and stored it itself
+  }
+  const int word = blockIdx.y * 256 + threadIdx.x; // of BM * BN / VEC
+  const int row = word / (BN / VEC), col = (word % (BN / VEC)) * VEC;
+  Vec sum;
+#pragma unroll
+  for (int q = 0; q < VEC; ++q)
+    sum[q] = T(0);
+  for (; g < blocks; ++g) {
+    const int64_t b = evenSharesStart(g, units, blocks);
+    if (b >= u1)
+      break;
+    const T *slot = W + (g * 2 + (b >= u0 ? 0 : 1)) * int64_t(BM * BN);
+    sum += *reinterpret_cast<const Vec *>(slot + row * BN + col);
+  }
+  const int gr = int(tile / tilesN) * BM + row, gc = int(tile % tilesN) * BN + col;
+  if (gr >= M)
+    return;
+  T *dst = C + int64_t(gr) * ldc + gc;
+#pragma unroll
+  for (int q = 0; q < VEC; ++q) {
+    if (gc + q < N) {
+      T v = alpha * sum[q];
+      if (beta != T(0))
+        v += beta * dst[q];
+      dst[q] = v;
     }
   }
 }
@@ -558,6 +672,22 @@ SplitPlan planSplit(int64_t tiles, int64_t K, int BK, int blocksPerCu) {
   return plan;
 }
 
+// Blocks of an even-shares launch over `tiles` block tiles of `slabs` K slabs
+// each on `slots` resident blocks, or 0 when whole tiles do as well: they
+// fill their rounds to nine tenths or more, or a block's share would be under
+// eight slabs (the pieces' trip through the workspace would cost more than
+// the idle CUs).
+int planEvenShares(int64_t tiles, int64_t slabs, int64_t slots) {
+  if (tiles <= 0 || slabs <= 0)
+    return 0;
+  const int64_t rounds = (tiles + slots - 1) / slots;
+  if (tiles * 10 >= rounds * slots * 9)
+    return 0;
+  if (tiles * slabs < 8 * slots)
+    return 0;
+  return int(slots);
+}
+
 enum WorkspaceKind { WORKSPACE_HEAP, WORKSPACE_FIXED };
 
 template <typename T> struct MemrefOf;
@@ -648,12 +778,37 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
     }
     return static_cast<T *>(p);
   };
+  // Workspace of an even-shares launch: two BM x BN slots a block; the
+  // shares are given up (0 blocks) when there is no room.
+  auto evenWorkspace = [&](int &blocks, int bm, int bn) -> T * {
+    if (blocks <= 0)
+      return nullptr;
+    void *p = heapWorkspace(device, size_t(blocks) * 2 * size_t(bm) * size_t(bn) * sizeof(T));
+    if (!p)
+      blocks = 0;
+    return static_cast<T *>(p);
+  };
+  const int64_t slots = 512; // resident blocks of the 128 x 128 tiles: two a CU
   auto fold = [&](const SplitPlan &plan, const T *W, int64_t m, int64_t n,
                   int64_t ldw, int64_t ldz, T *Z) {
     const int64_t words = m * ((n + Mfma<T>::VEC - 1) / Mfma<T>::VEC);
     hipLaunchKernelGGL(gemm_splitk_fold<T>, dim3(unsigned((words + 255) / 256)),
                        dim3(256), 0, stream, W, plan.slices, m * ldw, ldw, Z,
                        int(m), int(n), ldz, alpha, beta);
+  };
+
+  auto evenFold = [&](const T *W, int blocks, int slabs, int64_t tilesM, int64_t tilesN,
+                      int tile, int64_t m, int64_t n, int64_t ldz, T *Z) {
+    const int64_t units = tilesM * tilesN * slabs;
+    dim3 grid(unsigned(tilesM * tilesN), unsigned(tile * tile / Mfma<T>::VEC / 256));
+    if (tile == 256)
+      hipLaunchKernelGGL((gemm_even_fold<T, 256, 256>), grid, dim3(256), 0, stream, W,
+                         int64_t(blocks), slabs, int(tilesN), units, Z, int(m), int(n),
+                         ldz, alpha, beta);
+    else
+      hipLaunchKernelGGL((gemm_even_fold<T, 128, 128>), grid, dim3(256), 0, stream, W,
+                         int64_t(blocks), slabs, int(tilesN), units, Z, int(m), int(n),
+                         ldz, alpha, beta);
   };
 
   if (M > 0 && N > 0) {
@@ -687,8 +842,16 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       // large tile advances K in slabs of 2 BK where K allows (half the
       // barriers; 144 against 142 TFLOP/s on 4096^3).
       const int64_t Mt = Mz - Mz % 128, Nt = Nz - Nz % 128, Kt = K - K % BK;
-      const bool big = sizeof(T) == 4 && Mt % 256 == 0 && Nt % 256 == 0 &&
-                       (Mt / 256) * (Nt / 256) >= 192;
+      // Where whole tiles would leave CUs idle (too few of them, or a last
+      // round that is mostly empty) and K is long enough, the blocks take
+      // even shares of the K slabs of all tiles instead (planEvenShares).
+      const bool bigFits = sizeof(T) == 4 && Mt % 256 == 0 && Nt % 256 == 0;
+      const int64_t bigTiles = (Mt / 256) * (Nt / 256);
+      const int bigSlab = Kt % (2 * BK) == 0 ? 2 * BK : BK;
+      const int bigEven = bigFits && workspaceKind == WORKSPACE_HEAP
+                              ? planEvenShares(bigTiles, Kt / bigSlab, 256)
+                              : 0;
+      const bool big = bigFits && (bigEven > 0 || bigTiles >= 192);
       const int BM = big ? 256 : 128, BN = BM;
       const bool unitOk = (xk == 1 || xm == 1) && (yk == 1 || yn == 1);
       // worth it when the tiled part is most of the work and fills at least
@@ -712,16 +875,28 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           ldx > 0 && ldy > 0 && aligned16(X) && aligned16(Y) && M <= 0x7fffffff &&
           N <= 0x7fffffff && K <= 0x7fffffff - 64 && tilesM <= 65535 &&
           tilesM * tilesN >= 16) {
-        SplitPlan plan = planSplit(tilesM * tilesN, K, BK, sizeof(T) == 8 ? 2 : 1);
+        const int slabs = int((K + BK - 1) / BK);
+        int evenBlocks = workspaceKind == WORKSPACE_HEAP
+                             ? planEvenShares(tilesM * tilesN, slabs, slots)
+                             : 0;
+        T *W = evenWorkspace(evenBlocks, 128, 128);
+        SplitPlan plan;
+        if (!evenBlocks)
+          plan = planSplit(tilesM * tilesN, K, BK, sizeof(T) == 8 ? 2 : 1);
         const int64_t ldw = (Nz + VEC - 1) / VEC * VEC;
-        T *W = workspaceFor(plan, Mz, ldw);
+        if (!evenBlocks)
+          W = workspaceFor(plan, Mz, ldw);
         if (tooLarge)
           return 1;
+        const EvenShares even{evenBlocks ? slabs : 0, int(tilesN)};
         dim3 grid(unsigned(tilesN), unsigned(tilesM), unsigned(plan.slices));
+        if (evenBlocks)
+          grid = dim3(unsigned(evenBlocks), 1, 1);
 #define NMHIP_GEMM_RAGGED(TM, TN, XKC, YNC)                                    \
   hipLaunchKernelGGL((gemm_mfma<T, BK, TM, TN, XKC, YNC, true>), grid,         \
                      dim3(256), 0, stream, X, Y, cData, int(Mz), int(Nz),      \
-                     int(K), ldx, ldy, ldz, alpha, beta, plan.sliceK, W, ldw)
+                     int(K), ldx, ldy, ldz, alpha, beta, plan.sliceK, W, ldw,  \
+                     even)
 #define NMHIP_GEMM_RAGGED_LAYOUTS(TM, TN)                                      \
   do {                                                                         \
     if (xKc && yNc)                                                            \
@@ -735,14 +910,18 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
   } while (0)
         if constexpr (sizeof(T) == 4) {
           NMHIP_GEMM_RAGGED_LAYOUTS(2, 2);
-          lastKernel = plan.slices > 1 ? "sgemm_mfma_128x128_ragged_splitk"
-                                       : "sgemm_mfma_128x128_ragged";
+          lastKernel = evenBlocks        ? "sgemm_mfma_128x128_ragged_even"
+                       : plan.slices > 1 ? "sgemm_mfma_128x128_ragged_splitk"
+                                         : "sgemm_mfma_128x128_ragged";
         } else {
           NMHIP_GEMM_RAGGED_LAYOUTS(4, 4);
-          lastKernel = plan.slices > 1 ? "dgemm_mfma_128x128_ragged_splitk"
-                                       : "dgemm_mfma_128x128_ragged";
+          lastKernel = evenBlocks        ? "dgemm_mfma_128x128_ragged_even"
+                       : plan.slices > 1 ? "dgemm_mfma_128x128_ragged_splitk"
+                                         : "dgemm_mfma_128x128_ragged";
         }
-        if (plan.slices > 1)
+        if (evenBlocks)
+          evenFold(W, evenBlocks, slabs, tilesM, tilesN, 128, Mz, Nz, ldz, cData);
+        else if (plan.slices > 1)
           fold(plan, W, Mz, Nz, ldw, ldz, cData);
 #undef NMHIP_GEMM_RAGGED_LAYOUTS
 #undef NMHIP_GEMM_RAGGED
@@ -751,17 +930,31 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           ldx % VEC == 0 && ldy % VEC == 0 && ldx > 0 && ldy > 0 &&
           aligned16(X) && aligned16(Y) && M <= 0x7fffffff && N <= 0x7fffffff &&
           K <= 0x7fffffff && Mz <= 65535 * 32) {
+        const int slabK = big ? bigSlab : BK;
+        const int slabs = int(Kt / slabK);
+        int evenBlocks = big ? bigEven
+                         : workspaceKind == WORKSPACE_HEAP
+                             ? planEvenShares((Mt / BM) * (Nt / BN), slabs, slots)
+                             : 0;
+        T *W = evenWorkspace(evenBlocks, BM, BN);
+        if (big && !evenBlocks && bigTiles < 192)
+          fatal("mkl_gemm_device: no workspace for %lld tiles of 256 x 256\n",
+                (long long)bigTiles);
         SplitPlan plan;
-        if (!big)
+        if (!big && !evenBlocks) {
           plan = planSplit((Mt / BM) * (Nt / BN), Kt, BK, sizeof(T) == 8 ? 2 : 1);
-        T *W = workspaceFor(plan, Mt, Nt);
+          W = workspaceFor(plan, Mt, Nt);
+        }
         if (tooLarge)
           return 1;
+        const EvenShares even{evenBlocks ? slabs : 0, int(Nt / BN)};
         dim3 grid(unsigned(Nt / BN), unsigned(Mt / BM), unsigned(plan.slices));
+        if (evenBlocks)
+          grid = dim3(unsigned(evenBlocks), 1, 1);
 #define NMHIP_GEMM_LAUNCH(SLAB, TM, TN, XKC, YNC)                              \
   hipLaunchKernelGGL((gemm_mfma<T, SLAB, TM, TN, XKC, YNC>), grid, dim3(256),  \
                      0, stream, X, Y, cData, int(Mt), int(Nt), int(Kt), ldx,   \
-                     ldy, ldz, alpha, beta, plan.sliceK, W, int64_t(Nt))
+                     ldy, ldz, alpha, beta, plan.sliceK, W, int64_t(Nt), even)
 #define NMHIP_GEMM_LAYOUTS(SLAB, TM, TN)                                       \
   do {                                                                         \
     if (xKc && yNc)                                                            \
@@ -774,29 +967,35 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       NMHIP_GEMM_LAUNCH(SLAB, TM, TN, false, false);                           \
   } while (0)
         if constexpr (sizeof(T) == 4) {
-          if (big && Kt % (2 * BK) == 0) {
+          if (big && bigSlab == 2 * BK)
             NMHIP_GEMM_LAYOUTS(2 * BK, 4, 4);
-            lastKernel = whole ? "sgemm_mfma_256x256" : "sgemm_mfma_256x256+edges";
-          } else if (big) {
+          else if (big)
             NMHIP_GEMM_LAYOUTS(BK, 4, 4);
-            lastKernel = whole ? "sgemm_mfma_256x256" : "sgemm_mfma_256x256+edges";
-          } else {
+          else
             NMHIP_GEMM_LAYOUTS(BK, 2, 2);
-            lastKernel = plan.slices > 1
-                             ? (whole ? "sgemm_mfma_128x128_splitk"
-                                      : "sgemm_mfma_128x128_splitk+edges")
-                             : (whole ? "sgemm_mfma_128x128"
-                                      : "sgemm_mfma_128x128+edges");
-          }
+          static const char *const names[2][4][2] = {
+              {{"sgemm_mfma_128x128", "sgemm_mfma_128x128+edges"},
+               {"sgemm_mfma_128x128_splitk", "sgemm_mfma_128x128_splitk+edges"},
+               {"sgemm_mfma_128x128_even", "sgemm_mfma_128x128_even+edges"},
+               {"", ""}},
+              {{"sgemm_mfma_256x256", "sgemm_mfma_256x256+edges"},
+               {"", ""},
+               {"sgemm_mfma_256x256_even", "sgemm_mfma_256x256_even+edges"},
+               {"", ""}}};
+          lastKernel = names[big ? 1 : 0][evenBlocks ? 2 : plan.slices > 1 ? 1 : 0][whole ? 0 : 1];
         } else {
           NMHIP_GEMM_LAYOUTS(BK, 4, 4);
-          lastKernel = plan.slices > 1
+          lastKernel = evenBlocks ? (whole ? "dgemm_mfma_128x128_even"
+                                           : "dgemm_mfma_128x128_even+edges")
+                       : plan.slices > 1
                            ? (whole ? "dgemm_mfma_128x128_splitk"
                                     : "dgemm_mfma_128x128_splitk+edges")
                            : (whole ? "dgemm_mfma_128x128"
                                     : "dgemm_mfma_128x128+edges");
         }
-        if (plan.slices > 1)
+        if (evenBlocks)
+          evenFold(W, evenBlocks, slabs, Mt / BM, Nt / BN, BM, Mt, Nt, ldz, cData);
+        else if (plan.slices > 1)
           fold(plan, W, Mt, Nt, Nt, ldz, cData);
 #undef NMHIP_GEMM_LAYOUTS
 #undef NMHIP_GEMM_LAUNCH

@@ -22,9 +22,10 @@ def env(hip):
 
 
 def _kernel(mrt):
-    """Name of the last gemm kernel without the split-K marker (whether K is
-    cut into slices depends only on how many tiles the shape has)."""
-    return mrt.last_kernel().replace("_splitk", "")
+    """Name of the last gemm kernel without the marker of how K was shared
+    out (split into slices, or even shares of the slabs of all tiles: that
+    depends only on how many tiles the shape has)."""
+    return mrt.last_kernel().replace("_splitk", "").replace("_even", "")
 
 
 def _printed(x):
@@ -301,7 +302,7 @@ def test_split_k(env, dtype, ta, tb, tc, m, n, k):
     for _ in range(2):
         d_c = _to_dev(hip, lay(c0, tc))
         ops.gemm(d_a, d_b, d_c, 1.5, -0.5)
-        assert "_splitk" in mrt.last_kernel(), mrt.last_kernel()
+        assert "_splitk" in mrt.last_kernel() or "_even" in mrt.last_kernel(), mrt.last_kernel()
         runs.append(d_c.asnumpy())
     assert np.array_equal(runs[0], runs[1])
     _check_scaled(runs[0], a, b, c0, 1.5, -0.5, 1e-5 if dtype == np.float32 else 1e-13)
@@ -315,3 +316,55 @@ def test_split_k_beta_zero_ignores_c(env):
     ops.gemm(hip.asarray(a), hip.asarray(b), c, 1.0, 0.0)
     assert "_splitk" in mrt.last_kernel()
     assert (c.asnumpy() == 2048).all()
+
+
+# ---- even shares: the K slabs of all tiles dealt out to the resident blocks ------
+
+@pytest.mark.parametrize("dtype,m,n,k,kernel", [
+    # 576 tiles of 256 x 256, eight slabs each: a share is 2.25 tiles (the end
+    # of one, a whole one, the beginning of the next)
+    (np.float32, 6144, 6144, 256, "sgemm_mfma_256x256_even"),
+    # 16 tiles on 256 blocks: every tile in sixteen pieces
+    (np.float32, 1024, 1024, 4096, "sgemm_mfma_256x256_even"),
+    (np.float32, 2048, 2048, 2048 + 16, "sgemm_mfma_256x256_even"),   # slabs of 16
+    (np.float32, 1536, 1408, 2056, "sgemm_mfma_128x128_even+edges"),  # the rest of K beside
+    (np.float32, 1000, 1100, 1200, "sgemm_mfma_128x128_ragged_even"),
+    (np.float32, 2000, 2300, 2600, "sgemm_mfma_128x128_ragged_even"),
+    (np.float64, 3072, 3072, 512, "dgemm_mfma_128x128_even"),         # 1.125 rounds
+    (np.float64, 1024, 1024, 4096, "dgemm_mfma_128x128_even"),
+    (np.float64, 1000, 1100, 1200, "dgemm_mfma_128x128_ragged_even"),  # the reference's preset
+    (np.float64, 2500, 2750, 3000, "dgemm_mfma_128x128_ragged_even"),
+])
+@pytest.mark.parametrize("ta,tb,tc", [(False, False, False), (True, False, True),
+                                      (False, True, False)])
+def test_even_shares(env, dtype, m, n, k, kernel, ta, tb, tc):
+    """Whole tiles that would leave most CUs idle (too few, or a nearly empty
+    last round): the blocks take equal shares of all K slabs, pieces of tiles
+    meet in the workspace and are added in K order.  Every element against
+    float64, alpha and beta applied once, the same bits on a second run."""
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(m + 3 * n + 7 * k)
+    a = rng.standard_normal((m, k)).astype(dtype)
+    b = rng.standard_normal((k, n)).astype(dtype)
+    c0 = rng.standard_normal((m, n)).astype(dtype)
+    lay = lambda x, t: np.asfortranarray(x) if t else x
+    d_a, d_b = _to_dev(hip, lay(a, ta)), _to_dev(hip, lay(b, tb))
+    runs = []
+    for _ in range(2):
+        d_c = _to_dev(hip, lay(c0, tc))
+        ops.gemm(d_a, d_b, d_c, 1.5, -0.5)
+        if not tc:       # (a column-major C swaps the operands: another tile count)
+            assert mrt.last_kernel() == kernel
+        runs.append(d_c.asnumpy())
+    assert np.array_equal(runs[0], runs[1])
+    _check_scaled(runs[0], a, b, c0, 1.5, -0.5, 1e-5 if dtype == np.float32 else 1e-13)
+
+
+def test_even_shares_beta_zero_ignores_c_and_the_no_alloc_entry_keeps_slices(env):
+    hip, ops, _, mrt = env
+    a = np.ones((1024, 4096), np.float32)
+    b = np.ones((4096, 1024), np.float32)
+    c = hip.asarray(np.full((1024, 1024), np.nan, np.float32))
+    ops.gemm(hip.asarray(a), hip.asarray(b), c, 1.0, 0.0)
+    assert "_even" in mrt.last_kernel()
+    assert (c.asnumpy() == 4096).all()

@@ -73,11 +73,17 @@ def test_two_calls_in_a_row_match_the_allocating_entry_point(gemm_entry_points):
         status, got, ref, k_ref, k_got, (a, b, c0) = _both(
             hip, lib, mrt, m, n, k, alpha, beta, seed=m + n + k)
         assert status == 0
-        assert k_got == k_ref
         assert ("_splitk" in k_got) == (k > 64)
-        assert np.array_equal(got, ref), (m, n, k)
+        # The allocating entry point may share K out differently (even shares
+        # of the slabs need a larger workspace than the fixed one): the same
+        # kernel gives the same bits, another one the same product to
+        # float32's accuracy.
+        assert k_got == k_ref or "_even" in k_ref, (k_got, k_ref)
+        if k_got == k_ref:
+            assert np.array_equal(got, ref), (m, n, k)
         truth = beta * c0.astype(np.float64) + alpha * (
             a.astype(np.float64) @ b.astype(np.float64))
         scale = abs(beta) * np.abs(c0) + abs(alpha) * (
             np.abs(a).astype(np.float64) @ np.abs(b))
         assert (np.abs(got - truth) <= 1e-4 * scale + 1e-30).all()
+        assert (np.abs(got - ref) <= 1e-4 * scale + 1e-30).all()
