@@ -39,15 +39,16 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 WAKE_SECONDS = 0.1
 
 MEASURED_TRAFFIC = {
-    "nmk_black_scholes_f32_w64": 335662062,
-    "nmk_black_scholes_f32_w32": 335623055,
-    "nmk_map2_rowbcast_add_f64": 268501394,
-    "nmk_sum_axis1_wide_f32": 537392364,
-    "nmk_norm2_f32": 536915968,
-    "nmk_sum_axis0_i32_i64": 538008372,
-    "nmk_twin_pairwise_f64_rows": 540444027,
+    "nmk_black_scholes_f32_w64": 335614484,
+    "bench_streams_3r2w_f32": 335526234,
+    "nmk_black_scholes_f32_w32": 335607299,
+    "nmk_map2_rowbcast_add_f64": 268470962,
+    "nmk_sum_axis1_wide_f32": 537392134,
+    "nmk_norm2_f32": 536915846,
+    "nmk_sum_axis0_i32_i64": 538008264,
+    "nmk_twin_pairwise_f64_rows": 540497146,
     "nmk_copy_b128": 536870912,
-    "sgemm_mfma_256x256": 671497896,
+    "sgemm_mfma_256x256": 671624029,
 }
 
 
