@@ -55,11 +55,14 @@ void mkl_gemm_float64_device(void *queue, const NmhipMemref2F64 *a,
 /*
  * mkl_gemm_float32_device for callers that cannot allocate device memory
  * (code under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc).  No counterpart in the reference.  Same arguments, same
- * kernels, same results as mkl_gemm_float32_device bit for bit; it calls no
- * hipMalloc / hipFree.  Where that entry point takes split-K workspace from
- * a heap block it grows on demand, this one uses a fixed 16 MiB array that
- * lives in the library's device image on every GPU it runs on.  The first
+ * hipMalloc).  No counterpart in the reference.  Same arguments as
+ * mkl_gemm_float32_device; it calls no hipMalloc / hipFree.  Where that
+ * entry point takes its workspace from a heap block it grows on demand, this
+ * one uses a fixed 16 MiB array that lives in the library's device image on
+ * every GPU it runs on, and shares K out over the blocks by split K only
+ * (the even shares of K slabs the allocating entry point may take instead
+ * need up to 128 MiB): where both run the same kernel the results agree bit
+ * for bit, elsewhere to float32's accuracy.  The first
  * call on a device looks the array's address up (no allocation).  Returns 0,
  * or 1 -- with a message on stderr and nothing launched -- when the product
  * would need more split-K workspace than the array holds.  Only shapes with
@@ -68,8 +71,10 @@ void mkl_gemm_float64_device(void *queue, const NmhipMemref2F64 *a,
  * (1024 x 1024 with k >= 512 does), so the limit is a guard, not a case a
  * float32 caller meets.  The array is shared by every call on a GPU and
  * keeps the last call's partial products; nothing in it needs clearing,
- * each slice is written before it is read.  Calls that overlap on one GPU
- * race on it.
+ * each slice is written before it is read.  Calls from several host
+ * threads take turns on it (the library holds a lock while a call's kernels
+ * run); launches captured into graphs and replayed side by side on one GPU
+ * would race on it.
  */
 int mkl_gemm_float32_device_noalloc(void *queue, const NmhipMemref2F32 *a,
                                     const NmhipMemref2F32 *b, float alpha,
@@ -82,7 +87,8 @@ void nmrtMathRuntimeFinalize(void);
 /* Name of the device kernel the most recent gemm call on this thread ran
  * ("sgemm_mfma_256x256", "sgemm_mfma_128x128", "dgemm_mfma_128x128",
  * "sgemm_generic", "dgemm_generic"; "<tile kernel>_ragged" for the guarded
- * instance that takes shapes which are not whole tiles, "_splitk" after
+ * instance that takes shapes which are not whole tiles, "_even" after the
+ * tile kernel's name when the blocks took even shares of all K slabs, "_splitk" after
  * either when K was cut into slices, "<tile kernel>+edges" when the strided
  * kernel completed what the tiles left); for tests and profiling. */
 const char *nmhipMathLastKernel(void);

@@ -584,6 +584,10 @@ struct DeviceWorkspace {
 };
 DeviceWorkspace workspaces[kMaxDevices];
 std::mutex workspaceMutex;
+// Held by a call from the moment it asks for a device's workspace (heap or
+// fixed) until its kernels have finished: calls from several host threads,
+// on whatever queues, take turns on the one workspace of a device.
+std::mutex workspaceInUse[kMaxDevices];
 
 DeviceWorkspace &workspaceOf(int device) {
   if (device < 0 || device >= kMaxDevices)
@@ -753,9 +757,16 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
   // leaves plan unsplit when the heap has no room, reports the fixed array
   // as too small through tooLarge.
   bool tooLarge = false;
+  std::unique_lock<std::mutex> workspaceTurn; // (released when the call returns)
+  auto takeTurn = [&]() {
+    (void)workspaceOf(device); // (checks the ordinal)
+    if (!workspaceTurn.owns_lock())
+      workspaceTurn = std::unique_lock<std::mutex>(workspaceInUse[device]);
+  };
   auto workspaceFor = [&](SplitPlan &plan, int64_t m, int64_t ldw) -> T * {
     if (plan.slices < 2)
       return nullptr;
+    takeTurn();
     const size_t bytes = size_t(plan.slices) * size_t(m) * size_t(ldw) * sizeof(T);
     void *p = nullptr;
     if (workspaceKind == WORKSPACE_FIXED) {
@@ -783,6 +794,7 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
   auto evenWorkspace = [&](int &blocks, int bm, int bn) -> T * {
     if (blocks <= 0)
       return nullptr;
+    takeTurn();
     void *p = heapWorkspace(device, size_t(blocks) * 2 * size_t(bm) * size_t(bn) * sizeof(T));
     if (!p)
       blocks = 0;

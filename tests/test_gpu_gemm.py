@@ -368,3 +368,61 @@ def test_even_shares_beta_zero_ignores_c_and_the_no_alloc_entry_keeps_slices(env
     ops.gemm(hip.asarray(a), hip.asarray(b), c, 1.0, 0.0)
     assert "_even" in mrt.last_kernel()
     assert (c.asnumpy() == 4096).all()
+
+
+def test_calls_from_two_threads_take_turns_on_the_workspace(env):
+    """Two host threads, each with a queue of its own, multiply at the same
+    time through the raw C-ABI (ctypes drops the GIL for the call): products
+    that go through the device's one workspace must not mix."""
+    import ctypes
+    import threading
+    hip, ops, _, mrt = env
+    from numba_mlir_amd.mlir import gpu_runtime
+
+    class Memref2(ctypes.Structure):
+        _fields_ = [("userData", ctypes.c_void_p), ("data", ctypes.c_void_p),
+                    ("offset", ctypes.c_size_t), ("dims", ctypes.c_size_t * 2),
+                    ("strides", ctypes.c_size_t * 2)]
+
+    def memref(arr):
+        r = Memref2()
+        r.userData, r.data, r.offset = None, arr.ptr, 0
+        r.dims[0], r.dims[1] = arr.shape
+        r.strides[0], r.strides[1] = arr.elem_strides
+        return r
+
+    lib = mrt.runtime_hip_lib
+    gemm = lib.mkl_gemm_float32_device
+    gemm.restype = None
+    gemm.argtypes = [ctypes.c_void_p, ctypes.POINTER(Memref2), ctypes.POINTER(Memref2),
+                     ctypes.c_float, ctypes.c_float, ctypes.POINTER(Memref2)]
+    rt = gpu_runtime.runtime_lib
+    shapes = [(1024, 1024, 2048), (640, 768, 4096)]      # both share K out over the blocks
+    work = []
+    for seed, (m, n, k) in enumerate(shapes):
+        rng = np.random.default_rng(seed)
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        b = rng.standard_normal((k, n)).astype(np.float32)
+        work.append((a, b, hip.asarray(a), hip.asarray(b),
+                     hip.asarray(np.zeros((m, n), np.float32)), rt.gpuxQueueCreate(None)))
+    errors = []
+
+    def run(item):
+        a, b, d_a, d_b, d_c, queue = item
+        try:
+            for _ in range(25):
+                gemm(queue, memref(d_a), memref(d_b), 1.0, 0.0, memref(d_c))
+        except Exception as exc:      # noqa: BLE001
+            errors.append(exc)
+
+    threads = [threading.Thread(target=run, args=(item,)) for item in work]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors
+    for a, b, d_a, d_b, d_c, queue in work:
+        truth = a.astype(np.float64) @ b.astype(np.float64)
+        scale = np.abs(a).astype(np.float64) @ np.abs(b)
+        assert (np.abs(d_c.asnumpy() - truth) <= 1e-4 * scale).all()
+        rt.gpuxQueueDestroy(queue)
