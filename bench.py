@@ -253,6 +253,28 @@ def black_scholes_body(price, strike, t, rate, volatility, call, put):
     put[:] = r - P + Se
 
 
+def black_scholes_loop_body(nopt, price, strike, t, rate, volatility, call, put):
+    mr = -rate
+    sig_sig_two = volatility * volatility * 2
+    for i in prange(nopt):        # noqa: F821 -- bound in generated_kernels()
+        P = price[i]
+        S = strike[i]
+        T = t[i]
+        a = math.log(P / S)
+        b = T * mr
+        z = T * sig_sig_two
+        c = 0.25 * z
+        y = 1.0 / math.sqrt(z)
+        w1 = (a - b + c) * y
+        w2 = (a - b - c) * y
+        d1 = 0.5 + 0.5 * math.erf(w1)
+        d2 = 0.5 + 0.5 * math.erf(w2)
+        Se = math.exp(b) * S
+        r = P * d1 - Se * d2
+        call[i] = r
+        put[i] = r - P + Se
+
+
 def scaled_add_body(a, b):
     return a * 2.0 + b
 
@@ -615,6 +637,7 @@ def generated_kernels(b, workloads):
     """The same workloads through the decorators: the body is translated,
     compiled for gfx950 and launched through gpuxLaunchKernel; timed like the
     hand-written kernels, on the generated kernel alone."""
+    from numba_mlir_amd import decorators
     from numba_mlir_amd import kernel as kapi
     from numba_mlir_amd.decorators import njit
 
@@ -654,7 +677,13 @@ def generated_kernels(b, workloads):
         f(*sets[0])
         timed("bs_njit", "Black-Scholes, 2^24 float32 options, the reference's test "
               "body under @njit", 20 * nopt, f.last_plan, sets)
-        del sets
+        globals()["prange"] = decorators.prange
+        loop = njit(parallel=True)(black_scholes_loop_body)
+        loop_sets = [[nopt] + s for s in sets]
+        loop(*loop_sets[0])
+        timed("bs_prange", "Black-Scholes, 2^24 float32 options, the same body as one "
+              "prange loop under @njit(parallel=True)", 20 * nopt, loop.last_plan, loop_sets)
+        del sets, loop_sets
 
         a, _ = workloads.broadcast_add()
         sets = [[da.asarray(a), da.asarray(a)] for _ in range(3)]

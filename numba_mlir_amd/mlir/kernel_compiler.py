@@ -484,6 +484,7 @@ class FunctionTranslator:
         # elementwise 1-d maps over dense arrays: a lane takes ADJACENT
         # elements, 128-bit loads and stores (see translate_kernel)
         self.adjacent = False
+        self.unit_loop_var = None    # parallel mode: the variable of a prange(n) grid loop
         self.adjacent_outs = {}      # output array (code) -> (element ctype, pointer)
         self.speculates = False      # some call of the body has a plain and a careful form
 
@@ -633,7 +634,7 @@ class FunctionTranslator:
         """Template argument of the routines that come in a plain and a
         careful form, where the body is computed under speculation (a fused
         map over adjacent elements), else the empty string."""
-        if self.adjacent and self.mode == "elementwise" and self.is_kernel:
+        if self.adjacent and self.mode in ("elementwise", "parallel") and self.is_kernel:
             self.speculates = True
             return "<decltype(nmk_careful)::value>"
         return ""
@@ -641,6 +642,14 @@ class FunctionTranslator:
     def outputs_are_float32(self):
         """A fused map all of whose results are float32 arrays: its float64
         intermediates need float32's accuracy and a margin, not their own."""
+        if self.is_kernel and self.mode == "parallel":
+            # a loop without reductions that stores into float32 arrays only
+            stored = {n.value.id for n in ast.walk(self.node)
+                      if isinstance(n, ast.Subscript) and isinstance(n.ctx, ast.Store) and
+                      isinstance(n.value, ast.Name)}
+            types = dict(zip(self.params, self.arg_types))
+            return bool(stored) and not self.reductions and all(
+                isinstance(types.get(n), Array) and types[n].elem is FLOAT32 for n in stored)
         if not (self.is_kernel and self.mode == "elementwise") or self.opaque_write:
             return False
         outs = [t.elem for p, t in zip(self.params, self.arg_types)
@@ -657,11 +666,16 @@ class FunctionTranslator:
         (What the body does with them is found out while its statements are
         written: _NotAdjacent.  Maps over 8-byte elements measured faster with
         a lane's elements a block apart.)"""
-        if not (self.is_kernel and self.mode == "elementwise" and self.ndim == 1 and
-                self.noalias and self.elements_per_thread == 4) or \
+        if not (self.is_kernel and self.mode in ("elementwise", "parallel") and
+                self.ndim == 1 and self.noalias and self.elements_per_thread == 4) or \
                 self.m.communicates or self.m.boundscheck or self.reductions or \
                 self.opaque_write:
             return False
+        if self.mode == "parallel":
+            # one prange(n) loop: iteration g is work-item g.  Which arrays it
+            # reads and stores at its own index is settled while the body is
+            # written (check_adjacent_operands).
+            return self.unit_loop_var is not None and len(self.grid_loops) == 1
         elems = [t.elem for t in self.arg_types if isinstance(t, Array)]
         if any(isinstance(t, Array) and (t.layout != "C" or t.ndim != 1)
                for t in self.arg_types):
@@ -669,6 +683,22 @@ class FunctionTranslator:
         if self.ret_type is not None:
             elems.append(self.ret_type)
         return all(e.ctype in self._WORD_CTYPES for e in elems)
+
+    def check_adjacent_operands(self):
+        """After the body has been written: every array loaded ahead of it and
+        every array it stores must be dense with 4-byte elements, and
+        something must be stored."""
+        types = dict(zip(self.params, self.arg_types))
+        for name in self.prefetched:
+            t = types.get(name)
+            if not (isinstance(t, Array) and t.layout == "C" and t.ndim == 1 and
+                    t.elem.ctype in self._WORD_CTYPES):
+                raise _NotAdjacent(f"'{name}' is not a dense array of 4-byte elements")
+        if not self.adjacent_outs:
+            raise _NotAdjacent("no array is assigned at every index")
+        for ctype, _ in self.adjacent_outs.values():
+            if ctype not in self._WORD_CTYPES:
+                raise _NotAdjacent("an assigned array has 8-byte elements")
 
     def adjacent_rounds(self, pf, body):
         """The rounds of a fused map over adjacent elements.  A lane loads its
@@ -1577,7 +1607,21 @@ class FunctionTranslator:
         if not isinstance(v.type, Scalar):
             self.err(node, "Only scalars can be stored into an array element")
         if self.adjacent and self.emitting:
-            raise _NotAdjacent("the body stores single elements")
+            # a prange(n) loop that stores p[i] = value for its own i, in the
+            # loop body itself: the lane's four values leave in one store
+            name = target.value.id if isinstance(target.value, ast.Name) else None
+            t = dict(zip(self.params, self.arg_types)).get(name)
+            if not (self.mode == "parallel" and self.unit_loop_var is not None and
+                    isinstance(target.slice, ast.Name) and
+                    target.slice.id == self.unit_loop_var and
+                    self.loop_kinds == ["grid"] and self.indent == 2 and
+                    name in self.store_only_params() and isinstance(t, Array) and
+                    t.ndim == 1 and t.layout == "C"):
+                raise _NotAdjacent("the body stores single elements")
+            c = self.cname(name)
+            self.adjacent_outs[c] = (elem.ctype, f"{c}_p")
+            self.emit(f"nmk_out.{c} = ({elem.ctype})({cast(v, elem).code});")
+            return
         if self.noalias and self.stream and self.last_elem_gid is not None and \
                 isinstance(target.value, ast.Name) and \
                 target.value.id in self.store_only_params():
@@ -1697,6 +1741,8 @@ class FunctionTranslator:
                 # what every iteration reads at its own index is loaded for
                 # all of a lane's iterations before the first one runs
                 self.ahead_nodes = self.loads_ahead_of(node)
+                if self.store_count.get(name) == 1:
+                    self.unit_loop_var = name      # iteration g is work-item g
             if self.emitting:
                 self.emit(f"{self.cname(name)} = {start.code} + nmk_gid{depth} * {step.code};")
             self.indent -= 1
@@ -1946,8 +1992,7 @@ class FunctionTranslator:
         if self.adjacent:
             try:
                 lines = self.run_emit(body)
-                if not self.adjacent_outs:
-                    raise _NotAdjacent("no array is assigned as a whole")
+                self.check_adjacent_operands()
             except _NotAdjacent:
                 self.adjacent = False
         if not self.adjacent:

@@ -70,12 +70,19 @@ def test_black_scholes_body_unaligned_views_and_ragged_ends(env):
     np.testing.assert_allclose(got[0][1][1:], got[1][1][:-1], rtol=1e-6, atol=1e-6)
 
 
-def test_black_scholes_body_odd_operands(env):
+@pytest.mark.parametrize("form", ["arrays", "loop"])
+def test_black_scholes_body_odd_operands(env, form):
     """Zeros, infinities, NaNs, negative, huge, tiny and denormal operands and
     a discount factor that underflows: the wave computes its options again
     with the general routines and matches the oracle; the everyday options
-    that share a wave with an odd one keep their prices."""
+    that share a wave with an odd one keep their prices.  Both forms of the
+    body: whole arrays, and one prange loop that stores call[i], put[i]."""
     hip, ops, orc, workloads = env
+    if form == "arrays":
+        compiled = njit(cases.black_scholes_arrays)
+    else:
+        loop = njit(parallel=True)(cases.black_scholes_loop)
+        compiled = lambda p, s, t, rate, vol, call, put: loop(len(p), p, s, t, rate, vol, call, put)
     inf, nan = np.inf, np.nan
     price = np.array([30, 0, 30, 0, inf, 30, nan, 30, 30, 1e-30, 50, 10, 1e38, 1e-38, 1e-42,
                       30, 30, -30, 30, 2.0 ** 60, 2.0 ** -61, 30, 1e20], np.float32)
@@ -83,7 +90,7 @@ def test_black_scholes_body_odd_operands(env):
                        1e38, 1e-38, 30, -30, 2.0 ** 59, 2.0 ** -60, 30, 1e-20], np.float32)
     t = np.array([1.5, 1, 1, 1, 1, 1, 1, 1, 0, 1, 2, 1, 1, 1, 1, 1, 1, 1, 1, 1.5, 1.5, 1000, 1],
                  np.float32)
-    f = njit(cases.black_scholes_arrays)
+    f = compiled
     n = len(price)
     d = [hip.asarray(x) for x in (price, strike, t, np.zeros(n, np.float32),
                                   np.zeros(n, np.float32))]

@@ -352,6 +352,32 @@ def test_fused_maps_take_several_elements_per_lane(K, tmp_path, monkeypatch):
     assert "v_a = nmk::logQuotientF32(nmk_pf_price, nmk_pf_strike);" in ck.source
     assert "nmkjit::cdfTableLoad();" in ck.source and "__launch_bounds__(1024)" in ck.source
     assert kc.build_code_object(ck)[:4] == b"\x7fELF"
+    # the loop form of the same body: prange(n), reads p[i], stores call[i], put[i]
+    mode2, ndim2, types2 = _njit_types("black_scholes_loop")
+    ck = kc.translate(njit_cases.black_scholes_loop, types2, ndim2, K, mode=mode2,
+                      noalias=True, elements_per_thread=4)
+    assert "nmk_out.v_call = (float)" in ck.source and "nmk_words" in ck.source
+    assert ("v_a = nmkjit::logQuotientF32m<decltype(nmk_careful)::value>(v_P, v_S, nmk_ok);"
+            in ck.source)
+    assert "v_d2 = nmkjit::cdfTermF64(v_w2);" in ck.source
+    assert ("__builtin_nontemporal_store(nmk_vec_v_put, "
+            "reinterpret_cast<nmk_out_t_v_put *>(v_put_p) + nmk_i);") in ck.source
+    assert kc.build_code_object(ck)[:4] == b"\x7fELF"
+    # ... but not when a store sits under a condition, or at another index
+    def guarded(n, a, out):
+        for i in njit_cases.prange(n):
+            if a[i] > 0:
+                out[i] = a[i]
+
+    def shifted(n, a, out):
+        for i in njit_cases.prange(n):
+            out[i + 1] = a[i]
+
+    f32c1 = kc.Array(kc.FLOAT32, 1, layout="C")
+    for body in (guarded, shifted):
+        ck = kc.translate(body, [kc.INT64, f32c1, f32c1], 1, K, mode="parallel", noalias=True,
+                          elements_per_thread=4)
+        assert "nmk_words" not in ck.source
     # a body that stores single elements keeps one element per lane and trip
     def by_index(a, b, c):
         for i in range(len(a)):
@@ -384,7 +410,15 @@ def test_prange_loops_load_what_every_iteration_reads_ahead(K):
     mode, ndim, types = _njit_types("black_scholes_loop")
     ck = kc.translate(njit_cases.black_scholes_loop, types, ndim, K, mode=mode, noalias=True,
                       elements_per_thread=4)
-    assert "nmk_ahead_price[nmk_rep] = *(&v_price_p[g]);" in ck.source
+    # (dense float32 arrays stored at the loop's own index: four adjacent
+    # iterations a lane, the loads in one 128-bit word per array)
+    assert "nmk_in_price = __builtin_nontemporal_load(" in ck.source
+    assert "v_P = nmk_pf_price;" in ck.source and "v_T = nmk_pf_t;" in ck.source
+    # arrays with a stride: a lane's iterations a block apart
+    strided = [kc.Array(t.elem, 1) if isinstance(t, kc.Array) else t for t in types]
+    ck = kc.translate(njit_cases.black_scholes_loop, strided, ndim, K, mode=mode, noalias=True,
+                      elements_per_thread=4)
+    assert "nmk_ahead_price[nmk_rep] = *(&v_price_p[g * v_price_t0]);" in ck.source
     assert "v_P = nmk_pf_price;" in ck.source and "v_T = nmk_pf_t;" in ck.source
     # overlapping arguments, or one element per lane: every load where it is written
     for kw in ({"noalias": False, "elements_per_thread": 4},
