@@ -90,7 +90,9 @@ void nmrtMathRuntimeFinalize(void);
  * instance that takes shapes which are not whole tiles, "_even" after the
  * tile kernel's name when the blocks took even shares of all K slabs, "_splitk" after
  * either when K was cut into slices, "<tile kernel>+edges" when the strided
- * kernel completed what the tiles left); for tests and profiling. */
+ * kernel completed what the tiles left, "+packed" when an operand whose rows
+ * do not begin and end on 128-bit words was first copied into padded rows);
+ * for tests and profiling. */
 const char *nmhipMathLastKernel(void);
 
 #ifdef __cplusplus

@@ -43,6 +43,7 @@ void checkHip(hipError_t err, const char *what) {
 }
 
 thread_local const char *lastKernel = "";
+thread_local bool lastPacked = false; // operands went through gemm_pack_rows
 
 // ---------------------------------------------------------------------------
 // C[M,N] = alpha * A[M,K] * B[K,N] + beta * C with C row-major (ldc) on the
@@ -563,6 +564,32 @@ gemm_generic(const T *A, const T *B, T *C, int64_t M, int64_t N, int64_t K,
 }
 
 // ---------------------------------------------------------------------------
+// A copy of an operand that the tile kernels can read in 128-bit words: the
+// R rows of C elements at src (row stride ld, unit stride along a row) go to
+// rows of Cp = C rounded up to whole words, dense, 16-byte aligned, the tail
+// of every row filled with zeros.  For operands whose rows do not begin or
+// end on a word (an odd extent or leading dimension, a view that starts
+// inside a word).  One thread per destination word.
+template <typename T>
+__global__ __launch_bounds__(256) void
+gemm_pack_rows(const T *__restrict__ src, int64_t ld, int64_t R, int64_t C,
+               T *__restrict__ dst, int64_t Cp) {
+  typedef typename Mfma<T>::Vec Vec;
+  constexpr int VEC = Mfma<T>::VEC;
+  const int64_t wordsPerRow = Cp / VEC;
+  const int64_t word = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (word >= R * wordsPerRow)
+    return;
+  const int64_t r = word / wordsPerRow, c = (word % wordsPerRow) * VEC;
+  const T *row = src + r * ld;
+  Vec v;
+#pragma unroll
+  for (int q = 0; q < VEC; ++q)
+    v[q] = c + q < C ? row[c + q] : T(0);
+  *reinterpret_cast<Vec *>(dst + r * Cp + c) = v;
+}
+
+// ---------------------------------------------------------------------------
 // Workspace of the split-K path, per device.
 //
 // mkl_gemm_<dtype>_device keeps one hipMalloc'ed block per device, grown on
@@ -757,6 +784,9 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
   // leaves plan unsplit when the heap has no room, reports the fixed array
   // as too small through tooLarge.
   bool tooLarge = false;
+  // Bytes at the start of the heap workspace that hold repacked operands
+  // (gemm_pack_rows); the partial products come behind them.
+  size_t packBytes = 0;
   std::unique_lock<std::mutex> workspaceTurn; // (released when the call returns)
   auto takeTurn = [&]() {
     (void)workspaceOf(device); // (checks the ordinal)
@@ -783,9 +813,11 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       }
       p = fixedWorkspace(device);
     } else {
-      p = heapWorkspace(device, bytes);
+      p = heapWorkspace(device, packBytes + bytes);
       if (!p)
         plan = SplitPlan();
+      else
+        p = static_cast<unsigned char *>(p) + packBytes;
     }
     return static_cast<T *>(p);
   };
@@ -795,9 +827,12 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
     if (blocks <= 0)
       return nullptr;
     takeTurn();
-    void *p = heapWorkspace(device, size_t(blocks) * 2 * size_t(bm) * size_t(bn) * sizeof(T));
+    void *p = heapWorkspace(
+        device, packBytes + size_t(blocks) * 2 * size_t(bm) * size_t(bn) * sizeof(T));
     if (!p)
       blocks = 0;
+    else
+      p = static_cast<unsigned char *>(p) + packBytes;
     return static_cast<T *>(p);
   };
   const int64_t slots = 512; // resident blocks of the 128 x 128 tiles: two a CU
@@ -823,6 +858,7 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
                          ldz, alpha, beta);
   };
 
+  lastPacked = false;
   if (M > 0 && N > 0) {
     bool launched = false;
     {
@@ -883,10 +919,31 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       // (only K ragged: the tiles as they are plus the rest of K on the
       // strided kernel is faster, 116 against 106 TFLOP/s on 4096 x 4096 x 4100)
       const bool onlyK = Mt == Mz && Nt == Nz && mostly;
-      if (!whole && !onlyK && unitOk && wordsWhole && K > 0 && ldx % VEC == 0 && ldy % VEC == 0 &&
-          ldx > 0 && ldy > 0 && aligned16(X) && aligned16(Y) && M <= 0x7fffffff &&
+      // An operand whose rows do not begin and end on 128-bit words (an odd
+      // extent or leading dimension, a base inside a word) is copied once
+      // into word-aligned rows padded with zeros (gemm_pack_rows) and the same
+      // guarded tiles run on the copy: reading and writing each operand once
+      // more is small beside the product (4094^3 float32: 27 -> 110 TFLOP/s).
+      // Needs the heap workspace.
+      const int64_t xC = xKc ? K : Mz, xR = xKc ? Mz : K; // X: contiguous extent, rows
+      const int64_t yC = yNc ? Nz : K, yR = yNc ? K : Nz;
+      auto offWords = [&](const T *base, int64_t ld, int64_t C) {
+        return ld % VEC != 0 || !aligned16(base) || C % VEC != 0;
+      };
+      const bool canPack = workspaceKind == WORKSPACE_HEAP && unitOk && ldx > 0 && ldy > 0;
+      const bool packX = canPack && offWords(X, ldx, xC);
+      const bool packY = canPack && offWords(Y, ldy, yC);
+      const bool wordsOk = (packX || !offWords(X, ldx, xC)) && (packY || !offWords(Y, ldy, yC));
+      (void)wordsWhole;
+      if (((!whole && !onlyK) || packX || packY) && unitOk && wordsOk && K > 0 &&
+          ldx > 0 && ldy > 0 && M <= 0x7fffffff &&
           N <= 0x7fffffff && K <= 0x7fffffff - 64 && tilesM <= 65535 &&
           tilesM * tilesN >= 16) {
+        auto roundUp = [](int64_t v, int64_t to) { return (v + to - 1) / to * to; };
+        const int64_t xCp = roundUp(xC, VEC), yCp = roundUp(yC, VEC);
+        const size_t xBytes = packX ? size_t(roundUp(xR * xCp * int64_t(sizeof(T)), 256)) : 0;
+        const size_t yBytes = packY ? size_t(roundUp(yR * yCp * int64_t(sizeof(T)), 256)) : 0;
+        packBytes = xBytes + yBytes;
         const int slabs = int((K + BK - 1) / BK);
         int evenBlocks = workspaceKind == WORKSPACE_HEAP
                              ? planEvenShares(tilesM * tilesN, slabs, slots)
@@ -900,6 +957,34 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           W = workspaceFor(plan, Mz, ldw);
         if (tooLarge)
           return 1;
+        if (packBytes) {
+          // (one block for the copies and the partial products: asked for
+          // once, before anything is launched into it)
+          unsigned char *base = W ? reinterpret_cast<unsigned char *>(W) - packBytes : nullptr;
+          if (!base) {
+            takeTurn();
+            base = static_cast<unsigned char *>(heapWorkspace(device, packBytes));
+            if (!base)
+              fatal("mkl_gemm_device: no device memory for %zu bytes of repacked operands\n",
+                    packBytes);
+          }
+          auto pack = [&](const T *src, int64_t ld, int64_t R, int64_t C, int64_t Cp, T *dst) {
+            const int64_t words = R * (Cp / VEC);
+            hipLaunchKernelGGL(gemm_pack_rows<T>, dim3(unsigned((words + 255) / 256)),
+                               dim3(256), 0, stream, src, ld, R, C, dst, Cp);
+          };
+          if (packX) {
+            T *dst = reinterpret_cast<T *>(base);
+            pack(X, ldx, xR, xC, xCp, dst);
+            X = dst;
+          }
+          if (packY) {
+            T *dst = reinterpret_cast<T *>(base + xBytes);
+            pack(Y, ldy, yR, yC, yCp, dst);
+            Y = dst;
+          }
+        }
+        const int64_t ldxk = packX ? xCp : ldx, ldyk = packY ? yCp : ldy;
         const EvenShares even{evenBlocks ? slabs : 0, int(tilesN)};
         dim3 grid(unsigned(tilesN), unsigned(tilesM), unsigned(plan.slices));
         if (evenBlocks)
@@ -907,7 +992,7 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
 #define NMHIP_GEMM_RAGGED(TM, TN, XKC, YNC)                                    \
   hipLaunchKernelGGL((gemm_mfma<T, BK, TM, TN, XKC, YNC, true>), grid,         \
                      dim3(256), 0, stream, X, Y, cData, int(Mz), int(Nz),      \
-                     int(K), ldx, ldy, ldz, alpha, beta, plan.sliceK, W, ldw,  \
+                     int(K), ldxk, ldyk, ldz, alpha, beta, plan.sliceK, W, ldw,\
                      even)
 #define NMHIP_GEMM_RAGGED_LAYOUTS(TM, TN)                                      \
   do {                                                                         \
@@ -931,6 +1016,7 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
                        : plan.slices > 1 ? "dgemm_mfma_128x128_ragged_splitk"
                                          : "dgemm_mfma_128x128_ragged";
         }
+        lastPacked = packBytes != 0;
         if (evenBlocks)
           evenFold(W, evenBlocks, slabs, tilesM, tilesN, 128, Mz, Nz, ldz, cData);
         else if (plan.slices > 1)
@@ -1081,4 +1167,10 @@ NMHIP_MATH_EXPORT void nmrtMathRuntimeFinalize(void) {
   releaseHeapWorkspaces();
 }
 
-NMHIP_MATH_EXPORT const char *nmhipMathLastKernel(void) { return lastKernel; }
+NMHIP_MATH_EXPORT const char *nmhipMathLastKernel(void) {
+  if (!lastPacked)
+    return lastKernel;
+  thread_local char name[96];
+  std::snprintf(name, sizeof(name), "%s+packed", lastKernel);
+  return name;
+}

@@ -25,7 +25,7 @@ def _kernel(mrt):
     """Name of the last gemm kernel without the marker of how K was shared
     out (split into slices, or even shares of the slabs of all tiles: that
     depends only on how many tiles the shape has)."""
-    return mrt.last_kernel().replace("_splitk", "").replace("_even", "")
+    return mrt.last_kernel().replace("_splitk", "").replace("_even", "").replace("+packed", "")
 
 
 def _printed(x):
@@ -160,10 +160,10 @@ def test_ragged_k_alone_keeps_the_tiles(env, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-def test_ragged_shapes_split_into_tiles_and_edges(env, dtype):
-    """Operands whose rows do not end on a 128-bit word (views of wider
-    arrays): the tiled part runs on the matrix cores, the rest of K, the last
-    rows and the last columns on the strided kernel."""
+def test_operands_off_the_word_grid_are_repacked(env, dtype):
+    """Operands whose rows do not begin or end on a 128-bit word (views of
+    wider arrays, odd extents, a base inside a word) are copied once into
+    word-aligned rows padded with zeros and run on the guarded tiles."""
     hip, ops, orc, mrt = env
     m, n, k = 1540, 2052, 1001
     rng = np.random.default_rng(5)
@@ -173,9 +173,34 @@ def test_ragged_shapes_split_into_tiles_and_edges(env, dtype):
     d_a = hip.asarray(a_wide)[:, :k]
     d_c = hip.asarray(c0)
     ops.gemm(d_a, hip.asarray(b), d_c, 1.5, -0.5)
-    assert _kernel(mrt).endswith("_mfma_128x128+edges")
+    assert mrt.last_kernel().endswith("+packed") and "_mfma_128x128_ragged" in mrt.last_kernel()
     _check_scaled(d_c.asnumpy(), a_wide[:, :k], b, c0, 1.5, -0.5,
                   1e-5 if dtype == np.float32 else 1e-13)
+    tol = 1e-5 if dtype == np.float32 else 1e-13
+    lay = lambda x, t: np.asfortranarray(x) if t else x
+    for (m, n, k), ta, tb, tc in (((1001, 1003, 1005), False, False, False),
+                                  ((1001, 1003, 1005), True, False, True),
+                                  ((777, 1025, 2049), True, True, False),
+                                  ((513, 2047, 300), False, False, False),
+                                  ((2047, 2049, 2051), False, False, False)):
+        a = rng.standard_normal((m, k)).astype(dtype)
+        b = rng.standard_normal((k, n)).astype(dtype)
+        c0 = rng.standard_normal((m, n)).astype(dtype)
+        d_c = _to_dev(hip, lay(c0, tc))
+        ops.gemm(_to_dev(hip, lay(a, ta)), _to_dev(hip, lay(b, tb)), d_c, 1.5, -0.5)
+        assert mrt.last_kernel().endswith("+packed"), mrt.last_kernel()
+        _check_scaled(d_c.asnumpy(), a, b, c0, 1.5, -0.5, tol)
+    # whole tiles, but the first operand starts one element into a word
+    m = n = k = 1024
+    a = rng.standard_normal((m, k)).astype(dtype)
+    b = rng.standard_normal((k, n)).astype(dtype)
+    flat = np.zeros(m * k + 1, dtype)
+    flat[1:] = a.ravel()
+    d_a = hip.asarray(flat)[1:].reshape(m, k)
+    d_c = hip.asarray(np.full((m, n), np.nan, dtype))
+    ops.gemm(d_a, hip.asarray(b), d_c, 1.0, 0.0)
+    assert mrt.last_kernel().endswith("+packed")
+    _check_scaled(d_c.asnumpy(), a, b, np.zeros((m, n), dtype), 1.0, 0.0, tol)
 
 
 # Tolerance for float32 matmul: |gpu - truth| <= 1e-4 * (|a| @ |b|) elementwise

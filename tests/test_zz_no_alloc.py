@@ -87,3 +87,27 @@ def test_two_calls_in_a_row_match_the_allocating_entry_point(gemm_entry_points):
             np.abs(a).astype(np.float64) @ np.abs(b))
         assert (np.abs(got - truth) <= 1e-4 * scale + 1e-30).all()
         assert (np.abs(got - ref) <= 1e-4 * scale + 1e-30).all()
+
+
+def test_operands_off_the_word_grid_stay_on_tiles_and_edges(gemm_entry_points):
+    """The allocating entry point repacks an operand whose rows do not end on
+    a 128-bit word into its workspace; this one cannot, and runs the whole
+    tiles on the matrix cores and the rest on the strided kernel."""
+    hip, lib, mrt = gemm_entry_points
+    m, n, k = 1540, 2052, 1001
+    rng = np.random.default_rng(5)
+    a_wide = rng.standard_normal((m, k + 3), dtype=np.float32)
+    b = rng.standard_normal((k, n), dtype=np.float32)
+    d_a, d_b = hip.asarray(a_wide)[:, :k], hip.asarray(b)
+    outs = []
+    for entry in (lib.mkl_gemm_float32_device, lib.mkl_gemm_float32_device_noalloc):
+        d_c = hip.asarray(np.zeros((m, n), np.float32))
+        status = entry(d_a.ctx.queue, _memref(d_a), _memref(d_b), 1.0, 0.0, _memref(d_c))
+        assert not status
+        outs.append((mrt.last_kernel(), d_c.asnumpy()))
+    assert outs[0][0].endswith("+packed") and outs[1][0] == "sgemm_mfma_128x128+edges"
+    a = a_wide[:, :k]
+    truth = a.astype(np.float64) @ b.astype(np.float64)
+    scale = np.abs(a).astype(np.float64) @ np.abs(b)
+    for _, got in outs:
+        assert (np.abs(got - truth) <= 1e-4 * scale + 1e-30).all()
