@@ -355,6 +355,10 @@ def test_split_k_beta_zero_ignores_c(env):
     (np.float32, 1536, 1408, 2056, "sgemm_mfma_128x128_even+edges"),  # the rest of K beside
     (np.float32, 1000, 1100, 1200, "sgemm_mfma_128x128_ragged_even"),
     (np.float32, 2000, 2300, 2600, "sgemm_mfma_128x128_ragged_even"),
+    # from 192 padded tiles on, ragged float32 shapes run on the large tile over
+    # zero-padded copies of both operands: 210 tiles in even shares, 256 as they are
+    (np.float32, 3560, 3800, 1020, "sgemm_mfma_256x256_even+packed"),
+    (np.float32, 4000, 4000, 530, "sgemm_mfma_256x256+packed"),
     (np.float64, 3072, 3072, 512, "dgemm_mfma_128x128_even"),         # 1.125 rounds
     (np.float64, 1024, 1024, 4096, "dgemm_mfma_128x128_even"),
     (np.float64, 1000, 1100, 1200, "dgemm_mfma_128x128_ragged_even"),  # the reference's preset
