@@ -626,28 +626,42 @@ DeviceWorkspace &workspaceOf(int device) {
   return workspaces[device];
 }
 
-// Grown on demand; nullptr when the device has no memory left (the caller
-// then runs without splitting K).  The device must be current.
+// Grown on demand; nullptr when the device has no room for the larger block
+// (the block it has stays as it is: the caller then runs without what it
+// asked for).  The device must be current, and the caller holds the
+// device's turn, so no kernel of another call reads the block that is freed.
 void *heapWorkspace(int device, size_t bytes) {
   std::lock_guard<std::mutex> lock(workspaceMutex);
   DeviceWorkspace &w = workspaceOf(device);
   if (bytes <= w.heapBytes)
     return w.heap;
-  if (w.heap) {
-    checkHip(hipDeviceSynchronize(), "hipDeviceSynchronize");
-    checkHip(hipFree(w.heap), "hipFree");
-    w.heap = nullptr;
-    w.heapBytes = 0;
-  }
   const size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : bytes;
   void *p = nullptr;
   if (hipMalloc(&p, want) != hipSuccess) {
     (void)hipGetLastError();
     return nullptr;
   }
+  if (w.heap) {
+    checkHip(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    checkHip(hipFree(w.heap), "hipFree");
+  }
   w.heap = p;
   w.heapBytes = want;
   return p;
+}
+
+// A call whose repacked operands made the block larger than this gives it
+// back when it returns (its stream is idle by then): a device keeps at most
+// 1 GiB between calls.
+constexpr size_t kHeapKeptBytes = size_t(1) << 30;
+void trimHeapWorkspace(int device) {
+  std::lock_guard<std::mutex> lock(workspaceMutex);
+  DeviceWorkspace &w = workspaceOf(device);
+  if (w.heapBytes <= kHeapKeptBytes)
+    return;
+  checkHip(hipFree(w.heap), "hipFree");
+  w.heap = nullptr;
+  w.heapBytes = 0;
 }
 
 // Device address of the fixed array on the current device (set up on the
@@ -903,7 +917,14 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       const int bigEven = bigFits && workspaceKind == WORKSPACE_HEAP
                               ? planEvenShares(bigTiles, Kt / bigSlab, 256)
                               : 0;
-      const bool big = bigFits && (bigEven > 0 || bigTiles >= 192);
+      bool big = bigFits && (bigEven > 0 || bigTiles >= 192);
+      if (big && bigTiles < 192) {
+        // (fewer large tiles than CUs only pay in even shares: without room
+        // for those, the 128 x 128 tiles take the shape)
+        int blocks = bigEven;
+        (void)evenWorkspace(blocks, 256, 256);
+        big = blocks > 0;
+      }
       const int BM = big ? 256 : 128, BN = BM;
       const bool unitOk = (xk == 1 || xm == 1) && (yk == 1 || yn == 1);
       // worth it when the tiled part is most of the work and fills at least
@@ -1010,17 +1031,27 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           }
         }
       }
+      // (the guarded tiles below need every operand on the word grid: copies
+      // of those that are not, or none of this when there is no room for them)
+      size_t packXBytes = 0, packYBytes = 0;
+      bool copiesFit = true;
+      if (!paddedBig && (packX || packY)) {
+        auto roundUp = [](int64_t v, int64_t to) { return (v + to - 1) / to * to; };
+        packXBytes = packX ? size_t(roundUp(xR * roundUp(xC, VEC) * int64_t(sizeof(T)), 256)) : 0;
+        packYBytes = packY ? size_t(roundUp(yR * roundUp(yC, VEC) * int64_t(sizeof(T)), 256)) : 0;
+        takeTurn();
+        copiesFit = heapWorkspace(device, packXBytes + packYBytes) != nullptr;
+      }
       if (paddedBig) {
         // (done)
-      } else if (((!whole && !onlyK) || packX || packY) && unitOk && wordsOk && K > 0 &&
+      } else if (((!whole && !onlyK) || packX || packY) && copiesFit && unitOk && wordsOk && K > 0 &&
           ldx > 0 && ldy > 0 && M <= 0x7fffffff &&
           N <= 0x7fffffff && K <= 0x7fffffff - 64 && tilesM <= 65535 &&
           tilesM * tilesN >= 16) {
         auto roundUp = [](int64_t v, int64_t to) { return (v + to - 1) / to * to; };
         const int64_t xCp = roundUp(xC, VEC), yCp = roundUp(yC, VEC);
-        const size_t xBytes = packX ? size_t(roundUp(xR * xCp * int64_t(sizeof(T)), 256)) : 0;
-        const size_t yBytes = packY ? size_t(roundUp(yR * yCp * int64_t(sizeof(T)), 256)) : 0;
-        packBytes = xBytes + yBytes;
+        const size_t xBytes = packXBytes;
+        packBytes = packXBytes + packYBytes;
         const int slabs = int((K + BK - 1) / BK);
         int evenBlocks = workspaceKind == WORKSPACE_HEAP
                              ? planEvenShares(tilesM * tilesN, slabs, slots)
@@ -1037,14 +1068,10 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
         if (packBytes) {
           // (one block for the copies and the partial products: asked for
           // once, before anything is launched into it)
-          unsigned char *base = W ? reinterpret_cast<unsigned char *>(W) - packBytes : nullptr;
-          if (!base) {
-            takeTurn();
-            base = static_cast<unsigned char *>(heapWorkspace(device, packBytes));
-            if (!base)
-              fatal("mkl_gemm_device: no device memory for %zu bytes of repacked operands\n",
-                    packBytes);
-          }
+          // (a workspace request that found no room left the block as it
+          // was: the copies still fit, as checked above)
+          unsigned char *base = W ? reinterpret_cast<unsigned char *>(W) - packBytes
+                                  : static_cast<unsigned char *>(heapWorkspace(device, packBytes));
           auto pack = [&](const T *src, int64_t ld, int64_t R, int64_t C, int64_t Cp, T *dst) {
             const int64_t words = R * (Cp / VEC);
             hipLaunchKernelGGL(gemm_pack_rows<T>, dim3(unsigned((words + 255) / 256)),
@@ -1112,9 +1139,6 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
                              ? planEvenShares((Mt / BM) * (Nt / BN), slabs, slots)
                              : 0;
         T *W = evenWorkspace(evenBlocks, BM, BN);
-        if (big && !evenBlocks && bigTiles < 192)
-          fatal("mkl_gemm_device: no workspace for %lld tiles of 256 x 256\n",
-                (long long)bigTiles);
         SplitPlan plan;
         if (!big && !evenBlocks) {
           plan = planSplit((Mt / BM) * (Nt / BN), Kt, BK, sizeof(T) == 8 ? 2 : 1);
@@ -1210,6 +1234,8 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
   }
   // The reference call returns only when C is complete (.wait(), 127/145).
   checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
+  if (workspaceTurn.owns_lock() && workspaceKind == WORKSPACE_HEAP)
+    trimHeapWorkspace(device);
   return 0;
 }
 

@@ -203,6 +203,42 @@ def test_operands_off_the_word_grid_are_repacked(env, dtype):
     _check_scaled(d_c.asnumpy(), a, b, np.zeros((m, n), dtype), 1.0, 0.0, tol)
 
 
+def test_copies_above_a_gigabyte_are_given_back(env):
+    """The device keeps its gemm workspace between calls, but not more than
+    1 GiB of it: a product whose padded copies need more (1.2 GB here) frees
+    the block when it returns.  Rows of the result against float64."""
+    import ctypes
+    hip, ops, _, mrt = env
+    hiprt = ctypes.CDLL("libamdhip64.so")
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert hiprt.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    m, n, k = 12290, 12294, 12289
+    rng = np.random.default_rng(11)
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    b = rng.standard_normal((k, n), dtype=np.float32)
+    d_a, d_b = hip.asarray(a), hip.asarray(b)
+    d_c = hip.asarray(np.zeros((m, n), np.float32))
+    ops.gemm(d_a, d_b, d_c, 1.0, 0.0)        # (whatever an earlier test left is freed too)
+    before = free_bytes()
+    for _ in range(2):
+        ops.gemm(d_a, d_b, d_c, 1.0, 0.0)
+        assert mrt.last_kernel() == "sgemm_mfma_256x256+packed"
+        assert free_bytes() >= before - (64 << 20)
+    got = d_c.asnumpy()
+    rows = np.array([0, 1, 255, 256, 6000, m - 2, m - 1])
+    truth = a[rows].astype(np.float64) @ b.astype(np.float64)
+    scale = np.abs(a[rows]).astype(np.float64) @ np.abs(b).astype(np.float64)
+    assert (np.abs(got[rows] - truth) <= 1e-5 * scale).all()
+    cols = np.array([0, 255, 256, n - 1])
+    truth = a.astype(np.float64) @ b[:, cols].astype(np.float64)
+    scale = np.abs(a).astype(np.float64) @ np.abs(b[:, cols]).astype(np.float64)
+    assert (np.abs(got[:, cols] - truth) <= 1e-5 * scale).all()
+
+
 # Tolerance for float32 matmul: |gpu - truth| <= 1e-4 * (|a| @ |b|) elementwise
 # against a float64 ground truth, and relative 1e-4 in the Frobenius norm.
 def _check(got, a, b):
