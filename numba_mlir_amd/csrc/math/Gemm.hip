@@ -960,33 +960,41 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       const bool packY = canPack && offWords(Y, ldy, yC);
       const bool wordsOk = (packX || !offWords(X, ldx, xC)) && (packY || !offWords(Y, ldy, yC));
       (void)wordsWhole;
-      // float32 shapes that are not whole 256 x 256 tiles of whole words, but
-      // large enough that padding them to such tiles costs under a tenth more
-      // arithmetic: both operands are copied into zero-padded rows (whole
-      // tiles, whole K slabs) and the large tile runs on the copies with only
-      // its stores guarded (4000^3: 117 -> 126 TFLOP/s, 4094^3: 117 -> 131).
-      // From 192 padded tiles on: below that the guarded 128 x 128 tiles in
-      // even shares are as fast or faster (3000^3: 107 against 104).
+      // Large shapes that are not whole tiles of whole words (256 x 256 for
+      // float32, 128 x 128 for float64), where padding them to such tiles
+      // costs under a tenth more arithmetic: both operands are copied into
+      // zero-padded rows (whole tiles, whole K slabs) and the tiles run on the
+      // copies with only their stores guarded.  float32 4000^3: 117 -> 126
+      // TFLOP/s, 4094^3: 117 -> 131; float64 4000^3: 56 -> 62, 7000 x 7500 x
+      // 8000: 61 -> 65.  From 192 padded tiles on in float32 (below that the
+      // guarded 128 x 128 tiles in even shares are as fast or faster, 3000^3:
+      // 107 against 104), from 256 in float64 (the same tile either way: the
+      // copies have to be won back from the guards on the loads alone).
       bool paddedBig = false;
-      if constexpr (sizeof(T) == 4) {
+      {
+        // float32: 256 x 256 tiles, K slabs of 32; float64: 128 x 128, slabs of 16
+        constexpr int PT = sizeof(T) == 4 ? 256 : 128;
+        constexpr int PSLAB = sizeof(T) == 4 ? 2 * BK : BK;
+        const int64_t padSlots = sizeof(T) == 4 ? 256 : slots;
+        const int64_t minTiles = sizeof(T) == 4 ? 192 : 256;
         auto roundUp = [](int64_t v, int64_t to) { return (v + to - 1) / to * to; };
-        const int64_t Mp = roundUp(Mz, 256), Np = roundUp(Nz, 256), Kp = roundUp(K, 2 * BK);
+        const int64_t Mp = roundUp(Mz, PT), Np = roundUp(Nz, PT), Kp = roundUp(K, PSLAB);
         const bool fitsAsIs = Mz == Mp && Nz == Np && K % BK == 0 && !offWords(X, ldx, xC) &&
                               !offWords(Y, ldy, yC);
-        const int64_t padTiles = (Mp / 256) * (Np / 256);
-        const int slabs = int(Kp / (2 * BK));
-        int evenBlocks = planEvenShares(padTiles, slabs, 256);
-        if (canPack && !fitsAsIs && (!whole || packX || packY) && K >= 256 && padTiles >= 192 &&
-            Mp / 256 <= 65535 && Mz <= 0x7fffffff - 256 &&
+        const int64_t padTiles = (Mp / PT) * (Np / PT);
+        const int slabs = int(Kp / PSLAB);
+        int evenBlocks = planEvenShares(padTiles, slabs, padSlots);
+        if (canPack && !fitsAsIs && (!whole || packX || packY) && K >= 256 && padTiles >= minTiles &&
+            Mp / PT <= 65535 && Mz <= 0x7fffffff - 256 &&
             Nz <= 0x7fffffff - 256 && K <= 0x7fffffff - 64 &&
             double(Mp) * double(Np) * double(Kp) <= 1.10 * double(Mz) * double(Nz) * double(K)) {
           // X as [rows x contiguous extent], padded; the same for Y
           const int64_t xRp = xKc ? Mp : Kp, xCp = xKc ? Kp : Mp;
           const int64_t yRp = yNc ? Kp : Np, yCp = yNc ? Np : Kp;
-          const size_t xBytes = size_t(roundUp(xRp * xCp * 4, 256));
-          const size_t yBytes = size_t(roundUp(yRp * yCp * 4, 256));
+          const size_t xBytes = size_t(roundUp(xRp * xCp * int64_t(sizeof(T)), 256));
+          const size_t yBytes = size_t(roundUp(yRp * yCp * int64_t(sizeof(T)), 256));
           packBytes = xBytes + yBytes;
-          T *W = evenWorkspace(evenBlocks, 256, 256);
+          T *W = evenWorkspace(evenBlocks, PT, PT);
           unsigned char *base = W ? reinterpret_cast<unsigned char *>(W) - packBytes : nullptr;
           if (!base) {
             evenBlocks = 0;
@@ -1003,12 +1011,12 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
             T *Xp = reinterpret_cast<T *>(base), *Yp = reinterpret_cast<T *>(base + xBytes);
             pack(X, ldx, xR, xC, xRp, xCp, Xp);
             pack(Y, ldy, yR, yC, yRp, yCp, Yp);
-            const EvenShares even{evenBlocks ? slabs : 0, int(Np / 256)};
-            dim3 grid(unsigned(Np / 256), unsigned(Mp / 256), 1);
+            const EvenShares even{evenBlocks ? slabs : 0, int(Np / PT)};
+            dim3 grid(unsigned(Np / PT), unsigned(Mp / PT), 1);
             if (evenBlocks)
               grid = dim3(unsigned(evenBlocks), 1, 1);
 #define NMHIP_GEMM_PADDED(XKC, YNC)                                            \
-  hipLaunchKernelGGL((gemm_mfma<T, 2 * BK, 4, 4, XKC, YNC, 2>), grid,          \
+  hipLaunchKernelGGL((gemm_mfma<T, PSLAB, 4, 4, XKC, YNC, 2>), grid,          \
                      dim3(256), 0, stream, Xp, Yp, cData, int(Mz), int(Nz),    \
                      int(Kp), xCp, yCp, ldz, alpha, beta, 0, W, int64_t(0),    \
                      even)
@@ -1022,8 +1030,10 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
               NMHIP_GEMM_PADDED(false, false);
 #undef NMHIP_GEMM_PADDED
             if (evenBlocks)
-              evenFold(W, evenBlocks, slabs, Mp / 256, Np / 256, 256, Mz, Nz, ldz, cData);
-            lastKernel = evenBlocks ? "sgemm_mfma_256x256_even" : "sgemm_mfma_256x256";
+              evenFold(W, evenBlocks, slabs, Mp / PT, Np / PT, PT, Mz, Nz, ldz, cData);
+            lastKernel = sizeof(T) == 4
+                             ? (evenBlocks ? "sgemm_mfma_256x256_even" : "sgemm_mfma_256x256")
+                             : (evenBlocks ? "dgemm_mfma_128x128_even" : "dgemm_mfma_128x128");
             lastPacked = true;
             launched = paddedBig = true;
           } else {

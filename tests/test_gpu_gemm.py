@@ -398,7 +398,10 @@ def test_split_k_beta_zero_ignores_c(env):
     (np.float64, 3072, 3072, 512, "dgemm_mfma_128x128_even"),         # 1.125 rounds
     (np.float64, 1024, 1024, 4096, "dgemm_mfma_128x128_even"),
     (np.float64, 1000, 1100, 1200, "dgemm_mfma_128x128_ragged_even"),  # the reference's preset
-    (np.float64, 2500, 2750, 3000, "dgemm_mfma_128x128_ragged_even"),
+    (np.float64, 1500, 1700, 1200, "dgemm_mfma_128x128_ragged_even"),
+    # float64 from 256 padded tiles on: the same tile over zero-padded copies
+    (np.float64, 2500, 2750, 3000, "dgemm_mfma_128x128_even+packed"),
+    (np.float64, 2040, 4090, 600, "dgemm_mfma_128x128+packed"),
 ])
 @pytest.mark.parametrize("ta,tb,tc", [(False, False, False), (True, False, True),
                                       (False, True, False)])
