@@ -393,6 +393,26 @@ template <bool CAREFUL> __device__ __forceinline__ double rsqrtF64m(double z, bo
   const double e = __builtin_fma(-z, y * y, 1.0); // 1 - z y^2
   return __builtin_fma(y * e, __builtin_fma(0.375, e, 0.5), y);
 }
+// (plain form: the polynomial of a NaN is some number, so a NaN sends the
+// wave to the careful form instead of being put back by a select)
+template <bool CAREFUL> __device__ __forceinline__ double cdfTermF64m(double x, bool &ok) {
+  if (CAREFUL)
+    return cdfTermF64(x);
+  ok = ok & (x == x);
+  const double ax = __builtin_fmin(__builtin_fabs(x), 6.0);
+  const double t = ax + 0x1.8p48;
+  const int node = __double2loint(t);
+  const double u = ax - (t - 0x1.8p48);
+  const cdf_word *row = cdfLds + __mul24(node, 3);
+  const cdf_word c01 = row[0], c23 = row[1], c45 = row[2];
+  double p = c45[1];
+  p = __builtin_fma(p, u, c45[0]);
+  p = __builtin_fma(p, u, c23[1]);
+  p = __builtin_fma(p, u, c23[0]);
+  p = __builtin_fma(p, u, c01[1]);
+  p = __builtin_fma(p, u, c01[0]);
+  return 0.5 + __builtin_copysign(p, x);
+}
 template <bool CAREFUL> __device__ __forceinline__ double sqrtF64m(double d, bool &ok) {
   if (CAREFUL)
     return sqrt(d);

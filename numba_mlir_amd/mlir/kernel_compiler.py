@@ -1023,7 +1023,9 @@ class FunctionTranslator:
                             return v
                         if sym == "+" and other.tag[0] == "halferf" and \
                                 self.emitting and self.outputs_are_float32():
-                            return Val(f"nmkjit::cdfTermF64({other.tag[1]})", t, nonneg=True)
+                            spec = self.speculation()
+                            return Val(f"nmkjit::cdfTermF64m{spec}({other.tag[1]}, nmk_ok)" if spec
+                                       else f"nmkjit::cdfTermF64({other.tag[1]})", t, nonneg=True)
             gid = None
             if t is INT64:                # id + constant still runs along the id
                 if sym in "+-" and a.gid is not None and y.const is not None:
@@ -2109,7 +2111,7 @@ class FunctionTranslator:
         text = "\n".join(self.m.device_code + lines)
         if "nmkjit::erfF64(" in text:
             out.append("  nmkjit::erfTableLoad();")
-        if "nmkjit::cdfTermF64(" in text:
+        if "nmkjit::cdfTermF64(" in text or "nmkjit::cdfTermF64m<" in text:
             out.append("  nmkjit::cdfTableLoad();")
         body = ["    " + v for v in views]
         body += ["    " + d for d in self.declarations() + self.private_decls]

@@ -329,7 +329,8 @@ def test_fused_maps_take_several_elements_per_lane(K, tmp_path, monkeypatch):
     assert "if (__builtin_amdgcn_ballot_w64(!nmk_ok) != 0) {" in ck.source
     assert "__attribute__((noinline)) -> nmk_results {" in ck.source
     # 0.5 + 0.5 * erf(w) with float32 results only: one table term, its own table
-    assert "v_d1 = nmkjit::cdfTermF64(v_w1);" in ck.source
+    assert ("v_d1 = nmkjit::cdfTermF64m<decltype(nmk_careful)::value>(v_w1, nmk_ok);"
+            in ck.source)
     assert "nmkjit::cdfTableLoad();" in ck.source and "erfTableLoad" not in ck.source
     assert kc.build_code_object(ck)[:4] == b"\x7fELF"
     small = kc.translate(njit_cases.black_scholes_arrays, types, ndim, K, mode=mode,
@@ -359,7 +360,8 @@ def test_fused_maps_take_several_elements_per_lane(K, tmp_path, monkeypatch):
     assert "nmk_out.v_call = (float)" in ck.source and "nmk_words" in ck.source
     assert ("v_a = nmkjit::logQuotientF32m<decltype(nmk_careful)::value>(v_P, v_S, nmk_ok);"
             in ck.source)
-    assert "v_d2 = nmkjit::cdfTermF64(v_w2);" in ck.source
+    assert ("v_d2 = nmkjit::cdfTermF64m<decltype(nmk_careful)::value>(v_w2, nmk_ok);"
+            in ck.source)
     assert ("__builtin_nontemporal_store(nmk_vec_v_put, "
             "reinterpret_cast<nmk_out_t_v_put *>(v_put_p) + nmk_i);") in ck.source
     assert kc.build_code_object(ck)[:4] == b"\x7fELF"
