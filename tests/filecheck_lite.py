@@ -51,3 +51,20 @@ def check(output, directives):
         else:
             raise ValueError(f"unsupported directive {kind}")
         matched = True
+
+
+LLVM_FILECHECK = "/opt/rocm/llvm/bin/FileCheck"
+
+
+def llvm_filecheck(output, directives, workdir):
+    """The same question put to LLVM's own FileCheck, where the ROCm image has
+    one: (accepted, its message)."""
+    import os
+    import subprocess
+    checks = os.path.join(str(workdir), "checks.txt")
+    with open(checks, "w") as f:
+        for kind, text in directives:
+            f.write(f"// {kind}: {text}\n")
+    r = subprocess.run([LLVM_FILECHECK, checks], input=output, capture_output=True, text=True,
+                       timeout=60)
+    return r.returncode == 0, r.stderr

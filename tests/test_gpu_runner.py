@@ -18,7 +18,7 @@ with open(os.path.join(ROOT, "tests", "golden", "l0_runner_checks.json")) as f:
 
 
 @pytest.mark.parametrize("case", sorted(CHECKS))
-def test_runner_case_matches_the_reference_checks(hip, case):
+def test_runner_case_matches_the_reference_checks(hip, case, tmp_path):
     from numba_mlir_amd import build
     runner = os.path.join(build.HERE, build.RUNNER)
     assert os.path.exists(runner), "hip-runner is not built"
@@ -27,7 +27,11 @@ def test_runner_case_matches_the_reference_checks(hip, case):
          "-shared-libs=" + os.path.join(build.HERE, build.RUNTIME_LIB)],
         capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stdout + r.stderr
-    filecheck_lite.check(r.stdout, [tuple(c) for c in CHECKS[case]["checks"]])
+    directives = [tuple(c) for c in CHECKS[case]["checks"]]
+    filecheck_lite.check(r.stdout, directives)
+    if os.path.exists(filecheck_lite.LLVM_FILECHECK):     # LLVM's own, as the reference runs it
+        accepted, message = filecheck_lite.llvm_filecheck(r.stdout, directives, tmp_path)
+        assert accepted, message
 
 
 # -- the same programs through the decorators ---------------------------------

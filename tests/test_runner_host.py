@@ -100,3 +100,54 @@ def test_filecheck_subset():
         filecheck_lite.check(out, [("CHECK", "[1, 2"), ("CHECK-SAME", "[5")])
     with pytest.raises(AssertionError, match="not found"):
         filecheck_lite.check(out, [("CHECK", "rank = 2")])
+
+
+def _conforming_output(directives):
+    """Printed output that satisfies the directives: each CHECK or CHECK-NEXT
+    pattern on a line of its own, CHECK-SAME continuing the line, a regex
+    block replaced by text it matches (an address, one digit)."""
+    import re
+    lines = []
+    for kind, text in directives:
+        text = re.sub(r"\{\{(.*?)\}\}",
+                      lambda m: "2" if m.group(1) == "." else "0xdeadbeef", text)
+        if kind == "CHECK-SAME":
+            lines[-1] += " " + text
+        else:
+            lines.append(text)
+    return "\n".join(lines) + "\n"
+
+
+@pytest.mark.skipif(not os.path.exists(filecheck_lite.LLVM_FILECHECK),
+                    reason="no LLVM FileCheck in this image")
+def test_filecheck_subset_agrees_with_llvm_filecheck(tmp_path):
+    """The directives of every runner test of the reference, against output
+    that conforms and against the same output with one printed digit changed,
+    one line dropped, one line inserted ahead of a CHECK-NEXT: the Python
+    subset and LLVM's FileCheck give the same verdict each time."""
+    with open(os.path.join(ROOT, "tests", "golden", "l0_runner_checks.json")) as f:
+        cases = {k: v for k, v in json.load(f).items() if not k.startswith("_")}
+    compared = 0
+    for name, case in sorted(cases.items()):
+        directives = [tuple(c) for c in case["checks"]]
+        good = _conforming_output(directives)
+        lines = good.splitlines()
+        variants = [good]
+        last = lines[-1]
+        digit = next((k for k in range(len(last) - 1, -1, -1) if last[k].isdigit()), None)
+        if digit is not None:
+            changed = last[:digit] + str((int(last[digit]) + 1) % 10) + last[digit + 1:]
+            variants.append("\n".join(lines[:-1] + [changed]) + "\n")
+        variants.append("\n".join(lines[:-1]) + "\n")
+        variants.append("\n".join(lines[:1] + ["something else"] + lines[1:]) + "\n")
+        for out in variants:
+            try:
+                filecheck_lite.check(out, directives)
+                mine = True
+            except AssertionError:
+                mine = False
+            theirs, message = filecheck_lite.llvm_filecheck(out, directives, tmp_path)
+            assert mine == theirs, (name, out, message)
+            compared += 1
+        assert filecheck_lite.llvm_filecheck(good, directives, tmp_path)[0], name
+    assert compared >= 3 * len(cases)
