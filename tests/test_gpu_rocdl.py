@@ -56,15 +56,21 @@ class _Session:
         view[:] = values
         return res.ptr, view
 
-    def launch(self, name, blocks, pointers):
+    def launch(self, name, blocks, pointers, block=1, local_bytes=None):
+        """``pointers`` as ptr params; ``local_bytes``: one more ptr param with
+        no data, the reference's form of a workgroup-memory argument."""
         kern = self.lib.gpuxKernelGet(self.mod, name.encode())
-        descs = (self.g.GPUParamDesc * (len(pointers) + 1))()
+        count = len(pointers) + (local_bytes is not None)
+        descs = (self.g.GPUParamDesc * (count + 1))()
         keep = [ctypes.c_void_p(p) for p in pointers]
         for i, val in enumerate(keep):
             descs[i].data = ctypes.cast(ctypes.pointer(val), ctypes.c_void_p)
             descs[i].size = ctypes.sizeof(val)
             descs[i].type = 8
-        ev = self.lib.gpuxLaunchKernel(self.q, kern, blocks, 1, 1, 1, 1, 1, NO_DEPS, descs)
+        if local_bytes is not None:
+            descs[len(keep)].data, descs[len(keep)].size = None, local_bytes
+            descs[len(keep)].type = 8
+        ev = self.lib.gpuxLaunchKernel(self.q, kern, blocks, 1, 1, block, 1, 1, NO_DEPS, descs)
         self.lib.gpuxWait(self.q, ev)
         self.lib.gpuxDestroyEvent(self.q, ev)
         self.lib.gpuxKernelDestroy(kern)
@@ -104,4 +110,20 @@ def test_fused_map_module_with_a_device_library_call(rt, dtype, kernel):
     s.launch(kernel, gold["n"], [a, coeff, o])
     assert np.array_equal(_printed(out), np.full(gold["n"], gold["printed"]))
     assert np.abs(out - (1 + 4 / (np.exp(12.0) + 1))).max() < (2e-6 if dtype is np.float32 else 1e-14)
+    s.close()
+
+
+def test_workgroup_memory_argument_and_barrier_from_llvm_ir(rt):
+    """A ptr param without data (GpuRuntimeToLlvm.cpp:507-536) reaches a
+    kernel built from LLVM IR as an offset into dynamic LDS: every group's
+    sum in index order, bit for bit."""
+    lib, g = rt
+    s = _Session(lib, g, rb.serialize(_ir("group_sum")))
+    groups = 300
+    x = np.random.default_rng(3).standard_normal(groups * 256).astype(np.float32)
+    src, _ = s.shared(x)
+    dst, out = s.shared(np.zeros(groups, np.float32))
+    s.launch("group_sum_f32", groups, [src, dst], block=256, local_bytes=256 * 4)
+    expect = np.cumsum(x.reshape(groups, 256), axis=1, dtype=np.float32)[:, -1]
+    assert np.array_equal(out, expect)
     s.close()

@@ -59,3 +59,13 @@ def test_every_optimisation_level_and_errors():
         rb.serialize("define void @broken( {")
     with pytest.raises(ValueError):
         rb.kernel_names(b"not an elf")
+
+
+def test_workgroup_memory_stays_dynamic():
+    """The external workgroup-memory array takes no static LDS: the launch
+    supplies the bytes."""
+    blob = rb.serialize(_ir("group_sum"))
+    assert rb.kernel_names(blob) == ["group_sum_f32"]
+    at = blob.index(b".group_segment_fixed_size")
+    # msgpack: the key, then a positive fixint 0
+    assert blob[at + len(b".group_segment_fixed_size")] == 0
