@@ -737,6 +737,18 @@ int planEvenShares(int64_t tiles, int64_t slabs, int64_t slots) {
   return int(slots);
 }
 
+// Whether cutting K into plan.slices equal slices goes ahead of even shares:
+// when the slices fill the resident blocks to 0.86 (measured: from 0.875 up
+// the slices are 4-17 % faster than even shares of the same tiles -- their
+// partial products are whole tiles that one streaming pass adds up -- at 0.84
+// and below the shares win), or when there are so few tiles that shares
+// would cut each into more than 16 pieces.
+bool splitFills(const SplitPlan &plan, int64_t tiles, int blocksPerCu) {
+  if (plan.slices < 2)
+    return false;
+  return tiles * plan.slices * 100 >= int64_t(256) * blocksPerCu * 86 || plan.slices >= 16;
+}
+
 enum WorkspaceKind { WORKSPACE_HEAP, WORKSPACE_FIXED };
 
 template <typename T> struct MemrefOf;
@@ -920,7 +932,9 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       bool big = bigFits && (bigEven > 0 || bigTiles >= 192);
       if (big && bigTiles < 192) {
         // (fewer large tiles than CUs only pay in even shares: without room
-        // for those, the 128 x 128 tiles take the shape)
+        // for those, the 128 x 128 tiles take the shape.  Slices of K on the
+        // large tile were measured and gain nothing over its even shares:
+        // 2048^3 160 against 158 us.)
         int blocks = bigEven;
         (void)evenWorkspace(blocks, 256, 256);
         big = blocks > 0;
@@ -1063,13 +1077,14 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
         const size_t xBytes = packXBytes;
         packBytes = packXBytes + packYBytes;
         const int slabs = int((K + BK - 1) / BK);
-        int evenBlocks = workspaceKind == WORKSPACE_HEAP
+        SplitPlan plan = planSplit(tilesM * tilesN, K, BK, sizeof(T) == 8 ? 2 : 1);
+        int evenBlocks = workspaceKind == WORKSPACE_HEAP &&
+                                 !splitFills(plan, tilesM * tilesN, sizeof(T) == 8 ? 2 : 1)
                              ? planEvenShares(tilesM * tilesN, slabs, slots)
                              : 0;
         T *W = evenWorkspace(evenBlocks, 128, 128);
-        SplitPlan plan;
-        if (!evenBlocks)
-          plan = planSplit(tilesM * tilesN, K, BK, sizeof(T) == 8 ? 2 : 1);
+        if (evenBlocks)
+          plan = SplitPlan();
         const int64_t ldw = (Nz + VEC - 1) / VEC * VEC;
         if (!evenBlocks)
           W = workspaceFor(plan, Mz, ldw);
@@ -1144,16 +1159,19 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           K <= 0x7fffffff && Mz <= 65535 * 32) {
         const int slabK = big ? bigSlab : BK;
         const int slabs = int(Kt / slabK);
+        SplitPlan plan;
+        if (!big)
+          plan = planSplit((Mt / BM) * (Nt / BN), Kt, BK, sizeof(T) == 8 ? 2 : 1);
         int evenBlocks = big ? bigEven
-                         : workspaceKind == WORKSPACE_HEAP
+                         : workspaceKind == WORKSPACE_HEAP &&
+                                 !splitFills(plan, (Mt / BM) * (Nt / BN), sizeof(T) == 8 ? 2 : 1)
                              ? planEvenShares((Mt / BM) * (Nt / BN), slabs, slots)
                              : 0;
         T *W = evenWorkspace(evenBlocks, BM, BN);
-        SplitPlan plan;
-        if (!big && !evenBlocks) {
-          plan = planSplit((Mt / BM) * (Nt / BN), Kt, BK, sizeof(T) == 8 ? 2 : 1);
+        if (evenBlocks)
+          plan = SplitPlan();
+        else if (!big)
           W = workspaceFor(plan, Mt, Nt);
-        }
         if (tooLarge)
           return 1;
         const EvenShares even{evenBlocks ? slabs : 0, int(Nt / BN)};

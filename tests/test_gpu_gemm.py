@@ -396,9 +396,12 @@ def test_split_k_beta_zero_ignores_c(env):
     (np.float32, 3560, 3800, 1020, "sgemm_mfma_256x256_even+packed"),
     (np.float32, 4000, 4000, 530, "sgemm_mfma_256x256+packed"),
     (np.float64, 3072, 3072, 512, "dgemm_mfma_128x128_even"),         # 1.125 rounds
-    (np.float64, 1024, 1024, 4096, "dgemm_mfma_128x128_even"),
-    (np.float64, 1000, 1100, 1200, "dgemm_mfma_128x128_ragged_even"),  # the reference's preset
-    (np.float64, 1500, 1700, 1200, "dgemm_mfma_128x128_ragged_even"),
+    (np.float64, 1536, 1536, 2048, "dgemm_mfma_128x128_even"),        # 144 tiles: 3 slices fill 0.84
+    (np.float64, 1500, 1500, 1200, "dgemm_mfma_128x128_ragged_even"),
+    # equal slices of K go first where they fill the blocks: 64 tiles x 8, 72 x 7
+    (np.float64, 1024, 1024, 4096, "dgemm_mfma_128x128_splitk"),
+    (np.float64, 1000, 1100, 1200, "dgemm_mfma_128x128_ragged_splitk"),  # the reference's preset
+    (np.float32, 1152, 1152, 1152, "sgemm_mfma_128x128_splitk"),
     # float64 from 256 padded tiles on: the same tile over zero-padded copies
     (np.float64, 2500, 2750, 3000, "dgemm_mfma_128x128_even+packed"),
     (np.float64, 2040, 4090, 600, "dgemm_mfma_128x128+packed"),
