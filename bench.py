@@ -20,6 +20,7 @@ import ctypes
 import json
 import math
 import os
+import re
 import sys
 import time
 
@@ -39,17 +40,29 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 WAKE_SECONDS = 0.1
 
 MEASURED_TRAFFIC = {
-    "nmk_black_scholes_f32_w64": 335614484,
-    "bench_streams_3r2w_f32": 335526234,
-    "nmk_black_scholes_f32_w32": 335607299,
-    "nmk_map2_rowbcast_add_f64": 268470962,
-    "nmk_sum_axis1_wide_f32": 537392134,
-    "nmk_norm2_f32": 536915846,
-    "nmk_sum_axis0_i32_i64": 538008264,
-    "nmk_twin_pairwise_f64_rows": 540497146,
+    "nmk_black_scholes_f32_w64": 335612006,
+    "bench_streams_3r2w_f32": 335528195,
+    "nmk_black_scholes_f32_w32": 335609034,
+    "nmk_map2_rowbcast_add_f64": 268477666,
+    "nmk_sum_axis1_wide_f32": 537392240,
+    "nmk_norm2_f32": 536915851,
+    "nmk_sum_axis0_i32_i64": 538008276,
+    "nmk_twin_pairwise_f64_rows": 540432684,
     "nmk_copy_b128": 536870912,
-    "sgemm_mfma_256x256": 671624029,
+    "sgemm_mfma_256x256": 671826722,
+    # generated kernels, without the hash of the body at the end of their names
+    "nmkjit_black_scholes_body": 335599967,
+    "nmkjit_black_scholes_loop_body": 335613367,
+    "nmkjit_scaled_add_body": 402631780,
+    "nmkjit_pairwise_body": 540511466,
 }
+
+
+def measured_traffic(kernel):
+    """HBM bytes per launch of ``kernel`` from the counter runs, or None."""
+    if kernel in MEASURED_TRAFFIC:
+        return MEASURED_TRAFFIC[kernel]
+    return MEASURED_TRAFFIC.get(re.sub(r"_[0-9a-f]{12}$", "", kernel or ""))
 
 
 def parse_args():
@@ -304,7 +317,7 @@ def hbm_entry(name, workload, alg_bytes, wall_ms, ev_ms, kernel, extra=None):
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC.get(kernel)},
+                     "traffic": measured_traffic(kernel)},
     }
     if extra:
         e.update(extra)
@@ -504,8 +517,7 @@ def run(args):
             "roofline": {"bound": "mfma", "achieved": round(tf, 2),
                          "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4),
-                         "traffic": MEASURED_TRAFFIC.get(
-                             math_runtime.last_kernel())},
+                         "traffic": measured_traffic(math_runtime.last_kernel())},
         }
         if orc:
             # The reference's CPU np.dot is MKL cblas_sgemm on all cores
