@@ -191,7 +191,8 @@ void nmhipPairwiseF64(void *ctx, const double *X1, const double *X2, double *D,
 const void *nmhipKernelBlob(const char *family, size_t *size);
 
 /* Overrides a launch-shape knob ("rowbcast_rows", "map_blocks", "bs_blocks",
- * "reduce_blocks", "axis0_rows", "pairwise_rows"); 0 restores the default. */
+ * "reduce_blocks", "axis0_rows", "cols_blocks", "pairwise_rows"); 0 restores
+ * the default. */
 void nmhipSetTuning(const char *knob, int64_t value);
 
 #ifdef __cplusplus

@@ -302,52 +302,176 @@ nmk_sum_all_f32(const float *x, float *out, int64_t n, int32_t vec,
 // Generic strided reduction: out[k * so] = fold_r op(x[k * sk + r * sr]) for
 // k < nKeep, r < nRed, accumulating in ACC starting from `init`.  One wave per
 // kept index; lanes stride over the reduced axis, then a wave butterfly.
-// Covers every (op, dtype, axis) combination at modest speed; a full
-// reduction is nKeep == 1.
+// Covers every (op, dtype, axis) combination; a full reduction is nKeep == 1.
+// vec != 0 (the host has checked: sr == 1, x 16-byte aligned, sk a multiple
+// of the elements in a 128-bit word): lanes read 128-bit words, four in
+// flight, the elements beyond the last whole word one by one.
+template <typename IN> struct WordOf {
+  static constexpr int N = 16 / sizeof(IN);
+  typedef IN type __attribute__((ext_vector_type(16 / sizeof(IN))));
+};
+
+template <typename IN, typename ACC, typename Op>
+__device__ __forceinline__ ACC foldWord(ACC acc, typename WordOf<IN>::type w, Op op) {
+#pragma unroll
+  for (int q = 0; q < WordOf<IN>::N; ++q)
+    acc = op(acc, ACC(w[q]));
+  return acc;
+}
+
+// Fold of x[0 .. n), x 16-byte aligned, by LANES lanes (a wave's 64 or a
+// block's 256) that read consecutive 128-bit words, four in flight a lane:
+// the lanes together stream LANES x 64 contiguous bytes per trip.  `id` is
+// the lane's index among them; every lane returns its share.
+template <int LANES, typename IN, typename ACC, typename Op>
+__device__ __forceinline__ ACC foldWords(const IN *__restrict__ x, int64_t n, int id,
+                                         ACC init, Op op) {
+  typedef typename WordOf<IN>::type Word;
+  constexpr int N = WordOf<IN>::N;
+  const Word *w = reinterpret_cast<const Word *>(x);
+  const int64_t words = n / N;
+  ACC a0 = init, a1 = init, a2 = init, a3 = init;
+  int64_t i = id;
+  for (; i + 3 * LANES < words; i += 4 * LANES) {
+    const Word v0 = __builtin_nontemporal_load(w + i);
+    const Word v1 = __builtin_nontemporal_load(w + i + LANES);
+    const Word v2 = __builtin_nontemporal_load(w + i + 2 * LANES);
+    const Word v3 = __builtin_nontemporal_load(w + i + 3 * LANES);
+    a0 = foldWord<IN>(a0, v0, op);
+    a1 = foldWord<IN>(a1, v1, op);
+    a2 = foldWord<IN>(a2, v2, op);
+    a3 = foldWord<IN>(a3, v3, op);
+  }
+  for (; i < words; i += LANES)
+    a0 = foldWord<IN>(a0, __builtin_nontemporal_load(w + i), op);
+  for (int64_t r = words * N + id; r < n; r += LANES)
+    a1 = op(a1, ACC(x[r]));
+  return op(op(a0, a1), op(a2, a3));
+}
+
+// The same over elements `stride` apart, one element a load.
+template <int LANES, typename IN, typename ACC, typename Op>
+__device__ __forceinline__ ACC foldElements(const IN *__restrict__ x, int64_t n,
+                                            int64_t stride, int id, ACC init, Op op) {
+  ACC a0 = init, a1 = init, a2 = init, a3 = init;
+  int64_t r = id;
+  for (; r + 3 * LANES < n; r += 4 * LANES) {
+    const IN v0 = x[r * stride], v1 = x[(r + LANES) * stride],
+             v2 = x[(r + 2 * LANES) * stride], v3 = x[(r + 3 * LANES) * stride];
+    a0 = op(a0, ACC(v0));
+    a1 = op(a1, ACC(v1));
+    a2 = op(a2, ACC(v2));
+    a3 = op(a3, ACC(v3));
+  }
+  for (; r < n; r += LANES)
+    a0 = op(a0, ACC(x[r * stride]));
+  return op(op(a0, a1), op(a2, a3));
+}
+
+// mode bit 0 (the host has checked: sr == 1, x 16-byte aligned, sk a multiple
+// of the elements in a 128-bit word): 128-bit loads.  mode bit 1: a block,
+// not a wave, per kept index (long rows: the block streams 16 KiB of its row
+// per trip).
 template <typename IN, typename ACC, typename Op>
 __device__ __forceinline__ void
 reduceStrided(const IN *x, ACC *out, int64_t nKeep, int64_t nRed, int64_t sk,
-              int64_t sr, int64_t so, ACC init, Op op) {
+              int64_t sr, int64_t so, int32_t mode, ACC init, Op op) {
+  __shared__ ACC slots[256 / NMK_WAVE];
+  const bool vec = mode & 1;
+  if (mode & 2) {
+    const int64_t k = blockIdx.x;
+    const IN *p = x + k * sk;
+    ACC acc = vec ? foldWords<256, IN, ACC>(p, nRed, threadIdx.x, init, op)
+                  : foldElements<256, IN, ACC>(p, nRed, sr, threadIdx.x, init, op);
+    acc = blockAllReduce<256>(acc, op, slots);
+    if (threadIdx.x == 0)
+      out[k * so] = acc;
+    return;
+  }
   const int lane = threadIdx.x % NMK_WAVE;
   const int64_t k =
       int64_t(blockIdx.x) * (blockDim.x / NMK_WAVE) + threadIdx.x / NMK_WAVE;
   if (k >= nKeep)
     return;
-  ACC acc = init, a1 = init, a2 = init, a3 = init;
   const IN *p = x + k * sk;
-  int64_t r = lane;
-  for (; r + 3 * NMK_WAVE < nRed; r += 4 * NMK_WAVE) { // four loads in flight
-    const IN v0 = p[r * sr], v1 = p[(r + NMK_WAVE) * sr],
-             v2 = p[(r + 2 * NMK_WAVE) * sr], v3 = p[(r + 3 * NMK_WAVE) * sr];
-    acc = op(acc, ACC(v0));
-    a1 = op(a1, ACC(v1));
-    a2 = op(a2, ACC(v2));
-    a3 = op(a3, ACC(v3));
-  }
-  for (; r < nRed; r += NMK_WAVE)
-    acc = op(acc, ACC(p[r * sr]));
-  acc = waveAllReduce(op(op(acc, a1), op(a2, a3)), op);
+  ACC acc = vec ? foldWords<NMK_WAVE, IN, ACC>(p, nRed, lane, init, op)
+                : foldElements<NMK_WAVE, IN, ACC>(p, nRed, sr, lane, init, op);
+  acc = waveAllReduce(acc, op);
   if (lane == 0)
     out[k * so] = acc;
 }
 
 // Generic reduction over the slow axis of a matrix whose kept index has unit
 // stride (column sums of a row-major matrix, row sums of a column-major one):
-// out[chunk * nKeep + k] = fold_{r in chunk} op(x[r * ld + k]).  A block owns
-// 256 consecutive kept indices (adjacent lanes read adjacent elements) and one
-// chunk of rowsPerChunk reduced indices, eight loads in flight per lane; with
-// more than one chunk the same kernel folds the partial results.
+// out[chunk * nKeep + k] = fold_{r in chunk} op(x[r * ld + k]); with more than
+// one chunk the same kernel folds the partial results.
+// vec == 0: a block owns 256 consecutive kept indices, one a lane, and a
+// chunk of rowsPerChunk reduced indices, eight loads in flight per lane.
+// vec != 0 (the host has checked: x 16-byte aligned, ld and nKeep multiples
+// of the elements in a 128-bit word): a block owns a strip of 64 words (1 KiB
+// of every row), a word a lane; its four waves take interleaved rows of the
+// chunk, eight loads in flight per lane, and meet in LDS.
 template <typename IN, typename ACC, typename Op>
 __device__ __forceinline__ void
 reduceColumns(const IN *__restrict__ x, ACC *__restrict__ out, int64_t nRed,
-              int64_t nKeep, int64_t ld, int64_t rowsPerChunk, ACC init, Op op) {
-  const int64_t k = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (k >= nKeep)
-    return;
+              int64_t nKeep, int64_t ld, int64_t rowsPerChunk, int32_t vec, ACC init,
+              Op op) {
   int64_t r = int64_t(blockIdx.y) * rowsPerChunk;
   int64_t rEnd = r + rowsPerChunk;
   if (rEnd > nRed)
     rEnd = nRed;
+  if (vec) {
+    typedef typename WordOf<IN>::type Word;
+    constexpr int N = WordOf<IN>::N;
+    constexpr int WAVES = 256 / NMK_WAVE;
+    constexpr int U = 8;
+    __shared__ ACC meet[WAVES][NMK_WAVE * N];
+    const int lane = threadIdx.x % NMK_WAVE;
+    const int wave = threadIdx.x / NMK_WAVE;
+    const int64_t k = (int64_t(blockIdx.x) * NMK_WAVE + lane) * N;
+    ACC a[N];
+#pragma unroll
+    for (int q = 0; q < N; ++q)
+      a[q] = init;
+    if (k < nKeep) {
+      r += wave;
+      const IN *p = x + r * ld + k;
+      const int64_t step = WAVES * ld;
+      for (; r + WAVES * (U - 1) < rEnd; r += WAVES * U) {
+        Word v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          v[u] = __builtin_nontemporal_load(reinterpret_cast<const Word *>(p + u * step));
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int q = 0; q < N; ++q)
+            a[q] = op(a[q], ACC(v[u][q]));
+        p += U * step;
+      }
+      for (; r < rEnd; r += WAVES) {
+        const Word v = __builtin_nontemporal_load(reinterpret_cast<const Word *>(p));
+#pragma unroll
+        for (int q = 0; q < N; ++q)
+          a[q] = op(a[q], ACC(v[q]));
+        p += step;
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < N; ++q)
+      meet[wave][lane * N + q] = a[q];
+    __syncthreads();
+    for (int c = threadIdx.x; c < NMK_WAVE * N; c += 256) {
+      const int64_t kc = int64_t(blockIdx.x) * NMK_WAVE * N + c;
+      if (kc < nKeep)
+        out[int64_t(blockIdx.y) * nKeep + kc] =
+            op(op(meet[0][c], meet[1][c]), op(meet[2][c], meet[3][c]));
+    }
+    return;
+  }
+  const int64_t k = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (k >= nKeep)
+    return;
   const IN *p = x + r * ld + k;
   ACC a[8];
 #pragma unroll
@@ -372,35 +496,27 @@ reduceColumns(const IN *__restrict__ x, ACC *__restrict__ out, int64_t nRed,
 }
 
 // Generic reduction of a long contiguous run in chunks: out[c] = fold of
-// x[c * chunk .. min(n, (c + 1) * chunk)), one wave per chunk, four loads in
-// flight per lane.  A full reduction is this kernel followed by the strided
-// one over the partial results.
+// x[c * chunk .. min(n, (c + 1) * chunk)), one block per chunk (its 256
+// lanes stream 16 KiB per trip).  A full reduction is this kernel followed by
+// the strided one over the partial results.  vec != 0 (the host has checked:
+// x 16-byte aligned, chunk a multiple of the elements in a 128-bit word):
+// 128-bit loads.
 template <typename IN, typename ACC, typename Op>
 __device__ __forceinline__ void
 reduceChunks(const IN *__restrict__ x, ACC *__restrict__ out, int64_t n,
-             int64_t chunk, int64_t nChunks, ACC init, Op op) {
-  const int lane = threadIdx.x % NMK_WAVE;
-  const int64_t c =
-      int64_t(blockIdx.x) * (blockDim.x / NMK_WAVE) + threadIdx.x / NMK_WAVE;
+             int64_t chunk, int64_t nChunks, int32_t vec, ACC init, Op op) {
+  __shared__ ACC slots[256 / NMK_WAVE];
+  const int64_t c = blockIdx.x;
   if (c >= nChunks)
     return;
-  int64_t i = c * chunk + lane;
+  const int64_t i = c * chunk;
   int64_t end = (c + 1) * chunk;
   if (end > n)
     end = n;
-  ACC a0 = init, a1 = init, a2 = init, a3 = init;
-  for (; i + 3 * NMK_WAVE < end; i += 4 * NMK_WAVE) {
-    const IN v0 = x[i], v1 = x[i + NMK_WAVE], v2 = x[i + 2 * NMK_WAVE],
-             v3 = x[i + 3 * NMK_WAVE];
-    a0 = op(a0, ACC(v0));
-    a1 = op(a1, ACC(v1));
-    a2 = op(a2, ACC(v2));
-    a3 = op(a3, ACC(v3));
-  }
-  for (; i < end; i += NMK_WAVE)
-    a0 = op(a0, ACC(x[i]));
-  ACC acc = waveAllReduce(op(op(a0, a1), op(a2, a3)), op);
-  if (lane == 0)
+  ACC acc = vec ? foldWords<256, IN, ACC>(x + i, end - i, threadIdx.x, init, op)
+                : foldElements<256, IN, ACC>(x + i, end - i, 1, threadIdx.x, init, op);
+  acc = blockAllReduce<256>(acc, op, slots);
+  if (threadIdx.x == 0)
     out[c] = acc;
 }
 
@@ -408,20 +524,22 @@ reduceChunks(const IN *__restrict__ x, ACC *__restrict__ out, int64_t n,
   NMK_KERNEL(256)                                                              \
   nmk_reduce_##OPNAME##_##TNAME(const IN *x, ACC *out, int64_t nKeep,          \
                                 int64_t nRed, int64_t sk, int64_t sr,          \
-                                int64_t so) {                                  \
-    reduceStrided<IN, ACC>(x, out, nKeep, nRed, sk, sr, so, ACC(INIT), OP());  \
+                                int64_t so, int32_t vec) {                     \
+    reduceStrided<IN, ACC>(x, out, nKeep, nRed, sk, sr, so, vec, ACC(INIT),    \
+                           OP());                                              \
   }                                                                            \
   NMK_KERNEL(256)                                                              \
   nmk_reducecols_##OPNAME##_##TNAME(const IN *x, ACC *out, int64_t nRed,       \
                                     int64_t nKeep, int64_t ld,                 \
-                                    int64_t rowsPerChunk) {                    \
-    reduceColumns<IN, ACC>(x, out, nRed, nKeep, ld, rowsPerChunk, ACC(INIT),   \
-                           OP());                                              \
+                                    int64_t rowsPerChunk, int32_t vec) {       \
+    reduceColumns<IN, ACC>(x, out, nRed, nKeep, ld, rowsPerChunk, vec,         \
+                           ACC(INIT), OP());                                   \
   }                                                                            \
   NMK_KERNEL(256)                                                              \
   nmk_reducechunks_##OPNAME##_##TNAME(const IN *x, ACC *out, int64_t n,        \
-                                      int64_t chunk, int64_t nChunks) {        \
-    reduceChunks<IN, ACC>(x, out, n, chunk, nChunks, ACC(INIT), OP());         \
+                                      int64_t chunk, int64_t nChunks,          \
+                                      int32_t vec) {                           \
+    reduceChunks<IN, ACC>(x, out, n, chunk, nChunks, vec, ACC(INIT), OP());    \
   }
 
 NMK_DEFINE_REDUCE(sum, AddOp, 0, i32, int32_t, int64_t)

