@@ -428,6 +428,16 @@ class Dispatcher:
                 self._names.update(table)
         return self._names.get(name)
 
+    def _callee(self, node):
+        """The Python object a call's function expression names: a name, or
+        attributes of one (``numba_mlir.prange``), else None."""
+        if isinstance(node, ast.Name):
+            return self._resolve(node.id)
+        if isinstance(node, ast.Attribute):
+            base = self._callee(node.value)
+            return getattr(base, node.attr, None) if base is not None else None
+        return None
+
     def _served(self, how, result, ctx):
         self.last_launch = {"path": how, "kernel": ctx.last_kernel()}
         return result
@@ -438,9 +448,8 @@ class Dispatcher:
             self._parallel_loop = False
             if not isinstance(self._node, ast.Lambda):
                 for stmt in self._node.body:
-                    if isinstance(stmt, ast.For) and isinstance(stmt.iter, ast.Call) and \
-                            isinstance(stmt.iter.func, ast.Name):
-                        target = self._resolve(stmt.iter.func.id)
+                    if isinstance(stmt, ast.For) and isinstance(stmt.iter, ast.Call):
+                        target = self._callee(stmt.iter.func)
                         if getattr(target, "_nmk_prange", False):
                             self._parallel_loop = True
         return self._parallel_loop
@@ -475,8 +484,8 @@ class Dispatcher:
             while rank < 3 and len(loop.body) == 1 and isinstance(loop.body[0], ast.For):
                 inner = loop.body[0]
                 it = inner.iter
-                if not (isinstance(it, ast.Call) and isinstance(it.func, ast.Name) and
-                        getattr(self._resolve(it.func.id), "_nmk_prange", False)):
+                if not (isinstance(it, ast.Call) and
+                        getattr(self._callee(it.func), "_nmk_prange", False)):
                     break
                 used = {n.id for a in it.args for n in ast.walk(a) if isinstance(n, ast.Name)}
                 if used & seen or not isinstance(inner.target, ast.Name):

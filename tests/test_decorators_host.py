@@ -1,0 +1,50 @@
+"""Host-side logic of ``njit`` that needs no GPU: which functions are taken as
+one parallel loop."""
+
+import numpy as np
+
+from numba_mlir_amd import decorators
+from numba_mlir_amd.decorators import njit, prange
+
+
+def _by_name(x):
+    s = 0.0
+    for i in prange(x.shape[0]):
+        s += x[i]
+    return s
+
+
+def _by_attribute(x):
+    s = 0.0
+    for i in decorators.prange(x.shape[0]):
+        s += x[i]
+    return s
+
+
+def _nested_by_attribute(a):
+    for h in decorators.prange(a.shape[0]):
+        for w in decorators.prange(a.shape[1]):
+            a[h, w] = h + w
+
+
+def _sequential(x):
+    s = 0.0
+    for i in range(x.shape[0]):
+        s += x[i]
+    return s
+
+
+def _unknown_callee(x):
+    for i in np.nothing_of_that_name(3):
+        pass
+
+
+def test_prange_is_found_by_name_and_through_a_module():
+    """``for i in prange(n)`` and ``for i in module.prange(n)`` are the same
+    loop (the reference's users write ``numba.prange``)."""
+    assert njit(parallel=True)(_by_name)._has_parallel_loop()
+    assert njit(parallel=True)(_by_attribute)._has_parallel_loop()
+    nested = njit(parallel=True)(_nested_by_attribute)
+    assert nested._has_parallel_loop() and nested._grid_rank() == 2
+    assert not njit(parallel=True)(_sequential)._has_parallel_loop()
+    assert not njit(parallel=True)(_unknown_callee)._has_parallel_loop()
