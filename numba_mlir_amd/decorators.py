@@ -908,6 +908,49 @@ class Dispatcher:
             raise kernel_compiler.KernelCompileError(f"{where}: np.{op}: {exc}") from exc
 
     # -- 4. elementwise fusion -----------------------------------------------
+    def _refuse_sequential_array_loops(self, args):
+        """A ``for ... in range(...)`` whose bounds are taken from an array
+        argument (``x.shape[0]``, ``len(x)``, ``x.size``) walks that array in
+        order: on the host that is a sequential loop, which is not offloaded
+        -- as one work-item's loop inside a fused map it would run once per
+        element.  Such a function must say ``prange``."""
+        arrays = {name for name, a in zip(self._params(), args) if isinstance(a, HipNdArray)}
+
+        def sized_by_array(node):
+            for n in ast.walk(node):
+                if isinstance(n, ast.Attribute) and n.attr in ("shape", "size") and \
+                        isinstance(n.value, ast.Name) and n.value.id in arrays:
+                    return n.value.id
+                if isinstance(n, ast.Call) and isinstance(n.func, ast.Name) and \
+                        n.func.id == "len" and len(n.args) == 1 and \
+                        isinstance(n.args[0], ast.Name) and n.args[0].id in arrays:
+                    return n.args[0].id
+            return None
+
+        # names bound to such extents first (n = len(x); for i in range(n))
+        extents = {}
+        for n in ast.walk(self._node):
+            if isinstance(n, ast.Assign) and len(n.targets) == 1 and \
+                    isinstance(n.targets[0], ast.Name):
+                owner = sized_by_array(n.value)
+                if owner:
+                    extents[n.targets[0].id] = owner
+        for n in ast.walk(self._node):
+            if not (isinstance(n, ast.For) and isinstance(n.iter, ast.Call) and
+                    self._callee(n.iter.func) is range):
+                continue
+            owner = None
+            for a in n.iter.args:
+                owner = owner or sized_by_array(a)
+                for m in ast.walk(a):
+                    if isinstance(m, ast.Name) and m.id in extents:
+                        owner = owner or extents[m.id]
+            if owner:
+                raise kernel_compiler.KernelCompileError(
+                    f"{self.py_func.__name__}, line {n.lineno}: a range loop over the extent of "
+                    f"array argument '{owner}' is sequential and is not offloaded; write it "
+                    "with prange")
+
     def _elementwise(self, args):
         ctx = kernel_impl.check_device_args(args)
         # Everything but addresses and scalar values is fixed by the argument
@@ -930,6 +973,7 @@ class Dispatcher:
                 self.last_plan = plan
                 return ret
 
+        self._refuse_sequential_array_loops(args)
         arrays = [a for a in args if isinstance(a, HipNdArray)]
         shape = np.broadcast_shapes(*[a.shape for a in arrays])
         views = [a.broadcast_to(shape) if isinstance(a, HipNdArray) else a for a in args]

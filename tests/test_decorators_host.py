@@ -48,3 +48,32 @@ def test_prange_is_found_by_name_and_through_a_module():
     assert nested._has_parallel_loop() and nested._grid_rank() == 2
     assert not njit(parallel=True)(_sequential)._has_parallel_loop()
     assert not njit(parallel=True)(_unknown_callee)._has_parallel_loop()
+
+
+def _n_first(x):
+    n = len(x)
+    s = 0.0
+    for i in range(1, n):
+        s += x[i]
+    return s
+
+
+def _small_inner_loop(x, y):
+    acc = x * 0.0
+    for k in range(3):
+        acc = acc * y + x
+    return acc
+
+
+def test_sequential_loops_over_an_array_are_refused_not_run_per_element():
+    """Without prange such a loop is host code in the reference; as the loop
+    of every work-item of a fused map it would be quadratic."""
+    import pytest
+    from numba_mlir_amd.mlir import kernel_compiler
+    from numba_mlir_amd.mlir.device_array import HipNdArray
+    x = HipNdArray.__new__(HipNdArray)          # (only its type is looked at)
+    for func in (_sequential, _n_first):
+        with pytest.raises(kernel_compiler.KernelCompileError, match="write it with prange"):
+            njit(func)._refuse_sequential_array_loops([x])
+    njit(_small_inner_loop)._refuse_sequential_array_loops([x, x])
+    njit(_by_name)._refuse_sequential_array_loops([x])      # (prange is not range)
