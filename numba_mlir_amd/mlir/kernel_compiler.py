@@ -634,7 +634,10 @@ class FunctionTranslator:
         """Template argument of the routines that come in a plain and a
         careful form, where the body is computed under speculation (a fused
         map over adjacent elements), else the empty string."""
-        if self.adjacent and self.mode in ("elementwise", "parallel") and self.is_kernel:
+        if self.adjacent and self.mode in ("elementwise", "parallel") and self.is_kernel \
+                and not self.reductions:
+            # (a loop with reduction variables keeps them in registers of one
+            # inlined body: no second, out-of-line form)
             self.speculates = True
             return "<decltype(nmk_careful)::value>"
         return ""
@@ -668,8 +671,9 @@ class FunctionTranslator:
         a lane's elements a block apart.)"""
         if not (self.is_kernel and self.mode in ("elementwise", "parallel") and
                 self.ndim == 1 and self.noalias and self.elements_per_thread == 4) or \
-                self.m.communicates or self.m.boundscheck or self.reductions or \
-                self.opaque_write:
+                self.m.communicates or self.m.boundscheck or self.opaque_write:
+            return False
+        if self.reductions and self.mode != "parallel":
             return False
         if self.mode == "parallel":
             # one prange(n) loop: iteration g is work-item g.  Which arrays it
@@ -694,7 +698,7 @@ class FunctionTranslator:
             if not (isinstance(t, Array) and t.layout == "C" and t.ndim == 1 and
                     t.elem.ctype in self._WORD_CTYPES):
                 raise _NotAdjacent(f"'{name}' is not a dense array of 4-byte elements")
-        if not self.adjacent_outs:
+        if not self.adjacent_outs and not (self.reductions and self.prefetched):
             raise _NotAdjacent("no array is assigned at every index")
         for ctype, _ in self.adjacent_outs.values():
             if ctype not in self._WORD_CTYPES:
@@ -728,26 +732,43 @@ class FunctionTranslator:
         names = "".join(f", nmk_pf_{n}" for n, _, _ in ins)
         # The careful form is kept out of line (and the closures hold copies,
         # not addresses): inlined, it would cost the plain form registers.
+        # With reduction variables there is one form only, inlined, that adds
+        # to them where they are.
+        reducing = bool(self.reductions)
         out += [
-            "  auto nmk_item = [=](const int64_t nmk_gid0, auto nmk_careful, bool &nmk_ok"
-            f"{extra}) -> nmk_results {{",
+            f"  auto nmk_item = [{'&' if reducing else '='}](const int64_t nmk_gid0, "
+            f"auto nmk_careful, bool &nmk_ok{extra}) -> nmk_results {{",
             "    (void)nmk_gid0; (void)nmk_ok;",
             "    nmk_results nmk_out = {};",
         ] + body + [
             "    return nmk_out;",
             "  };",
-            f"  auto nmk_item_careful = [=](const int64_t nmk_gid0{extra}) "
-            "__attribute__((noinline)) -> nmk_results {",
-            "    bool nmk_unused = true;",
-            f"    return nmk_item(nmk_gid0, nmkjit::Yes(), nmk_unused{names});",
-            "  };",
+        ]
+        if reducing:
+            out += [
+                f"  auto nmk_item_careful = [&](const int64_t nmk_gid0{extra}) -> nmk_results {{",
+                "    bool nmk_unused = true;",
+                f"    return nmk_item(nmk_gid0, nmkjit::Yes(), nmk_unused{names});",
+                "  };",
+            ]
+        else:
+            out += [
+                f"  auto nmk_item_careful = [=](const int64_t nmk_gid0{extra}) "
+                "__attribute__((noinline)) -> nmk_results {",
+                "    bool nmk_unused = true;",
+                f"    return nmk_item(nmk_gid0, nmkjit::Yes(), nmk_unused{names});",
+                "  };",
+            ]
+        out += [
             "  const bool nmk_words = ((" + " | ".join(
                 f"reinterpret_cast<uintptr_t>({p})" for p in pointers) + ") & 15u) == 0;",
             "  const int64_t nmk_nvec = nmk_words ? nmk_gsz0 / 4 : 0;",
             "  const int64_t nmk_lane = nmk_grp0 * nmk_lsz0 + nmk_lid0;",
             "  const int64_t nmk_lanes = int64_t(gridDim.x) * nmk_lsz0;",
-            "  for (int64_t nmk_i = nmk_lane; nmk_i < nmk_nvec; nmk_i += nmk_lanes) {",
         ]
+        # (two words of every operand in flight a lane were measured for loops
+        # that only reduce: slower, 88 against 79 us for 512 MiB)
+        out.append("  for (int64_t nmk_i = nmk_lane; nmk_i < nmk_nvec; nmk_i += nmk_lanes) {")
         for n, ct, c in ins:
             src = f"reinterpret_cast<const nmk_in_t_{n} *>({c}_p) + nmk_i"
             load = f"__builtin_nontemporal_load({src})" if nt else f"*({src})"
@@ -761,6 +782,7 @@ class FunctionTranslator:
             "    for (int nmk_k = 0; nmk_k < 4; ++nmk_k) {",
             f"      const nmk_results nmk_r = nmk_item(nmk_i * 4 + nmk_k, nmkjit::No(), nmk_ok"
             f"{args});",
+            "      (void)nmk_r;",
         ] + keep + [
             "    }",
         ]
@@ -783,6 +805,7 @@ class FunctionTranslator:
             "  }",
             "  for (int64_t g = nmk_nvec * 4 + nmk_lane; g < nmk_gsz0; g += nmk_lanes) {",
             f"    const nmk_results nmk_r = nmk_item_careful(g{scalars});",
+            "    (void)nmk_r;",
         ] + [f"    {ptr}[g] = nmk_r.{code};" for code, (_, ptr) in outs] + [
             "  }",
         ]

@@ -453,7 +453,19 @@ def test_prange_reductions(K, tmp_path, monkeypatch):
     assert ck.return_source == "(total / n, above)"
     assert "int64_t *nmk_part_above, double *nmk_part_total" in ck.source
     assert ck.source.count("nmkjit::blockReduceStore<") == 2
+    # dense float32 operands read at the loop's own index: a 128-bit word of
+    # four adjacent iterations a lane, the sums kept where they are (one
+    # inlined form of the body, closures by reference)
+    assert ("const nmk_in_t_x nmk_in_x = __builtin_nontemporal_load("
+            "reinterpret_cast<const nmk_in_t_x *>(v_x_p) + nmk_i);") in ck.source
+    assert "auto nmk_item = [&](const int64_t nmk_gid0, auto nmk_careful" in ck.source
+    assert "noinline" not in ck.source and "ballot" not in ck.source
     assert kc.build_code_object(ck)[:4] == b"\x7fELF"
+    # (float64 operands: a lane's elements a block apart, as before)
+    f64 = kc.Array(kc.FLOAT64, 1, layout="C")
+    ck64 = kc.translate(njit_cases.sum_of_squares, [f64], 1, K, mode="parallel",
+                        noalias=True, elements_per_thread=4)
+    assert "nmk_in_t_x" not in ck64.source and "nmk_ahead_x[4]" in ck64.source
     ck = kc.translate(njit_cases.product, [f32], 1, K, mode="parallel")
     assert ck.reductions == [("p", np.dtype(np.float64), "mul")]
     assert "double v_p = (double)1;" in ck.source
