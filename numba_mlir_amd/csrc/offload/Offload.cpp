@@ -844,9 +844,9 @@ NMHIP_EXPORT void nmhipReduce(void *ctx, int op, int dtype, const void *x,
                  Arg::I64(0), Arg::I64(1), Arg::I64(1), Arg::I32(0)});
       return;
     }
-    // (a block per kept index where the reduced run is long and the kept
-    // indices alone fill the GPU; a wave per kept index otherwise)
-    const bool wide = nRed >= 4096 && nKeep >= 512;
+    // (a block per kept index where the reduced run is long, a wave per
+    // kept index otherwise)
+    const bool wide = nRed >= 4096;
     const int mode = ((sr == 1 && aligned16(x) && (nKeep == 1 || sk % word == 0)) ? 1 : 0) |
                      (wide ? 2 : 0);
     c->launch(std::string("nmk_reduce_") + opNames[op] + "_" + dtypeName(dtype),

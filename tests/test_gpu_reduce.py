@@ -189,6 +189,7 @@ _ROUTES = [
     ("rows, a block each, words", (600, 4100), False),
     ("rows, a block each, odd leading dimension", (520, 4099), False),
     ("rows, a wave each", (37, 1500), False),
+    ("few long rows", (5, 70000), False),
     ("columns on words", (4100, 516), False),
     ("columns on single elements", (4100, 515), False),
     ("one run in chunks", (1, 1000003), False),
