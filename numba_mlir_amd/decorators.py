@@ -558,6 +558,7 @@ class Dispatcher:
             counts = trip_counts(compiled)
         count = math.prod(counts)
         partials = []
+        read_back = None
 
         def make_partials(blocks):
             for _, dtype, _ in compiled.reductions:
@@ -574,9 +575,19 @@ class Dispatcher:
                     ctx, compiled, self.py_func.__name__, counts, args,
                     make_partials=make_partials if compiled.reductions else None)
                 plan.run()
+                read_back = [part.asnumpy() for part in partials]   # (before others see the plan)
                 if len(entry["plans"]) >= MAX_PLANS:
                     entry["plans"].clear()
                 entry["plans"][(compiled.name, counts)] = plan
+            elif compiled.reductions and plan.partials_free.acquire(blocking=False):
+                # the launch's own arrays of partial results, read back before
+                # another call of this thread or any other may write them
+                try:
+                    partials = plan.partials
+                    plan.run(args, partials=partials)
+                    read_back = [part.asnumpy() for part in partials]
+                finally:
+                    plan.partials_free.release()
             else:
                 if compiled.reductions:
                     make_partials(math.prod(plan.grid))
@@ -586,8 +597,9 @@ class Dispatcher:
         self.last_launch = dict(info, path="parallel loop")
         # fold the per-block partial results, in block order, onto the values
         # the reduction variables had before the loop
-        for (name, dtype, op), part in zip(compiled.reductions, partials):
-            blocks = part.asnumpy()
+        if read_back is None:
+            read_back = [part.asnumpy() for part in partials]
+        for (name, dtype, op), blocks in zip(compiled.reductions, read_back):
             start = np.dtype(dtype).type(scope[name])
             with np.errstate(over="ignore"):
                 fold = blocks.sum(dtype=dtype) if op == "add" else blocks.prod(dtype=dtype)
@@ -706,14 +718,21 @@ class Dispatcher:
         if first.size == 0 or not all(
                 env[n].shape == first.shape and env[n].is_c_contiguous() for n in arrays):
             return NotImplemented
-        # the type the map stage itself would give its result
-        try:
-            sub, params = self._stage_dispatcher(k - 1, source, scope)
-            flat = [env[p].reshape((first.size,)) if p in arrays else env[p] for p in params]
-            dtype = sub._compile("elementwise", flat, 1, False).ret_dtype
-        except kernel_compiler.KernelCompileError:
-            return NotImplemented
+        # the type the map stage itself would give its result (it follows from
+        # the operands' types: looked up once per combination)
+        type_key = ("map dtype", k, kernel_impl.captured_constants(self.py_func), tuple(
+            (v.dtype, v.ndim) if isinstance(v, HipNdArray) else type(v) for v in values))
+        dtype = self._stage_funcs.get(type_key)
         if dtype is None:
+            try:
+                sub, params = self._stage_dispatcher(k - 1, source, scope)
+                flat = [env[p].reshape((first.size,)) if p in arrays else env[p]
+                        for p in params]
+                dtype = sub._compile("elementwise", flat, 1, False).ret_dtype
+            except kernel_compiler.KernelCompileError:
+                return NotImplemented
+            self._stage_funcs[type_key] = dtype if dtype is not None else False
+        if dtype is None or dtype is False:
             return NotImplemented
         dtype = np.dtype(dtype)
         if dtype.kind not in "fiub":

@@ -457,7 +457,9 @@ class LaunchPlan:
             else:
                 self._arg_slots.append(params.add_scalar(a))
         self._ret_slot = params.add_array(ret) if ret is not None else None
-        # one pointer per reduction variable
+        # one pointer per reduction variable (the arrays stay with the plan)
+        self.partials = list(partials)
+        self.partials_free = threading.Lock()   # held from a launch into them to their read-back
         self._partial_slots = [params._add(ctypes.c_void_p(part.ptr), lowered.PARAM_PTR)
                                for part in partials]
         for nbytes in compiled.local_bytes:
