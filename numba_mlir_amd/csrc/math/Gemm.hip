@@ -866,6 +866,31 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
     return static_cast<T *>(p);
   };
   const int64_t slots = 512; // resident blocks of the 128 x 128 tiles: two a CU
+  // Equal slices of K for `tiles` 128 x 128 tiles, and whether they go ahead
+  // of even shares.  float64 blocks share a CU in pairs; float32 ones may
+  // (186 registers a lane), which pays where one block a CU would not fill
+  // the GPU but two do (72 tiles: 3 slices fill 0.84 of 256 blocks, 7 fill
+  // 0.98 of 512; 1000 x 1100 x 1200 58 -> 52 us, 1280^3 64 -> 59), and not
+  // otherwise (1024^3: 4 slices on 256 blocks 40 us, 8 on 512 43).  The
+  // entry point that may not allocate keeps to 256 blocks: the fixed
+  // workspace is sized for those.
+  auto planSlices = [&](int64_t tiles, int64_t k, bool &fills) {
+    if (sizeof(T) == 8) {
+      const SplitPlan two = planSplit(tiles, k, Mfma<T>::BK, 2);
+      fills = splitFills(two, tiles, 2);
+      return two;
+    }
+    const SplitPlan one = planSplit(tiles, k, Mfma<T>::BK, 1);
+    fills = splitFills(one, tiles, 1);
+    if (fills || workspaceKind != WORKSPACE_HEAP)
+      return one;
+    const SplitPlan two = planSplit(tiles, k, Mfma<T>::BK, 2);
+    if (splitFills(two, tiles, 2)) {
+      fills = true;
+      return two;
+    }
+    return one;
+  };
   auto fold = [&](const SplitPlan &plan, const T *W, int64_t m, int64_t n,
                   int64_t ldw, int64_t ldz, T *Z) {
     const int64_t words = m * ((n + Mfma<T>::VEC - 1) / Mfma<T>::VEC);
@@ -1077,9 +1102,9 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
         const size_t xBytes = packXBytes;
         packBytes = packXBytes + packYBytes;
         const int slabs = int((K + BK - 1) / BK);
-        SplitPlan plan = planSplit(tilesM * tilesN, K, BK, sizeof(T) == 8 ? 2 : 1);
-        int evenBlocks = workspaceKind == WORKSPACE_HEAP &&
-                                 !splitFills(plan, tilesM * tilesN, sizeof(T) == 8 ? 2 : 1)
+        bool slicesFill = false;
+        SplitPlan plan = planSlices(tilesM * tilesN, K, slicesFill);
+        int evenBlocks = workspaceKind == WORKSPACE_HEAP && !slicesFill
                              ? planEvenShares(tilesM * tilesN, slabs, slots)
                              : 0;
         T *W = evenWorkspace(evenBlocks, 128, 128);
@@ -1160,11 +1185,11 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
         const int slabK = big ? bigSlab : BK;
         const int slabs = int(Kt / slabK);
         SplitPlan plan;
+        bool slicesFill = false;
         if (!big)
-          plan = planSplit((Mt / BM) * (Nt / BN), Kt, BK, sizeof(T) == 8 ? 2 : 1);
+          plan = planSlices((Mt / BM) * (Nt / BN), Kt, slicesFill);
         int evenBlocks = big ? bigEven
-                         : workspaceKind == WORKSPACE_HEAP &&
-                                 !splitFills(plan, (Mt / BM) * (Nt / BN), sizeof(T) == 8 ? 2 : 1)
+                         : workspaceKind == WORKSPACE_HEAP && !slicesFill
                              ? planEvenShares((Mt / BM) * (Nt / BN), slabs, slots)
                              : 0;
         T *W = evenWorkspace(evenBlocks, BM, BN);

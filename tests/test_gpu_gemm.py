@@ -389,7 +389,8 @@ def test_split_k_beta_zero_ignores_c(env):
     (np.float32, 1024, 1024, 4096, "sgemm_mfma_256x256_even"),
     (np.float32, 2048, 2048, 2048 + 16, "sgemm_mfma_256x256_even"),   # slabs of 16
     (np.float32, 1536, 1408, 2056, "sgemm_mfma_128x128_even+edges"),  # the rest of K beside
-    (np.float32, 1000, 1100, 1200, "sgemm_mfma_128x128_ragged_even"),
+    (np.float32, 1500, 1500, 1200, "sgemm_mfma_128x128_ragged_even"),
+    (np.float32, 1000, 1100, 1200, "sgemm_mfma_128x128_ragged_splitk"),  # 72 tiles x 7 on 512 blocks
     (np.float32, 2000, 2300, 2600, "sgemm_mfma_128x128_ragged_even"),
     # from 192 padded tiles on, ragged float32 shapes run on the large tile over
     # zero-padded copies of both operands: 210 tiles in even shares, 256 as they are
