@@ -954,7 +954,11 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       const int bigEven = bigFits && workspaceKind == WORKSPACE_HEAP
                               ? planEvenShares(bigTiles, Kt / bigSlab, 256)
                               : 0;
-      bool big = bigFits && (bigEven > 0 || bigTiles >= 192);
+      // (from 64 large tiles on: below, the 128 x 128 tiles in slices or
+      // shares are as fast or faster -- 1792^3 120 against 131 us, 1024 x
+      // 1024 x 4096 92 against 99 -- and from 121 on the large tile wins,
+      // 3072^3 456 against 474)
+      bool big = bigFits && bigTiles >= 64 && (bigEven > 0 || bigTiles >= 192);
       if (big && bigTiles < 192) {
         // (fewer large tiles than CUs only pay in even shares: without room
         // for those, the 128 x 128 tiles take the shape.  Slices of K on the

@@ -385,8 +385,10 @@ def test_split_k_beta_zero_ignores_c(env):
     # 576 tiles of 256 x 256, eight slabs each: a share is 2.25 tiles (the end
     # of one, a whole one, the beginning of the next)
     (np.float32, 6144, 6144, 256, "sgemm_mfma_256x256_even"),
-    # 16 tiles on 256 blocks: every tile in sixteen pieces
-    (np.float32, 1024, 1024, 4096, "sgemm_mfma_256x256_even"),
+    # 64 tiles on 256 blocks: every tile in four pieces
+    (np.float32, 2048, 2048, 1024, "sgemm_mfma_256x256_even"),
+    # (fewer than 64 large tiles: the small ones, here in four slices of K)
+    (np.float32, 1024, 1024, 4096, "sgemm_mfma_128x128_splitk"),
     (np.float32, 2048, 2048, 2048 + 16, "sgemm_mfma_256x256_even"),   # slabs of 16
     (np.float32, 1536, 1408, 2056, "sgemm_mfma_128x128_even+edges"),  # the rest of K beside
     (np.float32, 1500, 1500, 1200, "sgemm_mfma_128x128_ragged_even"),
@@ -434,12 +436,12 @@ def test_even_shares(env, dtype, m, n, k, kernel, ta, tb, tc):
 
 def test_even_shares_beta_zero_ignores_c_and_the_no_alloc_entry_keeps_slices(env):
     hip, ops, _, mrt = env
-    a = np.ones((1024, 4096), np.float32)
-    b = np.ones((4096, 1024), np.float32)
-    c = hip.asarray(np.full((1024, 1024), np.nan, np.float32))
+    a = np.ones((2048, 1024), np.float32)
+    b = np.ones((1024, 2048), np.float32)
+    c = hip.asarray(np.full((2048, 2048), np.nan, np.float32))
     ops.gemm(hip.asarray(a), hip.asarray(b), c, 1.0, 0.0)
     assert "_even" in mrt.last_kernel()
-    assert (c.asnumpy() == 4096).all()
+    assert (c.asnumpy() == 1024).all()
 
 
 def test_calls_from_two_threads_take_turns_on_the_workspace(env):
