@@ -237,11 +237,11 @@ __device__ __forceinline__ T groupReduce(T *slots, T v, bool clipped, Op op) {
 }
 
 // Reduction of one value per lane over the whole block (every lane calls it,
-// lanes outside the global size with the neutral element); lane 0 stores the
-// block's result at partial[block index].  The tree is fixed by the block
-// shape, so repeated launches give the same bits.
+// lanes outside the global size with the neutral element): lane 0 gets the
+// block's result.  The tree is fixed by the block shape, so repeated launches
+// give the same bits.
 template <typename T, typename Op>
-__device__ __forceinline__ void blockReduceStore(T v, Op op, T *partial) {
+__device__ __forceinline__ T blockReduce(T v, Op op) {
   __shared__ T slots[kMaxGroup];
   const int tid = linearLocalId();
   const int n = localCount();
@@ -256,8 +256,99 @@ __device__ __forceinline__ void blockReduceStore(T v, Op op, T *partial) {
       slots[tid] = op(slots[tid], slots[tid + s]);
     __syncthreads();
   }
-  if (tid == 0)
-    partial[blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)] = slots[0];
+  return slots[0];
+}
+
+// A launch's reduction variables finish on the device (the reference stores
+// per-workgroup partial results to host-shared memory and adds them in a host
+// loop, mlir/lib/Conversion/GpuToGpuRuntime.cpp:2161-2277).  Every block
+// leaves its partial result at partial[block index] with a store that is
+// visible device-wide once acknowledged; the block that draws the last ticket
+// reads all of them back past its own caches, folds them -- a fixed tree over
+// the block index, so repeated launches give the same bits -- and leaves the
+// total at partial[number of blocks].  No value is accumulated with an
+// atomic: the ticket only orders the blocks.
+__device__ __forceinline__ int64_t blockCount() {
+  return int64_t(gridDim.x) * gridDim.y * gridDim.z;
+}
+
+template <typename T, typename Op>
+__device__ __forceinline__ void blockReduceStore(T v, Op op, T *partial) {
+  const T total = blockReduce(v, op);
+  if (linearLocalId() == 0)
+    __hip_atomic_store(
+        partial + (blockIdx.x + gridDim.x * (blockIdx.y + int64_t(gridDim.y) * blockIdx.z)),
+        total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// After the blockReduceStore calls of a kernel: true in every lane of the
+// block that arrived last (all partial results are then visible to it).
+// Device-wide atomics on one 256-byte line of memory are served one after
+// the other, about 7 ns each, and the blocks of a streaming kernel all end
+// together: 2048 tickets from one counter, or from sixteen counters next to
+// each other, add 16 us to a launch of 79 us.  So the tickets are drawn in
+// two steps from counters 256 bytes apart: a block draws from one of
+// kTicketGroups counters (its index modulo their number), and only the last
+// of each group draws from the counter behind them (with that, 2 us).
+// `ticket`: (kTicketGroups + 1) * kTicketStride counters, zero between
+// launches (the block that empties a counter puts it back).
+constexpr int kTicketGroups = 16;
+constexpr int kTicketStride = 64; // counters 256 bytes apart
+
+__device__ __forceinline__ bool drewLastTicket(uint32_t *ticket) {
+  __shared__ uint32_t last;
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+  __builtin_amdgcn_s_waitcnt(0); // the partial results are acknowledged
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+  __syncthreads();
+  if (linearLocalId() == 0) {
+    const int64_t blocks = blockCount();
+    const int64_t me = blockIdx.x + gridDim.x * (blockIdx.y + int64_t(gridDim.y) * blockIdx.z);
+    const int64_t group = me % kTicketGroups;
+    const int64_t inGroup = (blocks - group + kTicketGroups - 1) / kTicketGroups;
+    const int64_t groups = blocks < kTicketGroups ? blocks : kTicketGroups;
+    uint32_t mine = __hip_atomic_fetch_add(ticket + group * kTicketStride, 1u, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+    last = 0u;
+    if (mine == uint32_t(inGroup - 1)) {
+      __hip_atomic_store(ticket + group * kTicketStride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      mine = __hip_atomic_fetch_add(ticket + kTicketGroups * kTicketStride, 1u, __ATOMIC_RELAXED,
+                                    __HIP_MEMORY_SCOPE_AGENT);
+      if (mine == uint32_t(groups - 1)) {
+        __hip_atomic_store(ticket + kTicketGroups * kTicketStride, 0u, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        last = 1u;
+      }
+    }
+  }
+  __syncthreads();
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+  return last != 0;
+}
+
+// In the last block: partial[number of blocks] = fold of partial[0 ..).
+template <typename T, typename Op>
+__device__ __forceinline__ void foldPartials(T *partial, Op op, T neutral) {
+  const int64_t blocks = blockCount();
+  const int64_t n = localCount();
+  T acc = neutral;
+  // (eight loads in flight a lane: each comes from beyond the caches)
+  for (int64_t base = linearLocalId(); base < blocks; base += 8 * n) {
+    T v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int64_t i = base + u * n;
+      v[u] = i < blocks ? __hip_atomic_load(partial + i, __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT)
+                        : neutral;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      acc = op(acc, v[u]);
+  }
+  const T total = blockReduce(acc, op);
+  if (linearLocalId() == 0)
+    partial[blocks] = total;
 }
 
 // A store of a value that no work-item of the launch reads back.  `unit`:

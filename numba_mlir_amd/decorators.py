@@ -561,10 +561,15 @@ class Dispatcher:
         read_back = None
 
         def make_partials(blocks):
+            # (a slot per block and one for the total, which the launch's last
+            # block leaves there)
             for _, dtype, _ in compiled.reductions:
-                partials.append(HipNdArray.empty((max(blocks, 1),), dtype,
+                partials.append(HipNdArray.empty((max(blocks, 1) + 1,), dtype,
                                                  device=ctx.device))
             return partials
+
+        def totals(arrays):
+            return [part[part.shape[0] - 1:].asnumpy()[0] for part in arrays]
 
         if count == 0 and compiled.reductions:
             info = {"kernel": compiled.name, "grid": (0, 0, 0), "block": (0, 0, 0)}
@@ -575,7 +580,7 @@ class Dispatcher:
                     ctx, compiled, self.py_func.__name__, counts, args,
                     make_partials=make_partials if compiled.reductions else None)
                 plan.run()
-                read_back = [part.asnumpy() for part in partials]   # (before others see the plan)
+                read_back = totals(partials)         # (before others see the plan)
                 if len(entry["plans"]) >= MAX_PLANS:
                     entry["plans"].clear()
                 entry["plans"][(compiled.name, counts)] = plan
@@ -585,7 +590,7 @@ class Dispatcher:
                 try:
                     partials = plan.partials
                     plan.run(args, partials=partials)
-                    read_back = [part.asnumpy() for part in partials]
+                    read_back = totals(partials)
                 finally:
                     plan.partials_free.release()
             else:
@@ -595,14 +600,14 @@ class Dispatcher:
             info = plan.info
             self.last_plan = plan
         self.last_launch = dict(info, path="parallel loop")
-        # fold the per-block partial results, in block order, onto the values
-        # the reduction variables had before the loop
+        # the totals of the reduction variables (added up by the launch's last
+        # block) onto the values the variables had before the loop
         if read_back is None:
-            read_back = [part.asnumpy() for part in partials]
-        for (name, dtype, op), blocks in zip(compiled.reductions, read_back):
+            read_back = totals(partials)
+        for (name, dtype, op), fold in zip(compiled.reductions, read_back):
             start = np.dtype(dtype).type(scope[name])
             with np.errstate(over="ignore"):
-                fold = blocks.sum(dtype=dtype) if op == "add" else blocks.prod(dtype=dtype)
+                fold = np.dtype(dtype).type(fold)
                 scope[name] = start + fold if op == "add" else start * fold
         return_code = self._host_code(compiled)[2]
         if return_code is not None:

@@ -2080,6 +2080,9 @@ class FunctionTranslator:
             neutral = "0" if self.reductions[name] == "add" else "1"
             red.append((name, t, neutral))
             params.append(f"{t.ctype} *nmk_part_{name}")
+        if red:
+            # (zeroed counters, one set per launch plan: which block finishes)
+            params.append("uint32_t *nmk_ticket")
         self.reduction_types = [(n, t) for n, t, _ in red]
         params += [f"uint64_t nmk_lds{k}" for k in range(len(self.local_arrays))]
         params += ["int64_t nmk_gsz0", "int64_t nmk_gsz1", "int64_t nmk_gsz2"]
@@ -2261,6 +2264,15 @@ class FunctionTranslator:
             op = "AddOp" if self.reductions[name] == "add" else "MulOp"
             out.append(f"  nmkjit::blockReduceStore<{t.ctype}>({self.cname(name)}, "
                        f"nmkjit::{op}(), nmk_part_{name});")
+        if red:
+            # the block that arrives last adds up the blocks' results: each
+            # array of partial results has one more element, for the total
+            out.append("  if (nmkjit::drewLastTicket(nmk_ticket)) {")
+            for name, t, neutral in red:
+                op = "AddOp" if self.reductions[name] == "add" else "MulOp"
+                out.append(f"    nmkjit::foldPartials<{t.ctype}>(nmk_part_{name}, nmkjit::{op}(), "
+                           f"({t.ctype}){neutral});")
+            out.append("  }")
         out.append("}")
         return "\n".join(out)
 

@@ -223,6 +223,7 @@ class _ParamList:
 NO_DEPS = (ctypes.c_void_p * 1)(None)
 MAX_SPECIALISATIONS = 16   # per kernel, before new shapes get the general form
 MAX_PLANS = 64             # stored launches per kernel
+TICKET_COUNTERS = 17 * 64  # of a generated reduction (jit_support.h: kTicketGroups + 1 counters, kTicketStride apart)
 REDUCTION_BLOCKS = 2048    # of a generated 1-d reduction: eight per compute unit
 
 
@@ -462,6 +463,13 @@ class LaunchPlan:
         self.partials_free = threading.Lock()   # held from a launch into them to their read-back
         self._partial_slots = [params._add(ctypes.c_void_p(part.ptr), lowered.PARAM_PTR)
                                for part in partials]
+        # the counters by which the launch's last block knows itself (zero
+        # between launches: the kernel puts them back)
+        self._ticket = None
+        if self.partials:
+            self._ticket = HipNdArray.from_numpy(np.zeros(TICKET_COUNTERS, np.uint32),
+                                                 device=ctx.device)
+            params._add(ctypes.c_void_p(self._ticket.ptr), lowered.PARAM_PTR)
         for nbytes in compiled.local_bytes:
             params.add_local(int(nbytes))
         for g in gsize3:

@@ -453,6 +453,10 @@ def test_prange_reductions(K, tmp_path, monkeypatch):
     assert ck.return_source == "(total / n, above)"
     assert "int64_t *nmk_part_above, double *nmk_part_total" in ck.source
     assert ck.source.count("nmkjit::blockReduceStore<") == 2
+    # the launch's last block adds the blocks' results up: nothing is summed on the host
+    assert "uint32_t *nmk_ticket" in ck.source
+    assert "if (nmkjit::drewLastTicket(nmk_ticket)) {" in ck.source
+    assert ck.source.count("nmkjit::foldPartials<") == 2
     # dense float32 operands read at the loop's own index: a 128-bit word of
     # four adjacent iterations a lane, the sums kept where they are (one
     # inlined form of the body, closures by reference)
