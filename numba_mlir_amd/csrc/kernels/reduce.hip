@@ -125,6 +125,13 @@ NMK_DEFINE_ROWSUM(nmk_norm2_axis1_wide_f32, true, 4)
 #define NMK_AX0_UNROLL 16 // row loads in flight per lane
 #endif
 
+// The counter of a strip: those of neighbouring strips, whose blocks end
+// together, lie 256 bytes apart (device-wide atomics on one such line are
+// served one after the other).  strip < 4096.
+__device__ __forceinline__ uint32_t *stripTicket(uint32_t *tickets, int64_t strip) {
+  return tickets + (strip % 64) * 64 + strip / 64;
+}
+
 NMK_KERNEL(256)
 nmk_sum_axis0_i32_i64(const int32_t *__restrict__ x, int64_t *__restrict__ out,
                       int64_t rows, int64_t cols, int64_t ld,
@@ -181,7 +188,7 @@ nmk_sum_axis0_i32_i64(const int32_t *__restrict__ x, int64_t *__restrict__ out,
   awaitStores();
   __syncthreads();
   if (threadIdx.x == 0)
-    isLast = drawLastTicket(&tickets[strip], gridDim.y) ? 1u : 0u;
+    isLast = drawLastTicket(stripTicket(tickets, strip), gridDim.y) ? 1u : 0u;
   __syncthreads();
   if (!isLast)
     return;
@@ -204,7 +211,7 @@ nmk_sum_axis0_i32_i64(const int32_t *__restrict__ x, int64_t *__restrict__ out,
     out[myCol] = s;
   }
   if (threadIdx.x == 0)
-    publish(&tickets[strip], 0u);
+    publish(stripTicket(tickets, strip), 0u);
 }
 
 // ---------------------------------------------------------------------------
@@ -271,7 +278,7 @@ fullSumF32(const float *__restrict__ x, float *__restrict__ out, int64_t n,
   if (threadIdx.x == 0) {
     publish(partial + blockIdx.x, total);
     awaitStores();
-    isLast = drawLastTicket(ticket, gridDim.x) ? 1u : 0u;
+    isLast = drawLastTicketSpread(ticket, gridDim.x, blockIdx.x) ? 1u : 0u;
   }
   __syncthreads();
   if (!isLast)
@@ -280,10 +287,8 @@ fullSumF32(const float *__restrict__ x, float *__restrict__ out, int64_t n,
   for (int64_t b = threadIdx.x; b < int64_t(gridDim.x); b += blockDim.x)
     s += collect(partial + b);
   s = blockAllReduce<256>(s, AddOp(), slots);
-  if (threadIdx.x == 0) {
+  if (threadIdx.x == 0)
     out[0] = SQUARE_ROOT_OF_SQUARES ? sqrtf(s) : s;
-    publish(ticket, 0u);
-  }
 }
 
 NMK_KERNEL(256)
