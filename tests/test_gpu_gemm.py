@@ -284,6 +284,29 @@ def test_beta_zero_ignores_c(env):
     assert (c.asnumpy() == 16).all()
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_empty_extents(env, dtype):
+    """No rows or no columns: nothing to write.  No inner dimension: the
+    product is zero, so C becomes beta * C (and plain zeros for beta == 0,
+    whatever C held)."""
+    hip, ops, _, mrt = env
+    for m, n in ((0, 5), (5, 0), (0, 0)):
+        c = hip.asarray(np.zeros((m, n), dtype))
+        ops.gemm(hip.asarray(np.ones((m, 7), dtype)), hip.asarray(np.ones((7, n), dtype)),
+                 c, 1.0, 0.0)
+        assert c.asnumpy().shape == (m, n)
+    for m, n in ((5, 9), (130, 257)):
+        c0 = np.arange(m * n, dtype=dtype).reshape(m, n)
+        c = hip.asarray(c0)
+        ops.gemm(hip.asarray(np.ones((m, 0), dtype)), hip.asarray(np.ones((0, n), dtype)),
+                 c, 1.0, 2.0)
+        assert np.array_equal(c.asnumpy(), 2 * c0)
+        c = hip.asarray(np.full((m, n), np.nan, dtype))
+        ops.gemm(hip.asarray(np.ones((m, 0), dtype)), hip.asarray(np.ones((0, n), dtype)),
+                 c, 1.0, 0.0)
+        assert np.array_equal(c.asnumpy(), np.zeros((m, n), dtype))
+
+
 def test_identity_and_linearity_full_size(env):
     """Configuration 5 (4096^3): rows checked against float64, plus
     size-independent properties: A @ I == A exactly, and linearity."""
