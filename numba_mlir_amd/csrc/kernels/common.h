@@ -107,6 +107,14 @@ __device__ __forceinline__ T blockAllReduce(T v, Op op, T *slots) {
   return total;
 }
 
+// Index of the block in a launch whose blocks are counted along x, then y:
+// a launch may run at most 2^32 - 1 work-items along a dimension (the
+// dispatch packet counts them in 32 bits), so a kernel with a block per row
+// of a very tall matrix gets its blocks in an x-by-y grid.
+__device__ __forceinline__ int64_t blockLinearXY() {
+  return int64_t(blockIdx.x) + int64_t(gridDim.x) * blockIdx.y;
+}
+
 // ---------------------------------------------------------------------------
 // Hand-off of per-block partial results to the last block of a launch.
 //

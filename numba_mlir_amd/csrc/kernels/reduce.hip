@@ -40,7 +40,7 @@ rowSumF32(const float *__restrict__ x, float *__restrict__ out, int64_t rows,
   const int lane = threadIdx.x % NMK_WAVE;
   const int wave = threadIdx.x / NMK_WAVE;
   const int sub = wave % WPR; // this wave's share of the row
-  const int64_t row = int64_t(blockIdx.x) * (4 / WPR) + wave / WPR;
+  const int64_t row = blockLinearXY() * (4 / WPR) + wave / WPR;
   constexpr int STEP = NMK_WAVE * WPR;
   float total = 0.f;
   if (row < rows) {
@@ -384,7 +384,9 @@ reduceStrided(const IN *x, ACC *out, int64_t nKeep, int64_t nRed, int64_t sk,
   __shared__ ACC slots[256 / NMK_WAVE];
   const bool vec = mode & 1;
   if (mode & 2) {
-    const int64_t k = blockIdx.x;
+    const int64_t k = blockLinearXY();
+    if (k >= nKeep)
+      return;
     const IN *p = x + k * sk;
     ACC acc = vec ? foldWords<256, IN, ACC>(p, nRed, threadIdx.x, init, op)
                   : foldElements<256, IN, ACC>(p, nRed, sr, threadIdx.x, init, op);
@@ -395,7 +397,7 @@ reduceStrided(const IN *x, ACC *out, int64_t nKeep, int64_t nRed, int64_t sk,
   }
   const int lane = threadIdx.x % NMK_WAVE;
   const int64_t k =
-      int64_t(blockIdx.x) * (blockDim.x / NMK_WAVE) + threadIdx.x / NMK_WAVE;
+      blockLinearXY() * (blockDim.x / NMK_WAVE) + threadIdx.x / NMK_WAVE;
   if (k >= nKeep)
     return;
   const IN *p = x + k * sk;

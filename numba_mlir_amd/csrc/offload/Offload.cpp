@@ -278,6 +278,19 @@ public:
     launchDesc(name, grid, block, descs.data());
   }
 
+  // A launch of `blocks` blocks of 256 lanes whose kernel counts its blocks
+  // along x, then y (blockLinearXY): a dimension of a launch holds at most
+  // 2^32 - 1 work-items, 2^24 - 1 such blocks.
+  void launchBlocksXY(const std::string &name, int64_t blocks,
+                      std::initializer_list<Arg> args) {
+    const int64_t most = int64_t(1) << 23;
+    const int64_t gx = blocks < most ? blocks : most;
+    const int64_t gy = ceilDiv(blocks, gx);
+    if (gy > 65535)
+      fail("%s: %lld blocks are more than one launch holds", name.c_str(), (long long)blocks);
+    launch(name, size_t(gx), size_t(gy), 1, 256, 1, 1, args);
+  }
+
   void synchronize() {
     if (lastEvent) {
       retireEvent(lastEvent, true);
@@ -711,11 +724,11 @@ NMHIP_EXPORT void nmhipReduce(void *ctx, int op, int dtype, const void *x,
         n0 > 0 && n1 > 0) {
       const int vec = (aligned16(x) && s0 % 4 == 0 && n1 % 4 == 0) ? 1 : 0;
       // a block per row for long rows, a wave per row otherwise
-      const bool wide = n1 >= 4096 && n0 <= 0x7fffffff;
-      c->launch(wide ? "nmk_sum_axis1_wide_f32" : "nmk_sum_axis1_f32",
-                size_t(wide ? n0 : ceilDiv(n0, 4)), 1, 1, 256, 1, 1,
-                {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(n0), Arg::I64(n1),
-                 Arg::I64(s0), Arg::I32(vec)});
+      const bool wide = n1 >= 4096;
+      c->launchBlocksXY(wide ? "nmk_sum_axis1_wide_f32" : "nmk_sum_axis1_f32",
+                        wide ? n0 : ceilDiv(n0, 4),
+                        {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(n0), Arg::I64(n1),
+                         Arg::I64(s0), Arg::I32(vec)});
       return;
     }
     // int32 column sums into int64: column strips x row chunks, device finish.
@@ -849,10 +862,10 @@ NMHIP_EXPORT void nmhipReduce(void *ctx, int op, int dtype, const void *x,
     const bool wide = nRed >= 4096;
     const int mode = ((sr == 1 && aligned16(x) && (nKeep == 1 || sk % word == 0)) ? 1 : 0) |
                      (wide ? 2 : 0);
-    c->launch(std::string("nmk_reduce_") + opNames[op] + "_" + dtypeName(dtype),
-              size_t(wide ? nKeep : ceilDiv(nKeep, 4)), 1, 1, 256, 1, 1,
-              {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(nKeep), Arg::I64(nRed),
-               Arg::I64(sk), Arg::I64(sr), Arg::I64(1), Arg::I32(mode)});
+    c->launchBlocksXY(std::string("nmk_reduce_") + opNames[op] + "_" + dtypeName(dtype),
+                      wide ? nKeep : ceilDiv(nKeep, 4),
+                      {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(nKeep), Arg::I64(nRed),
+                       Arg::I64(sk), Arg::I64(sr), Arg::I64(1), Arg::I32(mode)});
   });
 }
 
@@ -866,11 +879,11 @@ NMHIP_EXPORT void nmhipNorm2RowsF32(void *ctx, const float *x, int64_t n0,
     if (n0 == 0)
       return;
     const int vec = (aligned16(x) && s0 % 4 == 0 && n1 % 4 == 0) ? 1 : 0;
-    const bool wide = n1 >= 4096 && n0 <= 0x7fffffff;
-    c->launch(wide ? "nmk_norm2_axis1_wide_f32" : "nmk_norm2_axis1_f32",
-              size_t(wide ? n0 : ceilDiv(n0, 4)), 1, 1, 256, 1, 1,
-              {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(n0), Arg::I64(n1),
-               Arg::I64(s0), Arg::I32(vec)});
+    const bool wide = n1 >= 4096;
+    c->launchBlocksXY(wide ? "nmk_norm2_axis1_wide_f32" : "nmk_norm2_axis1_f32",
+                      wide ? n0 : ceilDiv(n0, 4),
+                      {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(n0), Arg::I64(n1),
+                       Arg::I64(s0), Arg::I32(vec)});
   });
 }
 

@@ -485,6 +485,13 @@ public:
       if (blockX * blockY * blockZ > 1024)
         fail("Launch block (%zu, %zu, %zu) exceeds 1024 threads", blockX,
              blockY, blockZ);
+      // The dispatch packet counts the work-items of a dimension in 32 bits;
+      // a larger product would wrap without an error from the launch call.
+      if (gridX * blockX > 0xffffffffull || gridY * blockY > 0xffffffffull ||
+          gridZ * blockZ > 0xffffffffull)
+        fail("Launch of (%zu, %zu, %zu) blocks of (%zu, %zu, %zu) exceeds "
+             "4294967295 work-items along a dimension",
+             gridX, gridY, gridZ, blockX, blockY, blockZ);
       if (ldsBytes > 160 * 1024)
         fail("Launch needs %zu bytes of workgroup memory; gfx950 has 163840",
              ldsBytes);

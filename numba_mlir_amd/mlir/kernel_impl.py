@@ -446,6 +446,12 @@ class LaunchPlan:
                  ret=None, partials=()):
         self.ctx, self.compiled, self.kern, self.func_name = ctx, compiled, kern, func_name
         self.grid, self.block = tuple(grid), tuple(block)
+        for g, b in zip(self.grid, self.block):
+            if g * b > 2 ** 32 - 1:
+                # (the runtime would abort the process: say it here instead)
+                raise ValueError(
+                    f"kernel '{func_name}': {g} blocks of {b} work-items are more than the "
+                    "4294967295 work-items a launch holds along one dimension")
         self.info = {"kernel": compiled.name, "grid": self.grid, "block": self.block}
         self.empty = 0 in gsize3
         params = _ParamList()
@@ -615,6 +621,10 @@ def plan_compiled(ctx, compiled, func_name, global_size, args, ret=None,
     per_lane = getattr(compiled, "elements_per_thread", 1)
     lanes = [-(-int(global_size[0]) // per_lane)] + [int(g) for g in global_size[1:]]
     block, grid = _geometry(ctx, compiled, kern, lanes, ())
+    if getattr(compiled, "grid_stride", False):
+        # (a launch counts the work-items of a dimension in 32 bits; the
+        # kernel strides over the rest)
+        grid[0] = min(grid[0], (2 ** 32 - 1) // max(block[0], 1))
     if make_partials and getattr(compiled, "grid_stride", False):
         # a reduction: few, long-running blocks (one partial result each); the
         # more arrays they stream at once, the fewer (two arrays of 512 MiB:

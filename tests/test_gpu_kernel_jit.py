@@ -783,6 +783,9 @@ def test_large_1d_launch_ids_do_not_wrap(env):               # 2268-2283
     b = 2 ** 31 + 10
     K.kernel(func)[2 ** 31 + 11, 1024](arr, b)
     assert arr.asnumpy()[0] == np.float32(b)
+    # a dimension of a launch holds 2^32 - 1 work-items: more is an error, not a wrap
+    with pytest.raises(ValueError, match="4294967295 work-items"):
+        K.kernel(func)[2 ** 32 + 5, 1024](arr, b)
 
 
 def _all_kinds_f32(rng, n):

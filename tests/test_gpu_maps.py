@@ -318,3 +318,37 @@ def test_black_scholes_full_size(env):
     np.testing.assert_allclose(call, tc, rtol=5e-5, atol=1e-12)
     np.testing.assert_allclose(put, tp, rtol=5e-5, atol=1e-12)
     assert (call >= 0).all() and (put >= -1e-6).all()   # r - P + Se cancels
+
+
+def test_more_than_two_to_the_31_elements(env):
+    """Element counts and byte offsets past 2^31 (8 GiB of int32 an array): the
+    map and the reductions index in 64 bits.  Checked on the device: the ends
+    of the result, and its sums."""
+    hip, ops, _ = env
+    n = 2 ** 31 + 8
+    host = np.ones(n, np.int32)
+    host[-8:] = 7
+    a = hip.asarray(host)
+    del host
+    out = ops.add(a, a)
+    assert out.shape == (n,)
+    assert out[:8].asnumpy().tolist() == [2] * 8
+    assert out[n - 16:].asnumpy().tolist() == [2] * 8 + [14] * 8
+    # (a full reduction accumulates in int64 and is cast back to the array's
+    # type, numpy/funcs.py:183-185: the total modulo 2^32)
+    total = ops.sum(out)
+    assert total.dtype == np.int32
+    assert int(total) == int(np.int64(2 * (n - 8) + 14 * 8).astype(np.int32)) == 112
+    assert int(ops.amax(out)) == 14 and int(ops.amin(out)) == 2
+    wide = out.reshape((n // 8, 8))
+    assert ops.sum(wide, axis=0).asnumpy().tolist() == [2 * (n // 8 - 1) + 14] * 8
+    # (268 million rows of eight: more blocks than one dimension of a launch holds)
+    rows = ops.sum(wide, axis=1)
+    assert rows.shape == (n // 8,) and int(ops.amax(rows)) == 112 and int(ops.amin(rows)) == 16
+    assert rows[n // 8 - 2:].asnumpy().tolist() == [16, 112]
+    del rows, wide, out, a
+    tall = hip.asarray(np.ones((2 ** 27 + 3, 8), np.float32))
+    sums = ops.sum(tall, axis=1)
+    assert float(ops.amin(sums)) == 8.0 and float(ops.amax(sums)) == 8.0
+    norms = ops.l2_norm_rows(tall)
+    assert abs(float(ops.amin(norms)) - 8 ** 0.5) < 1e-6 and abs(float(ops.amax(norms)) - 8 ** 0.5) < 1e-6

@@ -495,6 +495,11 @@ FATAL = {
          "k = rt.gpuxKernelGet(m, b'k'); d, keep = make_params([]);"
          "rt.gpuxLaunchKernel(q, k, 1, 70000, 1, 1, 1, 1, NO_DEPS, d)",
          "exceeds the HIP limits"),
+    "more work-items along x than a launch counts":
+        ("q = rt.gpuxQueueCreate(None); m = rt.gpuxModuleLoad(q, ELF, len(ELF));"
+         "k = rt.gpuxKernelGet(m, b'k'); d, keep = make_params([]);"
+         "rt.gpuxLaunchKernel(q, k, 67108865, 1, 1, 256, 1, 1, NO_DEPS, d)",
+         "exceeds 4294967295 work-items along a dimension"),
     "foreign pointer":
         ("q = rt.gpuxQueueCreate(None); rt.gpuxDeAlloc(q, 0x40)",
          "was not allocated by gpuxAlloc"),
