@@ -531,8 +531,14 @@ gemm_generic(const T *A, const T *B, T *C, int64_t M, int64_t N, int64_t K,
   __shared__ T Bs[TILE][TILE + 1];
   const int tx = threadIdx.x % TILE; // column within the tile
   const int ty = threadIdx.x / TILE; // 0..7, rows ty, ty+8, ty+16, ty+24
-  const int64_t row0 = int64_t(blockIdx.y) * TILE;
-  const int64_t col = int64_t(blockIdx.x) * TILE + tx;
+  // The tiles in row-major order, counted along the grid's x, then y (a tall
+  // matrix has more tile rows than grid.y holds).
+  const int64_t tilesN = (N + TILE - 1) / TILE;
+  const int64_t tile = int64_t(blockIdx.x) + int64_t(gridDim.x) * blockIdx.y;
+  if (tile >= tilesN * ((M + TILE - 1) / TILE))
+    return;
+  const int64_t row0 = tile / tilesN * TILE;
+  const int64_t col = tile % tilesN * TILE + tx;
   T acc[4] = {T(0), T(0), T(0), T(0)};
   for (int64_t k0 = 0; k0 < K; k0 += TILE) {
 #pragma unroll
@@ -774,6 +780,20 @@ void requireUnitStride(const typename MemrefOf<T>::type *arr, char name) {
 
 bool aligned16(const void *p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+// Grid of gemm_generic for an m x n result: its 32 x 32 tiles along x, then y
+// (a dimension of a launch holds 2^32 - 1 work-items, 2^24 - 1 blocks of 256).
+dim3 genericGrid(int64_t m, int64_t n) {
+  const int64_t tiles = ((m + 31) / 32) * ((n + 31) / 32);
+  const int64_t most = int64_t(1) << 23;
+  const int64_t gx = tiles < most ? tiles : most;
+  const int64_t gy = (tiles + gx - 1) / gx;
+  if (gy > 65535)
+    fatal("mkl_gemm_device: a %lld x %lld result is more than one launch of the "
+          "strided kernel holds\n",
+          (long long)m, (long long)n);
+  return dim3(unsigned(gx), unsigned(gy), 1);
 }
 
 // Returns 0, or (WORKSPACE_FIXED only) 1 when the product would need more
@@ -1264,7 +1284,7 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
                         int64_t k, T bz) {
           if (m <= 0 || n <= 0)
             return;
-          dim3 g{unsigned((n + 31) / 32), unsigned((m + 31) / 32), 1};
+          const dim3 g = genericGrid(m, n);
           hipLaunchKernelGGL(gemm_generic<T>, g, dim3(256), 0, stream,
                              X + m0 * xm + k0 * xk, Y + k0 * yk + n0 * yn,
                              cData + m0 * ldz + n0, m, n, k, xm, xk, yk, yn, ldz,
@@ -1278,12 +1298,7 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       }
     }
     if (!launched) {
-      const int64_t gx = (N + 31) / 32, gy = (M + 31) / 32;
-      if (gy > 65535)
-        fatal("mkl_gemm_device: M = %lld is too large for the strided "
-              "kernel\n",
-              (long long)M);
-      dim3 grid{unsigned(gx), unsigned(gy), 1};
+      const dim3 grid = genericGrid(M, N);
       hipLaunchKernelGGL(gemm_generic<T>, grid, dim3(256), 0, stream, aData,
                          bData, cData, M, N, K, int64_t(a->strides[0]),
                          int64_t(a->strides[1]), int64_t(b->strides[0]),

@@ -307,6 +307,27 @@ def test_empty_extents(env, dtype):
         assert np.array_equal(c.asnumpy(), np.zeros((m, n), dtype))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_tall_and_skinny(env, dtype):
+    """2.2 million rows times an 8 x 8 matrix, and 9 million rows times a
+    40 x 130 one: more rows of tiles than a launch has along y."""
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(17)
+    for m, k, n in ((2_200_000, 8, 8), (9_000_000, 40, 130) if dtype is np.float32
+                    else (4_500_000, 40, 130)):
+        a = rng.standard_normal((m, k)).astype(dtype)
+        b = rng.standard_normal((k, n)).astype(dtype)
+        c = hip.asarray(np.full((m, n), np.nan, dtype))
+        ops.gemm(hip.asarray(a), hip.asarray(b), c, 1.0, 0.0)
+        got = c.asnumpy()
+        for rows in (slice(0, 4096), slice(m // 2, m // 2 + 4096), slice(m - 4096, m)):
+            truth = a[rows].astype(np.float64) @ b.astype(np.float64)
+            scale = np.abs(a[rows]).astype(np.float64) @ np.abs(b).astype(np.float64)
+            assert (np.abs(got[rows] - truth) <= (1e-5 if dtype is np.float32 else 1e-13)
+                    * scale).all(), (m, k, n, mrt.last_kernel())
+        assert np.isfinite(got).all()
+
+
 def test_identity_and_linearity_full_size(env):
     """Configuration 5 (4096^3): rows checked against float64, plus
     size-independent properties: A @ I == A exactly, and linearity."""
