@@ -134,7 +134,10 @@ mapStrided2(const T *a, int64_t sa0, int64_t sa1, const T *b, int64_t sb0,
             int64_t sb1, T *out, int64_t so0, int64_t so1, int64_t n0,
             int64_t n1) {
   const int64_t j = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-  const int64_t i = int64_t(blockIdx.y) * blockDim.y + threadIdx.y;
+  // (a launch has 65535 blocks along y: the rows of a taller array go on
+  // along z)
+  const int64_t i =
+      (int64_t(blockIdx.y) + int64_t(gridDim.y) * blockIdx.z) * blockDim.y + threadIdx.y;
   if (i >= n0 || j >= n1)
     return;
   out[i * so0 + j * so1] =

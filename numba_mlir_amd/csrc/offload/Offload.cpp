@@ -660,8 +660,15 @@ NMHIP_EXPORT void nmhipMapBinary(void *ctx, int op, int dtype, const void *a,
     uint32_t block[2] = {1, 1};
     SYM(SuggestBlockSize, "gpuxSuggestBlockSize")(c->queue, c->kernel(name),
                                                   global, block, 2);
-    c->launch(name, size_t(ceilDiv(n1, block[0])), size_t(ceilDiv(n0, block[1])),
-              1, block[0], block[1], 1,
+    int64_t gy = ceilDiv(n0, block[1]), gz = 1;
+    if (gy > 65535) {
+      gz = ceilDiv(gy, 65535);
+      gy = 65535;
+      if (gz > 65535)
+        fail("nmhipMapBinary: %lld rows are more than one launch holds", (long long)n0);
+    }
+    c->launch(name, size_t(ceilDiv(n1, block[0])), size_t(gy), size_t(gz), block[0],
+              block[1], 1,
               {Arg::Ptr(a), Arg::I64(aS[0]), Arg::I64(aS[1]), Arg::Ptr(b),
                Arg::I64(bS[0]), Arg::I64(bS[1]), Arg::Ptr(out), Arg::I64(oS[0]),
                Arg::I64(oS[1]), Arg::I64(n0), Arg::I64(n1)});

@@ -352,3 +352,14 @@ def test_more_than_two_to_the_31_elements(env):
     assert float(ops.amin(sums)) == 8.0 and float(ops.amax(sums)) == 8.0
     norms = ops.l2_norm_rows(tall)
     assert abs(float(ops.amin(norms)) - 8 ** 0.5) < 1e-6 and abs(float(ops.amax(norms)) - 8 ** 0.5) < 1e-6
+
+
+def test_tall_strided_operands(env):
+    """Views of ten million rows (two of three columns): more blocks of rows
+    than a launch has along y."""
+    hip, ops, _ = env
+    rng = np.random.default_rng(23)
+    a = rng.standard_normal((10_000_000, 3)).astype(np.float32)
+    b = rng.standard_normal((10_000_000, 3)).astype(np.float32)
+    got = ops.add(hip.asarray(a)[:, :2], hip.asarray(b)[:, :2]).asnumpy()
+    assert np.array_equal(got, a[:, :2] + b[:, :2])
