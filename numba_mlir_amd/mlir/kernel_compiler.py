@@ -2124,7 +2124,13 @@ class FunctionTranslator:
             "  const int64_t " + ", ".join(
                 f"nmk_lid{k} = " + ("0" if flat and dim[k] != "x" else f"threadIdx.{dim[k]}")
                 for k in range(3)) + ";",
-            "  const int64_t " + ", ".join(f"nmk_grp{k} = blockIdx.{dim[k]}" for k in range(3)) + ";",
+            # (a launch has 65535 blocks along y and z: a grid of one or two
+            # dimensions with more along y goes on along z)
+            "  const int64_t " + ", ".join(
+                f"nmk_grp{k} = " + (
+                    f"blockIdx.{dim[k]}" if self.ndim == 3 or dim[k] == "x" else
+                    "int64_t(blockIdx.y) + int64_t(gridDim.y) * blockIdx.z" if dim[k] == "y"
+                    else "0") for k in range(3)) + ";",
             "  const int64_t " + ", ".join(
                 f"nmk_lsz{k} = " + ("1" if flat and dim[k] != "x" else f"blockDim.{dim[k]}")
                 for k in range(3)) + ";",

@@ -432,6 +432,10 @@ def _geometry(ctx, compiled, kern, global_size, local_size):
     grid = [(g + b - 1) // b for g, b in zip(sizes, block)]
     if rows > 1:
         grid[1] = (grid[1] + rows - 1) // rows
+    if ndim <= 2 and grid[1] > 65535:
+        # (the generated kernels count their blocks along y, then z)
+        grid[2] = (grid[1] + 65534) // 65535
+        grid[1] = 65535
     return block, grid
 
 

@@ -788,6 +788,26 @@ def test_large_1d_launch_ids_do_not_wrap(env):               # 2268-2283
         K.kernel(func)[2 ** 32 + 5, 1024](arr, b)
 
 
+def test_more_rows_of_blocks_than_a_launch_has_along_y(env):
+    """A 2-d launch whose second dimension needs more than 65535 blocks: the
+    blocks go on along z."""
+    hip, sim = env
+
+    def func(a, out):
+        i = get_global_id(0)
+        j = get_global_id(1)
+        out[j, i] = a[j, i] * 2.0 + i
+
+    n = 9_000_000
+    a = np.random.default_rng(1).standard_normal((n, 3)).astype(np.float32)
+    d_out = hip.asarray(np.zeros((n, 3), np.float32))
+    K.kernel(func)[(3, n), ()](hip.asarray(a), d_out)
+    assert np.array_equal(d_out.asnumpy(), a * np.float32(2.0) + np.arange(3, dtype=np.float32))
+    d_out = hip.asarray(np.zeros((n, 3), np.float32))
+    K.kernel(func)[(3, n), (1, 64)](hip.asarray(a), d_out)
+    assert np.array_equal(d_out.asnumpy(), a * np.float32(2.0) + np.arange(3, dtype=np.float32))
+
+
 def _all_kinds_f32(rng, n):
     """float32 values of every kind: random bit patterns (all exponents, both
     signs, denormals, NaNs), a band around 1 and the special values."""

@@ -911,3 +911,15 @@ def test_maps_run_inside_axis_reductions(env, shape):
     run(cases.row_dots, ai, bi, fused=rows_fused)
     # a broadcast operand: the map and the reduction run separately
     run(cases.row_dots, a, rng.standard_normal(shape[1]), fused=False)
+
+
+def test_fused_map_over_tall_strided_views(env):
+    """Two of three columns of ten million rows: the fused map's grid has
+    more blocks of rows than a launch holds along y."""
+    hip = env[0] if isinstance(env, tuple) else env
+    rng = np.random.default_rng(29)
+    a = rng.standard_normal((10_000_000, 3))
+    b = rng.standard_normal((10_000_000, 3))
+    f = njit(lambda x, y: x * 2.0 + y)
+    got = f(hip.asarray(a)[:, :2], hip.asarray(b)[:, :2]).asnumpy()
+    assert np.array_equal(got, a[:, :2] * 2.0 + b[:, :2])
