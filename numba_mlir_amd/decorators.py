@@ -28,6 +28,7 @@ import ast
 import functools
 import inspect
 import math
+import re
 
 import numpy as np
 
@@ -428,6 +429,16 @@ class Dispatcher:
                 self._names.update(table)
         return self._names.get(name)
 
+    @property
+    def _stage_stem(self):
+        """The function's name as an identifier (a lambda's is not one): the
+        stem of the names of the kernels generated for its stages."""
+        name = self.py_func.__name__
+        if name.isidentifier():
+            return name
+        name = re.sub(r"\W", "_", name).strip("_") or "function"
+        return name if not name[0].isdigit() else "f" + name
+
     def _callee(self, node):
         """The Python object a call's function expression names: a name, or
         attributes of one (``numba_mlir.prange``), else None."""
@@ -685,7 +696,7 @@ class Dispatcher:
         entry = self._stage_funcs.get(key)
         if entry is None:
             func, params = staging.stage_function(
-                stage, f"{self.py_func.__name__}_stage{k}", scope)
+                stage, f"{self._stage_stem}_stage{k}", scope)
             entry = self._stage_funcs[key] = (
                 Dispatcher(func, boundscheck=self.boundscheck, **self.options), params)
         return entry
@@ -753,7 +764,7 @@ class Dispatcher:
             namespace = dict(scope, _nmk_prange=prange)
             try:
                 func, params = staging.reduction_function(
-                    source, f"{self.py_func.__name__}_stage{k}_sum", namespace, set(arrays),
+                    source, f"{self._stage_stem}_stage{k}_sum", namespace, set(arrays),
                     integer)
                 entry = (Dispatcher(func, parallel=True, boundscheck=self.boundscheck,
                                     **self.options), params)
@@ -811,7 +822,7 @@ class Dispatcher:
                              _nmk_global_id=kernel_impl.get_global_id,
                              _nmk_group=kernel_impl.group)
             make = staging.row_sum_function if along_rows else staging.column_sum_function
-            func, params = make(source, f"{self.py_func.__name__}_stage{k}_axis", namespace,
+            func, params = make(source, f"{self._stage_stem}_stage{k}_axis", namespace,
                                 set(arrays), integer)
             entry = self._stage_funcs[key] = kernel_impl.Kernel(
                 func, dict(boundscheck=self.boundscheck, **self.options))

@@ -77,3 +77,8 @@ def test_sequential_loops_over_an_array_are_refused_not_run_per_element():
             njit(func)._refuse_sequential_array_loops([x])
     njit(_small_inner_loop)._refuse_sequential_array_loops([x, x])
     njit(_by_name)._refuse_sequential_array_loops([x])      # (prange is not range)
+
+
+def test_stage_kernels_of_a_lambda_get_identifier_names():
+    f = njit(lambda a: np.sum(a * a, axis=1))
+    assert f._stage_stem == "lambda" and njit(_by_name)._stage_stem == "_by_name"

@@ -923,3 +923,13 @@ def test_fused_map_over_tall_strided_views(env):
     f = njit(lambda x, y: x * 2.0 + y)
     got = f(hip.asarray(a)[:, :2], hip.asarray(b)[:, :2]).asnumpy()
     assert np.array_equal(got, a[:, :2] * 2.0 + b[:, :2])
+
+
+def test_staged_reductions_of_a_lambda(env):
+    """A lambda's stages get kernels too (its name is no identifier)."""
+    hip = env[0]
+    x = np.random.default_rng(31).uniform(0.5, 1.5, (50_000, 3)).astype(np.float32)
+    got = njit(lambda a: np.sum(a * a, axis=1))(hip.asarray(x)).asnumpy()
+    np.testing.assert_allclose(got, (x.astype(np.float64) ** 2).sum(axis=1), rtol=1e-5)
+    got = njit(lambda a: np.mean(np.abs(a)))(hip.asarray(x))
+    np.testing.assert_allclose(got, np.abs(x).astype(np.float64).mean(), rtol=1e-5)
