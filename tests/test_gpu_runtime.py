@@ -226,3 +226,52 @@ def test_async_mode_keeps_order(hip):
     for _ in range(10):
         expect = expect + b
     assert out.asnumpy().tobytes() == expect.tobytes()
+
+
+@pytest.mark.parametrize("shared_queue", [False, True])
+def test_call_sequence_from_six_threads(rt, shared_queue):
+    """Compiled functions run on whatever Python thread calls them: six
+    threads repeat alloc -> launch -> wait -> read -> dealloc, each on a queue
+    of its own or all on one (ctypes drops the GIL during the calls)."""
+    import threading
+    lib, g, low = rt
+    blob = low.kernel_blob("twins")
+    one = lib.gpuxQueueCreate(None) if shared_queue else None
+    errors = []
+
+    def work(seed):
+        try:
+            q = one if shared_queue else lib.gpuxQueueCreate(None)
+            mod = lib.gpuxModuleLoad(q, blob, len(blob))
+            kern = lib.gpuxKernelGet(mod, b"nmk_twin_get_global_id_2")
+            for it in range(60):
+                r, c = 3 + (seed + it) % 5, 5 + (seed * 7 + it) % 11
+                ptr = _alloc(lib, g, q, r * c * 4, 1)
+                host = _host_view(ptr, r * c, np.int32)
+                host[:] = -1
+                descs, keep = _params(g, [
+                    (ctypes.c_void_p(ptr), 8), (ctypes.c_int64(r), 5), (ctypes.c_int64(c), 5),
+                    (ctypes.c_int64(c), 5), (ctypes.c_int64(1), 5),
+                    (ctypes.c_int64(r), 5), (ctypes.c_int64(c), 5), (ctypes.c_int64(1), 5)])
+                ev = lib.gpuxLaunchKernel(q, kern, 1, 1, 1, r, c, 1, NO_DEPS, descs)
+                lib.gpuxWait(q, ev)
+                lib.gpuxDestroyEvent(q, ev)
+                i, j = np.meshgrid(np.arange(r), np.arange(c), indexing="ij")
+                if not np.array_equal(host.reshape(r, c), i + 100 * j):
+                    errors.append((seed, it, host.copy()))
+                lib.gpuxDeAlloc(q, ptr)
+            lib.gpuxKernelDestroy(kern)
+            lib.gpuxModuleDestroy(mod)
+            if not shared_queue:
+                lib.gpuxQueueDestroy(q)
+        except Exception as exc:      # noqa: BLE001
+            errors.append(exc)
+
+    threads = [threading.Thread(target=work, args=(s,)) for s in range(6)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    if shared_queue:
+        lib.gpuxQueueDestroy(one)
+    assert not errors, errors[:2]
