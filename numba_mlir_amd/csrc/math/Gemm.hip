@@ -573,6 +573,94 @@ gemm_generic(const T *A, const T *B, T *C, int64_t M, int64_t N, int64_t K,
 }
 
 // ---------------------------------------------------------------------------
+// Z[M, N] = alpha X[M, K] Y[K, N] + beta Z for a tall X with few columns and a
+// small Y (K, N <= 32): coordinates times a small matrix.  The work is moving
+// X and Z once; a 128 x 128 tile would spend its time on rows of zeros and on
+// filling and draining its pipeline every four slabs.  A block takes tiles of
+// 128 rows or more in turn: the tile of X goes to LDS with coalesced loads, Y sits in
+// LDS for the whole launch, and every lane computes four adjacent columns of
+// one row at a time (one read of X and one 128-bit read of Y per four
+// multiply-adds).  X has unit stride along k, Z along n; Y any strides.
+template <typename T>
+__global__ __launch_bounds__(256) void
+gemm_skinny(const T *__restrict__ X, int64_t ldx, const T *__restrict__ Y, int64_t yk,
+            int64_t yn, T *__restrict__ Z, int64_t ldz, int64_t M, int N, int K, T alpha,
+            T beta, int wordStores) {
+  constexpr int MAXD = 32, XS_WORDS = 128 * (MAXD + 1);
+  typedef T Four __attribute__((ext_vector_type(4)));
+  __shared__ __attribute__((aligned(32))) T Ys[MAXD][MAXD];
+  // rows of K + 1 words (an odd pitch for K a power of two: lanes on
+  // different rows read different banks); the fewer columns, the more rows
+  // a tile holds, so that a block always has some 16 KiB of X in flight
+  __shared__ T Xs[XS_WORDS];
+  const int pitch = K + 1;
+  const int ROWS = XS_WORDS / pitch;
+  const int tid = threadIdx.x;
+  for (int i = tid; i < MAXD * MAXD; i += 256) {
+    const int k = i / MAXD, n = i % MAXD;
+    Ys[k][n] = (k < K && n < N) ? Y[k * yk + n * yn] : T(0);
+  }
+  // Lanes per row of X and per row of Z: the next powers of two (shifts and
+  // masks instead of divisions by K and N; the lanes beyond idle).
+  int kLanes = 1, kShift = 0;
+  while (kLanes < K)
+    kLanes <<= 1, ++kShift;
+  const int groups = (N + 3) / 4; // of four adjacent columns
+  int gLanes = 1, gShift = 0;
+  while (gLanes < groups)
+    gLanes <<= 1, ++gShift;
+  const int kk = tid & (kLanes - 1), rk = tid >> kShift, rkStep = 256 >> kShift;
+  const int gg = tid & (gLanes - 1), rg = tid >> gShift, rgStep = 256 >> gShift;
+  const int n0 = gg * 4;
+  const int64_t tiles = (M + ROWS - 1) / ROWS;
+  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const int64_t row0 = tile * ROWS;
+    __syncthreads(); // the last tile's rows are used up (and Ys is written)
+    if (kk < K)
+      for (int r = rk; r < ROWS; r += 8 * rkStep) { // eight loads in flight a lane
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int rr = r + u * rkStep;
+          v[u] = rr < ROWS && row0 + rr < M
+                     ? __builtin_nontemporal_load(X + (row0 + rr) * ldx + kk)
+                     : T(0);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int rr = r + u * rkStep;
+          if (rr < ROWS)
+            Xs[rr * pitch + kk] = v[u];
+        }
+      }
+    __syncthreads();
+    if (gg < groups)
+      for (int r = rg; r < ROWS && row0 + r < M; r += rgStep) {
+        Four acc = {T(0), T(0), T(0), T(0)};
+        const T *xr = Xs + r * pitch;
+        for (int k = 0; k < K; ++k)
+          acc += xr[k] * *reinterpret_cast<const Four *>(&Ys[k][n0]);
+        T *dst = Z + (row0 + r) * ldz + n0;
+        if (wordStores) {
+          Four v = alpha * acc;
+          if (beta != T(0))
+            v += beta * *reinterpret_cast<const Four *>(dst);
+          __builtin_nontemporal_store(v, reinterpret_cast<Four *>(dst));
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (n0 + j < N) {
+              T v = alpha * acc[j];
+              if (beta != T(0))
+                v += beta * dst[j];
+              dst[j] = v;
+            }
+        }
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // A copy of an operand that the tile kernels can read in 128-bit words: the
 // R rows of C elements at src (row stride ld, unit stride along a row) go to
 // rows of Cp = C rounded up to whole words, dense, 16-byte aligned, the tail
@@ -958,6 +1046,20 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       const bool xKc = xk == 1, yNc = yn == 1;
       const int64_t ldx = xKc ? xm : xk, ldy = yNc ? yk : yn;
       constexpr int VEC = Mfma<T>::VEC, BK = Mfma<T>::BK;
+      // Tall times small: gemm_skinny.
+      if (xKc && K >= 1 && K <= 32 && Nz <= 32 && Mz >= 4096 && ldx > 0) {
+        const int64_t rows = 128 * 33 / (K + 1); // of a tile (gemm_skinny)
+        const int64_t tiles = (Mz + rows - 1) / rows;
+        const unsigned blocks = unsigned(tiles < 2048 ? tiles : 2048);
+        // (whole rows of four-element words: one store a lane)
+        const int wordStores =
+            Nz % 4 == 0 && ldz % 4 == 0 &&
+            reinterpret_cast<uintptr_t>(cData) % (4 * sizeof(T)) == 0;
+        hipLaunchKernelGGL(gemm_skinny<T>, dim3(blocks), dim3(256), 0, stream, X, ldx, Y, yk,
+                           yn, cData, ldz, Mz, int(Nz), int(K), alpha, beta, wordStores);
+        lastKernel = sizeof(T) == 4 ? "sgemm_skinny" : "dgemm_skinny";
+        launched = true;
+      }
       // The matrix-core kernel takes the part of the problem that is whole
       // tiles, Z[0:Mt, 0:Nt] over k in [0, Kt); the strided kernel adds the
       // rest of K to that block and computes the rows and columns beyond it
@@ -1051,7 +1153,8 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
         const int64_t padTiles = (Mp / PT) * (Np / PT);
         const int slabs = int(Kp / PSLAB);
         int evenBlocks = planEvenShares(padTiles, slabs, padSlots);
-        if (canPack && !fitsAsIs && (!whole || packX || packY) && K >= 256 && padTiles >= minTiles &&
+        if (!launched && canPack && !fitsAsIs && (!whole || packX || packY) && K >= 256 &&
+            padTiles >= minTiles &&
             Mp / PT <= 65535 && Mz <= 0x7fffffff - 256 &&
             Nz <= 0x7fffffff - 256 && K <= 0x7fffffff - 64 &&
             double(Mp) * double(Np) * double(Kp) <= 1.10 * double(Mz) * double(Nz) * double(K)) {
@@ -1112,14 +1215,14 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       // of those that are not, or none of this when there is no room for them)
       size_t packXBytes = 0, packYBytes = 0;
       bool copiesFit = true;
-      if (!paddedBig && (packX || packY)) {
+      if (!launched && !paddedBig && (packX || packY)) {
         auto roundUp = [](int64_t v, int64_t to) { return (v + to - 1) / to * to; };
         packXBytes = packX ? size_t(roundUp(xR * roundUp(xC, VEC) * int64_t(sizeof(T)), 256)) : 0;
         packYBytes = packY ? size_t(roundUp(yR * roundUp(yC, VEC) * int64_t(sizeof(T)), 256)) : 0;
         takeTurn();
         copiesFit = heapWorkspace(device, packXBytes + packYBytes) != nullptr;
       }
-      if (paddedBig) {
+      if (paddedBig || launched) {
         // (done)
       } else if (((!whole && !onlyK) || packX || packY) && copiesFit && unitOk && wordsOk && K > 0 &&
           ldx > 0 && ldy > 0 && M <= 0x7fffffff &&

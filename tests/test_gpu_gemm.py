@@ -328,6 +328,30 @@ def test_tall_and_skinny(env, dtype):
         assert np.isfinite(got).all()
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("m,k,n", [(4096, 1, 1), (5000, 3, 3), (100_003, 8, 8), (70_001, 16, 5),
+                                   (33_333, 32, 32), (65_537, 7, 29)])
+def test_tall_times_small(env, dtype, m, k, n):
+    """Coordinates times a small matrix (K, N <= 32): the streaming kernel.
+    Row-major, a view of wider rows, a transposed small operand, alpha and
+    beta; every element against float64."""
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(m + k + n)
+    wide = rng.standard_normal((m, k + 3)).astype(dtype)
+    b = rng.standard_normal((k, n)).astype(dtype)
+    c0 = rng.standard_normal((m, n + 2)).astype(dtype)
+    tol = 1e-5 if dtype == np.float32 else 1e-13
+    for a_view, b_dev in ((hip.asarray(np.ascontiguousarray(wide[:, :k])), hip.asarray(b)),
+                          (hip.asarray(wide)[:, :k], hip.asarray(np.asfortranarray(b)))):
+        d_c = hip.asarray(c0)[:, :n]
+        ops.gemm(a_view, b_dev, d_c, 1.5, -0.5)
+        assert mrt.last_kernel() == ("sgemm_skinny" if dtype == np.float32 else "dgemm_skinny")
+        _check_scaled(d_c.asnumpy(), wide[:, :k], b, c0[:, :n], 1.5, -0.5, tol)
+        d_c = hip.asarray(np.full((m, n), np.nan, dtype))
+        ops.gemm(a_view, b_dev, d_c, 1.0, 0.0)
+        _check_scaled(d_c.asnumpy(), wide[:, :k], b, np.zeros((m, n), dtype), 1.0, 0.0, tol)
+
+
 def test_identity_and_linearity_full_size(env):
     """Configuration 5 (4096^3): rows checked against float64, plus
     size-independent properties: A @ I == A exactly, and linearity."""
