@@ -661,6 +661,53 @@ gemm_skinny(const T *__restrict__ X, int64_t ldx, const T *__restrict__ Y, int64
 }
 
 // ---------------------------------------------------------------------------
+// The same the other way round: Z[M, N] = alpha X[M, K] Y[K, N] + beta Z for a
+// small X (M, K <= 32) and a long Y with unit stride along n.  A lane owns a
+// column n: it reads Y(k, n) for every k (adjacent lanes adjacent words),
+// keeps the M sums of its column in registers and stores them down the
+// column.  X sits in LDS.  MB: M rounded up to 4, 8, 16 or 32, the
+// accumulators a lane holds.
+template <typename T, int MB>
+__global__ __launch_bounds__(256) void
+gemm_wide(const T *__restrict__ X, int64_t xm, int64_t xk, const T *__restrict__ Y,
+          int64_t ldy, T *__restrict__ Z, int64_t ldz, int M, int64_t N, int K, T alpha,
+          T beta) {
+  typedef T Four __attribute__((ext_vector_type(4)));
+  // X transposed and padded with zeros: four sums advance with one 128-bit
+  // read that is the same for every lane
+  __shared__ __attribute__((aligned(32))) T Xs[32][MB];
+  for (int i = threadIdx.x; i < 32 * MB; i += 256) {
+    const int k = i / MB, m = i % MB;
+    Xs[k][m] = (k < K && m < M) ? X[m * xm + k * xk] : T(0);
+  }
+  __syncthreads();
+  const int64_t n = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (n >= N)
+    return;
+  Four acc[MB / 4];
+#pragma unroll
+  for (int q = 0; q < MB / 4; ++q)
+    acc[q] = Four{T(0), T(0), T(0), T(0)};
+  const T *y = Y + n;
+#pragma unroll 4
+  for (int k = 0; k < K; ++k) {
+    const T v = __builtin_nontemporal_load(y + k * ldy);
+#pragma unroll
+    for (int q = 0; q < MB / 4; ++q)
+      acc[q] += *reinterpret_cast<const Four *>(&Xs[k][4 * q]) * v;
+  }
+  T *z = Z + n;
+#pragma unroll
+  for (int m = 0; m < MB; ++m)
+    if (m < M) {
+      T v = alpha * acc[m / 4][m % 4];
+      if (beta != T(0))
+        v += beta * z[m * ldz];
+      __builtin_nontemporal_store(v, z + m * ldz);
+    }
+}
+
+// ---------------------------------------------------------------------------
 // A copy of an operand that the tile kernels can read in 128-bit words: the
 // R rows of C elements at src (row stride ld, unit stride along a row) go to
 // rows of Cp = C rounded up to whole words, dense, 16-byte aligned, the tail
@@ -1058,6 +1105,24 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
         hipLaunchKernelGGL(gemm_skinny<T>, dim3(blocks), dim3(256), 0, stream, X, ldx, Y, yk,
                            yn, cData, ldz, Mz, int(Nz), int(K), alpha, beta, wordStores);
         lastKernel = sizeof(T) == 4 ? "sgemm_skinny" : "dgemm_skinny";
+        launched = true;
+      }
+      // Small times long: gemm_wide.
+      if (!launched && yNc && K >= 1 && K <= 32 && Mz <= 32 && Nz >= 4096 && ldy > 0) {
+        const dim3 grid(unsigned((Nz + 255) / 256));
+#define NMHIP_GEMM_WIDE(MB)                                                    \
+  hipLaunchKernelGGL((gemm_wide<T, MB>), grid, dim3(256), 0, stream, X, xm, xk, \
+                     Y, ldy, cData, ldz, int(Mz), Nz, int(K), alpha, beta)
+        if (Mz <= 4)
+          NMHIP_GEMM_WIDE(4);
+        else if (Mz <= 8)
+          NMHIP_GEMM_WIDE(8);
+        else if (Mz <= 16)
+          NMHIP_GEMM_WIDE(16);
+        else
+          NMHIP_GEMM_WIDE(32);
+#undef NMHIP_GEMM_WIDE
+        lastKernel = sizeof(T) == 4 ? "sgemm_wide" : "dgemm_wide";
         launched = true;
       }
       // The matrix-core kernel takes the part of the problem that is whole

@@ -352,6 +352,30 @@ def test_tall_times_small(env, dtype, m, k, n):
         _check_scaled(d_c.asnumpy(), wide[:, :k], b, np.zeros((m, n), dtype), 1.0, 0.0, tol)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("m,k,n", [(1, 1, 4096), (3, 3, 5000), (8, 8, 100_003), (5, 16, 70_001),
+                                   (32, 32, 33_333), (29, 7, 65_537)])
+def test_small_times_long(env, dtype, m, k, n):
+    """A small matrix times a long one (M, K <= 32): a lane per column.
+    Row-major, views of wider rows, a transposed small operand, alpha and
+    beta; every element against float64."""
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(m + k + n)
+    a = rng.standard_normal((m, k)).astype(dtype)
+    wide = rng.standard_normal((k, n + 5)).astype(dtype)
+    c0 = rng.standard_normal((m, n + 3)).astype(dtype)
+    tol = 1e-5 if dtype == np.float32 else 1e-13
+    for a_dev, b_view in ((hip.asarray(a), hip.asarray(np.ascontiguousarray(wide[:, :n]))),
+                          (hip.asarray(np.asfortranarray(a)), hip.asarray(wide)[:, :n])):
+        d_c = hip.asarray(c0)[:, :n]
+        ops.gemm(a_dev, b_view, d_c, 1.5, -0.5)
+        assert mrt.last_kernel() == ("sgemm_wide" if dtype == np.float32 else "dgemm_wide")
+        _check_scaled(d_c.asnumpy(), a, wide[:, :n], c0[:, :n], 1.5, -0.5, tol)
+        d_c = hip.asarray(np.full((m, n), np.nan, dtype))
+        ops.gemm(a_dev, b_view, d_c, 1.0, 0.0)
+        _check_scaled(d_c.asnumpy(), a, wide[:, :n], np.zeros((m, n), dtype), 1.0, 0.0, tol)
+
+
 def test_identity_and_linearity_full_size(env):
     """Configuration 5 (4096^3): rows checked against float64, plus
     size-independent properties: A @ I == A exactly, and linearity."""
