@@ -708,6 +708,288 @@ gemm_wide(const T *__restrict__ X, int64_t xm, int64_t xk, const T *__restrict__
 }
 
 // ---------------------------------------------------------------------------
+// A long matrix times a thin one (a matrix times a vector or a few of them):
+// the work is reading the long matrix once.  W elements a load: the 128-bit
+// word when the rows of the long matrix begin and end on words, 1 otherwise.
+template <typename T, int W> struct ThinWord {
+  typedef T Type __attribute__((ext_vector_type(W)));
+  __device__ static __forceinline__ void load(const T *p, T (&out)[W]) {
+    const Type v = __builtin_nontemporal_load(reinterpret_cast<const Type *>(p));
+#pragma unroll
+    for (int q = 0; q < W; ++q)
+      out[q] = v[q];
+  }
+};
+template <typename T> struct ThinWord<T, 1> {
+  __device__ static __forceinline__ void load(const T *p, T (&out)[1]) {
+    out[0] = __builtin_nontemporal_load(p);
+  }
+};
+
+// O(r, j) = alpha * sum_k S(r, k) P(k, j) + beta * O(r, j) for a long S with
+// unit stride along k (rows `ld` apart) and a thin P (n <= NB columns, any
+// strides).  G adjacent lanes (a power of two up to a wave, or the 256 of the
+// block when there are few rows) share a set of R rows: each takes every G-th
+// word along k of those rows and the rows of P that go with it (P is read by
+// every group: it stays in the caches), the G partial sums meet through lane
+// exchanges (and LDS, for the block), and the first lane of the group stores.
+// R rows at once divide the reads of P by R; 8 / R steps along k are in
+// flight at once, eight loads of S a lane.  PV: how P is read -- 0 by
+// element; 1 by rows (unit stride along j, n == NB, rows aligned to
+// min(16, row) bytes); 2 by words along k (unit stride along k, columns
+// aligned to the word; W > 1).
+template <typename T, int NB, int R, int W, int PV>
+__global__ __launch_bounds__(256) void
+gemm_thin_rows(const T *__restrict__ S, int64_t ld, int64_t rows, int64_t K,
+               const T *__restrict__ P, int64_t pk, int64_t pn, int n, T *__restrict__ O,
+               int64_t orow, int64_t ocol, T alpha, T beta, int G, int gShift) {
+  constexpr int U = R < 8 ? 8 / R : 1;
+  constexpr int ROW_BYTES = NB * int(sizeof(T)) < 16 ? NB * int(sizeof(T)) : 16;
+  typedef T PRow __attribute__((ext_vector_type(NB), aligned(ROW_BYTES)));
+  typedef T PWord __attribute__((ext_vector_type(W)));
+  __shared__ T cross[4][R * NB];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const bool wholeBlock = G == 256;
+  const int g = wholeBlock ? int(threadIdx.x) : lane & (G - 1);
+  const int64_t set = wholeBlock ? int64_t(blockIdx.x)
+                                 : (int64_t(blockIdx.x) * 4 + wave) * (64 >> gShift) +
+                                       (lane >> gShift);
+  const int64_t r0 = set * R;
+  const T *row[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) // (rows beyond the last read the last: nothing of theirs is stored)
+    row[r] = S + (r0 + r < rows ? r0 + r : rows - 1) * ld;
+  T acc[R][NB];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+      acc[r][j] = T(0);
+  const int64_t words = K / W;
+  for (int64_t w0 = g; w0 < words; w0 += int64_t(G) * U) {
+    T x[U][R][W];
+    T p[U][W][NB];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t w = w0 + int64_t(u) * G;
+      if (w < words) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          ThinWord<T, W>::load(row[r] + w * W, x[u][r]);
+        if (PV == 1) {
+#pragma unroll
+          for (int q = 0; q < W; ++q) {
+            const PRow v = *reinterpret_cast<const PRow *>(P + (w * W + q) * pk);
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+              p[u][q][j] = v[j];
+          }
+        } else if (PV == 2) {
+#pragma unroll
+          for (int j = 0; j < NB; ++j)
+            if (j < n) {
+              const PWord v = *reinterpret_cast<const PWord *>(P + w * W + j * pn);
+#pragma unroll
+              for (int q = 0; q < W; ++q)
+                p[u][q][j] = v[q];
+            }
+        } else {
+#pragma unroll
+          for (int q = 0; q < W; ++q)
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+              if (j < n)
+                p[u][q][j] = P[(w * W + q) * pk + j * pn];
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t w = w0 + int64_t(u) * G;
+      if (w < words) {
+#pragma unroll
+        for (int q = 0; q < W; ++q)
+#pragma unroll
+          for (int j = 0; j < NB; ++j)
+            if (j < n) {
+#pragma unroll
+              for (int r = 0; r < R; ++r)
+                acc[r][j] += x[u][r][q] * p[u][q][j];
+            }
+      }
+    }
+  }
+  if (W > 1 && g == 0) // the elements behind the last whole word
+    for (int64_t k = words * W; k < K; ++k)
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        if (j < n) {
+          const T v = P[k * pk + j * pn];
+#pragma unroll
+          for (int r = 0; r < R; ++r)
+            acc[r][j] += row[r][k] * v;
+        }
+  const int inWave = G < 64 ? G : 64;
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      T v = acc[r][j];
+      for (int step = inWave >> 1; step > 0; step >>= 1)
+        v += __shfl_xor(v, step, 64);
+      acc[r][j] = v;
+    }
+  if (wholeBlock) { // (the same for every lane of the launch)
+    if (lane == 0)
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          cross[wave][r * NB + j] = acc[r][j];
+    __syncthreads();
+    if (threadIdx.x == 0)
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          acc[r][j] = ((cross[0][r * NB + j] + cross[1][r * NB + j]) + cross[2][r * NB + j]) +
+                      cross[3][r * NB + j];
+  }
+  if (g == 0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        if (r0 + r < rows && j < n) {
+          T *dst = O + (r0 + r) * orow + j * ocol;
+          T v = alpha * acc[r][j];
+          if (beta != T(0))
+            v += beta * *dst;
+          *dst = v;
+        }
+  }
+}
+
+// The value that lane `from` (the same for the whole wave) holds in v.
+__device__ __forceinline__ float fromLane(float v, int from) {
+  return __builtin_bit_cast(float,
+                            __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), from));
+}
+__device__ __forceinline__ double fromLane(double v, int from) {
+  const uint64_t bits = __builtin_bit_cast(uint64_t, v);
+  const uint32_t lo = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(bits)), from));
+  const uint32_t hi = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(bits >> 32)), from));
+  return __builtin_bit_cast(double, (uint64_t(hi) << 32) | lo);
+}
+
+// O(i, c) = alpha * sum_k P(i, k) S(k, c) + beta * O(i, c) for a thin P
+// (m <= MB rows, any strides) and a long S with unit stride along c (rows
+// `ld` apart): a lane owns W adjacent columns, each of the four waves of a
+// block takes every fourth k of the block's slice of K (eight loads of S in
+// flight a lane) and the four add up through LDS in wave order.  P(i, k) is
+// the same for the whole wave: the lanes fetch those of 64 steps at a time,
+// one each, and hand them round.  With one slice (part == nullptr) the block stores to O;
+// with more, slice z stores its m x cPitch partial sums at part + z m cPitch
+// and gemm_thin_fold adds the slices in index order.
+template <typename T, int MB, int W>
+__global__ __launch_bounds__(256) void
+gemm_thin_cols(const T *__restrict__ S, int64_t ld, int64_t C, int64_t K, int64_t sliceK,
+               const T *__restrict__ P, int64_t pm, int64_t pk, int m, T *__restrict__ O,
+               int64_t oi, int64_t oc, T alpha, T beta, T *__restrict__ part,
+               int64_t cPitch) {
+  constexpr int U = 8, STRIP = 64 * W;
+  __shared__ T sums[4][MB][STRIP];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t strip0 = int64_t(blockIdx.x) * STRIP;
+  const int64_t c0 = strip0 + lane * W;
+  const bool live = c0 < C; // (W > 1: C is a multiple of W)
+  const int64_t sliceBegin = int64_t(blockIdx.y) * sliceK;
+  const int64_t sliceEnd = sliceBegin + sliceK < K ? sliceBegin + sliceK : K;
+  // this wave's rows of S: every fourth of the slice (the four waves of a
+  // block read four adjacent rows at a time)
+  const int64_t kBegin = sliceBegin + wave;
+  const int64_t steps = kBegin < sliceEnd ? (sliceEnd - kBegin + 3) / 4 : 0;
+  T acc[MB][W];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int q = 0; q < W; ++q)
+      acc[i][q] = T(0);
+  const T *col = S + (live ? c0 : 0);
+  for (int64_t t64 = 0; t64 < steps; t64 += 64) {
+    T mine[MB]; // P(i, k) of step t64 + lane
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+      mine[i] = i < m && t64 + lane < steps ? P[i * pm + (kBegin + 4 * (t64 + lane)) * pk]
+                                            : T(0);
+    const int count = steps - t64 < 64 ? int(steps - t64) : 64;
+    for (int t0 = 0; t0 < count; t0 += U) {
+      T s[U][W];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (t0 + u < count)
+          ThinWord<T, W>::load(col + (kBegin + 4 * (t64 + t0 + u)) * ld, s[u]);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (t0 + u < count) {
+#pragma unroll
+          for (int i = 0; i < MB; ++i)
+            if (i < m) {
+              const T v = fromLane(mine[i], t0 + u);
+#pragma unroll
+              for (int q = 0; q < W; ++q)
+                acc[i][q] += v * s[u][q];
+            }
+        }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int q = 0; q < W; ++q)
+      sums[wave][i][lane * W + q] = acc[i][q];
+  __syncthreads();
+  for (int e = threadIdx.x; e < m * STRIP; e += 256) {
+    const int i = e / STRIP, cc = e % STRIP;
+    const int64_t c = strip0 + cc;
+    if (c >= C)
+      continue;
+    const T sum = ((sums[0][i][cc] + sums[1][i][cc]) + sums[2][i][cc]) + sums[3][i][cc];
+    if (part) {
+      part[(int64_t(blockIdx.y) * m + i) * cPitch + c] = sum;
+    } else {
+      T *dst = O + i * oi + c * oc;
+      T v = alpha * sum;
+      if (beta != T(0))
+        v += beta * *dst;
+      *dst = v;
+    }
+  }
+}
+
+// O(i, c) = alpha * (part[0](i, c) + part[1](i, c) + ...) + beta * O(i, c):
+// the slices of gemm_thin_cols in index order, one thread per element.
+template <typename T>
+__global__ __launch_bounds__(256) void
+gemm_thin_fold(const T *__restrict__ part, int slices, int m, int64_t C, int64_t cPitch,
+               T *__restrict__ O, int64_t oi, int64_t oc, T alpha, T beta) {
+  const int64_t c = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  const int i = blockIdx.y;
+  if (c >= C)
+    return;
+  const T *src = part + int64_t(i) * cPitch + c;
+  T sum = src[0];
+  for (int z = 1; z < slices; ++z)
+    sum += src[int64_t(z) * m * cPitch];
+  T *dst = O + i * oi + c * oc;
+  T v = alpha * sum;
+  if (beta != T(0))
+    v += beta * *dst;
+  *dst = v;
+}
+
+// ---------------------------------------------------------------------------
 // A copy of an operand that the tile kernels can read in 128-bit words: the
 // R rows of C elements at src (row stride ld, unit stride along a row) go to
 // rows of Cp = C rounded up to whole words, dense, 16-byte aligned, the tail
@@ -1124,6 +1406,144 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
 #undef NMHIP_GEMM_WIDE
         lastKernel = sizeof(T) == 4 ? "sgemm_wide" : "dgemm_wide";
         launched = true;
+      }
+      // A long matrix times a thin one (at most eight columns, or rows):
+      // gemm_thin_rows when the long one has unit stride along k,
+      // gemm_thin_cols when along its other dimension.
+      if (!launched && K > 32) {
+        constexpr int64_t kLong = 1024, kThin = 8;
+        auto wordsOk = [&](const T *S, int64_t ld) { return aligned16(S) && ld % VEC == 0; };
+        auto thinRows = [&](const T *S, int64_t ld, int64_t rows, const T *P, int64_t pk,
+                            int64_t pn, int n, int64_t orow, int64_t ocol) {
+          const bool vec = wordsOk(S, ld);
+          const int64_t words = vec ? K / VEC : K;
+          int G = 64, gShift = 6;
+          while (G > 1 && 2 * G > words)
+            G >>= 1, --gShift;
+          const int NB = n <= 1 ? 1 : n <= 2 ? 2 : n <= 4 ? 4 : 8;
+          auto wavesWith = [&](int R) { return ((rows + R - 1) / R * G + 63) / 64; };
+          // Four rows a group where that leaves 2048 waves or more, and for
+          // more than one column of P always (fewer reads of P: as many
+          // elements of P as of S at most); the four
+          // waves of a block on one set of rows where there are few rows.
+          const int R = NB == 8 ? 8 : NB > 1 || wavesWith(4) >= 2048 ? 4 : 1;
+          if (wavesWith(R) < 2048 && words >= 512)
+            G = 256, gShift = 8;
+          const int64_t sets = (rows + R - 1) / R;
+          const int64_t perBlock = G == 256 ? 1 : 4 * (64 / G);
+          const int64_t blocks = (sets + perBlock - 1) / perBlock;
+          if (blocks >= (int64_t(1) << 24))
+            return false;
+          // How P is read (gemm_thin_rows).
+          const size_t rowBytes = size_t(NB) * sizeof(T) < 16 ? size_t(NB) * sizeof(T) : 16;
+          int PV = 0;
+          if (NB > 1 && n == NB && pn == 1 &&
+              reinterpret_cast<uintptr_t>(P) % rowBytes == 0 &&
+              size_t(pk) * sizeof(T) % rowBytes == 0)
+            PV = 1;
+          else if (vec && pk == 1 && aligned16(P) && pn % VEC == 0)
+            PV = 2;
+          const dim3 grid{unsigned(blocks)};
+#define NMHIP_THIN_ROWS(NB_, R_, W_, PV_)                                      \
+  hipLaunchKernelGGL((gemm_thin_rows<T, NB_, R_, W_, PV_>), grid, dim3(256), 0, \
+                     stream, S, ld, rows, K, P, pk, pn, n, cData, orow, ocol,  \
+                     alpha, beta, G, gShift)
+#define NMHIP_THIN_ROWS_P(NB_, R_)                                             \
+  do {                                                                         \
+    if (vec && PV == 2)                                                        \
+      NMHIP_THIN_ROWS(NB_, R_, VEC, 2);                                        \
+    else if (vec && PV == 1)                                                   \
+      NMHIP_THIN_ROWS(NB_, R_, VEC, (NB_ > 1 ? 1 : 0));                          \
+    else if (vec)                                                              \
+      NMHIP_THIN_ROWS(NB_, R_, VEC, 0);                                        \
+    else if (PV == 1)                                                          \
+      NMHIP_THIN_ROWS(NB_, R_, 1, (NB_ > 1 ? 1 : 0));                            \
+    else                                                                       \
+      NMHIP_THIN_ROWS(NB_, R_, 1, 0);                                          \
+  } while (0)
+          if (NB == 1) {
+            if (R == 4)
+              NMHIP_THIN_ROWS_P(1, 4);
+            else
+              NMHIP_THIN_ROWS_P(1, 1);
+          } else if (NB == 2) {
+            NMHIP_THIN_ROWS_P(2, 4);
+          } else if (NB == 4) {
+            NMHIP_THIN_ROWS_P(4, 4);
+          } else {
+            NMHIP_THIN_ROWS_P(8, 8);
+          }
+#undef NMHIP_THIN_ROWS_P
+#undef NMHIP_THIN_ROWS
+          lastKernel = sizeof(T) == 4 ? "sgemm_thin_rows" : "dgemm_thin_rows";
+          return true;
+        };
+        auto thinCols = [&](const T *S, int64_t ld, int64_t C, const T *P, int64_t pm,
+                            int64_t pk, int m, int64_t oi, int64_t oc) {
+          const bool vec = wordsOk(S, ld) && C % VEC == 0;
+          const int64_t strip = vec ? 64 * VEC : 64;
+          const int64_t strips = (C + strip - 1) / strip;
+          if (strips >= (int64_t(1) << 24))
+            return false;
+          // Slices of K so that some 2048 blocks are at work, each wave with
+          // sixteen rows of S or more; the partial sums within the fixed
+          // workspace's size whichever workspace serves.
+          const int64_t cPitch = strips * strip;
+          int64_t slices = 2048 / strips;
+          if (slices > K / 64)
+            slices = K / 64;
+          if (slices > 64)
+            slices = 64;
+          while (slices > 1 &&
+                 size_t(slices) * size_t(m) * size_t(cPitch) * sizeof(T) > kScratchBytes)
+            --slices;
+          int64_t sliceK = K;
+          if (slices > 1) {
+            sliceK = ((K + slices - 1) / slices + 3) / 4 * 4;
+            slices = (K + sliceK - 1) / sliceK;
+          }
+          SplitPlan plan;
+          plan.slices = int(slices < 1 ? 1 : slices);
+          T *part = workspaceFor(plan, m, cPitch);
+          if (!part)
+            plan.slices = 1, sliceK = K;
+          const dim3 grid(unsigned(strips), unsigned(plan.slices));
+#define NMHIP_THIN_COLS(MB, W)                                                 \
+  hipLaunchKernelGGL((gemm_thin_cols<T, MB, W>), grid, dim3(256), 0, stream, S, \
+                     ld, C, K, sliceK, P, pm, pk, m, cData, oi, oc, alpha,     \
+                     beta, part, cPitch)
+#define NMHIP_THIN_COLS_W(MB)                                                  \
+  do {                                                                         \
+    if (vec)                                                                   \
+      NMHIP_THIN_COLS(MB, VEC);                                                \
+    else                                                                       \
+      NMHIP_THIN_COLS(MB, 1);                                                  \
+  } while (0)
+          if (m <= 1)
+            NMHIP_THIN_COLS_W(1);
+          else if (m <= 2)
+            NMHIP_THIN_COLS_W(2);
+          else if (m <= 4)
+            NMHIP_THIN_COLS_W(4);
+          else
+            NMHIP_THIN_COLS_W(8);
+#undef NMHIP_THIN_COLS_W
+#undef NMHIP_THIN_COLS
+          if (part)
+            hipLaunchKernelGGL(gemm_thin_fold<T>, dim3(unsigned((C + 255) / 256), unsigned(m)),
+                               dim3(256), 0, stream, part, plan.slices, m, C, cPitch, cData,
+                               oi, oc, alpha, beta);
+          lastKernel = sizeof(T) == 4 ? "sgemm_thin_cols" : "dgemm_thin_cols";
+          return true;
+        };
+        if (Nz <= kThin && Mz >= kLong)
+          launched = xKc       ? thinRows(X, xm, Mz, Y, yk, yn, int(Nz), ldz, 1)
+                     : xm == 1 ? thinCols(X, xk, Mz, Y, yn, yk, int(Nz), 1, ldz)
+                               : false;
+        else if (Mz <= kThin && Nz >= kLong)
+          launched = yNc       ? thinCols(Y, yk, Nz, X, xm, xk, int(Mz), ldz, 1)
+                     : yk == 1 ? thinRows(Y, yn, Nz, X, xk, xm, int(Mz), 1, ldz)
+                               : false;
       }
       // The matrix-core kernel takes the part of the problem that is whole
       // tiles, Z[0:Mt, 0:Nt] over k in [0, Kt); the strided kernel adds the

@@ -325,13 +325,13 @@ class Dispatcher:
             # a @ b, np.dot(a, b)
             if isinstance(expr, ast.BinOp) and isinstance(expr.op, ast.MatMult):
                 a, b = array(expr.left), array(expr.right)
-                if a is not None and b is not None:
-                    return self._served("library", ops.dot(a, b), a.ctx)
+                if a is not None and b is not None and a.ndim <= 2 and b.ndim <= 2:
+                    return self._served("library", _dot(a, b), a.ctx)
             call = np_call(expr, ("dot",))
             if call and len(call[1]) == 2 and not call[2]:
                 a, b = array(call[1][0]), array(call[1][1])
-                if a is not None and b is not None and a.ndim == b.ndim == 2:
-                    return self._served("library", ops.dot(a, b), a.ctx)
+                if a is not None and b is not None and a.ndim <= 2 and b.ndim <= 2:
+                    return self._served("library", _dot(a, b), a.ctx)
             # np.dot(a, b, c), np.dot(a, b, out=c) (test_gpu.py:2101-2138)
             if call and len(call[1]) + len(call[2]) == 3 and \
                     all(k.arg == "out" for k in call[2]):

@@ -376,6 +376,70 @@ def test_small_times_long(env, dtype, m, k, n):
         _check_scaled(d_c.asnumpy(), a, wide[:, :n], np.zeros((m, n), dtype), 1.0, 0.0, tol)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("long,k,thin", [(1500, 100, 1), (1025, 33, 3), (2000, 1001, 8),
+                                         (5000, 4099, 5), (1100, 70_000, 2), (40_000, 260, 4)])
+def test_long_times_thin(env, dtype, long, k, thin):
+    """A long matrix times a thin one (a vector, or up to eight of them) and a
+    thin one times a long one, K > 32: the long operand is read once, by rows
+    when it has unit stride along k, by columns otherwise.  Every layout of
+    the three operands, rows that are and are not whole 128-bit words (views
+    of wider rows), alpha and beta, a C of NaNs under beta = 0; every element
+    against float64."""
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(long + k + thin)
+    tol = 1e-5 if dtype == np.float32 else 1e-13
+    prefix = "s" if dtype == np.float32 else "d"
+    for m, n in ((long, thin), (thin, long)):
+        a = rng.standard_normal((m, k)).astype(dtype)
+        b = rng.standard_normal((k, n)).astype(dtype)
+        c0 = rng.standard_normal((m, n)).astype(dtype)
+        for fa in (False, True):
+            for fb in (False, True):
+                # the long operand decides: by rows when its unit stride is k's
+                long_by_rows = (not fa) if m == long else fb
+                want = prefix + ("gemm_thin_rows" if long_by_rows else "gemm_thin_cols")
+                for fc in (False, True):
+                    d_a = _to_dev(hip, a.T.copy().T if fa else a)
+                    d_b = _to_dev(hip, b.T.copy().T if fb else b)
+                    d_c = _to_dev(hip, c0.T.copy().T if fc else c0)
+                    ops.gemm(d_a, d_b, d_c, 1.5, -0.5)
+                    assert mrt.last_kernel() == want, (m, n, fa, fb, fc)
+                    _check_scaled(d_c.asnumpy(), a, b, c0, 1.5, -0.5, tol)
+        # views of rows three and four elements wider, and beta = 0 over NaNs
+        for pad in (3, 4):
+            wide_a = rng.standard_normal((m, k + pad)).astype(dtype)
+            wide_b = rng.standard_normal((k, n + pad)).astype(dtype)
+            d_a, d_b = hip.asarray(wide_a)[:, :k], hip.asarray(wide_b)[:, :n]
+            d_c = hip.asarray(np.full((m, n), np.nan, dtype))
+            ops.gemm(d_a, d_b, d_c, 1.0, 0.0)
+            assert "gemm_thin" in mrt.last_kernel()
+            _check_scaled(d_c.asnumpy(), wide_a[:, :k], wide_b[:, :n], np.zeros((m, n), dtype),
+                          1.0, 0.0, tol)
+
+
+def test_thin_products_do_not_mix_in_what_lies_beyond(env):
+    """An infinity in the long operand's padding, or in the thin one's, stays
+    out of the sums (a product with zero would make it a NaN)."""
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(11)
+    m, k = 3000, 1030
+    wide = rng.standard_normal((m, k + 2)).astype(np.float32)
+    wide[:, k:] = np.inf
+    v = rng.standard_normal((k + 1, 1)).astype(np.float32)
+    v[k] = np.inf
+    d_c = hip.asarray(np.zeros((m, 1), np.float32))
+    ops.gemm(hip.asarray(wide)[:, :k], hip.asarray(v)[:k], d_c, 1.0, 0.0)
+    assert mrt.last_kernel() == "sgemm_thin_rows"
+    _check_scaled(d_c.asnumpy(), wide[:, :k], v[:k], np.zeros((m, 1), np.float32), 1.0, 0.0, 1e-5)
+    d_r = hip.asarray(np.zeros((1, m), np.float32))
+    row = hip.asarray(np.ascontiguousarray(v.T))[:, :k]
+    ops.gemm(row, _to_dev(hip, wide.T)[:k], d_r, 1.0, 0.0)
+    assert "gemm_thin" in mrt.last_kernel()
+    _check_scaled(d_r.asnumpy(), v[:k].T, wide[:, :k].T, np.zeros((1, m), np.float32), 1.0, 0.0,
+                  1e-5)
+
+
 def test_identity_and_linearity_full_size(env):
     """Configuration 5 (4096^3): rows checked against float64, plus
     size-independent properties: A @ I == A exactly, and linearity."""

@@ -704,6 +704,35 @@ def test_dot_into_an_existing_array(env, func):
     np.testing.assert_array_equal(res.asnumpy(), [[22, 28], [49, 64]])
 
 
+def _matmul_operator(a, b):
+    return a @ b
+
+
+def _np_dot(a, b):
+    return np.dot(a, b)
+
+
+@pytest.mark.parametrize("func", [_matmul_operator, _np_dot])
+def test_products_with_vectors(env, func):
+    """A matrix times a vector, a vector times a matrix and two vectors
+    (numpy/funcs.py:879-930: rank 1 operands of dot and of ``@`` take the
+    rank numpy gives the result)."""
+    hip = env[0]
+    rng = np.random.default_rng(3)
+    A = rng.standard_normal((1300, 700))
+    v, w = rng.standard_normal(700), rng.standard_normal(1300)
+    f = njit(func)
+    got = f(hip.asarray(A), hip.asarray(v))
+    assert f.last_launch["path"] == "library" and got.shape == (1300,)
+    np.testing.assert_allclose(got.asnumpy(), A @ v, rtol=1e-12, atol=1e-12)
+    got = f(hip.asarray(w), hip.asarray(A))
+    assert got.shape == (700,)
+    np.testing.assert_allclose(got.asnumpy(), w @ A, rtol=1e-12, atol=1e-12)
+    got = f(hip.asarray(v), hip.asarray(v))
+    assert np.shape(got) == ()
+    np.testing.assert_allclose(got, v @ v, rtol=1e-12)
+
+
 def test_pairwise_as_nested_prange_loops(env):
     """test_pairwise2 (test_gpu.py:2226-2266): the distance body as two
     prange loops around a serial one, on the reference's fixture."""

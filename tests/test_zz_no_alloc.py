@@ -111,3 +111,20 @@ def test_operands_off_the_word_grid_stay_on_tiles_and_edges(gemm_entry_points):
     scale = np.abs(a).astype(np.float64) @ np.abs(b)
     for _, got in outs:
         assert (np.abs(got - truth) <= 1e-4 * scale + 1e-30).all()
+
+
+def test_a_thin_product_keeps_its_partial_sums_in_the_fixed_array(gemm_entry_points):
+    """A few rows times a long matrix cuts K into slices whose partial sums
+    go through the workspace: both entry points cut alike and give the same
+    bits, the second call on a smaller problem."""
+    hip, lib, mrt = gemm_entry_points
+    for m, n, k in ((4, 4096, 4096), (2, 1100, 2048)):
+        status, got, ref, k_ref, k_got, (a, b, c0) = _both(
+            hip, lib, mrt, m, n, k, 1.5, -0.5, seed=m + n + k)
+        assert status == 0
+        assert k_got == k_ref == "sgemm_thin_cols"
+        assert np.array_equal(got, ref), (m, n, k)
+        truth = -0.5 * c0.astype(np.float64) + 1.5 * (
+            a.astype(np.float64) @ b.astype(np.float64))
+        scale = 0.5 * np.abs(c0) + 1.5 * (np.abs(a).astype(np.float64) @ np.abs(b))
+        assert (np.abs(got - truth) <= 1e-5 * scale + 1e-30).all()
