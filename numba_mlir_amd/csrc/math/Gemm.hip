@@ -525,7 +525,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void
 gemm_generic(const T *A, const T *B, T *C, int64_t M, int64_t N, int64_t K,
              int64_t as0, int64_t as1, int64_t bs0, int64_t bs1, int64_t cs0,
-             int64_t cs1, T alpha, T beta) {
+             int64_t cs1, T alpha, T beta, int64_t kSlice, T *part) {
   constexpr int TILE = 32;
   __shared__ T As[TILE][TILE + 1];
   __shared__ T Bs[TILE][TILE + 1];
@@ -540,7 +540,12 @@ gemm_generic(const T *A, const T *B, T *C, int64_t M, int64_t N, int64_t K,
   const int64_t row0 = tile / tilesN * TILE;
   const int64_t col = tile % tilesN * TILE + tx;
   T acc[4] = {T(0), T(0), T(0), T(0)};
-  for (int64_t k0 = 0; k0 < K; k0 += TILE) {
+  // blockIdx.z: the slice of K (multiples of the tile), whose partial sums go
+  // to part + z M N for gemm_thin_fold when there is more than one
+  const int64_t kBegin = int64_t(blockIdx.z) * kSlice;
+  if (kBegin + kSlice < K)
+    K = kBegin + kSlice;
+  for (int64_t k0 = kBegin; k0 < K; k0 += TILE) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int r = ty + 8 * i;
@@ -562,7 +567,9 @@ gemm_generic(const T *A, const T *B, T *C, int64_t M, int64_t N, int64_t K,
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int64_t row = row0 + ty + 8 * i;
-    if (row < M && col < N) {
+    if (row < M && col < N && part) {
+      part[(int64_t(blockIdx.z) * M + row) * N + col] = acc[i];
+    } else if (row < M && col < N) {
       T *dst = C + row * cs0 + col * cs1;
       T v = alpha * acc[i];
       if (beta != T(0))
@@ -968,20 +975,120 @@ gemm_thin_cols(const T *__restrict__ S, int64_t ld, int64_t C, int64_t K, int64_
   }
 }
 
-// O(i, c) = alpha * (part[0](i, c) + part[1](i, c) + ...) + beta * O(i, c):
-// the slices of gemm_thin_cols in index order, one thread per element.
+// A small product of long operands (m, n <= 8: the Gram matrix of a few
+// columns, a few columns against a right-hand side): block z takes a slice of
+// K, a lane every 256th k of it -- the m values of X and the n of Y at that k,
+// any strides, two k in flight -- and keeps all m n sums; they meet through
+// lane exchanges and LDS, in a fixed order, and go to part + z m n for
+// gemm_thin_fold.  ROWS: the m values of X at a k and the n of Y are adjacent
+// and aligned (m == MB, n == NB, rows of the transposed tall operands): read
+// as words (8 x 1048576 x 8 float32 73 -> 48 us).
+template <typename T, int MB, int NB, bool ROWS>
+__global__ __launch_bounds__(256) void
+gemm_inner(const T *__restrict__ X, int64_t xm, int64_t xk, const T *__restrict__ Y,
+           int64_t yk, int64_t yn, int m, int n, int64_t K, int64_t kSlice,
+           T *__restrict__ part) {
+  constexpr int U = 2;
+  __shared__ T cross[4][MB * NB];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t kBegin = int64_t(blockIdx.x) * kSlice;
+  const int64_t kEnd = kBegin + kSlice < K ? kBegin + kSlice : K;
+  T acc[MB][NB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+      acc[i][j] = T(0);
+  for (int64_t k0 = kBegin + threadIdx.x; k0 < kEnd; k0 += 256 * U) {
+    T x[U][MB], y[U][NB];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t k = k0 + 256 * u;
+      if (k < kEnd && ROWS) {
+        typedef T XRow __attribute__((ext_vector_type(MB), aligned(MB * sizeof(T) < 16 ? MB * sizeof(T) : 16)));
+        typedef T YRow __attribute__((ext_vector_type(NB), aligned(NB * sizeof(T) < 16 ? NB * sizeof(T) : 16)));
+        const XRow xv = __builtin_nontemporal_load(reinterpret_cast<const XRow *>(X + k * xk));
+        const YRow yv = __builtin_nontemporal_load(reinterpret_cast<const YRow *>(Y + k * yk));
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+          x[u][i] = xv[i];
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          y[u][j] = yv[j];
+      } else if (k < kEnd) {
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+          x[u][i] = i < m ? __builtin_nontemporal_load(X + i * xm + k * xk) : T(0);
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          y[u][j] = j < n ? __builtin_nontemporal_load(Y + k * yk + j * yn) : T(0);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (k0 + 256 * u < kEnd) {
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+          for (int j = 0; j < NB; ++j)
+            acc[i][j] += x[u][i] * y[u][j];
+      }
+  }
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      T v = acc[i][j];
+#pragma unroll
+      for (int step = 32; step > 0; step >>= 1)
+        v += __shfl_xor(v, step, 64);
+      if (lane == 0)
+        cross[wave][i * NB + j] = v;
+    }
+  __syncthreads();
+  if (int(threadIdx.x) < m * n) {
+    const int i = threadIdx.x / n, j = threadIdx.x % n, at = i * NB + j;
+    part[(int64_t(blockIdx.x) * m + i) * n + j] =
+        ((cross[0][at] + cross[1][at]) + cross[2][at]) + cross[3][at];
+  }
+}
+
+// O(i, c) = alpha * (part[0](i, c) + part[1](i, c) + ...) + beta * O(i, c),
+// the slices m cPitch elements apart: a block takes 16 adjacent elements of a
+// row; 16 lanes an element each add up every 16th slice (eight loads in
+// flight), then one adds the 16 sums in lane order -- a fixed order, so the
+// result does not depend on which block finished first, and thousands of
+// slices of a small result are not one lane's chain of loads.
 template <typename T>
 __global__ __launch_bounds__(256) void
 gemm_thin_fold(const T *__restrict__ part, int slices, int m, int64_t C, int64_t cPitch,
                T *__restrict__ O, int64_t oi, int64_t oc, T alpha, T beta) {
-  const int64_t c = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  __shared__ T sums[16][17];
+  const int el = threadIdx.x & 15, zl = threadIdx.x >> 4;
+  const int64_t c = int64_t(blockIdx.x) * 16 + el;
   const int i = blockIdx.y;
-  if (c >= C)
+  T sum = T(0);
+  if (c < C) {
+    const T *src = part + int64_t(i) * cPitch + c;
+    const int64_t stride = int64_t(m) * cPitch;
+    for (int z = zl; z < slices; z += 16 * 8) {
+      T v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        v[u] = z + 16 * u < slices ? src[(z + 16 * u) * stride] : T(0);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        sum += v[u];
+    }
+  }
+  sums[zl][el] = sum;
+  __syncthreads();
+  if (zl != 0 || c >= C)
     return;
-  const T *src = part + int64_t(i) * cPitch + c;
-  T sum = src[0];
-  for (int z = 1; z < slices; ++z)
-    sum += src[int64_t(z) * m * cPitch];
+  sum = sums[0][el];
+#pragma unroll
+  for (int z = 1; z < 16; ++z)
+    sum += sums[z][el];
   T *dst = O + i * oi + c * oc;
   T v = alpha * sum;
   if (beta != T(0))
@@ -1125,9 +1232,12 @@ SplitPlan planSplit(int64_t tiles, int64_t K, int BK, int blocksPerCu) {
   const int64_t slots = int64_t(256) * blocksPerCu; // resident blocks
   if (tiles <= 0 || tiles * 2 > slots)
     return plan;
+  // (at most 16 slices, or more of 512 elements each where K is that long:
+  // 128 x 262144 x 128 float32 1122 us in 16 slices)
   int64_t slices = slots / tiles;
-  if (slices > 16)
-    slices = 16;
+  const int64_t most = K / 512 > 16 ? K / 512 : 16;
+  if (slices > most)
+    slices = most;
   const int64_t minSlice = int64_t(8) * BK; // at least eight slabs a slice
   if (slices > K / minSlice)
     slices = K / minSlice;
@@ -1407,6 +1517,49 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
         lastKernel = sizeof(T) == 4 ? "sgemm_wide" : "dgemm_wide";
         launched = true;
       }
+      // A small product of long operands: gemm_inner, K in slices of 2048
+      // or more over at most 1024 blocks.
+      if (!launched && Mz <= 8 && Nz <= 8 && K >= 4096) {
+        SplitPlan plan;
+        plan.slices = int(K / 2048 < 1024 ? K / 2048 : 1024);
+        const int64_t kSlice = (K + plan.slices - 1) / plan.slices;
+        plan.slices = int((K + kSlice - 1) / kSlice);
+        if (T *part = workspaceFor(plan, Mz, Nz)) {
+          const dim3 grid{unsigned(plan.slices)};
+          auto rowsOf = [](const T *base, int64_t unit, int64_t step, int64_t extent) {
+            const size_t bytes = size_t(extent) * sizeof(T) < 16 ? size_t(extent) * sizeof(T) : 16;
+            return unit == 1 && (extent == 4 || extent == 8) &&
+                   reinterpret_cast<uintptr_t>(base) % bytes == 0 &&
+                   size_t(step) * sizeof(T) % bytes == 0;
+          };
+          const bool rowsXY = rowsOf(X, xm, xk, Mz) && rowsOf(Y, yn, yk, Nz);
+#define NMHIP_GEMM_INNER(MB, NB)                                               \
+  do {                                                                         \
+    if (rowsXY)                                                                \
+      hipLaunchKernelGGL((gemm_inner<T, MB, NB, true>), grid, dim3(256), 0,    \
+                         stream, X, xm, xk, Y, yk, yn, int(Mz), int(Nz), K,    \
+                         kSlice, part);                                        \
+    else                                                                       \
+      hipLaunchKernelGGL((gemm_inner<T, MB, NB, false>), grid, dim3(256), 0,   \
+                         stream, X, xm, xk, Y, yk, yn, int(Mz), int(Nz), K,    \
+                         kSlice, part);                                        \
+  } while (0)
+          if (Mz <= 4 && Nz <= 4)
+            NMHIP_GEMM_INNER(4, 4);
+          else if (Mz <= 4)
+            NMHIP_GEMM_INNER(4, 8);
+          else if (Nz <= 4)
+            NMHIP_GEMM_INNER(8, 4);
+          else
+            NMHIP_GEMM_INNER(8, 8);
+#undef NMHIP_GEMM_INNER
+          hipLaunchKernelGGL(gemm_thin_fold<T>, dim3(unsigned((Nz + 15) / 16), unsigned(Mz)),
+                             dim3(256), 0, stream, part, plan.slices, int(Mz), Nz, Nz, cData,
+                             ldz, int64_t(1), alpha, beta);
+          lastKernel = sizeof(T) == 4 ? "sgemm_inner" : "dgemm_inner";
+          launched = true;
+        }
+      }
       // A long matrix times a thin one (at most eight columns, or rows):
       // gemm_thin_rows when the long one has unit stride along k,
       // gemm_thin_cols when along its other dimension.
@@ -1530,7 +1683,7 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
 #undef NMHIP_THIN_COLS_W
 #undef NMHIP_THIN_COLS
           if (part)
-            hipLaunchKernelGGL(gemm_thin_fold<T>, dim3(unsigned((C + 255) / 256), unsigned(m)),
+            hipLaunchKernelGGL(gemm_thin_fold<T>, dim3(unsigned((C + 15) / 16), unsigned(m)),
                                dim3(256), 0, stream, part, plan.slices, m, C, cPitch, cData,
                                oi, oc, alpha, beta);
           lastKernel = sizeof(T) == 4 ? "sgemm_thin_cols" : "dgemm_thin_cols";
@@ -1707,12 +1860,15 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
         takeTurn();
         copiesFit = heapWorkspace(device, packXBytes + packYBytes) != nullptr;
       }
+      // (fewer than 16 tiles go to the strided kernel's 32 x 32 tiles, unless
+      // K is long and the result a quarter of a tile or more: slices of K fill
+      // the GPU then -- 300 x 65536 x 300 float32 15 -> 60 TFLOP/s)
       if (paddedBig || launched) {
         // (done)
       } else if (((!whole && !onlyK) || packX || packY) && copiesFit && unitOk && wordsOk && K > 0 &&
           ldx > 0 && ldy > 0 && M <= 0x7fffffff &&
           N <= 0x7fffffff && K <= 0x7fffffff - 64 && tilesM <= 65535 &&
-          tilesM * tilesN >= 16) {
+          (tilesM * tilesN >= 16 || (K >= 2048 && Mz * Nz >= 4096))) {
         auto roundUp = [](int64_t v, int64_t to) { return (v + to - 1) / to * to; };
         const int64_t xCp = roundUp(xC, VEC), yCp = roundUp(yC, VEC);
         const size_t xBytes = packXBytes;
@@ -1876,7 +2032,7 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           hipLaunchKernelGGL(gemm_generic<T>, g, dim3(256), 0, stream,
                              X + m0 * xm + k0 * xk, Y + k0 * yk + n0 * yn,
                              cData + m0 * ldz + n0, m, n, k, xm, xk, yk, yn, ldz,
-                             int64_t(1), alpha, bz);
+                             int64_t(1), alpha, bz, k, static_cast<T *>(nullptr));
         };
         if (Kt < K)
           edge(0, Mt, 0, Nt, Kt, K - Kt, T(1)); // the rest of K, on top
@@ -1886,13 +2042,36 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       }
     }
     if (!launched) {
-      const dim3 grid = genericGrid(M, N);
+      dim3 grid = genericGrid(M, N);
+      // A small product of long operands (a Gram matrix of a few columns):
+      // K in slices over some 2048 blocks, of 512 elements or more each;
+      // the partial sums (at most 16 MiB: a tile's are 8 KiB) are added in
+      // index order by gemm_thin_fold.
+      const int64_t tiles = int64_t(grid.x) * grid.y;
+      SplitPlan plan;
+      int64_t kSlice = K;
+      if (tiles <= 256 && K >= 2048) {
+        int64_t slices = 2048 / tiles;
+        if (slices > K / 512)
+          slices = K / 512;
+        kSlice = ((K + slices - 1) / slices + 31) / 32 * 32;
+        plan.slices = int((K + kSlice - 1) / kSlice);
+      }
+      T *part = workspaceFor(plan, M, N);
+      if (!part)
+        plan.slices = 1, kSlice = K;
+      grid.z = unsigned(plan.slices);
       hipLaunchKernelGGL(gemm_generic<T>, grid, dim3(256), 0, stream, aData,
                          bData, cData, M, N, K, int64_t(a->strides[0]),
                          int64_t(a->strides[1]), int64_t(b->strides[0]),
                          int64_t(b->strides[1]), int64_t(c->strides[0]),
-                         int64_t(c->strides[1]), alpha, beta);
-      lastKernel = sizeof(T) == 4 ? "sgemm_generic" : "dgemm_generic";
+                         int64_t(c->strides[1]), alpha, beta, kSlice, part);
+      if (part)
+        hipLaunchKernelGGL(gemm_thin_fold<T>, dim3(unsigned((N + 15) / 16), unsigned(M)),
+                           dim3(256), 0, stream, part, plan.slices, int(M), N, N, cData,
+                           int64_t(c->strides[0]), int64_t(c->strides[1]), alpha, beta);
+      lastKernel = part ? (sizeof(T) == 4 ? "sgemm_generic_splitk" : "dgemm_generic_splitk")
+                        : (sizeof(T) == 4 ? "sgemm_generic" : "dgemm_generic");
     }
     checkHip(hipGetLastError(), "gemm launch");
   }

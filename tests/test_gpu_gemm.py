@@ -440,6 +440,64 @@ def test_thin_products_do_not_mix_in_what_lies_beyond(env):
                   1e-5)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("k,m,n", [(1 << 18, 8, 8), (300_001, 8, 1), (1 << 20, 3, 3), (5000, 4, 8),
+                                   (70_000, 5, 2), (4096, 1, 1)])
+def test_small_products_of_long_operands(env, dtype, k, m, n):
+    """X.T @ Y for tall X and Y of a few columns (a Gram matrix, the right-hand
+    side of normal equations): slices of K on many blocks, partial sums added
+    in a fixed order.  Transposed views of row-major operands (rows read as
+    words where m and n are 4 or 8), row-major ones, views of wider rows,
+    alpha and beta, C in both layouts; every element against float64, and
+    twice the same bits."""
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(k + m + n)
+    x = rng.standard_normal((k, m + 1)).astype(dtype)
+    y = rng.standard_normal((k, n + 1)).astype(dtype)
+    c0 = rng.standard_normal((m, n)).astype(dtype)
+    tol = 1e-5 if dtype == np.float32 else 1e-13
+    name = "sgemm_inner" if dtype == np.float32 else "dgemm_inner"
+    xs, ys = np.ascontiguousarray(x[:, :m]), np.ascontiguousarray(y[:, :n])
+    cases = [(hip.asarray(xs).T, hip.asarray(ys)),                          # rows of m and n
+             (hip.asarray(x)[:, :m].T, hip.asarray(y)[:, :n]),              # of wider rows
+             (hip.asarray(np.ascontiguousarray(xs.T)), hip.asarray(ys)),    # X.T row-major
+             (hip.asarray(xs).T, hip.asarray(np.ascontiguousarray(ys.T)).T)]
+    for d_a, d_b in cases:
+        for fc in (False, True):
+            d_c = _to_dev(hip, c0.T.copy().T if fc else c0)
+            ops.gemm(d_a, d_b, d_c, 1.5, -0.5)
+            assert mrt.last_kernel() == name
+            first = d_c.asnumpy()
+            _check_scaled(first, xs.T, ys, c0, 1.5, -0.5, tol)
+            d_c = _to_dev(hip, c0.T.copy().T if fc else c0)
+            ops.gemm(d_a, d_b, d_c, 1.5, -0.5)
+            assert np.array_equal(d_c.asnumpy(), first)
+    d_c = hip.asarray(np.full((m, n), np.nan, dtype))
+    ops.gemm(cases[0][0], cases[0][1], d_c, 1.0, 0.0)
+    _check_scaled(d_c.asnumpy(), xs.T, ys, np.zeros((m, n), dtype), 1.0, 0.0, tol)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("m,k,n", [(16, 1 << 18, 16), (32, 100_003, 20), (100, 50_000, 60),
+                                   (128, 1 << 17, 128), (300, 1 << 15, 300), (10, 4099, 12)])
+def test_few_tiles_with_a_long_k(env, dtype, m, k, n):
+    """Results of a few tiles from long operands: K is cut into as many
+    slices as fill the GPU, on the strided kernel for the smallest results
+    and on the guarded tiles from a quarter of a tile on."""
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(m + k + n)
+    x = rng.standard_normal((k, m)).astype(dtype)
+    b = rng.standard_normal((k, n)).astype(dtype)
+    c0 = rng.standard_normal((m, n)).astype(dtype)
+    tol = 1e-5 if dtype == np.float32 else 1e-13
+    for d_a, a in ((hip.asarray(x).T, x.T), (hip.asarray(np.ascontiguousarray(x.T)), x.T)):
+        d_c = hip.asarray(c0)
+        ops.gemm(d_a, hip.asarray(b), d_c, 1.5, -0.5)
+        assert "_splitk" in mrt.last_kernel(), mrt.last_kernel()
+        assert ("generic" in mrt.last_kernel()) == (m * n < 4096)
+        _check_scaled(d_c.asnumpy(), a, b, c0, 1.5, -0.5, tol)
+
+
 def test_identity_and_linearity_full_size(env):
     """Configuration 5 (4096^3): rows checked against float64, plus
     size-independent properties: A @ I == A exactly, and linearity."""
