@@ -418,6 +418,36 @@ def test_long_times_thin(env, dtype, long, k, thin):
                           1.0, 0.0, tol)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("thin", [9, 12, 16])
+def test_up_to_sixteen_vectors_against_columns(env, dtype, thin):
+    """Nine to sixteen rows times a long matrix with unit stride along its
+    long dimension (and the transposed problem) stay on the column kernel;
+    with unit stride along k they go to the tiles."""
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(thin)
+    k, long = 1000, 3004
+    a = rng.standard_normal((thin, k)).astype(dtype)
+    b = rng.standard_normal((k, long)).astype(dtype)
+    c0 = rng.standard_normal((thin, long)).astype(dtype)
+    tol = 1e-5 if dtype == np.float32 else 1e-13
+    name = ("s" if dtype == np.float32 else "d") + "gemm_thin_cols"
+    d_c = hip.asarray(c0)
+    ops.gemm(hip.asarray(a), hip.asarray(b), d_c, 1.5, -0.5)
+    assert mrt.last_kernel() == name
+    _check_scaled(d_c.asnumpy(), a, b, c0, 1.5, -0.5, tol)
+    # (b.T a.T): the long operand first, its unit stride still along `long`
+    d_t = hip.asarray(np.ascontiguousarray(c0.T))
+    ops.gemm(hip.asarray(b).T, hip.asarray(a).T, d_t, 1.5, -0.5)
+    assert mrt.last_kernel() == name
+    _check_scaled(d_t.asnumpy(), b.T, a.T, c0.T, 1.5, -0.5, tol)
+    # unit stride along k: not this kernel's
+    d_c = hip.asarray(c0)
+    ops.gemm(hip.asarray(a), hip.asarray(np.ascontiguousarray(b.T)).T, d_c, 1.5, -0.5)
+    assert "thin" not in mrt.last_kernel()
+    _check_scaled(d_c.asnumpy(), a, b, c0, 1.5, -0.5, tol)
+
+
 def test_thin_products_do_not_mix_in_what_lies_beyond(env):
     """An infinity in the long operand's padding, or in the thin one's, stays
     out of the sums (a product with zero would make it a NaN)."""
