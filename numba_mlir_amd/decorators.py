@@ -112,6 +112,8 @@ def _reduce_nd(op, x, axis):
     integers, as NumPy does."""
     if x.dtype == np.bool_:
         x = _CAST_TO[np.int64](x)
+    if axis is None and not (x.is_c_contiguous() or x.is_f_contiguous()):
+        x = _copy(x)                      # a strided view: its elements, densely
     if x.ndim <= 2 or not x.is_c_contiguous():
         return op(x, axis=axis)
     if axis is None:
@@ -178,6 +180,171 @@ def _fill(array, value):
         _FILL.append(Dispatcher(_fill_body))
     _FILL[0]._run([array, value])
 
+
+
+def _copy(x):
+    """A dense C-ordered copy on x's device (numpy/funcs.py:255-262)."""
+    out = HipNdArray.empty(x.shape, x.dtype, device=x.ctx.device)
+    if out.size:
+        _fill(out, x)
+    return out
+
+
+def _arange_body(out, start, step):
+    i = kernel_impl.get_global_id(0)
+    out[i] = start + i * step
+
+
+def _eye_body(out, k):
+    i = kernel_impl.get_global_id(0)
+    j = kernel_impl.get_global_id(1)
+    out[i, j] = 1 if j - i == k else 0
+
+
+def _tril_body(a, out, k):
+    i = kernel_impl.get_global_id(0)
+    j = kernel_impl.get_global_id(1)
+    out[i, j] = a[i, j] if j - i <= k else 0
+
+
+def _triu_body(a, out, k):
+    i = kernel_impl.get_global_id(0)
+    j = kernel_impl.get_global_id(1)
+    out[i, j] = a[i, j] if j - i >= k else 0
+
+
+def _outer_body(a, b):
+    return a * b
+
+
+def _center_body(x, mean):
+    return x - mean
+
+
+def _scale_body(x, factor):
+    return x * factor
+
+
+class _LazyKernels(dict):
+    def __missing__(self, body):
+        self[body] = kernel_impl.kernel(body)
+        return self[body]
+
+
+class _LazyFunctions(dict):
+    def __missing__(self, body):
+        self[body] = Dispatcher(body)
+        return self[body]
+
+
+_KERNELS = _LazyKernels()
+_FUNCTIONS = _LazyFunctions()
+
+
+def _arange(ctx, *args, dtype=None):
+    """numpy.arange on the device (numpy/funcs.py:642-668): the same length
+    and type as NumPy gives, element i = start + i step."""
+    if not 1 <= len(args) <= 3:
+        raise TypeError("arange takes start, stop and step")
+    if len(args) == 1:
+        start, stop, step = 0, args[0], 1
+    else:
+        start, stop, step = args[0], args[1], args[2] if len(args) == 3 else 1
+    if step == 0:
+        raise ValueError("Maximum allowed size exceeded")
+    if dtype is None:
+        whole = all(isinstance(v, (int, np.integer)) for v in (start, stop, step))
+        dtype = np.int64 if whole else np.float64
+    dtype = np.dtype(dtype)
+    count = max(0, int(math.ceil((stop - start) / step)))
+    out = HipNdArray.empty((count,), dtype, device=ctx.device)
+    if count:
+        _KERNELS[_arange_body][(count,), ()](out, dtype.type(start), dtype.type(step))
+    return out
+
+
+def _eye(ctx, n, m=None, k=0, dtype=np.float64):
+    """numpy.eye (numpy/funcs.py:670-700)."""
+    m = n if m is None else m
+    out = HipNdArray.empty((int(n), int(m)), dtype, device=ctx.device)
+    if out.size:
+        _KERNELS[_eye_body][(int(n), int(m)), ()](out, int(k))
+    return out
+
+
+def _tri(x, k, lower):
+    """numpy.tril / triu of a matrix."""
+    if x.ndim != 2:
+        raise NotImplementedError("tril and triu are implemented for matrices")
+    out = HipNdArray.empty(x.shape, x.dtype, device=x.ctx.device)
+    if out.size:
+        _KERNELS[_tril_body if lower else _triu_body][x.shape, ()](x, out, int(k))
+    return out
+
+
+def _outer(a, b):
+    """numpy.outer: the operands flattened, one fused map over the product's shape."""
+    a = a if a.ndim == 1 else _copy(a).reshape((a.size,))
+    b = b if b.ndim == 1 else _copy(b).reshape((b.size,))
+    return _FUNCTIONS[_outer_body]._run([a.reshape((a.size, 1)), b.reshape((1, b.size))])
+
+
+def _concatenate(arrays, axis=0):
+    """numpy.concatenate: one strided store per piece into the new array."""
+    if not arrays:
+        raise ValueError("need at least one array to concatenate")
+    first = arrays[0]
+    if not -first.ndim <= axis < first.ndim:
+        raise ValueError(f"axis {axis} is out of bounds for array of dimension {first.ndim}")
+    axis %= first.ndim
+    for a in arrays[1:]:
+        if a.ndim != first.ndim or \
+                any(p != q for d, (p, q) in enumerate(zip(a.shape, first.shape)) if d != axis):
+            raise ValueError("all the input array dimensions except for the concatenation "
+                             "axis must match exactly")
+    shape = list(first.shape)
+    shape[axis] = sum(a.shape[axis] for a in arrays)
+    out = HipNdArray.empty(tuple(shape), np.result_type(*[a.dtype for a in arrays]),
+                           device=first.ctx.device)
+    at = 0
+    for a in arrays:
+        if a.size:
+            where = tuple(slice(at, at + a.shape[axis]) if d == axis else slice(None)
+                          for d in range(first.ndim))
+            _fill(out[where], a)
+        at += a.shape[axis]
+    return out
+
+
+def _cov(m, y=None, rowvar=True, bias=False, ddof=None):
+    """numpy.cov as the reference builds it (numpy/funcs.py:1455-1549): rows
+    are variables; the result keeps a floating input's type (integers become
+    float64); a single 1-d input gives a scalar."""
+    scalar = m.ndim == 1 and y is None
+    rows = []
+    for x in (m, y):
+        if x is None:
+            continue
+        if x.ndim > 2:
+            raise ValueError("m has more than 2 dimensions")
+        x = x.reshape((1, x.size)) if x.ndim < 2 else x
+        if not rowvar and (y is None or x.shape[0] != 1):
+            x = x.T
+        rows.append(x)
+    dtype = np.result_type(*[x.dtype for x in rows])
+    if dtype.kind != "f":
+        dtype = np.dtype(np.float64)
+    rows = [x if x.dtype == dtype else _CAST_TO[dtype.type]._run([x]) for x in rows]
+    X = rows[0] if len(rows) == 1 else _concatenate(rows, 0)
+    if ddof is None:
+        ddof = 0 if bias else 1
+    fact = max(X.shape[1] - ddof, 0.0)
+    mean = _mean(X, 1)
+    centered = _FUNCTIONS[_center_body]._run([X, mean.reshape((X.shape[0], 1))])
+    c = _dot(centered, centered.T)
+    with np.errstate(divide="ignore"):
+        c = _FUNCTIONS[_scale_body]._run([c, dtype.type(np.true_divide(1, fact))])
+    return c.asnumpy()[0, 0] if scalar else c
 
 
 def _mean(x, axis):
@@ -668,6 +835,12 @@ class Dispatcher:
                     scope = self._host_scope(())
                 env[stage.target] = self._stage_alloc(stage, env, scope, args)
                 continue
+            if stage.kind == "make":
+                if scope is None:
+                    scope = self._host_scope(())
+                env[stage.target] = self._stage_make(stage, env, scope, args)
+                launches.append({"path": "library", "op": stage.op})
+                continue
             if stage.kind == "call":
                 callee = self._resolve(stage.op)
                 value = callee._run([env[n] for n in stage.args])
@@ -684,6 +857,8 @@ class Dispatcher:
                 value = self._stage_map(k, stage, env, scope, launches)
             if stage.kind == "return":
                 self.last_launch = {"path": "staged", "stages": launches}
+                if isinstance(value, HipNdArray) and value.ndim == 0:
+                    value = value.asnumpy()[()]          # one indexed element
                 return value
             if stage.kind == "map":
                 env[stage.target] = value
@@ -888,9 +1063,68 @@ class Dispatcher:
             _fill(out, out.dtype.type(1 if stage.op.startswith("ones") else 0))
         return out
 
+    def _stage_make(self, stage, env, scope, call_args):
+        """np.arange / eye / tril / triu / outer / cov / concatenate / hstack /
+        vstack on the device of the call's arrays."""
+        def host(node):
+            expr = ast.fix_missing_locations(ast.Expression(body=node))
+            return eval(compile(expr, "<argument>", "eval"), scope, dict(env))  # noqa: S307
+
+        where = f"{self.py_func.__name__}, line {stage.node.lineno}"
+        arrays = [env[name] for name in stage.operands]
+        nodes, slots, keywords = stage.args
+        pos = [arrays[slot] if slot is not None else host(node)
+               for node, slot in zip(nodes, slots or [None] * len(nodes))]
+        kws = {key: arrays[value] if isinstance(value, int) else host(value)
+               for key, value in keywords}
+        op = stage.op
+        try:
+            if any(not isinstance(a, HipNdArray) for a in arrays):
+                raise TypeError("the array arguments must be device arrays")
+            ctx = kernel_impl.check_device_args(
+                [a for a in list(call_args) + list(env.values()) if isinstance(a, HipNdArray)])
+            if op == "arange":
+                return _arange(ctx, *pos, **kws)
+            if op == "eye":
+                return _eye(ctx, *pos, **kws)
+            if op in ("tril", "triu"):
+                k = pos[1] if len(pos) > 1 else kws.pop("k", 0)
+                if kws or len(pos) > 2:
+                    raise TypeError("takes an array and k")
+                return _tri(pos[0], k, op == "tril")
+            if op == "outer":
+                if kws or len(pos) != 2:
+                    raise TypeError("takes two arrays")
+                return _outer(*pos)
+            if op == "cov":
+                return _cov(*pos, **kws)
+            axis = pos[0] if pos else kws.pop("axis", 0)
+            if kws or len(pos) > 1:
+                raise TypeError("takes a tuple of arrays and an axis")
+            if op == "concatenate":
+                return _concatenate(arrays, axis)
+            if pos:
+                raise TypeError("takes a tuple of arrays")
+            if op == "hstack":
+                arrays = [a.reshape((1,)) if a.ndim == 0 else a for a in arrays]
+                return _concatenate(arrays, 0 if arrays and arrays[0].ndim == 1 else 1)
+            arrays = [a.reshape((1, a.size)) if a.ndim < 2 else a for a in arrays]
+            return _concatenate(arrays, 0)
+        except (TypeError, ValueError, NotImplementedError) as exc:
+            raise kernel_compiler.KernelCompileError(f"{where}: np.{op}: {exc}") from exc
+
     def _stage_view(self, stage, env, scope):
         x = env[stage.operands[0]]
         where = f"{self.py_func.__name__}, line {stage.node.lineno}"
+        if stage.op == "getitem":
+            node = ast.Subscript(value=ast.Name(id="_nmk_sliced", ctx=ast.Load()),
+                                 slice=stage.args[0], ctx=ast.Load())
+            expr = ast.fix_missing_locations(ast.Expression(body=node))
+            try:
+                return eval(compile(expr, "<index>", "eval"), scope,  # noqa: S307
+                            dict(env, _nmk_sliced=x))
+            except (TypeError, ValueError, IndexError, NotImplementedError) as exc:
+                raise kernel_compiler.KernelCompileError(f"{where}: {exc}") from exc
         args = []
         for node in stage.args:
             expr = ast.fix_missing_locations(ast.Expression(body=node))
@@ -902,6 +1136,10 @@ class Dispatcher:
                 return x.reshape(*args)
             if stage.op == "ravel":
                 return x.reshape((x.size,))
+            if stage.op in ("copy", "flatten"):
+                if args:
+                    raise NotImplementedError("the order argument is not supported")
+                return _copy(x) if stage.op == "copy" else _copy(x).reshape((x.size,))
             if stage.op == "flip":
                 # numpy.flip (numpy/funcs.py:236-253): negative strides
                 if len(args) > 1 or (args and not (args[0] is None or

@@ -19,7 +19,12 @@ import ast
 
 REDUCTIONS = ("sum", "prod", "min", "max", "amin", "amax", "mean")
 CONTRACTIONS = ("dot",)
-VIEWS = ("reshape", "transpose", "ravel", "flip")    # no data moves
+VIEWS = ("reshape", "transpose", "ravel", "flip",     # no data moves
+         "copy", "flatten")                           # a dense copy
+# np.<name>(...) that builds a new array on the device: which positional
+# arguments are arrays ("tuple": the first is a tuple of them)
+MAKERS = {"arange": (), "eye": (), "tril": (0,), "triu": (0,), "outer": (0, 1),
+          "cov": (0, 1), "concatenate": "tuple", "hstack": "tuple", "vstack": "tuple"}
 ALLOCATIONS = ("empty", "zeros", "ones", "empty_like", "zeros_like", "ones_like")
 # NumPy functions that take an `out` array after this many operands
 # (reference: numpy/funcs.py registers them with out="out")
@@ -116,6 +121,8 @@ class _Splitter(ast.NodeTransformer):
             self.plan.add(stage)
             self.plan.library_stages += 1
             return ast.copy_location(ast.Name(id=stage.target, ctx=ast.Load()), node)
+        if numpy_function and name in MAKERS:
+            return self._make(node, name)
         if numpy_function and name in OUT_AFTER:
             return self._with_out(node, OUT_AFTER[name])
         if name not in REDUCTIONS + CONTRACTIONS:
@@ -146,6 +153,55 @@ class _Splitter(ast.NodeTransformer):
                             node=node))
         self.plan.library_stages += 1
         return ast.copy_location(ast.Name(id=target, ctx=ast.Load()), node)
+
+    def _make(self, node, name):
+        """np.arange / eye / tril / triu / outer / cov / concatenate / hstack /
+        vstack (reference: numpy/funcs.py:255-310, 642-700, 1536-1549): the
+        array arguments become operands, the others stay host expressions."""
+        where = MAKERS[name]
+        args = list(node.args)
+        operands, slots = [], []          # slots: per positional, operand index or None
+        if where == "tuple":
+            if not args or not isinstance(args[0], (ast.Tuple, ast.List)):
+                raise NotStraightLine(f"line {node.lineno}: np.{name} takes a tuple of "
+                                      "arrays here")
+            operands = [self._operand(e) for e in args[0].elts]
+            args = args[1:]
+        else:
+            for at, arg in enumerate(args):
+                is_none = isinstance(arg, ast.Constant) and arg.value is None
+                if at in where and not is_none:
+                    slots.append(len(operands))
+                    operands.append(self._operand(arg))
+                else:
+                    slots.append(None)
+        keywords = []
+        for k in node.keywords:
+            if name == "cov" and k.arg == "y" and \
+                    not (isinstance(k.value, ast.Constant) and k.value.value is None):
+                keywords.append(("y", len(operands)))
+                operands.append(self._operand(k.value))
+            else:
+                keywords.append((k.arg, k.value))
+        stage = Stage("make", self.plan.fresh(), op=name, operands=operands, node=node)
+        stage.args = (args, slots, keywords)
+        self.plan.add(stage)
+        self.plan.library_stages += 1
+        return ast.copy_location(ast.Name(id=stage.target, ctx=ast.Load()), node)
+
+    def visit_Subscript(self, node):
+        """x[a:b], x[:, j], x[::2], x[i] of a local array: a view (of one
+        element when every axis is indexed)."""
+        self.generic_visit(node)
+        if not isinstance(node.ctx, ast.Load) or not isinstance(node.value, ast.Name) or \
+                node.value.id not in self.plan.locals or _is_whole_slice(node.slice):
+            return node
+        stage = Stage("view", self.plan.fresh(), op="getitem", operands=[node.value.id],
+                      node=node)
+        stage.args = [node.slice]
+        self.plan.add(stage)
+        self.plan.library_stages += 1
+        return ast.copy_location(ast.Name(id=stage.target, ctx=ast.Load()), node)
 
     def _with_out(self, node, operands):
         """np.add(a, b, out) / np.add(a, b, out=out): a store into ``out``,
@@ -291,10 +347,16 @@ class Plan:
                     [a for a in stage.args if isinstance(a, str)] + \
                     ([stage.kwargs["out"]] if "out" in stage.kwargs else []):
                 uses[name] = uses.get(name, 0) + 1
-            if stage.kind in ("view", "alloc"):
+            if stage.kind in ("view", "alloc", "make"):
                 # their argument expressions may name anything
-                nodes = stage.args[0] + [k.value for k in stage.args[1]] \
-                    if stage.kind == "alloc" else stage.args
+                if stage.kind == "alloc":
+                    nodes = stage.args[0] + [k.value for k in stage.args[1]]
+                elif stage.kind == "make":
+                    nodes = [a for a, slot in zip(stage.args[0], stage.args[1] or
+                                                  [None] * len(stage.args[0])) if slot is None] + \
+                        [v for _, v in stage.args[2] if isinstance(v, ast.AST)]
+                else:
+                    nodes = stage.args
                 for node in nodes:
                     for n in ast.walk(node):
                         if isinstance(n, ast.Name):

@@ -469,3 +469,98 @@ def row_mean_abs(a, b, s):
 
 def column_counts(a, b):
     return np.sum(a > b, axis=0)
+
+
+# -- arrays built and sliced inside a compiled function ----------------------
+# (numpy/funcs.py:236-310 views and copies, 642-700 arange and eye, 1455-1549
+# cov; tril/triu/outer/concatenate/hstack/vstack are registered there too)
+def built_arange_steps(a):
+    return a[:50] * np.arange(0.5, 25.5, 0.5)
+
+
+def built_arange_count(a):
+    return a + np.arange(5000)
+
+
+def built_arange_down(a):
+    return np.arange(10, 2, -3) + 0 * a[:3]
+
+
+def built_eye(a):
+    return a @ np.eye(200, 100, k=-3)
+
+
+def built_eye_square(a):
+    return a[:200] + np.eye(200)
+
+
+def built_triangles(a):
+    return np.triu(a, 2) - np.tril(a, -1)
+
+
+def built_outer(a, b):
+    return np.outer(a + 1, b * 2).sum(axis=0)
+
+
+def built_concatenate_columns(a, b):
+    return np.concatenate((a, b), axis=1)
+
+
+def built_concatenate_three(a, b):
+    return np.concatenate((a, b, a), axis=-2)
+
+
+def built_vstack(a, b):
+    return np.vstack((a, b))
+
+
+def built_hstack(a, b):
+    return np.hstack((a, b))
+
+
+def built_cov(a):
+    return np.cov(a)
+
+
+def built_cov_pair(a, b):
+    return np.cov(a, b)
+
+
+def built_cov_columns(a):
+    return np.cov(a, rowvar=False, bias=True)
+
+
+def sliced_sums(a):
+    return a[1:-1, ::2].sum() + a[:, 3].sum() + a[5].sum()
+
+
+def sliced_differences(a):
+    return (a[1:] - a[:-1]).sum(axis=0)
+
+
+def sliced_row(a):
+    return a[5] * 2.0
+
+
+def sliced_row_part(a):
+    return a[5, 1:4] * 2.0
+
+
+def sliced_element(a):
+    return a - a[0, 0]
+
+
+def sliced_element_returned(a):
+    return a[2, 3]
+
+
+def copied_transpose(a):
+    return np.copy(a.T)
+
+
+def copied_method(a):
+    return a.copy()
+
+
+def flattened_transpose(a):
+    return a.T.flatten()

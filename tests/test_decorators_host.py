@@ -82,3 +82,31 @@ def test_sequential_loops_over_an_array_are_refused_not_run_per_element():
 def test_stage_kernels_of_a_lambda_get_identifier_names():
     f = njit(lambda a: np.sum(a * a, axis=1))
     assert f._stage_stem == "lambda" and njit(_by_name)._stage_stem == "_by_name"
+
+
+def test_arrays_built_and_sliced_become_stages_of_their_own():
+    """np.concatenate / tril / outer / arange and basic indexing of a local
+    array split a straight-line body: array arguments become operands
+    (expressions materialised by a map first), the rest stays host
+    expressions."""
+    import ast
+
+    from numba_mlir_amd.mlir import staging
+
+    src = ("def f(a, b):\n"
+           "    c = np.concatenate((a, b + 1), axis=0)\n"
+           "    d = np.tril(c[1:5], -1)\n"
+           "    e = c[2] + d[0, 0]\n"
+           "    return np.outer(a, b).copy() + np.arange(3) + a.shape[0]\n")
+    plan = staging.plan_of(ast.parse(src).body[0], lambda name: name == "np")
+    kinds = [(st.kind, st.op) for st in plan.stages if st.kind in ("make", "view")]
+    assert kinds == [("make", "concatenate"), ("view", "getitem"), ("make", "tril"),
+                     ("view", "getitem"), ("view", "getitem"), ("make", "outer"),
+                     ("view", "copy"), ("make", "arange")]
+    concatenate = next(st for st in plan.stages if st.op == "concatenate")
+    assert concatenate.operands[0] == "a" and concatenate.operands[1].startswith("_nmk_t")
+    assert [key for key, _ in concatenate.args[2]] == ["axis"]
+    tril = next(st for st in plan.stages if st.op == "tril")
+    assert tril.args[1] == [0, None]          # the array, then k on the host
+    # a.shape[0] is not an index of a local array: it stays in the expression
+    assert "a.shape[0]" in ast.unparse(plan.stages[-1].expr)

@@ -733,6 +733,55 @@ def test_products_with_vectors(env, func):
     np.testing.assert_allclose(got, v @ v, rtol=1e-12)
 
 
+@pytest.mark.parametrize("name,operands", [
+    ("built_arange_steps", "x"), ("built_arange_count", "x"), ("built_arange_down", "x"),
+    ("built_eye", "A"), ("built_eye_square", "A"), ("built_triangles", "A"),
+    ("built_outer", "uv"), ("built_concatenate_columns", "AC"),
+    ("built_concatenate_three", "AR"), ("built_vstack", "AR"), ("built_hstack", "AC"),
+    ("built_cov", "S"), ("built_cov_pair", "ST"), ("built_cov_columns", "C"),
+    ("sliced_sums", "A"), ("sliced_differences", "A"), ("sliced_row", "A"),
+    ("sliced_row_part", "A"), ("sliced_element", "A"), ("sliced_element_returned", "A"),
+    ("copied_transpose", "A"), ("copied_method", "A"), ("flattened_transpose", "A")])
+def test_arrays_built_and_sliced_inside(env, name, operands):
+    """np.arange / eye / tril / triu / outer / concatenate / hstack / vstack /
+    cov / copy / flatten and basic indexing inside a compiled function: shape,
+    type and values as NumPy gives them for the same function."""
+    hip = env[0]
+    rng = np.random.default_rng(17)
+    A = rng.standard_normal((300, 200))
+    pool = {"x": rng.standard_normal(5000), "A": A, "u": rng.standard_normal(300),
+            "v": rng.standard_normal(200), "C": A[:, :7] * 2, "R": A[:9] * 2,
+            "S": A[:6], "T": A[10:12]}
+    func = getattr(cases, name)
+    host = [np.ascontiguousarray(pool[k]) for k in operands]
+    want = func(*host)
+    got = njit(func)(*[hip.asarray(a) for a in host])
+    got = got.asnumpy() if hasattr(got, "asnumpy") else got
+    assert np.shape(got) == np.shape(want)
+    assert np.asarray(got).dtype == np.asarray(want).dtype
+    np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-12)
+
+
+def test_cov_keeps_float32_and_one_variable_is_a_scalar(env):
+    """The reference's cov keeps the input's floating type (numpy/funcs.py:
+    1490-1527: only integers become float64) and returns a scalar for one
+    1-d variable (1547-1548)."""
+    hip = env[0]
+    rng = np.random.default_rng(18)
+    a = rng.standard_normal((5, 4000)).astype(np.float32)
+    f = njit(cases.built_cov)
+    got = f(hip.asarray(a)).asnumpy()
+    assert got.dtype == np.float32 and got.shape == (5, 5)
+    np.testing.assert_allclose(got, np.cov(a.astype(np.float64)), rtol=1e-4, atol=1e-5)
+    one = f(hip.asarray(a[0].astype(np.float64)))
+    assert np.shape(one) == ()
+    np.testing.assert_allclose(one, np.cov(a[0].astype(np.float64)), rtol=1e-12)
+    counts = rng.integers(0, 50, (3, 1000))
+    got = f(hip.asarray(counts)).asnumpy()
+    assert got.dtype == np.float64
+    np.testing.assert_allclose(got, np.cov(counts), rtol=1e-12)
+
+
 def test_pairwise_as_nested_prange_loops(env):
     """test_pairwise2 (test_gpu.py:2226-2266): the distance body as two
     prange loops around a serial one, on the reference's fixture."""
