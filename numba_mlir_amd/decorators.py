@@ -190,6 +190,26 @@ def _copy(x):
     return out
 
 
+_CASTS = {}
+
+
+def _astype(x, dtype):
+    """x converted element by element into a new dense array."""
+    if dtype == x.dtype:
+        return _copy(x)
+    name = dtype.name
+    if dtype.kind not in "iuf" or not hasattr(np, name):
+        raise NotImplementedError(f"conversion to {name} is not implemented")
+    if name not in _CASTS:
+        source = f"def _to_{name}(x):\n    return np.{name}(x)\n"
+        scope = {"np": np}
+        exec(source, scope)                                   # noqa: S102
+        func = scope[f"_to_{name}"]
+        func.__nmk_ast__ = ast.parse(source).body[0]
+        _CASTS[name] = func
+    return _CAST_TO_ANY[_CASTS[name]]._run([x])
+
+
 def _arange_body(out, start, step):
     i = kernel_impl.get_global_id(0)
     out[i] = start + i * step
@@ -239,6 +259,7 @@ class _LazyFunctions(dict):
 
 _KERNELS = _LazyKernels()
 _FUNCTIONS = _LazyFunctions()
+_CAST_TO_ANY = _LazyFunctions()
 
 
 def _arange(ctx, *args, dtype=None):
@@ -1105,6 +1126,10 @@ class Dispatcher:
                 return _concatenate(arrays, axis)
             if pos:
                 raise TypeError("takes a tuple of arrays")
+            if op == "dstack":
+                arrays = [a.reshape((1, a.size, 1)) if a.ndim < 2 else
+                          a.reshape(a.shape + (1,)) if a.ndim == 2 else a for a in arrays]
+                return _concatenate(arrays, 2)
             if op == "hstack":
                 arrays = [a.reshape((1,)) if a.ndim == 0 else a for a in arrays]
                 return _concatenate(arrays, 0 if arrays and arrays[0].ndim == 1 else 1)
@@ -1116,6 +1141,14 @@ class Dispatcher:
     def _stage_view(self, stage, env, scope):
         x = env[stage.operands[0]]
         where = f"{self.py_func.__name__}, line {stage.node.lineno}"
+        if stage.op == "len":
+            return len(x)
+        if stage.op in staging.ARRAY_FACTS:
+            if stage.op == "strides" and isinstance(x, HipNdArray):
+                return tuple(st * x.dtype.itemsize for st in x.elem_strides)
+            if stage.op == "itemsize" and isinstance(x, HipNdArray):
+                return x.dtype.itemsize
+            return getattr(x, stage.op)
         if stage.op == "getitem":
             node = ast.Subscript(value=ast.Name(id="_nmk_sliced", ctx=ast.Load()),
                                  slice=stage.args[0], ctx=ast.Load())
@@ -1140,6 +1173,13 @@ class Dispatcher:
                 if args:
                     raise NotImplementedError("the order argument is not supported")
                 return _copy(x) if stage.op == "copy" else _copy(x).reshape((x.size,))
+            if stage.op == "asfortranarray":
+                # (numpy/funcs.py:1243-1246: a copy; the layout is the compiler's)
+                return _copy(x.T).T
+            if stage.op == "astype":
+                if len(args) != 1:
+                    raise TypeError("astype takes a type")
+                return _astype(x, np.dtype(args[0]))
             if stage.op == "flip":
                 # numpy.flip (numpy/funcs.py:236-253): negative strides
                 if len(args) > 1 or (args and not (args[0] is None or

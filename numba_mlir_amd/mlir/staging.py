@@ -20,11 +20,14 @@ import ast
 REDUCTIONS = ("sum", "prod", "min", "max", "amin", "amax", "mean")
 CONTRACTIONS = ("dot",)
 VIEWS = ("reshape", "transpose", "ravel", "flip",     # no data moves
-         "copy", "flatten")                           # a dense copy
+         "copy", "flatten", "astype",                 # a dense copy
+         "asfortranarray")
+# what an array says about itself: host values (numpy/funcs.py:1197-1300)
+ARRAY_FACTS = ("shape", "size", "ndim", "itemsize", "strides", "dtype")
 # np.<name>(...) that builds a new array on the device: which positional
 # arguments are arrays ("tuple": the first is a tuple of them)
 MAKERS = {"arange": (), "eye": (), "tril": (0,), "triu": (0,), "outer": (0, 1),
-          "cov": (0, 1), "concatenate": "tuple", "hstack": "tuple", "vstack": "tuple"}
+          "cov": (0, 1), "concatenate": "tuple", "hstack": "tuple", "vstack": "tuple", "dstack": "tuple"}
 ALLOCATIONS = ("empty", "zeros", "ones", "empty_like", "zeros_like", "ones_like")
 # NumPy functions that take an `out` array after this many operands
 # (reference: numpy/funcs.py registers them with out="out")
@@ -79,6 +82,11 @@ def _is_whole_slice(node):
     return full(node)
 
 
+def _has_slice(node):
+    index = node.elts if isinstance(node, ast.Tuple) else [node]
+    return any(isinstance(e, ast.Slice) for e in index)
+
+
 class _Splitter(ast.NodeTransformer):
     def __init__(self, plan):
         self.plan = plan
@@ -108,6 +116,10 @@ class _Splitter(ast.NodeTransformer):
     def visit_Call(self, node):
         self.generic_visit(node)              # innermost stages first
         func = node.func
+        if isinstance(func, ast.Name) and func.id == "len" and "len" not in self.plan.locals \
+                and len(node.args) == 1 and not node.keywords and \
+                isinstance(node.args[0], ast.Name) and node.args[0].id in self.plan.locals:
+            return self._fact(node, "len", node.args[0].id)
         if not isinstance(func, ast.Attribute):
             return node
         name = func.attr
@@ -238,8 +250,20 @@ class _Splitter(ast.NodeTransformer):
         self.plan.library_stages += 1
         return ast.copy_location(ast.Name(id=stage.target, ctx=ast.Load()), node)
 
+    def _fact(self, node, name, operand):
+        """x.shape, len(x), ...: a host value taken from the array as it is at
+        that point (inside a fused map the array is seen per element, through
+        a view with its dimensions merged)."""
+        stage = Stage("view", self.plan.fresh(), op=name, operands=[operand], node=node)
+        self.plan.add(stage)
+        self.plan.library_stages += 1
+        return ast.copy_location(ast.Name(id=stage.target, ctx=ast.Load()), node)
+
     def visit_Attribute(self, node):
         self.generic_visit(node)
+        if node.attr in ARRAY_FACTS and isinstance(node.ctx, ast.Load) and \
+                isinstance(node.value, ast.Name) and node.value.id in self.plan.locals:
+            return self._fact(node, node.attr, node.value.id)
         if node.attr != "T" or not isinstance(node.ctx, ast.Load):
             return node
         if isinstance(node.value, ast.Name) and node.value.id not in self.plan.locals:
@@ -284,6 +308,15 @@ class Plan:
                 raise NotStraightLine("statements after the return")
             if isinstance(stmt, ast.Expr) and isinstance(stmt.value, ast.Constant):
                 continue                                       # a docstring
+            if isinstance(stmt, ast.AugAssign) and isinstance(stmt.target, ast.Subscript) and \
+                    isinstance(stmt.target.value, ast.Name) and _has_slice(stmt.target.slice):
+                # x[1:] += ...: x[1:] = x[1:] + ...
+                import copy
+                load = copy.deepcopy(stmt.target)
+                load.ctx = ast.Load()
+                value = ast.copy_location(ast.BinOp(left=load, op=stmt.op, right=stmt.value),
+                                          stmt)
+                stmt = ast.copy_location(ast.Assign(targets=[stmt.target], value=value), stmt)
             if isinstance(stmt, ast.AugAssign) and isinstance(stmt.target, ast.Name):
                 load = ast.copy_location(ast.Name(id=stmt.target.id, ctx=ast.Load()), stmt)
                 value = ast.copy_location(ast.BinOp(left=load, op=stmt.op, right=stmt.value),
@@ -316,6 +349,16 @@ class Plan:
                 if isinstance(target, ast.Subscript) and isinstance(target.value, ast.Name) \
                         and _is_whole_slice(target.slice):
                     self.add(Stage("store", target.value.id, value, node=stmt))
+                    continue
+                if isinstance(target, ast.Subscript) and isinstance(target.value, ast.Name) \
+                        and target.value.id in self.locals and _has_slice(target.slice):
+                    # x[1:5] = ..., x[:, 3] = ...: a store into a view of x
+                    view = Stage("view", self.fresh(), op="getitem",
+                                 operands=[target.value.id], node=stmt)
+                    view.args = [splitter.visit(target.slice)]
+                    self.add(view)
+                    self.library_stages += 1
+                    self.add(Stage("store", view.target, value, node=stmt))
                     continue
             elif isinstance(stmt, ast.Return):
                 if stmt.value is not None:

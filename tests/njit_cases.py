@@ -564,3 +564,52 @@ def copied_method(a):
 
 def flattened_transpose(a):
     return a.T.flatten()
+
+
+def facts_in_a_map(a):
+    return a * a.shape[0] + a.size + a.ndim
+
+
+def facts_after_a_reduction(a):
+    return np.sum(a, axis=0) / a.shape[0]
+
+
+def facts_of_layout(a):
+    return a * a.itemsize + a.strides[0] + len(a) + a.shape[1]
+
+
+def facts_dtype(a):
+    return np.zeros(a.shape, a.dtype) + a
+
+
+def converted(a):
+    return (a * 10).astype(np.int32).astype(np.float64) * 0.5
+
+
+def converted_down(a):
+    return a.astype(np.float32)
+
+
+def built_dstack(a, b):
+    return np.dstack((a, b))
+
+
+def copied_fortran(a):
+    return np.asfortranarray(a) * 2.0
+
+
+def store_slice(a, b):
+    a[1:5] = b[:4] * 2.0
+
+
+def store_column(a, b):
+    a[:, 3] = 1.5
+
+
+def store_block_and_update_row(a, b):
+    a[1:-1, 2:5] = b[:-2, :3] * 2.0
+    a[0, :] -= 1.0
+
+
+def update_shifted(a, b):
+    a[1:] += b[:-1]

@@ -102,11 +102,31 @@ def test_arrays_built_and_sliced_become_stages_of_their_own():
     kinds = [(st.kind, st.op) for st in plan.stages if st.kind in ("make", "view")]
     assert kinds == [("make", "concatenate"), ("view", "getitem"), ("make", "tril"),
                      ("view", "getitem"), ("view", "getitem"), ("make", "outer"),
-                     ("view", "copy"), ("make", "arange")]
+                     ("view", "copy"), ("make", "arange"), ("view", "shape"),
+                     ("view", "getitem")]
     concatenate = next(st for st in plan.stages if st.op == "concatenate")
     assert concatenate.operands[0] == "a" and concatenate.operands[1].startswith("_nmk_t")
     assert [key for key, _ in concatenate.args[2]] == ["axis"]
     tril = next(st for st in plan.stages if st.op == "tril")
     assert tril.args[1] == [0, None]          # the array, then k on the host
-    # a.shape[0] is not an index of a local array: it stays in the expression
-    assert "a.shape[0]" in ast.unparse(plan.stages[-1].expr)
+    # a.shape[0] is read from the array on the host, not inside the map (where
+    # the array is a view with its dimensions merged)
+    assert "shape" not in ast.unparse(plan.stages[-1].expr)
+
+
+def test_stores_into_slices_are_stores_into_views():
+    import ast
+
+    from numba_mlir_amd.mlir import staging
+
+    src = ("def f(a, b):\n"
+           "    a[1:-1, 2:5] = b[:-2, :3] * 2.0\n"
+           "    a[0, :] -= len(b)\n")
+    plan = staging.plan_of(ast.parse(src).body[0], lambda name: name == "np")
+    kinds = [(st.kind, st.op) for st in plan.stages]
+    assert kinds == [("view", "getitem"), ("view", "getitem"), ("store", None),
+                     ("view", "getitem"), ("view", "len"), ("view", "getitem"),
+                     ("store", None)]
+    # each store goes into the view made just before it
+    assert plan.stages[2].target == plan.stages[1].target
+    assert plan.stages[6].target == plan.stages[5].target

@@ -741,7 +741,10 @@ def test_products_with_vectors(env, func):
     ("built_cov", "S"), ("built_cov_pair", "ST"), ("built_cov_columns", "C"),
     ("sliced_sums", "A"), ("sliced_differences", "A"), ("sliced_row", "A"),
     ("sliced_row_part", "A"), ("sliced_element", "A"), ("sliced_element_returned", "A"),
-    ("copied_transpose", "A"), ("copied_method", "A"), ("flattened_transpose", "A")])
+    ("copied_transpose", "A"), ("copied_method", "A"), ("flattened_transpose", "A"),
+    ("facts_in_a_map", "A"), ("facts_after_a_reduction", "A"), ("facts_of_layout", "A"),
+    ("facts_dtype", "A"), ("converted", "x"), ("converted_down", "x"),
+    ("built_dstack", "AA"), ("copied_fortran", "A")])
 def test_arrays_built_and_sliced_inside(env, name, operands):
     """np.arange / eye / tril / triu / outer / concatenate / hstack / vstack /
     cov / copy / flatten and basic indexing inside a compiled function: shape,
@@ -760,6 +763,24 @@ def test_arrays_built_and_sliced_inside(env, name, operands):
     assert np.shape(got) == np.shape(want)
     assert np.asarray(got).dtype == np.asarray(want).dtype
     np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("name", ["store_slice", "store_column", "store_block_and_update_row",
+                                  "update_shifted"])
+def test_stores_into_slices(env, name):
+    """x[1:5] = ..., x[:, 3] = ..., x[1:] += ...: stores into views of the
+    array (array.__setitem__ with slices, numpy/funcs.py:1140-1195)."""
+    hip = env[0]
+    rng = np.random.default_rng(19)
+    flat = name in ("store_slice", "update_shifted")
+    a = rng.standard_normal(5000 if flat else (300, 200))
+    b = rng.standard_normal(a.shape)
+    func = getattr(cases, name)
+    want = a.copy()
+    func(want, b)
+    d_a = hip.asarray(a)
+    assert njit(func)(d_a, hip.asarray(b)) is None
+    np.testing.assert_allclose(d_a.asnumpy(), want, rtol=1e-13)
 
 
 def test_cov_keeps_float32_and_one_variable_is_a_scalar(env):
