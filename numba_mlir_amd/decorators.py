@@ -430,6 +430,7 @@ class Dispatcher:
         self._parallel_loop = None     # whether the body has a top-level prange loop
         self._library_form = None      # the one-expression pattern, parsed once
         self._rank = None              # grid dimensions of the prange nest
+        self._asked = None             # parameters whose shape or elements the body reads
         functools.update_wrapper(self, py_func)
 
     # -- entry ---------------------------------------------------------------
@@ -1264,6 +1265,25 @@ class Dispatcher:
                     f"array argument '{owner}' is sequential and is not offloaded; write it "
                     "with prange")
 
+    def _arrays_asked_about(self):
+        """Parameters whose shape, size, length or single elements the body
+        reads."""
+        if self._asked is None:
+            params, asked = set(self._params()), set()
+            for n in ast.walk(self._node):
+                if isinstance(n, ast.Attribute) and n.attr in staging.ARRAY_FACTS and \
+                        isinstance(n.value, ast.Name):
+                    asked.add(n.value.id)
+                elif isinstance(n, ast.Call) and isinstance(n.func, ast.Name) and \
+                        n.func.id == "len" and len(n.args) == 1 and \
+                        isinstance(n.args[0], ast.Name):
+                    asked.add(n.args[0].id)
+                elif isinstance(n, ast.Subscript) and isinstance(n.ctx, ast.Load) and \
+                        isinstance(n.value, ast.Name):
+                    asked.add(n.value.id)
+            self._asked = asked & params
+        return self._asked
+
     def _elementwise(self, args):
         ctx = kernel_impl.check_device_args(args)
         # Everything but addresses and scalar values is fixed by the argument
@@ -1291,7 +1311,24 @@ class Dispatcher:
         shape = np.broadcast_shapes(*[a.shape for a in arrays])
         views = [a.broadcast_to(shape) if isinstance(a, HipNdArray) else a for a in args]
         dense = all(v.is_c_contiguous() for v in views if isinstance(v, HipNdArray))
-        if dense:                         # one long row: the cheapest indexing
+        asked = [name for name, a in zip(self._params(), args)
+                 if isinstance(a, HipNdArray) and name in self._arrays_asked_about()]
+        if asked:
+            # the body reads x.shape, len(x) or x[i, j] of an array argument:
+            # the map must walk the arrays as they are, not merged into fewer
+            # dimensions, and x must not be stretched to a larger shape
+            for name, a in zip(self._params(), args):
+                if name in asked and a.shape != tuple(shape):
+                    raise kernel_compiler.KernelCompileError(
+                        f"{self.py_func.__name__}: '{name}' of shape {a.shape} is broadcast "
+                        f"to {tuple(shape)}; its shape, length or elements cannot be read "
+                        "inside the map")
+            if len(shape) > 3:
+                raise kernel_compiler.KernelCompileError(
+                    f"{self.py_func.__name__}: the shape, length or elements of an array of "
+                    "more than 3 dimensions cannot be read inside a map")
+            run_shape = tuple(shape)
+        elif dense:                       # one long row: the cheapest indexing
             run_shape = (math.prod(shape),)
             views = [v.reshape(run_shape) if isinstance(v, HipNdArray) else v
                      for v in views]

@@ -613,3 +613,17 @@ def store_block_and_update_row(a, b):
 
 def update_shifted(a, b):
     a[1:] += b[:-1]
+
+
+def facts_under_a_branch(a, flag):
+    r = a - a.shape[1]
+    if flag:
+        r = a * a.shape[0] + len(a)
+    return r
+
+
+def facts_of_a_stretched_operand(a, b, flag):
+    r = a
+    if flag:
+        r = a + b.shape[0]
+    return r

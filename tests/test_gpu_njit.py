@@ -783,6 +783,27 @@ def test_stores_into_slices(env, name):
     np.testing.assert_allclose(d_a.asnumpy(), want, rtol=1e-13)
 
 
+def test_shapes_read_inside_a_map_that_is_not_straight_line(env):
+    """A body with a branch is one fused map; where it reads an argument's
+    shape or length the map walks the arrays with their own dimensions (not
+    merged into one long row), and an argument that would be stretched to a
+    larger shape is refused rather than seen with that shape."""
+    hip = env[0]
+    rng = np.random.default_rng(20)
+    A = rng.standard_normal((300, 200))
+    f = njit(cases.facts_under_a_branch)
+    for host in (A, np.ascontiguousarray(A.T).T):
+        dev = hip.asarray(np.ascontiguousarray(host.T)).T if not host.flags.c_contiguous \
+            else hip.asarray(host)
+        for flag in (True, False):
+            np.testing.assert_allclose(f(dev, flag).asnumpy(),
+                                       cases.facts_under_a_branch(host, flag), rtol=1e-13)
+    assert f.last_launch["path"] == "elementwise"
+    g = njit(cases.facts_of_a_stretched_operand)
+    with pytest.raises(Exception, match="broadcast"):
+        g(hip.asarray(A), hip.asarray(A[0].copy()), True)
+
+
 def test_cov_keeps_float32_and_one_variable_is_a_scalar(env):
     """The reference's cov keeps the input's floating type (numpy/funcs.py:
     1490-1527: only integers become float64) and returns a scalar for one
