@@ -182,6 +182,26 @@ def _fill(array, value):
 
 
 
+def _span(x):
+    lo = hi = x._offset
+    for n, st in zip(x.shape, x.strides):
+        if n > 1:
+            lo += min(0, (n - 1) * st)
+            hi += max(0, (n - 1) * st)
+    return lo, hi
+
+
+def _overlaps(x, target):
+    """Whether x may share elements with target without being the same view
+    (the same view is read and written element by element, which is safe)."""
+    if x._buffer is not target._buffer or not x.size or not target.size:
+        return False
+    if x._offset == target._offset and x.shape == target.shape and x.strides == target.strides:
+        return False
+    (lo, hi), (tlo, thi) = _span(x), _span(target)
+    return lo <= thi and tlo <= hi
+
+
 def _copy(x):
     """A dense C-ordered copy on x's device (numpy/funcs.py:255-262)."""
     out = HipNdArray.empty(x.shape, x.dtype, device=x.ctx.device)
@@ -912,7 +932,14 @@ class Dispatcher:
             launches.append({"path": "host scalar"})
             return value
         sub, params = self._stage_dispatcher(k, stage, scope)
-        value = sub._run([env[p] for p in params])
+        values = [env[p] for p in params]
+        if stage.kind == "store" and isinstance(env.get(stage.target), HipNdArray):
+            # x[1:] += x[:-1]: an operand that shares memory with the target
+            # under another view is read in full first, as NumPy does
+            target = env[stage.target]
+            values = [_copy(v) if isinstance(v, HipNdArray) and _overlaps(v, target) else v
+                      for v in values]
+        value = sub._run(values)
         launches.append(sub.last_launch)
         return value
 

@@ -909,8 +909,11 @@ class FunctionTranslator:
         if isinstance(node.op, ast.Invert):
             if v.type.is_float:
                 self.err(node, "~ needs an integer")
+            if v.type.is_bool and v.const is None:
+                # an element of a boolean array: numpy.invert is logical not
+                return Val(f"(!{v.code})", BOOL)
             if v.type.is_bool:
-                v = cast(v, INT64)
+                v = cast(v, INT64)        # ~True of Python is -2
             return Val(f"(~{v.code})", v.type)
         self.err(node, "Unsupported unary operator")
 

@@ -627,3 +627,19 @@ def facts_of_a_stretched_operand(a, b, flag):
     if flag:
         r = a + b.shape[0]
     return r
+
+
+def update_overlapping(a):
+    a[1:] += a[:-1]
+
+
+def store_overlapping(a):
+    a[:-1] = a[1:] * 2
+
+
+def store_reversed_onto_itself(a):
+    a[:] = a[::-1] + 1.0
+
+
+def inverted(a):
+    return ~a

@@ -804,6 +804,32 @@ def test_shapes_read_inside_a_map_that_is_not_straight_line(env):
         g(hip.asarray(A), hip.asarray(A[0].copy()), True)
 
 
+@pytest.mark.parametrize("name", ["update_overlapping", "store_overlapping",
+                                  "store_reversed_onto_itself"])
+def test_a_store_whose_operand_overlaps_its_target(env, name):
+    """x[1:] += x[:-1]: NumPy reads the right-hand side in full before it
+    stores; every work-item storing while others still read would not."""
+    hip = env[0]
+    a = np.random.default_rng(21).standard_normal(100_000)
+    func = getattr(cases, name)
+    want = a.copy()
+    func(want)
+    d_a = hip.asarray(a)
+    njit(func)(d_a)
+    np.testing.assert_array_equal(d_a.asnumpy(), want)
+
+
+def test_invert_of_booleans_is_logical_not(env):
+    hip = env[0]
+    x = np.random.default_rng(22).standard_normal(5000)
+    f = njit(cases.inverted)
+    got = f(hip.asarray(x > 0)).asnumpy()
+    assert got.dtype == np.bool_
+    np.testing.assert_array_equal(got, ~(x > 0))
+    counts = (x * 100).astype(np.int64)
+    np.testing.assert_array_equal(f(hip.asarray(counts)).asnumpy(), ~counts)
+
+
 def test_cov_keeps_float32_and_one_variable_is_a_scalar(env):
     """The reference's cov keeps the input's floating type (numpy/funcs.py:
     1490-1527: only integers become float64) and returns a scalar for one
