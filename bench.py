@@ -72,7 +72,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", type=str, default="",
                     help="comma-separated subset of: add,bs,bs32,sum1,norm2,"
-                         "sum0,pairwise,matmul,dispatch,generated (plus copy, only on "
+                         "sum0,pairwise,matmul,gemv,dispatch,generated (plus copy, only on "
                          "request)")
     ap.add_argument("--no-cpu", action="store_true",
                     help="skip the CPU baseline legs")
@@ -537,6 +537,29 @@ def run(args):
                                         kind="port")
         per_config.append(e)
         del d_A, d_B, d_Cs
+
+    # -- a matrix times a vector: one read of the matrix ----------------------
+    if want("gemv"):
+        n = 16384
+        rng = np.random.default_rng(7)
+        A = rng.standard_normal((n, n), dtype=np.float32)
+        v = rng.standard_normal((n, 1), dtype=np.float32)
+        d_A, d_v = da.asarray(A), da.asarray(v)
+        d_ys = [da.empty((n, 1), np.float32) for _ in range(nsets)]
+        saved = b.steps
+        b.steps = max(5, min(saved, 20))
+        wall, ev, _ = b.measure([lambda d_y=d_y: ops.dot(d_A, d_v, out=d_y)
+                                 for d_y in d_ys], blocking=True)
+        b.steps = saved
+        e = hbm_entry("gemv", "np.dot float32 [16384,16384] x [16384,1]",
+                      (n * n + 2 * n) * 4, wall, ev, math_runtime.last_kernel())
+        if orc:
+            e["cpu_baseline"] = cpu_leg(lambda: np.dot(A, v), (n * n + 2 * n) * 4 / 1e9,
+                                        "GB/s", os.cpu_count() or 1,
+                                        "the whole product, NumPy/OpenBLAS sgemv standing in "
+                                        "for MKL", kind="port")
+        per_config.append(e)
+        del d_A, d_v, d_ys, A, v
 
     # -- per-call overhead of a launch (no roofline: eight elements) --------
     if want("dispatch"):
