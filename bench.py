@@ -40,21 +40,22 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 WAKE_SECONDS = 0.1
 
 MEASURED_TRAFFIC = {
-    "nmk_black_scholes_f32_w64": 335612006,
-    "bench_streams_3r2w_f32": 335528195,
-    "nmk_black_scholes_f32_w32": 335609034,
-    "nmk_map2_rowbcast_add_f64": 268477666,
-    "nmk_sum_axis1_wide_f32": 537392240,
-    "nmk_norm2_f32": 536915851,
-    "nmk_sum_axis0_i32_i64": 538008276,
-    "nmk_twin_pairwise_f64_rows": 540432684,
+    "nmk_black_scholes_f32_w64": 335618094,
+    "bench_streams_3r2w_f32": 335527416,
+    "nmk_black_scholes_f32_w32": 335620540,
+    "nmk_map2_rowbcast_add_f64": 268476301,
+    "nmk_sum_axis1_wide_f32": 537376784,
+    "nmk_norm2_f32": 536904611,
+    "nmk_sum_axis0_i32_i64": 538015461,
+    "nmk_twin_pairwise_f64_rows": 540445362,
     "nmk_copy_b128": 536870912,
-    "sgemm_mfma_256x256": 671826722,
+    "sgemm_mfma_256x256": 671612278,
+    "sgemm_thin_rows": 1074312045,
     # generated kernels, without the hash of the body at the end of their names
-    "nmkjit_black_scholes_body": 335599967,
-    "nmkjit_black_scholes_loop_body": 335613367,
-    "nmkjit_scaled_add_body": 402631780,
-    "nmkjit_pairwise_body": 540511466,
+    "nmkjit_black_scholes_body": 335600452,
+    "nmkjit_black_scholes_loop_body": 335614116,
+    "nmkjit_scaled_add_body": 402630989,
+    "nmkjit_pairwise_body": 540445096,
 }
 
 
