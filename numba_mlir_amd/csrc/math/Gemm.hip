@@ -538,7 +538,12 @@ gemm_generic(const T *A, const T *B, T *C, int64_t M, int64_t N, int64_t K,
   if (tile >= tilesN * ((M + TILE - 1) / TILE))
     return;
   const int64_t row0 = tile / tilesN * TILE;
-  const int64_t col = tile % tilesN * TILE + tx;
+  const int64_t col0 = tile % tilesN * TILE, col = col0 + tx;
+  // Adjacent lanes read along each operand's unit stride: A along k or along
+  // m, B along n or along k (a transposed tall operand, X.T @ Y, is read in
+  // whole rows instead of one element per row).
+  const bool aAlongM = as0 == 1 && as1 != 1;
+  const bool bAlongK = bs0 == 1 && bs1 != 1;
   T acc[4] = {T(0), T(0), T(0), T(0)};
   // blockIdx.z: the slice of K (multiples of the tile), whose partial sums go
   // to part + z M N for gemm_thin_fold when there is more than one
@@ -549,10 +554,20 @@ gemm_generic(const T *A, const T *B, T *C, int64_t M, int64_t N, int64_t K,
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int r = ty + 8 * i;
-      const int64_t ar = row0 + r, ak = k0 + tx;
-      As[r][tx] = (ar < M && ak < K) ? A[ar * as0 + ak * as1] : T(0);
-      const int64_t bk = k0 + r;
-      Bs[r][tx] = (bk < K && col < N) ? B[bk * bs0 + col * bs1] : T(0);
+      if (aAlongM) {
+        const int64_t ar = row0 + tx, ak = k0 + r;
+        As[tx][r] = (ar < M && ak < K) ? A[ar * as0 + ak * as1] : T(0);
+      } else {
+        const int64_t ar = row0 + r, ak = k0 + tx;
+        As[r][tx] = (ar < M && ak < K) ? A[ar * as0 + ak * as1] : T(0);
+      }
+      if (bAlongK) {
+        const int64_t bk = k0 + tx, bn = col0 + r;
+        Bs[tx][r] = (bk < K && bn < N) ? B[bk * bs0 + bn * bs1] : T(0);
+      } else {
+        const int64_t bk = k0 + r;
+        Bs[r][tx] = (bk < K && col < N) ? B[bk * bs0 + col * bs1] : T(0);
+      }
     }
     __syncthreads();
 #pragma unroll
