@@ -764,7 +764,8 @@ template <typename T, int NB, int R, int W, int PV>
 __global__ __launch_bounds__(256) void
 gemm_thin_rows(const T *__restrict__ S, int64_t ld, int64_t rows, int64_t K,
                const T *__restrict__ P, int64_t pk, int64_t pn, int n, T *__restrict__ O,
-               int64_t orow, int64_t ocol, T alpha, T beta, int G, int gShift) {
+               int64_t orow, int64_t ocol, T alpha, T beta, int G, int gShift,
+               int64_t sliceWords, T *__restrict__ part) {
   constexpr int U = R < 8 ? 8 / R : 1;
   constexpr int ROW_BYTES = NB * int(sizeof(T)) < 16 ? NB * int(sizeof(T)) : 16;
   typedef T PRow __attribute__((ext_vector_type(NB), aligned(ROW_BYTES)));
@@ -787,8 +788,13 @@ gemm_thin_rows(const T *__restrict__ S, int64_t ld, int64_t rows, int64_t K,
 #pragma unroll
     for (int j = 0; j < NB; ++j)
       acc[r][j] = T(0);
-  const int64_t words = K / W;
-  for (int64_t w0 = g; w0 < words; w0 += int64_t(G) * U) {
+  // blockIdx.y: the slice of K (sliceWords words each; the last one takes the
+  // elements behind the last whole word), whose sums go to part for
+  // gemm_thin_fold when there is more than one
+  const int64_t allWords = K / W;
+  const int64_t wordsBegin = int64_t(blockIdx.y) * sliceWords;
+  const int64_t words = wordsBegin + sliceWords < allWords ? wordsBegin + sliceWords : allWords;
+  for (int64_t w0 = wordsBegin + g; w0 < words; w0 += int64_t(G) * U) {
     T x[U][R][W];
     T p[U][W][NB];
 #pragma unroll
@@ -841,8 +847,8 @@ gemm_thin_rows(const T *__restrict__ S, int64_t ld, int64_t rows, int64_t K,
       }
     }
   }
-  if (W > 1 && g == 0) // the elements behind the last whole word
-    for (int64_t k = words * W; k < K; ++k)
+  if (W > 1 && g == 0 && blockIdx.y == gridDim.y - 1) // the elements behind the last whole word
+    for (int64_t k = allWords * W; k < K; ++k)
 #pragma unroll
       for (int j = 0; j < NB; ++j)
         if (j < n) {
@@ -882,7 +888,9 @@ gemm_thin_rows(const T *__restrict__ S, int64_t ld, int64_t rows, int64_t K,
     for (int r = 0; r < R; ++r)
 #pragma unroll
       for (int j = 0; j < NB; ++j)
-        if (r0 + r < rows && j < n) {
+        if (r0 + r < rows && j < n && part) {
+          part[(int64_t(blockIdx.y) * rows + r0 + r) * n + j] = acc[r][j];
+        } else if (r0 + r < rows && j < n) {
           T *dst = O + (r0 + r) * orow + j * ocol;
           T v = alpha * acc[r][j];
           if (beta != T(0))
@@ -1605,6 +1613,24 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           const int64_t blocks = (sets + perBlock - 1) / perBlock;
           if (blocks >= (int64_t(1) << 24))
             return false;
+          // Few rows of a long K: slices of K (four trips of a block or more
+          // each) bring the launch to some 2048 blocks; their sums are
+          // added in index order by gemm_thin_fold.
+          SplitPlan plan;
+          int64_t sliceWords = words > 0 ? words : 1;
+          if (G == 256 && blocks < 1024) {
+            const int64_t trip = int64_t(256) * (R < 8 ? 8 / R : 1);
+            int64_t slices = 2048 / blocks;
+            if (slices > words / (4 * trip))
+              slices = words / (4 * trip);
+            if (slices > 1) {
+              sliceWords = ((words + slices - 1) / slices + trip - 1) / trip * trip;
+              plan.slices = int((words + sliceWords - 1) / sliceWords);
+            }
+          }
+          T *part = workspaceFor(plan, rows, n);
+          if (!part)
+            plan.slices = 1, sliceWords = words > 0 ? words : 1;
           // How P is read (gemm_thin_rows).
           const size_t rowBytes = size_t(NB) * sizeof(T) < 16 ? size_t(NB) * sizeof(T) : 16;
           int PV = 0;
@@ -1614,11 +1640,11 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
             PV = 1;
           else if (vec && pk == 1 && aligned16(P) && pn % VEC == 0)
             PV = 2;
-          const dim3 grid{unsigned(blocks)};
+          const dim3 grid(unsigned(blocks), unsigned(plan.slices));
 #define NMHIP_THIN_ROWS(NB_, R_, W_, PV_)                                      \
   hipLaunchKernelGGL((gemm_thin_rows<T, NB_, R_, W_, PV_>), grid, dim3(256), 0, \
                      stream, S, ld, rows, K, P, pk, pn, n, cData, orow, ocol,  \
-                     alpha, beta, G, gShift)
+                     alpha, beta, G, gShift, sliceWords, part)
 #define NMHIP_THIN_ROWS_P(NB_, R_)                                             \
   do {                                                                         \
     if (vec && PV == 2)                                                        \
@@ -1646,6 +1672,10 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           }
 #undef NMHIP_THIN_ROWS_P
 #undef NMHIP_THIN_ROWS
+          if (part)
+            hipLaunchKernelGGL(gemm_thin_fold<T>, dim3(unsigned((n + 15) / 16), unsigned(rows)),
+                               dim3(256), 0, stream, part, plan.slices, int(rows), int64_t(n),
+                               int64_t(n), cData, orow, ocol, alpha, beta);
           lastKernel = sizeof(T) == 4 ? "sgemm_thin_rows" : "dgemm_thin_rows";
           return true;
         };
@@ -1663,8 +1693,8 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           int64_t slices = 2048 / strips;
           if (slices > K / 64)
             slices = K / 64;
-          if (slices > 64)
-            slices = 64;
+          if (slices > 1024)
+            slices = 1024;
           while (slices > 1 &&
                  size_t(slices) * size_t(m) * size_t(cPitch) * sizeof(T) > kScratchBytes)
             --slices;
@@ -1709,11 +1739,13 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           lastKernel = sizeof(T) == 4 ? "sgemm_thin_cols" : "dgemm_thin_cols";
           return true;
         };
-        if (Nz <= kThinCols && Mz >= kLong)
+        // (a long extent of 64 to 1023 too where K is long: slices of K fill the GPU)
+        const int64_t longEnough = K >= 8192 ? 64 : kLong;
+        if (Nz <= kThinCols && Mz >= longEnough)
           launched = xKc && Nz <= kThinRows ? thinRows(X, xm, Mz, Y, yk, yn, int(Nz), ldz, 1)
                      : !xKc && xm == 1      ? thinCols(X, xk, Mz, Y, yn, yk, int(Nz), 1, ldz)
                                             : false;
-        else if (Mz <= kThinCols && Nz >= kLong)
+        else if (Mz <= kThinCols && Nz >= longEnough)
           launched = yNc                         ? thinCols(Y, yk, Nz, X, xm, xk, int(Mz), ldz, 1)
                      : yk == 1 && Mz <= kThinRows ? thinRows(Y, yn, Nz, X, xk, xm, int(Mz), 1, ldz)
                                                   : false;

@@ -378,11 +378,14 @@ def test_small_times_long(env, dtype, m, k, n):
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("long,k,thin", [(1500, 100, 1), (1025, 33, 3), (2000, 1001, 8),
-                                         (5000, 4099, 5), (1100, 70_000, 2), (40_000, 260, 4)])
+                                         (5000, 4099, 5), (1100, 70_000, 2), (40_000, 260, 4),
+                                         (100, 70_000, 2), (64, 8192, 1), (700, 20_001, 8)])
 def test_long_times_thin(env, dtype, long, k, thin):
     """A long matrix times a thin one (a vector, or up to eight of them) and a
     thin one times a long one, K > 32: the long operand is read once, by rows
-    when it has unit stride along k, by columns otherwise.  Every layout of
+    when it has unit stride along k, by columns otherwise (a long extent of
+    64 to 1023 too where K is 8192 or more: K goes in slices over many blocks
+    then).  Every layout of
     the three operands, rows that are and are not whole 128-bit words (views
     of wider rows), alpha and beta, a C of NaNs under beta = 0; every element
     against float64."""
