@@ -794,7 +794,15 @@ gemm_thin_rows(const T *__restrict__ S, int64_t ld, int64_t rows, int64_t K,
   const int64_t allWords = K / W;
   const int64_t wordsBegin = int64_t(blockIdx.y) * sliceWords;
   const int64_t words = wordsBegin + sliceWords < allWords ? wordsBegin + sliceWords : allWords;
-  for (int64_t w0 = wordsBegin + g; w0 < words; w0 += int64_t(G) * U) {
+  // The trips along k start at a different place for every set of rows and
+  // wrap round: rows a power of two apart begin in the same memory channel,
+  // and sets that all walked from k = 0 would queue on it.
+  const int64_t tripWords = int64_t(G) * U;
+  const int64_t trips = words > wordsBegin ? (words - wordsBegin + tripWords - 1) / tripWords : 0;
+  const int64_t firstTrip = trips ? (set * 5) % trips : 0;
+  for (int64_t trip = 0; trip < trips; ++trip) {
+    const int64_t turned = trip + firstTrip < trips ? trip + firstTrip : trip + firstTrip - trips;
+    const int64_t w0 = wordsBegin + turned * tripWords + g;
     T x[U][R][W];
     T p[U][W][NB];
 #pragma unroll
