@@ -1646,7 +1646,7 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
               reinterpret_cast<uintptr_t>(P) % rowBytes == 0 &&
               size_t(pk) * sizeof(T) % rowBytes == 0)
             PV = 1;
-          else if (vec && pk == 1 && aligned16(P) && pn % VEC == 0)
+          else if (vec && pk == 1 && aligned16(P) && (n == 1 || pn % VEC == 0))
             PV = 2;
           const dim3 grid(unsigned(blocks), unsigned(plan.slices));
 #define NMHIP_THIN_ROWS(NB_, R_, W_, PV_)                                      \
