@@ -451,6 +451,35 @@ def test_up_to_sixteen_vectors_against_columns(env, dtype, thin):
     _check_scaled(d_c.asnumpy(), a, b, c0, 1.5, -0.5, tol)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_thin_and_small_products_of_views_that_start_inside_a_word(env, dtype):
+    """Operands that are views starting one element into a row: nothing is
+    aligned to a 128-bit word, every kernel of these families reads by
+    elements."""
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(31)
+    tol = 1e-5 if dtype == np.float32 else 1e-13
+    for m, k, n in ((2000, 1003, 3), (3, 1003, 2000), (5, 20_000, 7), (300, 9000, 1)):
+        wa = rng.standard_normal((m, k + 2)).astype(dtype)
+        wb = rng.standard_normal((k, n + 2)).astype(dtype)
+        wc = rng.standard_normal((m, n + 2)).astype(dtype)
+        d_a, d_b = hip.asarray(wa)[:, 1:k + 1], hip.asarray(wb)[:, 1:n + 1]
+        d_w = hip.asarray(wc)
+        ops.gemm(d_a, d_b, d_w[:, 1:n + 1], 1.5, -0.5)
+        assert "thin" in mrt.last_kernel() or "inner" in mrt.last_kernel(), mrt.last_kernel()
+        got = d_w.asnumpy()
+        _check_scaled(got[:, 1:n + 1], wa[:, 1:k + 1], wb[:, 1:n + 1], wc[:, 1:n + 1],
+                      1.5, -0.5, tol)
+        # the columns of C beside the view are untouched
+        assert np.array_equal(got[:, 0], wc[:, 0]) and np.array_equal(got[:, n + 1], wc[:, n + 1])
+        # the transposed long operand
+        d_at = hip.asarray(np.ascontiguousarray(wa.T))[1:k + 1].T
+        d_w = hip.asarray(wc)
+        ops.gemm(d_at, d_b, d_w[:, 1:n + 1], 1.0, 0.0)
+        _check_scaled(d_w.asnumpy()[:, 1:n + 1], wa[:, 1:k + 1], wb[:, 1:n + 1],
+                      np.zeros((m, n), dtype), 1.0, 0.0, tol)
+
+
 def test_thin_products_do_not_mix_in_what_lies_beyond(env):
     """An infinity in the long operand's padding, or in the thin one's, stays
     out of the sums (a product with zero would make it a NaN)."""
