@@ -480,6 +480,46 @@ def test_thin_and_small_products_of_views_that_start_inside_a_word(env, dtype):
                       np.zeros((m, n), dtype), 1.0, 0.0, tol)
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_shapes_drawn_round_the_limits_between_kernels(env, seed):
+    """Extents drawn next to the limits at which one kernel hands over to
+    another (thin extents of 8 and 16, long ones of 64, 1024 and 4096, K of
+    32, 2048, 4096 and 8192, tile counts of 16 and 256), every layout,
+    both types: whichever kernel serves, every element against float64."""
+    hip, ops, _, mrt = env
+    rng = np.random.default_rng(1000 + seed)
+    small = [1, 2, 3, 4, 5, 7, 8, 9, 12, 15, 16, 17, 31, 32, 33]
+    long = [63, 64, 65, 127, 129, 500, 1023, 1024, 1025, 4095, 4096, 4100]
+    depth = [31, 32, 33, 40, 255, 2047, 2048, 2050, 4095, 4096, 4097, 8191, 8192, 8200, 20_000]
+    for _ in range(16):
+        kind = rng.integers(0, 4)
+        if kind == 0:
+            m, n = rng.choice(long), rng.choice(small)
+        elif kind == 1:
+            m, n = rng.choice(small), rng.choice(long)
+        elif kind == 2:
+            m, n = rng.choice(small), rng.choice(small)
+        else:
+            m, n = rng.choice(long[:8]), rng.choice(long[:8])
+        k = int(rng.choice(depth))
+        m, n = int(m), int(n)
+        dtype = np.float32 if rng.integers(0, 2) else np.float64
+        fa, fb, fc = (bool(rng.integers(0, 2)) for _ in range(3))
+        alpha, beta = ((1.0, 0.0), (1.5, -0.5))[int(rng.integers(0, 2))]
+        a = rng.standard_normal((m, k)).astype(dtype)
+        b = rng.standard_normal((k, n)).astype(dtype)
+        c0 = rng.standard_normal((m, n)).astype(dtype)
+        d_a = _to_dev(hip, a.T.copy().T if fa else a)
+        d_b = _to_dev(hip, b.T.copy().T if fb else b)
+        d_c = _to_dev(hip, c0.T.copy().T if fc else c0)
+        ops.gemm(d_a, d_b, d_c, alpha, beta)
+        case = (m, k, n, np.dtype(dtype).name, fa, fb, fc, alpha, beta, mrt.last_kernel())
+        truth = beta * c0.astype(np.float64) + alpha * (a.astype(np.float64) @ b.astype(np.float64))
+        scale = abs(beta) * np.abs(c0) + abs(alpha) * (np.abs(a).astype(np.float64) @ np.abs(b))
+        rel = 1e-5 if dtype == np.float32 else 1e-13
+        assert (np.abs(d_c.asnumpy() - truth) <= rel * scale + 1e-30).all(), case
+
+
 def test_thin_products_do_not_mix_in_what_lies_beyond(env):
     """An infinity in the long operand's padding, or in the thin one's, stays
     out of the sums (a product with zero would make it a NaN)."""
