@@ -400,6 +400,44 @@ def _mean(x, axis):
     return _DIVIDE[0](total, float_t(x.shape[axis]))
 
 
+def _matmul_body(a, b, out):
+    i = kernel_impl.get_global_id(0)
+    j = kernel_impl.get_global_id(1)
+    acc = out[i, j] * 0
+    for k in range(a.shape[1]):
+        acc += a[i, k] * b[k, j]
+    out[i, j] = acc
+
+
+def _matmul(a, b, out=None):
+    """The product of two matrices: the gemm kernels for float32 and float64
+    (operands of two types are converted to their common type first), a plain
+    generated kernel, one work-item per element, for integers (the reference
+    lowers those to linalg.matmul, numpy/funcs.py:889-906)."""
+    dtype = np.result_type(a.dtype, b.dtype)
+    if dtype == np.bool_:
+        dtype = np.dtype(np.int64)
+    if dtype.kind == "f" and dtype.itemsize < 4:
+        dtype = np.dtype(np.float32)
+    if dtype.kind not in "iuf":
+        raise TypeError(f"no matrix product of {a.dtype} and {b.dtype}")
+    if out is not None and out.dtype != dtype:
+        raise TypeError(f"out must be of type {dtype}")
+    a = a if a.dtype == dtype else _astype(a, dtype)
+    b = b if b.dtype == dtype else _astype(b, dtype)
+    if dtype in (np.float32, np.float64):
+        return ops.dot(a, b, out=out)
+    if a.shape[1] != b.shape[0]:
+        raise ValueError(f"shapes {a.shape} and {b.shape} not aligned")
+    if out is None:
+        out = HipNdArray.empty((a.shape[0], b.shape[1]), dtype, device=a.ctx.device)
+    if out.size:
+        _fill(out, dtype.type(0))
+        if a.shape[1]:
+            _KERNELS[_matmul_body][out.shape, ()](a, b, out)
+    return out
+
+
 def _dot(a, b, out=None):
     """numpy.dot of device arrays of rank 1 or 2 through the matrix kernels."""
     if not (isinstance(a, HipNdArray) and isinstance(b, HipNdArray)):
@@ -408,7 +446,7 @@ def _dot(a, b, out=None):
         if out is not None and (not isinstance(out, HipNdArray) or
                                 out.shape != (a.shape[0], b.shape[1])):
             raise ValueError("out must be a device array of the product's shape")
-        return ops.dot(a, b, out=out)
+        return _matmul(a, b, out=out)
     if out is not None:
         raise NotImplementedError("out= is implemented for 2-d operands")
     if a.ndim == 1 and b.ndim == 1:
@@ -417,9 +455,9 @@ def _dot(a, b, out=None):
         total = ops.sum(ops.multiply(a, b))
         return total.asnumpy().reshape(-1)[0] if isinstance(total, HipNdArray) else total
     if a.ndim == 2 and b.ndim == 1:
-        return ops.dot(a, b.reshape((b.shape[0], 1))).reshape((a.shape[0],))
+        return _matmul(a, b.reshape((b.shape[0], 1))).reshape((a.shape[0],))
     if a.ndim == 1 and b.ndim == 2:
-        return ops.dot(a.reshape((1, a.shape[0])), b).reshape((b.shape[1],))
+        return _matmul(a.reshape((1, a.shape[0])), b).reshape((b.shape[1],))
     raise NotImplementedError("np.dot is implemented for rank 1 and 2")
 
 

@@ -207,6 +207,9 @@ def gemm(a, b, c, alpha, beta):
         raise ValueError("gemm needs 2-D arrays")
     if a.dtype != b.dtype or a.dtype != c.dtype:
         raise TypeError("gemm operands must share a dtype")
+    if a.dtype not in (np.float32, np.float64):
+        # (the reference binds mkl_gemm for these two only, numpy/funcs.py:848-864)
+        raise TypeError(f"gemm is implemented for float32 and float64, not {a.dtype}")
     m, k = a.shape
     k2, n = b.shape
     if k != k2 or c.shape != (m, n):

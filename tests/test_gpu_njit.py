@@ -850,6 +850,45 @@ def test_cov_keeps_float32_and_one_variable_is_a_scalar(env):
     np.testing.assert_allclose(got, np.cov(counts), rtol=1e-12)
 
 
+@pytest.mark.parametrize("left,right", [(np.int64, np.int64), (np.int32, np.int32),
+                                        (np.float32, np.float64), (np.float64, np.int64),
+                                        (np.int32, np.float32)])
+def test_products_of_integers_and_of_two_types(env, left, right):
+    """``@`` and np.dot of integer matrices (the reference lowers those to
+    linalg.matmul, numpy/funcs.py:889-906) and of operands of two types: the
+    type NumPy gives, exact for integers."""
+    hip = env[0]
+    rng = np.random.default_rng(23)
+
+    def draw(shape, dtype):
+        if np.dtype(dtype).kind == "i":
+            return rng.integers(-5, 6, shape).astype(dtype)
+        return rng.standard_normal(shape).astype(dtype)
+
+    a, b = draw((130, 70), left), draw((70, 45), right)
+    for func in (_matmul_operator, _np_dot):
+        f = njit(func)
+        for x, y in ((a, b), (a, b[:, 0].copy()), (a[0].copy(), b)):
+            want = func(x, y)
+            got = f(hip.asarray(x), hip.asarray(y)).asnumpy()
+            assert got.dtype == want.dtype and got.shape == want.shape
+            if want.dtype.kind == "i":
+                np.testing.assert_array_equal(got, want)
+            else:
+                np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+
+
+def test_gemm_refuses_other_types_with_an_exception(env):
+    """ops.gemm mirrors the reference's binding, which exists for float32 and
+    float64 (numpy/funcs.py:848-864): anything else is a TypeError, not an
+    abort inside the runtime."""
+    hip = env[0]
+    from numba_mlir_amd.mlir import ops
+    a = hip.asarray(np.ones((4, 4), np.int64))
+    with pytest.raises(TypeError, match="float32 and float64"):
+        ops.dot(a, a)
+
+
 def test_pairwise_as_nested_prange_loops(env):
     """test_pairwise2 (test_gpu.py:2226-2266): the distance body as two
     prange loops around a serial one, on the reference's fixture."""
