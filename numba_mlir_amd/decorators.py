@@ -112,6 +112,8 @@ def _reduce_nd(op, x, axis):
     integers, as NumPy does."""
     if x.dtype == np.bool_:
         x = _CAST_TO[np.int64](x)
+    if x.dtype in _NARROW_INTEGERS:
+        return _reduce_narrow(op, x, axis)
     if axis is None and not (x.is_c_contiguous() or x.is_f_contiguous()):
         x = _copy(x)                      # a strided view: its elements, densely
     if x.ndim <= 2 or not x.is_c_contiguous():
@@ -127,6 +129,27 @@ def _reduce_nd(op, x, axis):
                   axis=1).reshape(x.shape[:-1])
     raise NotImplementedError("reductions of arrays of rank > 2 run along the first or "
                               "the last axis")
+
+
+# Integer types the reduction kernels do not take as they are: widened to
+# int64 (every value fits) and reduced there.
+_NARROW_INTEGERS = tuple(np.dtype(t) for t in (np.int8, np.int16, np.uint8, np.uint16, np.uint32))
+
+
+def _reduce_narrow(op, x, axis):
+    """Sums and products come back in the type NumPy gives them along an axis
+    (int64, uint64 for unsigned input) and, like the other integer types
+    here, in the input's own type over everything (the reference casts a full
+    reduction back, numpy/funcs.py:163-229); minima and maxima in the input's
+    type."""
+    result = _reduce_nd(op, _astype(x, np.dtype(np.int64)), axis)
+    if op in (ops.amin, ops.amax) or axis is None:
+        back = x.dtype
+    else:
+        back = np.dtype(np.uint64 if x.dtype.kind == "u" else np.int64)
+    if isinstance(result, HipNdArray):
+        return result if result.dtype == back else _astype(result, back)
+    return np.asarray(result).astype(back)[()]
 
 
 _DIVIDE = []
@@ -389,6 +412,8 @@ def _cov(m, y=None, rowvar=True, bias=False, ddof=None):
 
 
 def _mean(x, axis):
+    if x.dtype in _NARROW_INTEGERS:
+        x = _astype(x, np.dtype(np.int64))        # (no wrap-round of the total)
     total = _reduce_nd(ops.sum, x, axis)
     float_t = x.dtype.type if x.dtype.kind == "f" else np.float64
     if axis is None:

@@ -889,6 +889,31 @@ def test_gemm_refuses_other_types_with_an_exception(env):
         ops.dot(a, a)
 
 
+@pytest.mark.parametrize("dtype", [np.int8, np.int16, np.uint8, np.uint16, np.uint32])
+def test_reductions_of_narrow_integers(env, dtype):
+    """Integer types narrower than the reduction kernels take are widened to
+    int64 first: along an axis the sums are NumPy's in value and type, minima
+    and maxima keep the input's type, the mean does not wrap round."""
+    hip = env[0]
+    rng = np.random.default_rng(24)
+    x = rng.integers(1, 100, (500, 40)).astype(dtype)
+    d_x = hip.asarray(x)
+    got = njit(lambda a: np.sum(a, axis=0))(d_x).asnumpy()
+    want = np.sum(x, axis=0)
+    assert got.dtype == want.dtype
+    np.testing.assert_array_equal(got, want)
+    got = njit(lambda a: a.max(axis=1))(d_x).asnumpy()
+    assert got.dtype == x.dtype
+    np.testing.assert_array_equal(got, x.max(axis=1))
+    assert njit(lambda a: np.min(a))(d_x) == x.min()
+    np.testing.assert_allclose(njit(lambda a: np.mean(a))(d_x), x.mean(), rtol=1e-12)
+    np.testing.assert_allclose(njit(lambda a: a.mean(axis=0))(d_x).asnumpy(), x.mean(axis=0),
+                               rtol=1e-12)
+    # over everything the total comes back in the input's type, as for int32
+    total = njit(lambda a: a.sum())(d_x)
+    assert total == np.sum(x).astype(dtype)
+
+
 def test_pairwise_as_nested_prange_loops(env):
     """test_pairwise2 (test_gpu.py:2226-2266): the distance body as two
     prange loops around a serial one, on the reference's fixture."""
