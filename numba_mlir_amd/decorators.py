@@ -452,6 +452,8 @@ def _matmul(a, b, out=None):
     b = b if b.dtype == dtype else _astype(b, dtype)
     if dtype in (np.float32, np.float64):
         return ops.dot(a, b, out=out)
+    if dtype.kind == "u" and dtype.itemsize == 8:
+        raise TypeError("no matrix product of uint64")
     if a.shape[1] != b.shape[0]:
         raise ValueError(f"shapes {a.shape} and {b.shape} not aligned")
     if out is None:
@@ -1245,8 +1247,12 @@ class Dispatcher:
                                  slice=stage.args[0], ctx=ast.Load())
             expr = ast.fix_missing_locations(ast.Expression(body=node))
             try:
-                return eval(compile(expr, "<index>", "eval"), scope,  # noqa: S307
+                view = eval(compile(expr, "<index>", "eval"), scope,  # noqa: S307
                             dict(env, _nmk_sliced=x))
+                if isinstance(stage.node, ast.Assign) and isinstance(view, HipNdArray) and \
+                        view.ndim == 0:
+                    view = view.reshape((1,))       # the target of x[i, j] = value
+                return view
             except (TypeError, ValueError, IndexError, NotImplementedError) as exc:
                 raise kernel_compiler.KernelCompileError(f"{where}: {exc}") from exc
         args = []

@@ -82,11 +82,6 @@ def _is_whole_slice(node):
     return full(node)
 
 
-def _has_slice(node):
-    index = node.elts if isinstance(node, ast.Tuple) else [node]
-    return any(isinstance(e, ast.Slice) for e in index)
-
-
 class _Splitter(ast.NodeTransformer):
     def __init__(self, plan):
         self.plan = plan
@@ -309,7 +304,8 @@ class Plan:
             if isinstance(stmt, ast.Expr) and isinstance(stmt.value, ast.Constant):
                 continue                                       # a docstring
             if isinstance(stmt, ast.AugAssign) and isinstance(stmt.target, ast.Subscript) and \
-                    isinstance(stmt.target.value, ast.Name) and _has_slice(stmt.target.slice):
+                    isinstance(stmt.target.value, ast.Name) and \
+                    not _is_whole_slice(stmt.target.slice):
                 # x[1:] += ...: x[1:] = x[1:] + ...
                 import copy
                 load = copy.deepcopy(stmt.target)
@@ -351,8 +347,8 @@ class Plan:
                     self.add(Stage("store", target.value.id, value, node=stmt))
                     continue
                 if isinstance(target, ast.Subscript) and isinstance(target.value, ast.Name) \
-                        and target.value.id in self.locals and _has_slice(target.slice):
-                    # x[1:5] = ..., x[:, 3] = ...: a store into a view of x
+                        and target.value.id in self.locals:
+                    # x[1:5] = ..., x[:, 3] = ..., x[5] = ...: a store into a view of x
                     view = Stage("view", self.fresh(), op="getitem",
                                  operands=[target.value.id], node=stmt)
                     view.args = [splitter.visit(target.slice)]

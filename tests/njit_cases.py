@@ -643,3 +643,10 @@ def store_reversed_onto_itself(a):
 
 def inverted(a):
     return ~a
+
+
+def store_row_and_elements(a, b):
+    a[5] = b[7] * 2.0
+    a[0, 1] = 3.5
+    a[2, 2] += 1.0
+    a[-1] -= b[0]

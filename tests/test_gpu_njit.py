@@ -766,7 +766,7 @@ def test_arrays_built_and_sliced_inside(env, name, operands):
 
 
 @pytest.mark.parametrize("name", ["store_slice", "store_column", "store_block_and_update_row",
-                                  "update_shifted"])
+                                  "update_shifted", "store_row_and_elements"])
 def test_stores_into_slices(env, name):
     """x[1:5] = ..., x[:, 3] = ..., x[1:] += ...: stores into views of the
     array (array.__setitem__ with slices, numpy/funcs.py:1140-1195)."""
