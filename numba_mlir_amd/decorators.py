@@ -1253,7 +1253,7 @@ class Dispatcher:
                         view.ndim == 0:
                     view = view.reshape((1,))       # the target of x[i, j] = value
                 return view
-            except (TypeError, ValueError, IndexError, NotImplementedError) as exc:
+            except (TypeError, ValueError, IndexError, NameError, NotImplementedError) as exc:
                 raise kernel_compiler.KernelCompileError(f"{where}: {exc}") from exc
         args = []
         for node in stage.args:
