@@ -282,6 +282,14 @@ class HipNdArray:
             shape = tuple(shape[0])
         if not self.is_c_contiguous():
             raise ValueError("reshape needs a C-contiguous device array")
+        shape = tuple(int(n) for n in shape)
+        if shape.count(-1) == 1:              # one extent left to be worked out
+            known = math.prod(n for n in shape if n != -1)
+            if known == 0 or self.size % known:
+                raise ValueError(f"cannot reshape array of size {self.size} into shape {shape}")
+            shape = tuple(self.size // known if n == -1 else n for n in shape)
+        if any(n < 0 for n in shape):
+            raise ValueError("negative dimensions are not allowed")
         strides = _dense_strides(shape, self.dtype.itemsize)
         if math.prod(int(n) for n in shape) != self.size:
             raise ValueError("cannot reshape: size mismatch")

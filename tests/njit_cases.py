@@ -650,3 +650,28 @@ def store_row_and_elements(a, b):
     a[0, 1] = 3.5
     a[2, 2] += 1.0
     a[-1] -= b[0]
+
+
+def distances_to_centres(X, C):
+    return (X * X).sum(axis=1).reshape(-1, 1) - 2 * X @ C.T + (C * C).sum(axis=1)
+
+
+def softmax_rows(x):
+    e = np.exp(x - x.max(axis=1).reshape(-1, 1))
+    return e / e.sum(axis=1).reshape(-1, 1)
+
+
+def covariance_of_columns(X):
+    Xc = X - X.mean(axis=0)
+    return Xc.T @ Xc / (X.shape[0] - 1)
+
+
+def ridge_gradient(X, y, w, lam):
+    r = X @ w - y
+    return X.T @ r / X.shape[0] + lam * w
+
+
+def cosine_to_centres(X, C):
+    xn = np.sqrt((X * X).sum(axis=1)).reshape(-1, 1)
+    cn = np.sqrt((C * C).sum(axis=1)).reshape(1, -1)
+    return (X @ C.T) / (xn * cn)

@@ -914,6 +914,27 @@ def test_reductions_of_narrow_integers(env, dtype):
     assert total == np.sum(x).astype(dtype)
 
 
+@pytest.mark.parametrize("name,operands", [
+    ("distances_to_centres", "XC"), ("softmax_rows", "X"), ("covariance_of_columns", "X"),
+    ("ridge_gradient", "Xywl"), ("cosine_to_centres", "XC")])
+def test_whole_array_recipes(env, name, operands):
+    """Recipes of a few lines over a tall matrix -- distances to centres, a
+    softmax per row, the covariance of columns, a gradient -- that mix
+    reductions, reshape(-1, 1), broadcasting and products with thin and
+    transposed operands: the values NumPy gives."""
+    hip = env[0]
+    rng = np.random.default_rng(25)
+    pool = {"X": rng.standard_normal((20000, 16)), "C": rng.standard_normal((8, 16)),
+            "y": rng.standard_normal(20000), "w": rng.standard_normal(16), "l": 0.1}
+    func = getattr(cases, name)
+    host = [pool[k] for k in operands]
+    want = func(*host)
+    got = njit(func)(*[hip.asarray(a) if isinstance(a, np.ndarray) else a for a in host])
+    got = got.asnumpy()
+    assert got.shape == want.shape and got.dtype == want.dtype
+    np.testing.assert_allclose(got, want, rtol=1e-9, atol=1e-9)
+
+
 def test_pairwise_as_nested_prange_loops(env):
     """test_pairwise2 (test_gpu.py:2226-2266): the distance body as two
     prange loops around a serial one, on the reference's fixture."""
