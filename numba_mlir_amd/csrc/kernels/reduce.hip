@@ -383,6 +383,25 @@ reduceStrided(const IN *x, ACC *out, int64_t nKeep, int64_t nRed, int64_t sk,
               int64_t sr, int64_t so, int32_t mode, ACC init, Op op) {
   __shared__ ACC slots[256 / NMK_WAVE];
   const bool vec = mode & 1;
+  if (mode & 4) {
+    // Short runs (a few coordinates or features a row): 2^(mode >> 8)
+    // adjacent lanes a kept index, so that a wave reads whole runs of
+    // neighbouring kept indices side by side; the group's lanes meet through
+    // lane exchanges.
+    const int gShift = mode >> 8, G = 1 << gShift;
+    const int g = threadIdx.x & (G - 1);
+    const int64_t k = (blockLinearXY() * blockDim.x + threadIdx.x) >> gShift;
+    const bool live = k < nKeep; // (the others still take part in the exchanges)
+    const IN *p = x + (live ? k : 0) * sk;
+    ACC acc = init;
+    for (int64_t r = g; r < nRed; r += G)
+      acc = op(acc, ACC(p[r * sr]));
+    for (int off = G >> 1; off > 0; off >>= 1)
+      acc = op(acc, __shfl_xor(acc, off, NMK_WAVE));
+    if (live && g == 0)
+      out[k * so] = acc;
+    return;
+  }
   if (mode & 2) {
     const int64_t k = blockLinearXY();
     if (k >= nKeep)

@@ -864,6 +864,20 @@ NMHIP_EXPORT void nmhipReduce(void *ctx, int op, int dtype, const void *x,
                  Arg::I64(0), Arg::I64(1), Arg::I64(1), Arg::I32(0)});
       return;
     }
+    // Many short runs (the rows of a tall matrix of a few columns): a group
+    // of 1 to 32 lanes a kept index, two elements or so a lane.
+    if (nRed >= 1 && nRed <= 64 && nKeep >= 4096) {
+      int gShift = 0;
+      while (sr == 1 && (int64_t(2) << gShift) < nRed && gShift < 5)
+        ++gShift; // (a lane a kept index where the run is strided: the lanes then
+                  // follow the kept index, which has the shorter stride)
+      const int mode = 4 | (gShift << 8);
+      c->launchBlocksXY(std::string("nmk_reduce_") + opNames[op] + "_" + dtypeName(dtype),
+                        ceilDiv(nKeep << gShift, 256),
+                        {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(nKeep), Arg::I64(nRed),
+                         Arg::I64(sk), Arg::I64(sr), Arg::I64(1), Arg::I32(mode)});
+      return;
+    }
     // (a block per kept index where the reduced run is long, a wave per
     // kept index otherwise)
     const bool wide = nRed >= 4096;

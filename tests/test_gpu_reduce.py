@@ -192,6 +192,10 @@ _ROUTES = [
     ("few long rows", (5, 70000), False),
     ("columns on words", (4100, 516), False),
     ("columns on single elements", (4100, 515), False),
+    ("many short rows, a group of lanes each", (70001, 16), False),
+    ("many rows of three", (50000, 3), False),
+    ("many rows of 64, base inside a word", (5000, 64), True),
+    ("many short columns, a lane each", (7, 70001), False),
     ("one run in chunks", (1, 1000003), False),
     ("one run in chunks, base inside a word", (1, 1000003), True),
 ]
