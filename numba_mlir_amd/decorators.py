@@ -1102,8 +1102,9 @@ class Dispatcher:
             (np.dtype(np.uint64) if dtype.kind == "u" else dtype)
         if stage.op == "mean":
             result_dtype = dtype if dtype.kind == "f" else np.dtype(np.float64)
-        short_rows = along_rows and cols <= staging.SHORT_ROW
-        key = ("axis", along_rows, short_rows, k, kernel_impl.captured_constants(self.py_func),
+        if along_rows and cols <= staging.SHORT_ROW and rows >= 4096:
+            return NotImplemented
+        key = ("axis", along_rows, k, kernel_impl.captured_constants(self.py_func),
                tuple(arrays), integer)
         entry = self._stage_funcs.get(key)
         if entry is None:
@@ -1111,8 +1112,7 @@ class Dispatcher:
                              _nmk_local_id=kernel_impl.get_local_id,
                              _nmk_global_id=kernel_impl.get_global_id,
                              _nmk_group=kernel_impl.group)
-            make = staging.short_row_sum_function if short_rows else \
-                staging.row_sum_function if along_rows else staging.column_sum_function
+            make = staging.row_sum_function if along_rows else staging.column_sum_function
             func, params = make(source, f"{self._stage_stem}_stage{k}_axis", namespace,
                                 set(arrays), integer)
             entry = self._stage_funcs[key] = kernel_impl.Kernel(
@@ -1126,8 +1126,7 @@ class Dispatcher:
             if along_rows:
                 total = HipNdArray.empty((rows,), acc_dtype if stage.op == "mean" else
                                          result_dtype, device=ctx.device)
-                launch = entry[(rows,), ()] if short_rows else \
-                    entry[(rows * staging.ROW_LANES,), (staging.ROW_LANES,)]
+                launch = entry[(rows * staging.ROW_LANES,), (staging.ROW_LANES,)]
                 launch(cols, *inputs, total)
             else:
                 # (more chunks cost partial-sum traffic, fewer leave the GPU idle:

@@ -582,30 +582,11 @@ def row_sum_function(stage, name, scope, arrays, integer):
     return _function(name, params, body, exprs, stage, scope), params
 
 
-SHORT_ROW = 64        # rows of up to this many columns: a work-item each
-
-
-def short_row_sum_function(stage, name, scope, arrays, integer):
-    """The same for rows of a few columns (coordinates, features): one
-    work-item per row walks its columns, two sums in turn -- a work-group
-    per row of 16 columns would be 240 idle lanes and a reduction for every
-    row.  Parameters as row_sum_function; ``scope`` must bind _nmk_global_id."""
-    row = ast.Name(id="_nmk_row", ctx=ast.Load())
-    exprs = [_indexed(stage.expr, arrays, [row, _offset("_nmk_j", k)]) for k in range(2)]
-    params = ["_nmk_cols"] + list(stage.inputs) + ["_nmk_out"]
-    zero = "0" if integer else "0.0"
-    body = f"""    _nmk_row = _nmk_global_id(0)
-    _nmk_a0 = {zero}
-    _nmk_a1 = {zero}
-    _nmk_whole = _nmk_cols - _nmk_cols % 2
-    for _nmk_j in range(0, _nmk_whole, 2):
-        _nmk_a0 += NMK_EXPR0
-        _nmk_a1 += NMK_EXPR1
-    for _nmk_j in range(_nmk_whole, _nmk_cols):
-        _nmk_a0 += NMK_EXPR0
-    _nmk_out[_nmk_row] = _nmk_a0 + _nmk_a1
-"""
-    return _function(name, params, body, exprs, stage, scope), params
+# Thousands of rows of up to this many columns are not summed inside the map: a work-group
+# per row would be mostly idle lanes and a work-item per row reads a cache
+# line per lane and trip (1,048,576 x 16 float64: 1244 and 133 us); the map
+# and the reduction kernels' short-row route take 45 + 42 us.
+SHORT_ROW = 64
 
 
 COLUMNS_PER_ITEM = 4      # adjacent columns per work-item of the column-sum kernel
