@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the offloaded hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME[,NAME]]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--regions R]
+                    [--only NAME[,NAME]]
 
 Prints ONE JSON line.  The headline metric is Black-Scholes options/s on
 2^24 float32 options (the configuration the metric is quoted on); every other
@@ -12,7 +13,9 @@ before the timed region.  Steps are enqueued back to back through the gpux*
 C-ABI (gpuxLaunchKernel returns an event; the wait happens after the last
 step) and the region is bracketed by queue synchronisation.  The per-kernel
 duration used for the roofline comes from HIP events recorded on the queue's
-own stream around the same region.
+own stream around the same region.  Each configuration times R such regions
+of exactly K steps; the median region is what "ms_per_step", "kernel_ms" and
+the roofline report, the fastest and slowest region are listed as "spread".
 """
 
 import argparse
@@ -73,8 +76,11 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", type=str, default="",
                     help="comma-separated subset of: add,bs,bs32,sum1,norm2,"
-                         "sum0,pairwise,matmul,gemv,dispatch,generated (plus copy, only on "
-                         "request)")
+                         "sum0,pairwise,matmul,gemv,dispatch,generated (plus copy and "
+                         "streams, only on request)")
+    ap.add_argument("--regions", type=int, default=5,
+                    help="timed regions of --steps launches per configuration; "
+                         "the median region is reported, the others as spread")
     ap.add_argument("--no-cpu", action="store_true",
                     help="skip the CPU baseline legs")
     ap.add_argument("--no-rotate", action="store_true",
@@ -121,8 +127,27 @@ class StreamTimer:
         self.lib.benchTimerDestroy(self.handle)
 
 
+class Timing:
+    """Median region of a measurement and the spread over its regions, in ms
+    per step: ``wall`` by the host clock around launch + synchronise, ``ev``
+    by HIP events on the stream."""
+
+    def __init__(self, walls, evs, kernel):
+        self.walls, self.evs, self.kernel = sorted(walls), sorted(evs), kernel
+        self.wall = self.walls[len(walls) // 2]
+        self.ev = self.evs[len(evs) // 2]
+
+    def __iter__(self):            # wall, ev, kernel = bench.measure(...)
+        return iter((self.wall, self.ev, self.kernel))
+
+    def spread(self):
+        return {"regions": len(self.evs),
+                "kernel_ms": [round(self.evs[0], 5), round(self.evs[-1], 5)],
+                "ms_per_step": [round(self.walls[0], 5), round(self.walls[-1], 5)]}
+
+
 class Bench:
-    def __init__(self, steps, warmup, rotate=True):
+    def __init__(self, steps, warmup, rotate=True, regions=5):
         from numba_mlir_amd import build as native_build
 
         if not native_build.libraries_present():
@@ -134,12 +159,14 @@ class Bench:
         self.lib = da.lib
         self.ctx = da.get_context()
         self.steps, self.warmup = steps, warmup
+        self.regions = max(1, regions)
         self.sets = ROTATE_SETS if rotate else 1
 
-    def measure(self, launches, blocking=False):
+    def measure(self, launches, blocking=False, regions=None):
         """``launches``: one callable per set of arrays (or a single callable);
-        step k runs launches[k % len].  Returns (wall ms/step, HIP-event
-        ms/step, kernel name)."""
+        step k runs launches[k % len].  After the warm-up, ``regions`` regions
+        of exactly ``steps`` launches are timed, each bracketed by queue
+        synchronisation; returns a Timing (median region, spread)."""
         ctx = self.ctx
         if callable(launches):
             launches = [launches]
@@ -163,18 +190,20 @@ class Bench:
             launch()
         ctx.synchronize()
         timer = StreamTimer(ctx.queue)
-        timer.start()
-        t0 = time.perf_counter()
-        for _ in range(self.steps):
-            launch()
-        timer.stop()
-        ctx.synchronize()
-        ev_ms = timer.elapsed_ms()
-        t1 = time.perf_counter()
+        walls, evs = [], []
+        for _ in range(regions or self.regions):
+            timer.start()
+            t0 = time.perf_counter()
+            for _ in range(self.steps):
+                launch()
+            timer.stop()
+            ctx.synchronize()
+            t1 = time.perf_counter()
+            evs.append(timer.elapsed_ms() / self.steps)
+            walls.append((t1 - t0) * 1e3 / self.steps)
         timer.close()
         ctx.set_async(False)
-        return ((t1 - t0) * 1e3 / self.steps, ev_ms / self.steps,
-                ctx.last_kernel())
+        return Timing(walls, evs, ctx.last_kernel())
 
 
 class Yardsticks:
@@ -309,15 +338,22 @@ def c_call(fn, *args):
     return lambda: fn(*args)
 
 
-def hbm_entry(name, workload, alg_bytes, wall_ms, ev_ms, kernel, extra=None):
-    achieved = alg_bytes / (ev_ms * 1e-3) / 1e9
+def hbm_entry(name, workload, alg_bytes, tm, kernel, extra=None):
+    """``tm``: the Timing of the configuration.  ``roofline.frac`` divides the
+    algorithmic bytes by the kernel's average duration between HIP events;
+    ``frac_wall`` by the host-clock time per step of the same region set
+    (launch overhead and the final synchronisation included)."""
+    achieved = alg_bytes / (tm.ev * 1e-3) / 1e9
+    achieved_wall = alg_bytes / (tm.wall * 1e-3) / 1e9
     e = {
         "name": name, "workload": workload, "kernel": kernel,
-        "ms_per_step": round(wall_ms, 5), "kernel_ms": round(ev_ms, 5),
+        "ms_per_step": round(tm.wall, 5), "kernel_ms": round(tm.ev, 5),
+        "spread": tm.spread(),
         "algorithmic_bytes": alg_bytes,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "frac_wall": round(achieved_wall / HBM_PEAK_GBS, 4),
                      "traffic": measured_traffic(kernel)},
     }
     if extra:
@@ -338,13 +374,58 @@ def cpu_leg(fn, units, unit, threads, sample, kind="port"):
             "sample": f"{sample}, {reps} passes"}
 
 
+def stream_placement_study(b):
+    """Do the relative positions of the five Black-Scholes arrays matter?
+
+    One slab per set of arrays; array k of a set starts at k * (64 MiB +
+    delta), so delta = 0 is five arrays that share every address bit below
+    2^26 (what separate large allocations give) and other deltas stagger
+    them over memory channels and banks.  Times the five-stream yardstick
+    and the Black-Scholes kernel on each placement, and the yardstick on a
+    grid of one trip per lane beside the kernel's two."""
+    import numpy as np
+
+    from numba_mlir_amd import workloads
+
+    da = b.da
+    nopt = 2 ** 24
+    nbytes = 4 * nopt
+    pad = 4 << 20
+    price, strike, t, rate, vol, _, _ = workloads.black_scholes(nopt)
+    slabs = [da.empty((5 * (nbytes + pad),), np.uint8) for _ in range(b.sets)]
+    yard = Yardsticks(b.ctx)
+    blocks2 = -(-(nopt // 4) // 256) // 2
+    rows = []
+    for delta in (0, 256, 1024, 4096, 4096 + 256, 8192, 12800, 65536, 65536 + 4096,
+                  1 << 19, 1 << 20, (1 << 20) + 4096):
+        ptrs = [[slab.ptr + k * (nbytes + delta) for k in range(5)] for slab in slabs]
+        for p in ptrs:
+            for k, host in enumerate((price, strike, t)):
+                b.lib.nmhipMemcpyHtoD(b.ctx.handle, p[k], host.ctypes.data, nbytes)
+        row = {"delta_bytes": delta}
+        for key, blocks in (("yardstick_2trips_us", blocks2), ("yardstick_1trip_us", 2 * blocks2)):
+            ty = b.measure([yard.launcher("bench_streams_3r2w_f32", blocks, 256, p, nopt)
+                            for p in ptrs], regions=3)
+            row[key] = round(ty.ev * 1e3, 2)
+        tk = b.measure([c_call(b.lib.nmhipBlackScholesF32, b.ctx.handle, p[0], p[1], p[2],
+                               float(rate), float(vol), p[3], p[4], nopt, 1)
+                        for p in ptrs], regions=3)
+        row["black_scholes_us"] = round(tk.ev * 1e3, 2)
+        rows.append(row)
+    yard.close()
+    return {"name": "streams",
+            "workload": "five float32 arrays of 2^24 elements carved from one slab, "
+                        "array k at k * (64 MiB + delta)",
+            "placements": rows}
+
+
 def run(args):
     import numpy as np
 
     from numba_mlir_amd import workloads
     from numba_mlir_amd.mlir import math_runtime
 
-    b = Bench(args.steps, args.warmup, rotate=not args.no_rotate)
+    b = Bench(args.steps, args.warmup, rotate=not args.no_rotate, regions=args.regions)
     da, ops = b.da, b.ops
     only = set(x for x in args.only.split(",") if x)
     want = lambda n: not only or n in only
@@ -372,12 +453,12 @@ def run(args):
                                d[1].ptr, d[2].ptr, float(rate), float(vol),
                                d[3].ptr, d[4].ptr, nopt, 1 if wide else 0)
                         for d in sets]
-            wall, ev, kern = b.measure(launches)
+            tm = b.measure(launches)
             e = hbm_entry(
                 key, f"Black-Scholes, 2^24 float32 options, literals typed "
                      f"{'float64 (reference typing)' if wide else 'float32'}",
-                alg, wall, ev, kern,
-                {"options_per_s": nopt / (wall * 1e-3)})
+                alg, tm, tm.kernel,
+                {"options_per_s": nopt / (tm.wall * 1e-3)})
             if orc:
                 e["cpu_baseline"] = cpu_leg(
                     lambda: orc.black_scholes(price, strike, t, rate, vol, wide, threads),
@@ -387,17 +468,29 @@ def run(args):
                 headline = (e, nopt)
                 # The same five streams (three arrays read, two written) with
                 # next to no arithmetic, on the same arrays and grid: the time
-                # the memory system needs for this access pattern.
+                # the memory system needs for this access pattern; and the
+                # rungs below it (fewer streams of the same arrays), which show
+                # what each stream adds.
                 yard = Yardsticks(b.ctx)
                 blocks = -(-(nopt // 4) // 256) // 2
-                wall_y, ev_y, _ = b.measure([yard.launcher(
-                    "bench_streams_3r2w_f32", blocks, 256, [x.ptr for x in d], nopt)
-                    for d in sets])
+                ladder = {}
+                for rung, streams in (("1r0w", 1), ("0r1w", 1), ("1r1w", 2), ("2r1w", 3),
+                                      ("3r1w", 4), ("3r2w", 5)):
+                    ty = b.measure([yard.launcher(
+                        f"bench_streams_{rung}_f32", blocks, 256, [x.ptr for x in d], nopt)
+                        for d in sets], regions=3)
+                    moved = 4 * nopt * streams
+                    ladder[rung] = {
+                        "kernel_ms": round(ty.ev, 5),
+                        "frac_of_peak": round(moved / (ty.ev * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                        "us_per_stream": round(ty.ev * 1e3 / streams, 2)}
                 yard.close()
+                ev_y = ladder["3r2w"]["kernel_ms"]
                 e["memory_floor"] = {
-                    "kernel": "bench_streams_3r2w_f32", "kernel_ms": round(ev_y, 5),
-                    "frac_of_peak": round(alg / (ev_y * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                    "kernel_over_floor": round(ev / ev_y, 4)}
+                    "kernel": "bench_streams_3r2w_f32", "kernel_ms": ev_y,
+                    "frac_of_peak": ladder["3r2w"]["frac_of_peak"],
+                    "kernel_over_floor": round(tm.ev / ev_y, 4)}
+                e["stream_ladder"] = ladder
         del sets
 
     # -- yardstick: plain copy of known size (scales the HBM counters) -------
@@ -405,11 +498,15 @@ def run(args):
         nbytes = 1 << 28
         pairs = [(da.empty((nbytes,), np.uint8), da.empty((nbytes,), np.uint8))
                  for _ in range(nsets)]
-        wall, ev, kern = b.measure([c_call(b.lib.nmhipCopy, b.ctx.handle, dst.ptr,
+        tm = b.measure([c_call(b.lib.nmhipCopy, b.ctx.handle, dst.ptr,
                                            src.ptr, nbytes) for src, dst in pairs])
         per_config.append(hbm_entry("copy", "device copy of 256 MiB",
-                                    2 * nbytes, wall, ev, kern))
+                                    2 * nbytes, tm, tm.kernel))
         del pairs
+
+    # -- study: where the five arrays start relative to each other -----------
+    if "streams" in only:
+        per_config.append(stream_placement_study(b))
 
     # -- config 1: broadcast add --------------------------------------------
     if want("add"):
@@ -421,9 +518,9 @@ def run(args):
                            i64x2(a.shape[1], 1), d_b.ptr, i64x2(0, 1), d_o.ptr,
                            i64x2(a.shape[1], 1), a.shape[0], a.shape[1])
                     for d_a, d_b, d_o in sets]
-        wall, ev, kern = b.measure(launches)
+        tm = b.measure(launches)
         alg = 2 * a.nbytes + bb.nbytes
-        e = hbm_entry("add", "a[4096,4096] + b[1,4096], float64", alg, wall, ev, kern)
+        e = hbm_entry("add", "a[4096,4096] + b[1,4096], float64", alg, tm, tm.kernel)
         if orc:
             e["cpu_baseline"] = cpu_leg(lambda: orc.add(a, bb, threads), alg / 1e9,
                                         "GB/s", threads, f"the whole array, {omp}")
@@ -439,10 +536,10 @@ def run(args):
             launches = [c_call(b.lib.nmhipReduce, b.ctx.handle, 0, 2, d_x.ptr,
                                x.shape[0], x.shape[1], x.shape[1], 1, 1, d_o.ptr)
                         for d_x in d_xs]
-            wall, ev, kern = b.measure(launches)
+            tm = b.measure(launches)
             alg = x.nbytes + 4 * x.shape[0]
             e = hbm_entry("sum1", "np.sum(x, axis=1), float32 [16384,8192]",
-                          alg, wall, ev, kern)
+                          alg, tm, tm.kernel)
             if orc:
                 e["cpu_baseline"] = cpu_leg(lambda: orc.sum_axis1_f32(x, threads),
                                             alg / 1e9, "GB/s", threads,
@@ -450,12 +547,12 @@ def run(args):
             per_config.append(e)
         if want("norm2"):
             d_o = da.empty((1,), np.float32)
-            wall, ev, kern = b.measure([c_call(
+            tm = b.measure([c_call(
                 b.lib.nmhipNorm2F32, b.ctx.handle, d_x.ptr, x.size, d_o.ptr)
                 for d_x in d_xs])
             alg = x.nbytes + 4
             e = hbm_entry("norm2", "np.sqrt(np.sum(x*x)), float32 [16384,8192]",
-                          alg, wall, ev, kern)
+                          alg, tm, tm.kernel)
             if orc:
                 e["cpu_baseline"] = cpu_leg(lambda: orc.norm2_f32(x, threads),
                                             alg / 1e9, "GB/s", threads,
@@ -469,10 +566,10 @@ def run(args):
         launches = [c_call(b.lib.nmhipReduce, b.ctx.handle, 0, 0, d_x.ptr,
                            xi.shape[0], xi.shape[1], xi.shape[1], 1, 0, d_o.ptr)
                     for d_x in d_xs]
-        wall, ev, kern = b.measure(launches)
+        tm = b.measure(launches)
         alg = xi.nbytes + 8 * xi.shape[1]
         e = hbm_entry("sum0", "np.sum(x, axis=0), int32 [16384,8192] -> int64",
-                      alg, wall, ev, kern)
+                      alg, tm, tm.kernel)
         if orc:
             e["cpu_baseline"] = cpu_leg(lambda: orc.sum_axis0_i32(xi, threads),
                                         alg / 1e9, "GB/s", threads,
@@ -485,12 +582,12 @@ def run(args):
         X, Y = workloads.pairwise()
         d_X, d_Y = da.asarray(X), da.asarray(Y)
         outs = [da.empty((X.shape[0], Y.shape[0]), np.float64) for _ in range(nsets)]
-        wall, ev, kern = b.measure([c_call(
+        tm = b.measure([c_call(
             b.lib.nmhipPairwiseF64, b.ctx.handle, d_X.ptr, d_Y.ptr, d_D.ptr,
             X.shape[0], Y.shape[0]) for d_D in outs])
         alg = X.nbytes + Y.nbytes + 8 * X.shape[0] * Y.shape[0]
         e = hbm_entry("pairwise", "pairwise distance @kernel, float64 [8192,3]^2",
-                      alg, wall, ev, kern)
+                      alg, tm, tm.kernel)
         if orc:
             e["cpu_baseline"] = cpu_leg(lambda: orc.pairwise(X, Y, threads), alg / 1e9,
                                         "GB/s", threads, f"all 8192^2 distances, {omp}")
@@ -505,19 +602,22 @@ def run(args):
         d_Cs = [da.empty((n, n), np.float32) for _ in range(nsets)]
         saved = b.steps
         b.steps = max(5, min(saved, 20))
-        wall, ev, _ = b.measure([lambda d_C=d_C: ops.dot(d_A, d_B, out=d_C)
-                                 for d_C in d_Cs], blocking=True)
+        tm = b.measure([lambda d_C=d_C: ops.dot(d_A, d_B, out=d_C)
+                        for d_C in d_Cs], blocking=True, regions=min(b.regions, 3))
         b.steps = saved
         flops = 2.0 * n ** 3
-        tf = flops / (ev * 1e-3) / 1e12
+        tf = flops / (tm.ev * 1e-3) / 1e12
+        tf_wall = flops / (tm.wall * 1e-3) / 1e12
         e = {
             "name": "matmul", "workload": "np.dot float32 [4096,4096]^2",
             "kernel": math_runtime.last_kernel(),
-            "ms_per_step": round(wall, 5), "kernel_ms": round(ev, 5),
+            "ms_per_step": round(tm.wall, 5), "kernel_ms": round(tm.ev, 5),
+            "spread": tm.spread(),
             "algorithmic_flops": flops,
             "roofline": {"bound": "mfma", "achieved": round(tf, 2),
                          "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4),
+                         "frac_wall": round(tf_wall / FP32_MFMA_PEAK_TFLOPS, 4),
                          "traffic": measured_traffic(math_runtime.last_kernel())},
         }
         if orc:
@@ -549,11 +649,11 @@ def run(args):
         d_ys = [da.empty((n, 1), np.float32) for _ in range(nsets)]
         saved = b.steps
         b.steps = max(5, min(saved, 20))
-        wall, ev, _ = b.measure([lambda d_y=d_y: ops.dot(d_A, d_v, out=d_y)
-                                 for d_y in d_ys], blocking=True)
+        tm = b.measure([lambda d_y=d_y: ops.dot(d_A, d_v, out=d_y)
+                        for d_y in d_ys], blocking=True)
         b.steps = saved
         e = hbm_entry("gemv", "np.dot float32 [16384,16384] x [16384,1]",
-                      (n * n + 2 * n) * 4, wall, ev, math_runtime.last_kernel())
+                      (n * n + 2 * n) * 4, tm, math_runtime.last_kernel())
         if orc:
             e["cpu_baseline"] = cpu_leg(lambda: np.dot(A, v), (n * n + 2 * n) * 4 / 1e9,
                                         "GB/s", os.cpu_count() or 1,
@@ -582,6 +682,7 @@ def run(args):
             "unit": "options/s",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": e["ms_per_step"],
+            "regions": e["spread"]["regions"], "spread": e["spread"],
             "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None,
             "dtype": "f32 (literal-bearing intermediates f64)",
@@ -697,10 +798,10 @@ def generated_kernels(b, workloads):
             if len(events) > 16:
                 plan.retire(events.pop(0))
 
-        wall, ev, _ = b.measure(launch)
+        tm = b.measure(launch)
         for event in events:
             plan.retire(event)
-        e = hbm_entry(name, workload, alg_bytes, wall, ev, plan.info["kernel"])
+        e = hbm_entry(name, workload, alg_bytes, tm, plan.info["kernel"])
         e["path"] = "generated"
         out.append(e)
 

@@ -32,6 +32,57 @@ bench_streams_3r2w_f32(const float *__restrict__ a, const float *__restrict__ b,
   }
 }
 
+// The ladder: R float32 arrays read and W written with the same accesses and
+// grid as above (1r0w, 0r1w, 1r1w, 2r1w, 3r1w; bench_streams_3r2w_f32 is the
+// top rung).  It shows what each additional stream costs on this memory
+// system, i.e. whether the five-stream mix is slower than fewer streams of
+// the same total size.  A read-only rung consumes what it loads through a
+// store that no input ever triggers.
+struct StreamSet {
+  const float4_y *r[3];
+  float4_y *w[2];
+};
+
+template <int R, int W>
+__device__ __forceinline__ void streamsBody(const StreamSet &p, int64_t n) {
+  const int64_t nvec = n / 4;
+  const int64_t stride = int64_t(gridDim.x) * blockDim.x;
+  for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec;
+       i += stride) {
+    float4_y acc = {1.f, 1.f, 1.f, 1.f};
+    float4_y v[R > 0 ? R : 1];
+#pragma unroll
+    for (int k = 0; k < R; ++k)
+      v[k] = __builtin_nontemporal_load(p.r[k] + i);
+#pragma unroll
+    for (int k = 0; k < R; ++k)
+      acc += v[k];
+    if (W == 0 && acc[0] == 12345.678f && acc[3] == -1.f)
+      p.w[0][i] = acc;
+#pragma unroll
+    for (int k = 0; k < W; ++k)
+      __builtin_nontemporal_store(acc * float(k + 1), p.w[k] + i);
+  }
+}
+
+#define BENCH_STREAMS(NAME, R, W)                                              \
+  extern "C" __global__ __launch_bounds__(256) void NAME(                      \
+      const float *a, const float *b, const float *c, float *x, float *y,      \
+      int64_t n) {                                                             \
+    StreamSet p;                                                               \
+    p.r[0] = reinterpret_cast<const float4_y *>(a);                            \
+    p.r[1] = reinterpret_cast<const float4_y *>(b);                            \
+    p.r[2] = reinterpret_cast<const float4_y *>(c);                            \
+    p.w[0] = reinterpret_cast<float4_y *>(x);                                  \
+    p.w[1] = reinterpret_cast<float4_y *>(y);                                  \
+    streamsBody<R, W>(p, n);                                                   \
+  }
+BENCH_STREAMS(bench_streams_1r0w_f32, 1, 0)
+BENCH_STREAMS(bench_streams_0r1w_f32, 0, 1)
+BENCH_STREAMS(bench_streams_1r1w_f32, 1, 1)
+BENCH_STREAMS(bench_streams_2r1w_f32, 2, 1)
+BENCH_STREAMS(bench_streams_3r1w_f32, 3, 1)
+
 // Dispatch-overhead yardsticks: eight work-items write their index into the
 // first of 1, 2, 6 or 12 int32 array arguments (the kernels of the
 // reference's kernel_dispatcher microbenchmark,
