@@ -278,31 +278,37 @@ template <> struct BsMath<double> {
   }
 };
 template <> struct BsMath<float> {
+  // 1 / sqrt(z) of a float with an exponent in [-60, 60): the hardware seed
+  // (one unit in the last place) with one Newton step, which leaves about
+  // half a unit -- what the two roundings of 1.0f / sqrtf(z) leave as well.
+  __device__ static __forceinline__ float rsqrtNormal(float z) {
+    const float y = __builtin_amdgcn_rsqf(z);
+    const float e = __builtin_fmaf(-(z * y), y, 1.0f); // 1 - z y^2
+    return __builtin_fmaf(y * e, 0.5f, y);
+  }
+  // Any z: the same value as rsqrtNormal where that applies, so a lane gets
+  // the same price whichever body its wave runs.
   __device__ static __forceinline__ float rsqrt_(float z) {
-    return 1.0f / sqrtf(z);
+    return (__float_as_uint(z) - 0x21800000u) < 0x3C000000u ? rsqrtNormal(z)
+                                                            : 1.0f / sqrtf(z);
   }
-  __device__ static __forceinline__ float cdfTerm(float x, const double2_lds *) {
-    return 0.5f + 0.5f * erff(x);
+  // 0.5 + 0.5 erf(x) rounded once to float32, from the float64 table (the
+  // library's erff, two multiply-adds and two roundings later, lands within
+  // one unit in the last place of the same value).
+  __device__ static __forceinline__ float cdfTerm(float x, const double2_lds *tab) {
+    return float(bsCdfTerm(double(x), tab));
   }
-  __device__ static __forceinline__ bool eitherNaN(float, float) {
-    return false; // erff propagates NaN by itself
+  __device__ static __forceinline__ bool eitherNaN(float a, float b) {
+    return __builtin_isunordered(a, b); // bsCdfTerm maps NaN to a number
   }
 };
 
-// The float32 steps log(P / S) and exp(b) without the range handling of the
-// general routines: the same operations in the same order, so log and exp
-// are bit-identical to logf and expf whenever bsEveryday() holds -- P and S
-// positive with exponents in [-60, 60) (the quotient and the reciprocal are
-// then normal numbers) and |b| <= 80 (exp(b) is normal).  The division is
-// the reciprocal times P with one residual correction: it equals the
-// correctly rounded quotient unless that quotient lies within 2e-7 units in
-// the last place of a rounding boundary.  Used by the all-float32 kernel.
-__device__ __forceinline__ bool bsEveryday(float P, float S, float b) {
-  const uint32_t lo = 0x21800000u;   // bits of 2^-60
-  const uint32_t span = 0x3C000000u; // up to, not including, 2^60
-  return (__float_as_uint(P) - lo) < span && (__float_as_uint(S) - lo) < span &&
-         __builtin_fabsf(b) <= 80.0f;
-}
+// P / S for positive P and S with exponents in [-60, 60) (the quotient and
+// the reciprocal are then normal numbers): the reciprocal times P with one
+// residual correction, which equals the correctly rounded quotient unless
+// that quotient lies within 2e-7 units in the last place of a rounding
+// boundary.  With logNormalF32 and expNormalF32 it gives the library's
+// log(P / S) and exp(b) bit for bit (NMK_BS_EXACT_F32_STEPS).
 __device__ __forceinline__ float bsDivEveryday(float P, float S) {
   const float y = __builtin_amdgcn_rcpf(S);
   const float q = P * y;
@@ -310,12 +316,13 @@ __device__ __forceinline__ float bsDivEveryday(float P, float S) {
   return __builtin_fmaf(e, y, q);
 }
 
-template <typename W, bool EVERYDAY>
+// One option by the general routines, any operands.
+template <typename W>
 __device__ __forceinline__ void
 blackScholesOne(float P, float S, float T, float mr, W sigSigTwo,
                 const double2_lds *erfTab, float &call, float &put) {
   const float b = T * mr;
-  const float a = EVERYDAY ? logNormalF32(bsDivEveryday(P, S)) : logf(P / S);
+  const float a = logf(P / S);
   const W z = W(T) * sigSigTwo;
   const W c = W(0.25) * z;
   const W y = BsMath<W>::rsqrt_(z);
@@ -324,7 +331,7 @@ blackScholesOne(float P, float S, float T, float mr, W sigSigTwo,
   const W w2 = (W(amb) - c) * y;
   const W d1 = BsMath<W>::cdfTerm(w1, erfTab); // 0.5 + 0.5 * erf(w1)
   const W d2 = BsMath<W>::cdfTerm(w2, erfTab);
-  const float Se = (EVERYDAY ? expNormalF32(b) : expf(b)) * S;
+  const float Se = expf(b) * S;
   const W r = W(P) * d1 - W(Se) * d2;
   const bool nan = BsMath<W>::eitherNaN(w1, w2);
   call = nan ? __builtin_nanf("") : float(r);
@@ -341,7 +348,7 @@ __device__ __attribute__((noinline)) BsPrices
 bsCareful(float P, float S, float T, float mr, double sigSigTwo,
           const double2_lds *erfTab) {
   BsPrices out;
-  blackScholesOne<double, false>(P, S, T, mr, sigSigTwo, erfTab, out.call, out.put);
+  blackScholesOne<double>(P, S, T, mr, sigSigTwo, erfTab, out.call, out.put);
   return out;
 }
 
@@ -385,10 +392,12 @@ bsPlain(float P, float S, float T, float mr, double sigSigTwo,
 // no option qualifies (tLimitBits == 0).
 struct BsPlainTest {
   uint32_t tLimitBits;
-  __device__ __forceinline__ BsPlainTest(float rate, float volatility) {
+  // |volatility| must lie in [1 / volSpan, volSpan]: 2^50 where z = 2 vol^2 T
+  // is a double, 2^30 where it is a float (z then stays a normal number).
+  __device__ __forceinline__ BsPlainTest(float rate, float volatility, float volSpan) {
     const float av = __builtin_fabsf(volatility);
-    const bool scalarsOk =
-        __builtin_fabsf(rate) < 0x1p60f && av >= 0x1p-50f && av <= 0x1p50f;
+    const bool scalarsOk = __builtin_fabsf(rate) < 0x1p60f &&
+                           av >= 1.0f / volSpan && av <= volSpan;
     const float bMax = NMK_BS_EXACT_F32_STEPS ? 80.0f : 1.0f;
     float tLimit =
         __builtin_fminf(0x1p60f, bMax * 0.999f / __builtin_fabsf(rate));
@@ -419,7 +428,60 @@ struct BsPlainTest {
     return least >= 0x21800000u /* 2^-60 */ && mostPS < 0x5D800000u /* 2^60 */ &&
            mostT < tLimitBits;
   }
+  // The same test for one option.
+  __device__ __forceinline__ bool lane(float P, float S, float T) const {
+    const uint32_t p = __float_as_uint(P), s = __float_as_uint(S), t = __float_as_uint(T);
+    return min(min(p, s), t) >= 0x21800000u && max(p, s) < 0x5D800000u &&
+           t < tLimitBits;
+  }
 };
+
+// ---- float32 typing: the same two bodies with every step in float32 --------
+// 0.5 + 0.5 erf comes from the float64 table in both (rounded once to
+// float32: the library's erff with its two further roundings lands within a
+// unit in the last place of it), so the float32 kernel's arithmetic is a
+// subset of the float64 one's and no longer bound by it.
+__device__ __forceinline__ void
+bsPlain32(float P, float S, float T, float mr, float sigSigTwo,
+          const double2_lds *erfTab, float &call, float &put) {
+  const float b = T * mr;
+#if NMK_BS_EXACT_F32_STEPS
+  const float a = logNormalF32(bsDivEveryday(P, S));
+  const float eb = expNormalF32(b);
+#else
+  const float a =
+      __builtin_amdgcn_logf(P * __builtin_amdgcn_rcpf(S)) * 0x1.62e430p-1f;
+  const float eb = __builtin_amdgcn_exp2f(b * 0x1.715476p+0f);
+#endif
+  const float z = T * sigSigTwo;
+  const float c = 0.25f * z;
+  const float y = BsMath<float>::rsqrtNormal(z);
+  const float amb = a - b;
+  const float w1 = (amb + c) * y;
+  const float w2 = (amb - c) * y;
+  const float d1 = BsMath<float>::cdfTerm(w1, erfTab);
+  const float d2 = BsMath<float>::cdfTerm(w2, erfTab);
+  const float Se = eb * S;
+  const float r = P * d1 - Se * d2;
+  call = r;
+  put = r - P + Se;
+}
+
+// Any option: the plain forms where the option qualifies for them (so that
+// it gets the same price whichever body its wave runs), the general routines
+// otherwise.  Out of line, like bsCareful.
+__device__ __attribute__((noinline)) BsPrices
+bsCareful32(float P, float S, float T, float mr, float sigSigTwo,
+            const double2_lds *erfTab, uint32_t tLimitBits) {
+  BsPrices out;
+  BsPlainTest test(0.f, 1.f, 2.f);
+  test.tLimitBits = tLimitBits;
+  if (test.lane(P, S, T))
+    bsPlain32(P, S, T, mr, sigSigTwo, erfTab, out.call, out.put);
+  else
+    blackScholesOne<float>(P, S, T, mr, sigSigTwo, erfTab, out.call, out.put);
+  return out;
+}
 
 // Copies the erf table into LDS (97 rows of three 128-bit words).
 __device__ __forceinline__ void bsStageTable(double2_lds *tab) {
@@ -440,7 +502,7 @@ blackScholesWide(const float *__restrict__ price, const float *__restrict__ stri
   bsStageTable(erfTab);
   const float mr = -rate;
   const double sigSigTwo = double(volatility * volatility) * 2.0;
-  const BsPlainTest isPlain(rate, volatility);
+  const BsPlainTest isPlain(rate, volatility, 0x1p50f);
   const int64_t nvec = n / 4;
   const int64_t stride = int64_t(gridDim.x) * blockDim.x;
   const float4_t *pv = reinterpret_cast<const float4_t *>(price);
@@ -483,15 +545,15 @@ blackScholesWide(const float *__restrict__ price, const float *__restrict__ stri
   }
 }
 
-// ---- float32 typing ---------------------------------------------------------
-// One trip of four options per lane.  The everyday forms are taken when every
-// lane of the wave qualifies, so each version stays one straight-line block.
 __device__ __forceinline__ void
 blackScholesNarrow(const float *__restrict__ price, const float *__restrict__ strike,
                    const float *__restrict__ t, float rate, float volatility,
                    float *__restrict__ call, float *__restrict__ put, int64_t n) {
+  __shared__ __attribute__((aligned(16))) double2_lds erfTab[NMK_ERF_NODES * 3];
+  bsStageTable(erfTab);
   const float mr = -rate;
   const float sigSigTwo = (volatility * volatility) * 2.0f;
+  const BsPlainTest isPlain(rate, volatility, 0x1p30f);
   const int64_t nvec = n / 4;
   const int64_t stride = int64_t(gridDim.x) * blockDim.x;
   const float4_t *pv = reinterpret_cast<const float4_t *>(price);
@@ -505,25 +567,21 @@ blackScholesNarrow(const float *__restrict__ price, const float *__restrict__ st
     const float4_t S = streamLoad(sv + i);
     const float4_t T = streamLoad(tv + i);
     float4_t c, u;
-    bool everyday = true;
-#pragma unroll
-    for (int k = 0; k < 4; ++k)
-      everyday = everyday && bsEveryday(P[k], S[k], T[k] * mr);
-    if (__builtin_amdgcn_ballot_w64(!everyday) == 0) {
+    if (__builtin_amdgcn_ballot_w64(!isPlain(P, S, T)) == 0) {
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         float ck, uk;
-        blackScholesOne<float, true>(P[k], S[k], T[k], mr, sigSigTwo, nullptr, ck, uk);
+        bsPlain32(P[k], S[k], T[k], mr, sigSigTwo, erfTab, ck, uk);
         c[k] = ck;
         u[k] = uk;
       }
     } else {
-#pragma unroll
+#pragma unroll 1
       for (int k = 0; k < 4; ++k) {
-        float ck, uk;
-        blackScholesOne<float, false>(P[k], S[k], T[k], mr, sigSigTwo, nullptr, ck, uk);
-        c[k] = ck;
-        u[k] = uk;
+        const BsPrices o =
+            bsCareful32(P[k], S[k], T[k], mr, sigSigTwo, erfTab, isPlain.tLimitBits);
+        c[k] = o.call;
+        u[k] = o.put;
       }
     }
     streamStore(c, cv + i);
@@ -531,11 +589,10 @@ blackScholesNarrow(const float *__restrict__ price, const float *__restrict__ st
   }
   const int64_t tail = nvec * 4 + threadIdx.x;
   if (blockIdx.x == 0 && tail < n) {
-    float ck, uk;
-    blackScholesOne<float, false>(price[tail], strike[tail], t[tail], mr, sigSigTwo,
-                                  nullptr, ck, uk);
-    call[tail] = ck;
-    put[tail] = uk;
+    const BsPrices o = bsCareful32(price[tail], strike[tail], t[tail], mr, sigSigTwo,
+                                   erfTab, isPlain.tLimitBits);
+    call[tail] = o.call;
+    put[tail] = o.put;
   }
 }
 
@@ -547,7 +604,8 @@ nmk_black_scholes_f32_w64(const float *price, const float *strike,
   blackScholesWide(price, strike, t, rate, volatility, call, put, n);
 }
 
-NMK_KERNEL(256)
+extern "C" __global__ __launch_bounds__(256)
+__attribute__((amdgpu_waves_per_eu(6, 8))) void
 nmk_black_scholes_f32_w32(const float *price, const float *strike,
                           const float *t, float rate, float volatility,
                           float *call, float *put, int64_t n) {

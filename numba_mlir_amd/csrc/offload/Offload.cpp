@@ -690,14 +690,12 @@ NMHIP_EXPORT void nmhipBlackScholesF32(void *ctx, const float *price,
       fail("nmhipBlackScholesF32: arrays must be 16-byte aligned");
     if (n < 0)
       fail("nmhipBlackScholesF32: negative extent");
-    // Four options per lane and trip.  The float64-typed kernel streams best
-    // from many short blocks, two trips a lane (8192 blocks at 2^24 options:
-    // 56.5 us against 59 us for 4096 blocks and for 16384); the float32 one
-    // is bound by its arithmetic and keeps 4096 long-running blocks.
+    // Four options per lane and trip.  Both kernels stream best from many
+    // short blocks, two trips a lane (8192 blocks at 2^24 options: 56.5 us
+    // against 59 us for 4096 blocks and for 16384, where staging the erf
+    // table once per block weighs more).
     const int64_t need = ceilDiv(ceilDiv(n, 4), 256);
-    int64_t blocks = tuning().bsBlocks ? tuning().bsBlocks
-                     : wide            ? ceilDiv(need, 2)
-                                       : 256 * 16;
+    int64_t blocks = tuning().bsBlocks ? tuning().bsBlocks : ceilDiv(need, 2);
     if (blocks > need)
       blocks = need;
     if (blocks > 0x7fffffff)
