@@ -187,12 +187,15 @@ void nmhipPairwiseF64(void *ctx, const double *X1, const double *X2, double *D,
 
 /* ---- code objects and tuning ------------------------------------------- */
 
-/* The embedded gfx950 code object of a family: "maps", "reduce", "twins". */
+/* The embedded gfx950 code object of a family: "maps", "reduce", "twins", or
+ * "reduce_release" (the reduction kernels with the release / acquire hand-off
+ * of partial results). */
 const void *nmhipKernelBlob(const char *family, size_t *size);
 
 /* Overrides a launch-shape knob ("rowbcast_rows", "map_blocks", "bs_blocks",
  * "reduce_blocks", "axis0_rows", "cols_blocks", "pairwise_rows"); 0 restores
- * the default. */
+ * the default.  "handoff_release" = 1 takes the reduction kernels from the
+ * "reduce_release" code object instead of "reduce". */
 void nmhipSetTuning(const char *knob, int64_t value);
 
 #ifdef __cplusplus

@@ -75,17 +75,25 @@ def _run(cmd):
         print(out, file=sys.stderr)
 
 
-def build_code_object(family):
+def build_code_object(family, variant="", defines=()):
     """One gfx950 ELF code object per kernel family.
 
     -ffp-contract=off keeps a*b+c as two roundings, matching the reference's
     CPU lowering (no fma without fastmath).
     """
     src = os.path.join(CSRC, "kernels", family + ".hip")
-    out = os.path.join(BUILD, family + ".hsaco")
+    out = os.path.join(BUILD, family + variant + ".hsaco")
     _run([HIPCC, "--genco", "--no-gpu-bundle-output", *DEVICE_FLAGS,
-          "-ffp-contract=off", "-o", out, src])
+          "-ffp-contract=off", *["-D" + d for d in defines], "-o", out, src])
     return out
+
+
+def build_reduce_release():
+    """The reduction kernels once more with the hand-off of partial results
+    written as the language's memory model asks (release on the ticket,
+    acquire in the last block): the code object the default one is checked
+    against (tuning knob "handoff_release")."""
+    return build_code_object("reduce", "_release", ["NMK_HANDOFF_RELEASE=1"])
 
 
 def build_runtime():
@@ -159,6 +167,7 @@ def build_all(jobs=4):
     os.makedirs(BUILD, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         futures = [pool.submit(build_code_object, f) for f in KERNEL_FAMILIES]
+        futures.append(pool.submit(build_reduce_release))
         futures.append(pool.submit(build_runtime))
         futures.append(pool.submit(build_math))
         futures.append(pool.submit(build_bench_timer))

@@ -142,7 +142,10 @@ __device__ __forceinline__ int64_t blockLinearXY() {
 //    memory model alone.  The release writes back the whole L2 of the XCD
 //    (buffer_wbl2) once per block, under the blocks that are still
 //    streaming; measured on MI355X: sqrt(sum(x*x)) over 512 MiB 78 -> 89 us,
-//    column sums 82 -> 89 us.  Kept for checking the default against.
+//    column sums 82 -> 89 us.  Built as a second code object of the
+//    reduction kernels ("reduce_release"), which the offload library carries
+//    and a tuning knob selects; a GPU test holds the two code objects to
+//    identical bits on the full-size benchmark reductions.
 #ifndef NMK_HANDOFF_RELEASE
 #define NMK_HANDOFF_RELEASE 0
 #endif

@@ -14,6 +14,12 @@ nmhip_blob_reduce:
 	.incbin "reduce.hsaco"
 nmhip_blob_reduce_end:
 	.balign 4096
+	.global nmhip_blob_reduce_release
+	.global nmhip_blob_reduce_release_end
+nmhip_blob_reduce_release:
+	.incbin "reduce_release.hsaco"
+nmhip_blob_reduce_release_end:
+	.balign 4096
 	.global nmhip_blob_twins
 	.global nmhip_blob_twins_end
 nmhip_blob_twins:

@@ -24,6 +24,8 @@
 // Code objects, embedded by Blobs.S.
 extern "C" const unsigned char nmhip_blob_maps[], nmhip_blob_maps_end[];
 extern "C" const unsigned char nmhip_blob_reduce[], nmhip_blob_reduce_end[];
+extern "C" const unsigned char nmhip_blob_reduce_release[],
+    nmhip_blob_reduce_release_end[];
 extern "C" const unsigned char nmhip_blob_twins[], nmhip_blob_twins_end[];
 
 namespace {
@@ -100,6 +102,10 @@ struct Tuning {
   int64_t pairwiseRows = 0;
   int64_t bsBlocks = 0;
   int64_t colsBlocks = 0;
+  // Non-zero: reduction kernels come from the code object whose hand-off of
+  // partial results uses release / acquire (slower; for checking the default
+  // hand-off against).
+  int64_t handoffRelease = 0;
 };
 
 Tuning &tuning() {
@@ -175,6 +181,8 @@ const Blob *findBlob(const char *family) {
   static const Blob blobs[] = {
       {"maps", nmhip_blob_maps, nmhip_blob_maps_end},
       {"reduce", nmhip_blob_reduce, nmhip_blob_reduce_end},
+      // reduce.hip built with NMK_HANDOFF_RELEASE=1 (csrc/kernels/common.h)
+      {"reduce_release", nmhip_blob_reduce_release, nmhip_blob_reduce_release_end},
       {"twins", nmhip_blob_twins, nmhip_blob_twins_end},
   };
   for (const Blob &b : blobs)
@@ -231,10 +239,13 @@ public:
   std::mutex mutex;
 
   void *kernel(const std::string &name) {
-    auto it = kernels.find(name);
+    const char *family = familyOf(name);
+    if (tuning().handoffRelease && std::strcmp(family, "reduce") == 0)
+      family = "reduce_release";
+    const std::string key = std::string(family) + ":" + name;
+    auto it = kernels.find(key);
     if (it != kernels.end())
       return it->second;
-    const char *family = familyOf(name);
     void *&mod = modules[family];
     if (!mod) {
       const Blob *blob = findBlob(family);
@@ -242,7 +253,7 @@ public:
           queue, blob->begin, static_cast<size_t>(blob->end - blob->begin));
     }
     void *k = SYM(KernelGet, "gpuxKernelGet")(mod, name.c_str());
-    kernels.emplace(name, k);
+    kernels.emplace(key, k);
     return k;
   }
 
@@ -1054,6 +1065,8 @@ NMHIP_EXPORT void nmhipSetTuning(const char *knob, int64_t value) {
       t.bsBlocks = value;
     else if (k == "cols_blocks")
       t.colsBlocks = value;
+    else if (k == "handoff_release")
+      t.handoffRelease = value;
     else
       fail("Unknown tuning knob '%s'", knob);
   });

@@ -255,3 +255,45 @@ def test_generic_reductions_on_every_route(env, dtype, what, shape, offset):
         for axis in (0, 1):       # (int64 wraps the same way in NumPy)
             got = ops.prod(fd, axis=axis).asnumpy()
             np.testing.assert_array_equal(got, np.prod(fa.astype(np.int64), axis=axis))
+
+
+def test_release_acquire_handoff_gives_the_same_bits(env):
+    """The reduction kernels hand per-block partial results to the launch's
+    last block through agent-scope accesses ordered by a wait for the stores'
+    acknowledgement.  The same kernels built with the hand-off the language's
+    memory model prescribes (release on the ticket, acquire in the last block:
+    the "reduce_release" code object) combine in the same fixed order, so the
+    three benchmark reductions at full size, and the generic kernels, must give
+    identical bits from both code objects."""
+    hip, ops, _ = env
+    from numba_mlir_amd.mlir import lowered
+    plain, release = lowered.kernel_blob("reduce"), lowered.kernel_blob("reduce_release")
+    assert plain != release                     # the build flag took effect
+    rng = np.random.Generator(np.random.PCG64(1003))
+    x = rng.standard_normal((16384, 8192), dtype=np.float32)
+    xi = np.random.Generator(np.random.PCG64(1013)).integers(
+        -1000, 1000, (16384, 8192), dtype=np.int32, endpoint=True)
+    d_x, d_xi = hip.asarray(x), hip.asarray(xi)
+    d_x64 = hip.asarray(x[:2048].astype(np.float64))
+
+    def results():
+        out = [ops.sum(d_x, axis=1).asnumpy(),
+               ops.sqrt_sum_squares(d_x.reshape((x.size,))).asnumpy(),
+               ops.sum(d_xi, axis=0).asnumpy()]
+        names = [hip.get_context().last_kernel()]
+        out += [ops.sum(d_x, axis=0).asnumpy(), np.asarray(ops.amax(d_x)),
+                ops.prod(d_x64, axis=0).asnumpy(), np.asarray(ops.sum(d_x64))]
+        return out, names
+
+    try:
+        base, names0 = results()
+        lowered.set_tuning("handoff_release", 1)
+        other, names1 = results()
+    finally:
+        lowered.set_tuning("handoff_release", 0)
+    assert names0 == names1 == ["nmk_sum_axis0_i32_i64"]
+    for a, b in zip(base, other):
+        assert a.dtype == b.dtype and a.shape == b.shape
+        assert a.tobytes() == b.tobytes()
+    # and the integer one is the exact column sum either way
+    assert np.array_equal(other[2], xi.sum(axis=0, dtype=np.int64))
