@@ -54,9 +54,11 @@ void mkl_gemm_float64_device(void *queue, const NmhipMemref2F64 *a,
 
 /*
  * mkl_gemm_float32_device for callers that cannot allocate device memory
- * (code under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc).  No counterpart in the reference.  Same arguments as
- * mkl_gemm_float32_device; it calls no hipMalloc / hipFree.  Where that
+ * (tight serving loops, harnesses that forbid hipMalloc).  No counterpart in
+ * the reference.  Same arguments as mkl_gemm_float32_device; it calls no
+ * hipMalloc / hipFree.  Like that entry point it returns when C is complete
+ * (it synchronises the queue's stream), so it cannot be issued on a stream
+ * that is being captured into a HIP graph.  Where that
  * entry point takes its workspace from a heap block it grows on demand, this
  * one uses a fixed 16 MiB array that lives in the library's device image on
  * every GPU it runs on, and shares K out over the blocks by split K only
@@ -73,8 +75,7 @@ void mkl_gemm_float64_device(void *queue, const NmhipMemref2F64 *a,
  * keeps the last call's partial products; nothing in it needs clearing,
  * each slice is written before it is read.  Calls from several host
  * threads take turns on it (the library holds a lock while a call's kernels
- * run); launches captured into graphs and replayed side by side on one GPU
- * would race on it.
+ * run).
  */
 int mkl_gemm_float32_device_noalloc(void *queue, const NmhipMemref2F32 *a,
                                     const NmhipMemref2F32 *b, float alpha,

@@ -27,6 +27,8 @@
 //    memory, no host loop, bit-identical from run to run.
 #include <mlir/Dialect/Arith/IR/Arith.h>
 #include <mlir/Dialect/GPU/IR/GPUDialect.h>
+#include <mlir/Dialect/LLVMIR/LLVMDialect.h>
+#include <mlir/IR/IRMapping.h>
 #include <mlir/Dialect/MemRef/IR/MemRef.h>
 #include <mlir/Dialect/SCF/IR/SCF.h>
 #include <mlir/Pass/Pass.h>
@@ -123,12 +125,52 @@ template <typename Base> struct ConvertGpuWaitPattern : public Base {
 
 // ---- 2. the last workgroup finishes the reduction -----------------------------
 // Replaces the body of LowerGPUGlobalReduce::matchAndRewrite from the
-// allocation on (GpuToGpuRuntime.cpp:2187-2277).  `combine(a, b)` clones the
-// reduction region; `neutral` is getNeutralValue()'s attribute.
+// allocation on (GpuToGpuRuntime.cpp:2187-2277); `neutral` is what
+// getNeutralValue() returned for the reduction region.
+//
+// Ordering.  The partial of a workgroup must be visible device-wide before
+// its ticket is, and the last workgroup must not read partials it fetched
+// before it drew the last ticket: an agent-scope release fence ahead of the
+// increment and an agent-scope acquire fence behind the last draw (LLVM
+// dialect fences, which pass through the ROCDL tail unchanged and become
+// buffer_wbl2 / buffer_inv around the global_atomic_add).
+
+// Workgroup (bx, by, bz) of a (gx, gy, gz) grid -> bx + gx * (by + gy * bz).
+inline mlir::Value linearGroupId(mlir::OpBuilder &b, mlir::Location loc,
+                                 const mlir::gpu::KernelDim3 &grid,
+                                 const mlir::gpu::KernelDim3 &id) {
+  mlir::Value yz = b.create<mlir::arith::AddIOp>(
+      loc, id.y, b.create<mlir::arith::MulIOp>(loc, grid.y, id.z));
+  return b.create<mlir::arith::AddIOp>(loc, id.x,
+                                       b.create<mlir::arith::MulIOp>(loc, grid.x, yz));
+}
+
+// True in the work-item whose three local ids are all zero.
+inline mlir::Value isFirstItem(mlir::OpBuilder &b, mlir::Location loc,
+                               const mlir::gpu::KernelDim3 &tid) {
+  mlir::Value zero = b.create<mlir::arith::ConstantIndexOp>(loc, 0);
+  mlir::Value any = b.create<mlir::arith::OrIOp>(
+      loc, tid.x, b.create<mlir::arith::OrIOp>(loc, tid.y, tid.z));
+  return b.create<mlir::arith::CmpIOp>(loc, mlir::arith::CmpIPredicate::eq, any, zero);
+}
+
+// acc (x) value by a clone of the reduction block `body` (two arguments, a
+// gpu.yield of the combined value), placed at b's insertion point.
+inline mlir::Value combineBy(mlir::OpBuilder &b, mlir::Block &body, mlir::Value acc,
+                             mlir::Value value) {
+  mlir::IRMapping map;
+  map.map(body.getArgument(0), acc);
+  map.map(body.getArgument(1), value);
+  for (mlir::Operation &inner : body.without_terminator())
+    b.clone(inner, map);
+  auto yield = mlir::cast<mlir::gpu::YieldOp>(body.getTerminator());
+  return map.lookupOrDefault(yield.getValues().front());
+}
+
 inline void finishOnDevice(mlir::PatternRewriter &rewriter, mlir::gpu::LaunchOp launch,
-                           gpu_runtime::GPUGlobalReduceOp op, mlir::TypedAttr neutral,
-                           llvm::function_ref<mlir::Value(mlir::Value, mlir::Value)> combine) {
+                           gpu_runtime::GPUGlobalReduceOp op, mlir::TypedAttr neutral) {
   auto loc = op.getLoc();
+  auto launchLoc = launch.getLoc();
   auto elemType = op.getValue().getType();
   auto i32 = rewriter.getI32Type();
   mlir::OpBuilder::InsertionGuard g(rewriter);
@@ -136,57 +178,80 @@ inline void finishOnDevice(mlir::PatternRewriter &rewriter, mlir::gpu::LaunchOp 
   // Before the launch: device arrays for the partials and the ticket.
   rewriter.setInsertionPoint(launch);
   mlir::Value groups = rewriter.create<mlir::arith::MulIOp>(
-      loc, rewriter.create<mlir::arith::MulIOp>(loc, launch.getGridSizeX(), launch.getGridSizeY()),
+      launchLoc,
+      rewriter.create<mlir::arith::MulIOp>(launchLoc, launch.getGridSizeX(),
+                                           launch.getGridSizeY()),
       launch.getGridSizeZ());
   auto partialsType = mlir::MemRefType::get({mlir::ShapedType::kDynamic}, elemType);
   auto ticketType = mlir::MemRefType::get({1}, i32);
-  mlir::Value partials = rewriter.create<mlir::gpu::AllocOp>(
-      loc, partialsType, nullptr, std::nullopt, groups, std::nullopt, /*hostShared=*/false)
-      .getMemref();
-  mlir::Value ticket = rewriter.create<mlir::gpu::AllocOp>(
-      loc, ticketType, nullptr, std::nullopt, std::nullopt, std::nullopt, false).getMemref();
-  mlir::Value zero = rewriter.create<mlir::arith::ConstantIndexOp>(loc, 0);
-  rewriter.create<mlir::gpu::MemsetOp>(loc, mlir::Type(), mlir::ValueRange(), ticket,
-                                       rewriter.create<mlir::arith::ConstantIntOp>(loc, 0, i32));
+  mlir::Value partials =
+      rewriter
+          .create<mlir::gpu::AllocOp>(launchLoc, partialsType, /*asyncToken*/ nullptr,
+                                      /*asyncDeps*/ std::nullopt, groups,
+                                      /*symbols*/ std::nullopt, /*hostShared*/ false)
+          .getMemref();
+  mlir::Value ticket =
+      rewriter
+          .create<mlir::gpu::AllocOp>(launchLoc, ticketType, nullptr, std::nullopt,
+                                      std::nullopt, std::nullopt, false)
+          .getMemref();
+  rewriter.create<mlir::gpu::MemsetOp>(
+      launchLoc, mlir::Type(), mlir::ValueRange(), ticket,
+      rewriter.create<mlir::arith::ConstantIntOp>(launchLoc, 0, i32));
 
-  // Inside the launch, in place of the global reduce.
+  // Inside the launch, in place of the global reduce: the workgroup's own
+  // reduction with the op's region as its body (2200-2215).
   rewriter.setInsertionPoint(op);
-  mlir::Value inGroup = rewriter.create<mlir::gpu::AllReduceOp>(
-      loc, op.getValue(), /*op=*/nullptr, /*uniform=*/true).getResult();
-  // (the all_reduce body is the cloned region, as at 2200-2215)
-  mlir::Value gid = /* linear workgroup id, computeGPUDimsProd-style */ zero;
-  mlir::Value isFirstLane = /* local linear id == 0 */ nullptr;
-  auto ifFirst = rewriter.create<mlir::scf::IfOp>(loc, isFirstLane, /*else=*/false);
+  auto inGroup = rewriter.create<mlir::gpu::AllReduceOp>(
+      loc, op.getValue(), mlir::gpu::AllReduceOperationAttr{}, /*uniform*/ true);
+  auto &region = inGroup.getRegion();
+  rewriter.inlineRegionBefore(op.getRegion(), region, region.end());
+  mlir::Block &body = region.front();
+  {
+    mlir::OpBuilder::InsertionGuard g1(rewriter);
+    auto term = mlir::cast<gpu_runtime::GPUGlobalReduceYieldOp>(body.getTerminator());
+    rewriter.setInsertionPoint(term);
+    rewriter.replaceOpWithNewOp<mlir::gpu::YieldOp>(term, term.getResult());
+  }
+
+  mlir::Value zero = rewriter.create<mlir::arith::ConstantIndexOp>(loc, 0);
+  mlir::Value one = rewriter.create<mlir::arith::ConstantIndexOp>(loc, 1);
+  mlir::Value gid = linearGroupId(rewriter, loc, launch.getGridSize(), launch.getBlockIds());
+  mlir::Value first = isFirstItem(rewriter, loc, launch.getThreadIds());
+
+  // One work-item a workgroup publishes the partial and draws a ticket.
+  auto ifFirst = rewriter.create<mlir::scf::IfOp>(loc, first, /*withElse*/ false);
   rewriter.setInsertionPointToStart(ifFirst.thenBlock());
-  rewriter.create<mlir::memref::StoreOp>(loc, inGroup, partials, gid);
-  // The partial must be visible device-wide before the ticket is taken:
-  // a release at agent scope on the increment (ROCDL: fence + atomicrmw add).
-  mlir::Value one = rewriter.create<mlir::arith::ConstantIntOp>(loc, 1, i32);
+  rewriter.create<mlir::memref::StoreOp>(loc, inGroup.getResult(), partials, gid);
+  rewriter.create<mlir::LLVM::FenceOp>(loc, mlir::LLVM::AtomicOrdering::release, "agent");
   mlir::Value taken = rewriter.create<mlir::memref::AtomicRMWOp>(
-      loc, mlir::arith::AtomicRMWKind::addi, one, ticket, mlir::ValueRange(zero));
+      loc, mlir::arith::AtomicRMWKind::addi,
+      rewriter.create<mlir::arith::ConstantIntOp>(loc, 1, i32), ticket,
+      mlir::ValueRange(zero));
   mlir::Value lastGroup = rewriter.create<mlir::arith::CmpIOp>(
       loc, mlir::arith::CmpIPredicate::eq,
       rewriter.create<mlir::arith::IndexCastOp>(loc, rewriter.getIndexType(), taken),
-      rewriter.create<mlir::arith::SubIOp>(
-          loc, groups, rewriter.create<mlir::arith::ConstantIndexOp>(loc, 1)));
-  auto ifLast = rewriter.create<mlir::scf::IfOp>(loc, lastGroup, false);
+      rewriter.create<mlir::arith::SubIOp>(loc, groups, one));
+
+  // The workgroup that drew the last ticket: every other one has published.
+  auto ifLast = rewriter.create<mlir::scf::IfOp>(loc, lastGroup, /*withElse*/ false);
   rewriter.setInsertionPointToStart(ifLast.thenBlock());
-  // Every other workgroup has published: fold in workgroup order.
+  rewriter.create<mlir::LLVM::FenceOp>(loc, mlir::LLVM::AtomicOrdering::acquire, "agent");
   mlir::Value init = rewriter.create<mlir::arith::ConstantOp>(loc, neutral);
   auto fold = rewriter.create<mlir::scf::ForOp>(
-      loc, zero, groups, rewriter.create<mlir::arith::ConstantIndexOp>(loc, 1),
-      mlir::ValueRange(init),
+      loc, zero, groups, one, mlir::ValueRange(init),
       [&](mlir::OpBuilder &b, mlir::Location l, mlir::Value i, mlir::ValueRange acc) {
         mlir::Value p = b.create<mlir::memref::LoadOp>(l, partials, i);
-        b.create<mlir::scf::YieldOp>(l, combine(acc[0], p));
+        b.create<mlir::scf::YieldOp>(l, combineBy(b, body, acc.front(), p));
       });
   rewriter.create<mlir::memref::StoreOp>(loc, fold.getResult(0), op.getTarget(),
                                          mlir::ValueRange());
+
   // After the launch: the two device arrays are released (in-order queue: no
   // wait needed before gpu.dealloc); the host loop of 2240-2270 is gone.
   rewriter.setInsertionPointAfter(launch);
-  rewriter.create<mlir::gpu::DeallocOp>(loc, mlir::Type(), mlir::ValueRange(), partials);
-  rewriter.create<mlir::gpu::DeallocOp>(loc, mlir::Type(), mlir::ValueRange(), ticket);
+  rewriter.create<mlir::gpu::DeallocOp>(launchLoc, mlir::Type(), mlir::ValueRange(), partials);
+  rewriter.create<mlir::gpu::DeallocOp>(launchLoc, mlir::Type(), mlir::ValueRange(), ticket);
   rewriter.eraseOp(op);
 }
 

@@ -625,25 +625,31 @@ nmk_copy_b128(const int4_t *__restrict__ src, int4_t *__restrict__ dst,
 }
 
 // Copy of nbytes bytes between any two device-visible buffers (host <-> device
-// staging: one side is pinned host memory).  128-bit words when both ends are
-// 16-byte aligned, single bytes otherwise and for the tail.
+// staging: one side is pinned host memory).  Where source and destination sit
+// alike within a 128-bit word (the host places the staged bytes so), the bytes
+// up to the first word boundary and behind the last one go singly and all
+// between as 128-bit words; otherwise everything goes by single bytes.
 NMK_KERNEL(256)
 nmk_copy_bytes(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
                int64_t nbytes) {
   const int64_t stride = int64_t(gridDim.x) * blockDim.x;
   const int64_t first = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-  const bool wide =
-      ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0;
-  int64_t done = 0;
-  if (wide) {
-    const int64_t nvec = nbytes / 16;
-    const int4_t *s = reinterpret_cast<const int4_t *>(src);
-    int4_t *d = reinterpret_cast<int4_t *>(dst);
-    for (int64_t i = first; i < nvec; i += stride)
-      d[i] = s[i];
-    done = nvec * 16;
+  const uintptr_t s = reinterpret_cast<uintptr_t>(src);
+  const uintptr_t d = reinterpret_cast<uintptr_t>(dst);
+  int64_t head = 0, nvec = 0;
+  if (((s ^ d) & 15u) == 0) {
+    head = int64_t((16u - (s & 15u)) & 15u);
+    if (head > nbytes)
+      head = nbytes;
+    nvec = (nbytes - head) / 16;
   }
-  for (int64_t i = done + first; i < nbytes; i += stride)
+  for (int64_t i = first; i < head; i += stride)
+    dst[i] = src[i];
+  const int4_t *sv = reinterpret_cast<const int4_t *>(src + head);
+  int4_t *dv = reinterpret_cast<int4_t *>(dst + head);
+  for (int64_t i = first; i < nvec; i += stride)
+    dv[i] = sv[i];
+  for (int64_t i = head + nvec * 16 + first; i < nbytes; i += stride)
     dst[i] = src[i];
 }
 

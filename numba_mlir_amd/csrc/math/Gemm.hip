@@ -1173,6 +1173,7 @@ struct DeviceWorkspace {
   void *fixed = nullptr; // device address of `scratch` on this device
   void *heap = nullptr;
   size_t heapBytes = 0;
+  int computeUnits = 0; // of the device (or of its partition), asked once
 };
 DeviceWorkspace workspaces[kMaxDevices];
 std::mutex workspaceMutex;
@@ -1185,6 +1186,20 @@ DeviceWorkspace &workspaceOf(int device) {
   if (device < 0 || device >= kMaxDevices)
     fatal("mkl_gemm_device: device ordinal %d out of range\n", device);
   return workspaces[device];
+}
+
+// Compute units of the current device: 256 on a whole MI355X, fewer on a
+// partition of one.  The launch plans below count resident blocks in them.
+int computeUnitsOf(int device) {
+  std::lock_guard<std::mutex> lock(workspaceMutex);
+  DeviceWorkspace &w = workspaceOf(device);
+  if (w.computeUnits <= 0) {
+    int n = 0;
+    checkHip(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device),
+             "hipDeviceGetAttribute(multiprocessor count)");
+    w.computeUnits = n > 0 ? n : 1;
+  }
+  return w.computeUnits;
 }
 
 // Grown on demand; nullptr when the device has no room for the larger block
@@ -1258,9 +1273,8 @@ struct SplitPlan {
   int slices = 1;
   int sliceK = 0;
 };
-SplitPlan planSplit(int64_t tiles, int64_t K, int BK, int blocksPerCu) {
+SplitPlan planSplit(int64_t tiles, int64_t K, int BK, int64_t slots /* resident blocks */) {
   SplitPlan plan;
-  const int64_t slots = int64_t(256) * blocksPerCu; // resident blocks
   if (tiles <= 0 || tiles * 2 > slots)
     return plan;
   // (at most 16 slices, or more of 512 elements each where K is that long:
@@ -1307,14 +1321,14 @@ int planEvenShares(int64_t tiles, int64_t slabs, int64_t slots) {
 // partial products are whole tiles that one streaming pass adds up -- at 0.84
 // and below the shares win), or when there are so few tiles that shares
 // would cut each into more than 16 pieces.
-bool splitFills(const SplitPlan &plan, int64_t tiles, int blocksPerCu) {
+bool splitFills(const SplitPlan &plan, int64_t tiles, int64_t slots) {
   if (plan.slices < 2)
     return false;
   // (two or three slices leave shares few pieces to add up, so the slices
   // must fill more: 225 tiles x 2 fill 0.88 and lose to shares, 149 against
   // 141 us for 1920^3 float32)
   const int64_t pct = plan.slices >= 4 ? 86 : 93;
-  return tiles * plan.slices * 100 >= int64_t(256) * blocksPerCu * pct || plan.slices >= 16;
+  return tiles * plan.slices * 100 >= slots * pct || plan.slices >= 16;
 }
 
 enum WorkspaceKind { WORKSPACE_HEAP, WORKSPACE_FIXED };
@@ -1405,13 +1419,21 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
     if (!workspaceTurn.owns_lock())
       workspaceTurn = std::unique_lock<std::mutex>(workspaceInUse[device]);
   };
-  auto workspaceFor = [&](SplitPlan &plan, int64_t m, int64_t ldw) -> T * {
+  // `required`: the caller cannot run unsplit (the tile kernels' plans count
+  // on their slices): the call then returns 1 before anything is launched.
+  // The other callers run unsplit on nullptr, whichever workspace was short.
+  auto workspaceFor = [&](SplitPlan &plan, int64_t m, int64_t ldw,
+                          bool required = false) -> T * {
     if (plan.slices < 2)
       return nullptr;
     takeTurn();
     const size_t bytes = size_t(plan.slices) * size_t(m) * size_t(ldw) * sizeof(T);
     void *p = nullptr;
     if (workspaceKind == WORKSPACE_FIXED) {
+      if (bytes > kScratchBytes && !required) {
+        plan = SplitPlan();
+        return nullptr;
+      }
       if (bytes > kScratchBytes) {
         std::fprintf(stderr,
                      "mkl_gemm_device_noalloc: [%lld,%lld] x [%lld,%lld] needs "
@@ -1447,7 +1469,8 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       p = static_cast<unsigned char *>(p) + packBytes;
     return static_cast<T *>(p);
   };
-  const int64_t slots = 512; // resident blocks of the 128 x 128 tiles: two a CU
+  const int64_t cus = computeUnitsOf(device);
+  const int64_t slots = 2 * cus; // resident blocks of the 128 x 128 tiles: two a CU
   // Equal slices of K for `tiles` 128 x 128 tiles, and whether they go ahead
   // of even shares.  float64 blocks share a CU in pairs; float32 ones may
   // (186 registers a lane), which pays where one block a CU would not fill
@@ -1458,16 +1481,16 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
   // workspace is sized for those.
   auto planSlices = [&](int64_t tiles, int64_t k, bool &fills) {
     if (sizeof(T) == 8) {
-      const SplitPlan two = planSplit(tiles, k, Mfma<T>::BK, 2);
-      fills = splitFills(two, tiles, 2);
+      const SplitPlan two = planSplit(tiles, k, Mfma<T>::BK, 2 * cus);
+      fills = splitFills(two, tiles, 2 * cus);
       return two;
     }
-    const SplitPlan one = planSplit(tiles, k, Mfma<T>::BK, 1);
-    fills = splitFills(one, tiles, 1);
+    const SplitPlan one = planSplit(tiles, k, Mfma<T>::BK, cus);
+    fills = splitFills(one, tiles, cus);
     if (fills || workspaceKind != WORKSPACE_HEAP)
       return one;
-    const SplitPlan two = planSplit(tiles, k, Mfma<T>::BK, 2);
-    if (splitFills(two, tiles, 2)) {
+    const SplitPlan two = planSplit(tiles, k, Mfma<T>::BK, 2 * cus);
+    if (splitFills(two, tiles, 2 * cus)) {
       fills = true;
       return two;
     }
@@ -1776,14 +1799,15 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       const int64_t bigTiles = (Mt / 256) * (Nt / 256);
       const int bigSlab = Kt % (2 * BK) == 0 ? 2 * BK : BK;
       const int bigEven = bigFits && workspaceKind == WORKSPACE_HEAP
-                              ? planEvenShares(bigTiles, Kt / bigSlab, 256)
+                              ? planEvenShares(bigTiles, Kt / bigSlab, cus)
                               : 0;
       // (from 64 large tiles on: below, the 128 x 128 tiles in slices or
       // shares are as fast or faster -- 1792^3 120 against 131 us, 1024 x
       // 1024 x 4096 92 against 99 -- and from 121 on the large tile wins,
       // 3072^3 456 against 474)
-      bool big = bigFits && bigTiles >= 64 && (bigEven > 0 || bigTiles >= 192);
-      if (big && bigTiles < 192) {
+      // (the tile counts below are a quarter and three quarters of the CUs)
+      bool big = bigFits && bigTiles * 4 >= cus && (bigEven > 0 || bigTiles * 4 >= 3 * cus);
+      if (big && bigTiles * 4 < 3 * cus) {
         // (fewer large tiles than CUs only pay in even shares: without room
         // for those, the 128 x 128 tiles take the shape.  Slices of K on the
         // large tile were measured and gain nothing over its even shares:
@@ -1842,8 +1866,8 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
         // float32: 256 x 256 tiles, K slabs of 32; float64: 128 x 128, slabs of 16
         constexpr int PT = sizeof(T) == 4 ? 256 : 128;
         constexpr int PSLAB = sizeof(T) == 4 ? 2 * BK : BK;
-        const int64_t padSlots = sizeof(T) == 4 ? 256 : slots;
-        const int64_t minTiles = sizeof(T) == 4 ? 192 : 256;
+        const int64_t padSlots = sizeof(T) == 4 ? cus : slots;
+        const int64_t minTiles = sizeof(T) == 4 ? 3 * cus / 4 : cus;
         auto roundUp = [](int64_t v, int64_t to) { return (v + to - 1) / to * to; };
         const int64_t Mp = roundUp(Mz, PT), Np = roundUp(Nz, PT), Kp = roundUp(K, PSLAB);
         const bool fitsAsIs = Mz == Mp && Nz == Np && K % BK == 0 && !offWords(X, ldx, xC) &&
@@ -1944,7 +1968,7 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
           plan = SplitPlan();
         const int64_t ldw = (Nz + VEC - 1) / VEC * VEC;
         if (!evenBlocks)
-          W = workspaceFor(plan, Mz, ldw);
+          W = workspaceFor(plan, Mz, ldw, true);
         if (tooLarge)
           return 1;
         if (packBytes) {
@@ -2028,7 +2052,7 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
         if (evenBlocks)
           plan = SplitPlan();
         else if (!big)
-          W = workspaceFor(plan, Mt, Nt);
+          W = workspaceFor(plan, Mt, Nt, true);
         if (tooLarge)
           return 1;
         const EvenShares even{evenBlocks ? slabs : 0, int(Nt / BN)};
@@ -2110,7 +2134,7 @@ int deviceGemm(void *queueObj, const typename MemrefOf<T>::type *a,
       const int64_t tiles = int64_t(grid.x) * grid.y;
       SplitPlan plan;
       int64_t kSlice = K;
-      if (tiles <= 256 && K >= 2048) {
+      if (tiles <= cus && K >= 2048) {
         int64_t slices = 2048 / tiles;
         if (slices > K / 512)
           slices = K / 512;

@@ -350,10 +350,14 @@ public:
   // alternate, so the host copies one while the kernel moves the other.
   static constexpr size_t kStagingHalf = size_t(16) << 20;
 
-  char *stagingHalf(int which) {
+  // Each half has 16 spare bytes: a transfer is staged at the offset within a
+  // 128-bit word that its device address has (`skew`, the same for every
+  // chunk: the chunks are whole words apart), so that the copy kernel moves
+  // words whatever the view's first byte.
+  char *stagingHalf(int which, size_t skew = 0) {
     if (!staging)
-      staging = static_cast<char *>(alloc(2 * kStagingHalf, GPUX_ALLOC_HOST));
-    return staging + size_t(which) * kStagingHalf;
+      staging = static_cast<char *>(alloc(2 * (kStagingHalf + 16), GPUX_ALLOC_HOST));
+    return staging + size_t(which) * (kStagingHalf + 16) + skew;
   }
 
   void *copyBytesAsync(const void *src, void *dst, size_t bytes) {
@@ -379,13 +383,14 @@ public:
     synchronize();
     void *pending[2] = {nullptr, nullptr};
     int half = 0;
+    const size_t skew = reinterpret_cast<uintptr_t>(dev) & 15u;
     for (size_t off = 0; off < bytes; off += kStagingHalf, half ^= 1) {
       const size_t n = bytes - off < kStagingHalf ? bytes - off : kStagingHalf;
       if (pending[half]) { // the kernel that last read this half
         retireEvent(pending[half], true);
         pending[half] = nullptr;
       }
-      char *stage = stagingHalf(half);
+      char *stage = stagingHalf(half, skew);
       std::memcpy(stage, static_cast<const char *>(host) + off, n);
       pending[half] = copyBytesAsync(stage, static_cast<char *>(dev) + off, n);
     }
@@ -398,12 +403,13 @@ public:
     synchronize();
     void *pending[2] = {nullptr, nullptr};
     size_t pendingOff[2] = {0, 0}, pendingBytes[2] = {0, 0};
+    const size_t skew = reinterpret_cast<uintptr_t>(dev) & 15u;
     auto drain = [&](int half) {
       if (!pending[half])
         return;
       retireEvent(pending[half], true);
       pending[half] = nullptr;
-      std::memcpy(static_cast<char *>(host) + pendingOff[half], stagingHalf(half),
+      std::memcpy(static_cast<char *>(host) + pendingOff[half], stagingHalf(half, skew),
                   pendingBytes[half]);
     };
     int half = 0;
@@ -411,7 +417,7 @@ public:
       const size_t n = bytes - off < kStagingHalf ? bytes - off : kStagingHalf;
       drain(half);
       pending[half] = copyBytesAsync(static_cast<const char *>(dev) + off,
-                                     stagingHalf(half), n);
+                                     stagingHalf(half, skew), n);
       pendingOff[half] = off;
       pendingBytes[half] = n;
       drain(half ^ 1); // the other half's kernel ran while this one was queued

@@ -70,8 +70,18 @@ def unbox(obj, ndim=None):
     what compiled code receives for the argument.  Raises what the unboxer
     set, or TypeError in the words of the reference's unboxing hook
     (dpctl_interop.py:252-259)."""
+    iface = obj.__hip_array_interface__
+    try:
+        rank = len(iface["shape"])
+    except (TypeError, KeyError):
+        rank = None                # malformed: the unboxer says what is wrong
     if ndim is None:
-        ndim = len(obj.__hip_array_interface__["shape"])
+        ndim = rank or 0
+    elif rank is not None and isinstance(iface["shape"], tuple) and ndim != rank:
+        # The unboxer writes 2 * rank trailing integers: a record typed for
+        # another rank would be overrun or left half filled.
+        raise TypeError(f"can't unbox a {rank}-dimensional array into a native "
+                        f"value of {ndim} dimensions")
     record = array_record(ndim)()
     code = runtime_lib.nmrtUnboxHipInterface(obj, ctypes.byref(record))
     if code != 0:

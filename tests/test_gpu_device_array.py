@@ -96,3 +96,25 @@ def test_l2_norm(env):
         got = ops.l2_norm_rows(hip.asarray(x)).asnumpy()
         truth = np.sqrt((x.astype(np.float64) ** 2).sum(axis=1))
         np.testing.assert_allclose(got, truth, rtol=1e-5)
+
+
+@pytest.mark.parametrize("first", [1, 3, 5, 8, 13, 16])
+def test_transfers_of_views_that_start_inside_a_word(env, first):
+    """A contiguous view whose first byte is not on a 16-byte boundary (and
+    whose last is not either) goes to the host and back in 128-bit words with
+    single bytes only at its two ends; what lies around it is untouched."""
+    hip = env[0]
+    n = (36 << 20) + 11                  # three staging chunks
+    rng = np.random.default_rng(first)
+    host = rng.integers(0, 255, n, dtype=np.uint8)
+    d = hip.asarray(host)
+    view = d[first:n - 7]
+    assert view.ptr % 16 == first % 16
+    np.testing.assert_array_equal(view.asnumpy(), host[first:n - 7])
+    fresh = rng.integers(0, 255, n - 7 - first, dtype=np.uint8)
+    view.copy_from_host(fresh)
+    expect = host.copy()
+    expect[first:n - 7] = fresh
+    np.testing.assert_array_equal(d.asnumpy(), expect)
+    small = d[first:first + 5]           # shorter than the distance to a boundary
+    np.testing.assert_array_equal(small.asnumpy(), expect[first:first + 5])

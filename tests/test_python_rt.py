@@ -79,6 +79,17 @@ def test_what_is_not_an_array_is_refused_with_a_reason():
     assert python_rt.unbox(Described(**fields)).nitems == 0
 
 
+def test_rank_must_match_the_record():
+    """The unboxer writes two integers per dimension of the OBJECT: a record
+    typed for fewer dimensions would be overrun."""
+    a = np.zeros((3, 5), np.float32)
+    obj = Described(**_iface(a))
+    for ndim in (0, 1, 3):
+        with pytest.raises(TypeError, match="2-dimensional"):
+            python_rt.unbox(obj, ndim=ndim)
+    assert tuple(python_rt.unbox(obj, ndim=2).shape) == (3, 5)
+
+
 def test_meminfo_carries_its_destructor():
     seen = []
     dtor_type = ctypes.CFUNCTYPE(None, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p)

@@ -128,3 +128,37 @@ def test_a_thin_product_keeps_its_partial_sums_in_the_fixed_array(gemm_entry_poi
             a.astype(np.float64) @ b.astype(np.float64))
         scale = 0.5 * np.abs(c0) + 1.5 * (np.abs(a).astype(np.float64) @ np.abs(b))
         assert (np.abs(got - truth) <= 1e-5 * scale + 1e-30).all()
+
+
+def test_the_entry_point_allocates_no_device_memory(gemm_entry_points):
+    """Free device memory, read with hipMemGetInfo, is the same before and
+    after calls on split-K shapes this process has not run before (a route
+    through the heap workspace would take at least 8 MiB for the first of
+    them and more for the second)."""
+    hip, lib, mrt = gemm_entry_points
+    hiprt = ctypes.CDLL("libamdhip64.so")
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert hiprt.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    rng = np.random.default_rng(3)
+    cases = []
+    for m, n, k in ((896, 1152, 1536), (1280, 768, 4096), (8, 2048, 8192)):
+        a = hip.asarray(rng.standard_normal((m, k), dtype=np.float32))
+        b = hip.asarray(rng.standard_normal((k, n), dtype=np.float32))
+        c = hip.asarray(np.zeros((m, n), np.float32))
+        cases.append((a, b, c))
+    mrt.runtime_hip_lib.nmrtMathRuntimeFinalize()    # the heap workspace, if any, goes
+    before = free_bytes()
+    for a, b, c in cases:
+        status = lib.mkl_gemm_float32_device_noalloc(
+            a.ctx.queue, _memref(a), _memref(b), 1.0, 0.0, _memref(c))
+        assert status == 0
+        assert "_splitk" in mrt.last_kernel() or mrt.last_kernel() == "sgemm_thin_cols"
+        assert free_bytes() == before, mrt.last_kernel()
+    # (and the allocating entry point does take its workspace from the heap)
+    a, b, c = cases[1]
+    lib.mkl_gemm_float32_device(a.ctx.queue, _memref(a), _memref(b), 1.0, 0.0, _memref(c))
+    assert free_bytes() < before
