@@ -1434,7 +1434,8 @@ class Dispatcher:
             run_shape, views = _collapse(shape, views)
         if len(run_shape) > 3:
             return self._elementwise_slices(ctx, args, shape, run_shape, views)
-        compiled = self._compile("elementwise", views, len(run_shape), len(run_shape) > 1)
+        compiled = self._compile("elementwise", views, len(run_shape),
+                                 kernel_impl.remap_mode(run_shape))
         for name, a, v in zip(self._params(), args, views):
             if isinstance(a, HipNdArray) and f"v_{name}" in compiled.written and \
                     a.shape != tuple(shape):
@@ -1471,7 +1472,8 @@ class Dispatcher:
         for index in np.ndindex(*outer):
             part = [v[index] if isinstance(v, HipNdArray) else v for v in views]
             if plan is None:
-                compiled = self._compile("elementwise", part, 3, True)
+                compiled = self._compile("elementwise", part, 3,
+                                         kernel_impl.remap_mode(run_shape[-3:]))
                 for name, a in zip(self._params(), args):
                     if isinstance(a, HipNdArray) and f"v_{name}" in compiled.written and \
                             a.shape != tuple(shape):

@@ -460,6 +460,7 @@ class FunctionTranslator:
         self.reductions = {}         # parallel mode: reduction variable -> "add" | "mul"
         self.return_node = None      # parallel mode: the return after the loop
         self.allow_remap = False     # kernels only: see translate_kernel
+        self.lanes_along_y = False   # remapped grids with a short x extent
         self.reversed = False
         self.rows_per_lane = 1
         self.grid_stride = False
@@ -2123,9 +2124,15 @@ class FunctionTranslator:
         rows = ROWS_PER_LANE if self.reversed else 1
         self.rows_per_lane = rows
         flat = self.reversed
+        # Where the extent along x is shorter than a wave (a tall result of a
+        # few columns), a flat block would leave most lanes of its wave idle:
+        # the block then has lanes along hardware y too -- a wave covers whole
+        # neighbouring rows -- and a lane's work-items lie a block's rows apart.
+        tall = self.lanes_along_y = bool(self.reversed and self.lanes_along_y)
+        thin = lambda k: flat and dim[k] != "x" and not (tall and dim[k] == "y")
         out += [
             "  const int64_t " + ", ".join(
-                f"nmk_lid{k} = " + ("0" if flat and dim[k] != "x" else f"threadIdx.{dim[k]}")
+                f"nmk_lid{k} = " + ("0" if thin(k) else f"threadIdx.{dim[k]}")
                 for k in range(3)) + ";",
             # (a launch has 65535 blocks along y and z: a grid of one or two
             # dimensions with more along y goes on along z)
@@ -2135,7 +2142,7 @@ class FunctionTranslator:
                     "int64_t(blockIdx.y) + int64_t(gridDim.y) * blockIdx.z" if dim[k] == "y"
                     else "0") for k in range(3)) + ";",
             "  const int64_t " + ", ".join(
-                f"nmk_lsz{k} = " + ("1" if flat and dim[k] != "x" else f"blockDim.{dim[k]}")
+                f"nmk_lsz{k} = " + ("1" if thin(k) else f"blockDim.{dim[k]}")
                 for k in range(3)) + ";",
             "  (void)nmk_lid0; (void)nmk_lid1; (void)nmk_lid2; (void)nmk_grp0; (void)nmk_grp1;",
             "  (void)nmk_grp2; (void)nmk_lsz0; (void)nmk_lsz1; (void)nmk_lsz2;",
@@ -2156,21 +2163,31 @@ class FunctionTranslator:
             others = [k for k in range(3) if k != ky]
             out += [f"  const int64_t nmk_gid{k} = nmk_grp{k} * nmk_lsz{k} + nmk_lid{k};"
                     for k in others]
+            # (flat blocks: a lane's rows are adjacent; with lanes along y they
+            # are a block's rows apart, so that each access of a wave covers
+            # adjacent rows)
+            first = f"nmk_grp{ky} * {rows}"
+            last = f"nmk_first + {rows}"
+            step = ""
+            if tall:
+                first = f"nmk_grp{ky} * ({rows} * nmk_lsz{ky}) + nmk_lid{ky}"
+                last = f"(nmk_grp{ky} + 1) * ({rows} * nmk_lsz{ky})"
+                step = f" * nmk_lsz{ky}"
             out += [
-                f"  const int64_t nmk_first = nmk_grp{ky} * {rows};",
+                f"  const int64_t nmk_first = {first};",
                 f"  auto nmk_item = [&](const int64_t nmk_gid{ky}, auto nmk_guarded) {{",
                 f"    if (decltype(nmk_guarded)::value && !(nmk_gid{ky} < nmk_gsz{ky})) return;",
             ] + body + [
                 "  };",
                 "  if (" + " && ".join(f"nmk_gid{k} < nmk_gsz{k}" for k in others) + ") {",
-                f"    if (nmk_first + {rows} <= nmk_gsz{ky}) {{",
+                f"    if ({last} <= nmk_gsz{ky}) {{",
                 "#pragma unroll",
                 f"      for (int nmk_row = 0; nmk_row < {rows}; ++nmk_row)",
-                "        nmk_item(nmk_first + nmk_row, nmkjit::No());",
+                f"        nmk_item(nmk_first + nmk_row{step}, nmkjit::No());",
                 "    } else {",
                 "#pragma unroll",
                 f"      for (int nmk_row = 0; nmk_row < {rows}; ++nmk_row)",
-                "        nmk_item(nmk_first + nmk_row, nmkjit::Yes());",
+                f"        nmk_item(nmk_first + nmk_row{step}, nmkjit::Yes());",
                 "    }",
                 "  }",
             ]
@@ -2316,7 +2333,9 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     parameter points at is set, so the launch can raise IndexError instead
     of faulting the GPU.  With ``remap`` a body whose work-items cannot
     observe their grouping gets global dimension ``ndim - 1`` on x
-    (``reversed_dims`` of the result tells the launcher).
+    (``reversed_dims`` of the result tells the launcher); ``remap="tall"``
+    says that this dimension is shorter than a wave, and the blocks get lanes
+    along the next dimension too (``lanes_along_y``).
 
     ``mode``: "kernel" for an @kernel body; "elementwise" for a function of
     whole arrays fused into one map over ``ndim`` dimensions (``ret_dtype`` of
@@ -2332,7 +2351,8 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     by it)."""
     module = Module(stubs, boundscheck)
     tr = FunctionTranslator(module, func, arg_types, True, ndim)
-    tr.allow_remap = remap
+    tr.allow_remap = bool(remap)
+    tr.lanes_along_y = remap == "tall"
     tr.mode = mode
     tr.noalias = noalias
     tr.stream = stream
@@ -2356,6 +2376,9 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     # many work-items along hardware y: the launcher divides that grid
     # dimension by it
     compiled.rows_per_lane = tr.rows_per_lane
+    # ... unless the grid is short along x: then the block has lanes along
+    # hardware y as well (x extent times as many as fill 256)
+    compiled.lanes_along_y = tr.lanes_along_y
     # a 1-d loop or map that strides over its iteration space by whole grids:
     # any number of blocks computes the same thing
     compiled.grid_stride = tr.grid_stride

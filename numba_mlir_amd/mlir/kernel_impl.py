@@ -363,7 +363,7 @@ class Kernel(KernelBase):
             # With a runtime-chosen block a body that cannot observe its
             # grouping is laid out for coalescing (last dimension on x), unless
             # that pushes a long dimension past the y / z grid limit.
-            remap = len(self.local_size) == 0 and ndim > 1
+            remap = len(self.local_size) == 0 and remap_mode(gsize3[:ndim])
             stream = streams([a for a in args if isinstance(a, HipNdArray)])
             compiled = self.compile(args, ndim, remap, noalias, stream)
             kern = _loaded_kernel(ctx, compiled)
@@ -406,6 +406,19 @@ class Kernel(KernelBase):
                         (ctypes.c_size_t * 3)(*block), descs)
 
 
+def remap_mode(global_size):
+    """How a grid of these extents is laid out on the lanes when the body
+    cannot observe its grouping: not at all (one dimension), last dimension
+    on x with flat blocks (True), or -- when that dimension is shorter than a
+    wave and the next one is not -- with lanes along the next dimension too
+    ("tall")."""
+    if len(global_size) < 2:
+        return False
+    if int(global_size[-1]) < 64 and int(global_size[-2]) >= 64:
+        return "tall"
+    return True
+
+
 def _geometry(ctx, compiled, kern, global_size, local_size):
     """Block and grid of a compiled kernel in hardware order (x, y, z)."""
     ndim = len(global_size)
@@ -420,6 +433,10 @@ def _geometry(ctx, compiled, kern, global_size, local_size):
         bsize = (ctypes.c_uint32 * 1)()
         runtime_lib.gpuxSuggestBlockSize(ctx.queue, kern, gsize, bsize, 1)
         block = [int(bsize[0])] + [1] * (ndim - 1)
+        if getattr(compiled, "lanes_along_y", False):
+            # a grid of a few columns: whole rows side by side in a wave, as
+            # many as bring the block to 256 lanes
+            block[1] = max(1, min(256 // max(block[0], 1), sizes[1]))
     elif len(local_size) != 0:
         block = [int(local_size[k]) for k in order]
     else:
@@ -431,7 +448,7 @@ def _geometry(ctx, compiled, kern, global_size, local_size):
     block += [1] * (3 - ndim)
     grid = [(g + b - 1) // b for g, b in zip(sizes, block)]
     if rows > 1:
-        grid[1] = (grid[1] + rows - 1) // rows
+        grid[1] = (grid[1] + rows - 1) // rows     # blocks of block[1] * rows rows
     if ndim <= 2 and grid[1] > 65535:
         # (the generated kernels count their blocks along y, then z)
         grid[2] = (grid[1] + 65534) // 65535

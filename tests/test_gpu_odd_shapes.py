@@ -141,3 +141,57 @@ def test_fused_axis_sums_of_a_tall_matrix(env):
                                (x.astype(np.float64) ** 2).sum(axis=1), rtol=1e-5)
     np.testing.assert_allclose(njit(_column_sums_of_squares)(d).asnumpy(),
                                (x.astype(np.float64) ** 2).sum(axis=0), rtol=1e-4)
+
+
+def _tall_body(a, b, c):
+    return a - 2.0 * b + c
+
+
+def _tall_store(a, b, c, out):
+    out[:] = a * b + c
+
+
+@pytest.mark.parametrize("cols", [1, 3, 8, 16, 33, 63, 64])
+@pytest.mark.parametrize("rows", [64, 1000, 100003])
+def test_tall_results_of_a_few_columns(env, rows, cols):
+    """A fused map over [rows, cols] with a column and a row operand (which
+    keeps the two dimensions apart): with fewer than 64 columns the blocks
+    have lanes along the rows too, so a wave works on whole neighbouring rows
+    instead of one short one."""
+    hip, _ = env
+    rng = np.random.default_rng(rows + cols)
+    a = rng.standard_normal((rows, 1))
+    b = rng.standard_normal((rows, cols))
+    c = rng.standard_normal(cols)
+    f = njit(_tall_body)
+    got = f(hip.asarray(a), hip.asarray(b), hip.asarray(c))
+    assert np.array_equal(_host(got), a - 2.0 * b + c)
+    block = f.last_launch["block"]
+    if cols < 64 and cols > 1:
+        assert block[:2] == (cols, min(256 // cols, rows)), block
+    out = hip.asarray(np.zeros((rows, cols), np.float32))
+    g = njit(_tall_store)
+    a32, b32, c32 = a.astype(np.float32), b.astype(np.float32), c.astype(np.float32)
+    g(hip.asarray(a32), hip.asarray(b32), hip.asarray(c32), out)
+    assert np.array_equal(out.asnumpy(), a32 * b32 + c32)
+
+
+def test_a_tall_kernel_grid_of_a_few_columns(env):
+    """The same layout for an @kernel body launched over (rows, 8) with a
+    block chosen by the runtime."""
+    hip, _ = env
+    from numba_mlir_amd import kernel as kapi
+
+    def body(x, y, out):
+        i = kapi.get_global_id(0)
+        j = kapi.get_global_id(1)
+        out[i, j] = x[i, j] * 3 + y[j] - i
+
+    rows, cols = 50001, 8
+    x = np.arange(rows * cols, dtype=np.int64).reshape(rows, cols)
+    y = np.arange(cols, dtype=np.int64) * 7
+    out = hip.asarray(np.zeros((rows, cols), np.int64))
+    k = kapi.kernel(body)[(rows, cols), ()]
+    k(hip.asarray(x), hip.asarray(y), out)
+    assert k.last_launch["block"][:2] == (8, 32)
+    assert np.array_equal(out.asnumpy(), x * 3 + y - np.arange(rows)[:, None])
