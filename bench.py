@@ -453,7 +453,11 @@ def run(args):
                                d[1].ptr, d[2].ptr, float(rate), float(vol),
                                d[3].ptr, d[4].ptr, nopt, 1 if wide else 0)
                         for d in sets]
-            tm = b.measure(launches)
+            # (this kernel's arithmetic hides under its memory time with little
+            # to spare, and the GPU alternates between faster and slower phases
+            # of some ten milliseconds: three times the regions, so that the
+            # median spans several phases)
+            tm = b.measure(launches, regions=3 * b.regions)
             e = hbm_entry(
                 key, f"Black-Scholes, 2^24 float32 options, literals typed "
                      f"{'float64 (reference typing)' if wide else 'float32'}",
@@ -782,7 +786,7 @@ def generated_kernels(b, workloads):
     out = []
     globals()["get_global_id"] = kapi.get_global_id    # what pairwise_body calls
 
-    def timed(name, workload, alg_bytes, plan, arg_sets, ret_sets=None):
+    def timed(name, workload, alg_bytes, plan, arg_sets, ret_sets=None, regions=None):
         """Launches rotate over several sets of arrays, so that inputs come
         from HBM and not from the 256 MiB memory-side cache (generated kernels
         read with ordinary loads; the hand-written ones bypass that cache)."""
@@ -798,7 +802,7 @@ def generated_kernels(b, workloads):
             if len(events) > 16:
                 plan.retire(events.pop(0))
 
-        tm = b.measure(launch)
+        tm = b.measure(launch, regions=regions)
         for event in events:
             plan.retire(event)
         e = hbm_entry(name, workload, alg_bytes, tm, plan.info["kernel"])
@@ -813,13 +817,14 @@ def generated_kernels(b, workloads):
         f = njit(black_scholes_body)
         f(*sets[0])
         timed("bs_njit", "Black-Scholes, 2^24 float32 options, the reference's test "
-              "body under @njit", 20 * nopt, f.last_plan, sets)
+              "body under @njit", 20 * nopt, f.last_plan, sets, regions=3 * b.regions)
         globals()["prange"] = decorators.prange
         loop = njit(parallel=True)(black_scholes_loop_body)
         loop_sets = [[nopt] + s for s in sets]
         loop(*loop_sets[0])
         timed("bs_prange", "Black-Scholes, 2^24 float32 options, the same body as one "
-              "prange loop under @njit(parallel=True)", 20 * nopt, loop.last_plan, loop_sets)
+              "prange loop under @njit(parallel=True)", 20 * nopt, loop.last_plan, loop_sets,
+              regions=3 * b.regions)
         del sets, loop_sets
 
         a, _ = workloads.broadcast_add()
