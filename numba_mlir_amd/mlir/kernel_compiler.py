@@ -461,6 +461,7 @@ class FunctionTranslator:
         self.return_node = None      # parallel mode: the return after the loop
         self.allow_remap = False     # kernels only: see translate_kernel
         self.lanes_along_y = False   # remapped grids with a short x extent
+        self.stages_table = False    # the kernel starts by copying a table into LDS
         self.reversed = False
         self.rows_per_lane = 1
         self.grid_stride = False
@@ -2151,10 +2152,13 @@ class FunctionTranslator:
             out.append(f"  {t.ctype} {self.cname(name)} = ({t.ctype}){neutral};")
         # tables in workgroup memory, staged by the routines' users
         text = "\n".join(self.m.device_code + lines)
+        self.stages_table = False
         if "nmkjit::erfF64(" in text:
             out.append("  nmkjit::erfTableLoad();")
+            self.stages_table = True
         if "nmkjit::cdfTermF64(" in text or "nmkjit::cdfTermF64m<" in text:
             out.append("  nmkjit::cdfTableLoad();")
+            self.stages_table = True
         body = ["    " + v for v in views]
         body += ["    " + d for d in self.declarations() + self.private_decls]
         body += lines
@@ -2382,6 +2386,9 @@ def translate(func, arg_types, ndim, stubs, boundscheck=False, remap=False,
     # a 1-d loop or map that strides over its iteration space by whole grids:
     # any number of blocks computes the same thing
     compiled.grid_stride = tr.grid_stride
+    # every block first copies a table into workgroup memory: worth two trips
+    # a lane instead of one
+    compiled.stages_table = tr.stages_table
     compiled.ret_dtype = tr.ret_type.dtype if (mode == "elementwise" and tr.ret_type) else None
     compiled.range_source = tr.range_source[1] if tr.range_source else None
     compiled.grid_sources = list(tr.grid_sources)   # per grid dimension

@@ -646,6 +646,12 @@ def plan_compiled(ctx, compiled, func_name, global_size, args, ret=None,
         # (a launch counts the work-items of a dimension in 32 bits; the
         # kernel strides over the rest)
         grid[0] = min(grid[0], (2 ** 32 - 1) // max(block[0], 1))
+    if getattr(compiled, "grid_stride", False) and getattr(compiled, "stages_table", False) \
+            and not make_partials and grid[0] >= 4096:
+        # Every block stages its table before its first element: half the
+        # blocks, two trips a lane (the Black-Scholes body over 2^24 options:
+        # 8192 blocks against 16384).
+        grid[0] = -(-grid[0] // 2)
     if make_partials and getattr(compiled, "grid_stride", False):
         # a reduction: few, long-running blocks (one partial result each); the
         # more arrays they stream at once, the fewer (two arrays of 512 MiB:
