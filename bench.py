@@ -137,9 +137,6 @@ class Timing:
         self.wall = self.walls[len(walls) // 2]
         self.ev = self.evs[len(evs) // 2]
 
-    def __iter__(self):            # wall, ev, kernel = bench.measure(...)
-        return iter((self.wall, self.ev, self.kernel))
-
     def spread(self):
         return {"regions": len(self.evs),
                 "kernel_ms": [round(self.evs[0], 5), round(self.evs[-1], 5)],

@@ -394,6 +394,9 @@ struct BsPlainTest {
   uint32_t tLimitBits;
   // |volatility| must lie in [1 / volSpan, volSpan]: 2^50 where z = 2 vol^2 T
   // is a double, 2^30 where it is a float (z then stays a normal number).
+  // (from the limit another instance worked out)
+  __device__ __forceinline__ explicit BsPlainTest(uint32_t limitBits)
+      : tLimitBits(limitBits) {}
   __device__ __forceinline__ BsPlainTest(float rate, float volatility, float volSpan) {
     const float av = __builtin_fabsf(volatility);
     const bool scalarsOk = __builtin_fabsf(rate) < 0x1p60f &&
@@ -474,8 +477,7 @@ __device__ __attribute__((noinline)) BsPrices
 bsCareful32(float P, float S, float T, float mr, float sigSigTwo,
             const double2_lds *erfTab, uint32_t tLimitBits) {
   BsPrices out;
-  BsPlainTest test(0.f, 1.f, 2.f);
-  test.tLimitBits = tLimitBits;
+  const BsPlainTest test(tLimitBits);
   if (test.lane(P, S, T))
     bsPlain32(P, S, T, mr, sigSigTwo, erfTab, out.call, out.put);
   else
