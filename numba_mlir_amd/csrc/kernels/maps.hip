@@ -231,6 +231,11 @@ NMK_DEFINE_MAP2_FAST(div, OpDiv, f64, double)
 // careful body, so a price can differ in the last places of float32 from what
 // the same option gets inside an all-plain wave; both are within the stated
 // tolerance of the reference (rel 1e-4), by orders of magnitude.
+//
+// The float32 kernel has the same two bodies with every step in float32 (its
+// 0.5 + 0.5 erf also comes from the float64 table, rounded once); there the
+// careful body takes the plain forms for each option that qualifies on its
+// own, so an option gets the same price whichever body its wave runs.
 #include "erf_table.inc"
 
 typedef double double2_lds __attribute__((ext_vector_type(2)));
@@ -278,16 +283,20 @@ template <> struct BsMath<double> {
   }
 };
 template <> struct BsMath<float> {
-  // 1 / sqrt(z) of a float with an exponent in [-60, 60): the hardware seed
-  // (one unit in the last place) with one Newton step, which leaves about
-  // half a unit -- what the two roundings of 1.0f / sqrtf(z) leave as well.
+  // 1 / sqrt(z) of a positive normal float whose exponent lies within
+  // [-120, 122) (z y y then neither overflows nor goes denormal; the plain
+  // body's z is the product of a T in [2^-60, 2^60) and 2 vol^2 in
+  // [2^-59, 2^61]): the hardware seed (one unit in the last place) with one
+  // Newton step, which leaves about half a unit -- what the two roundings of
+  // 1.0f / sqrtf(z) leave as well.
   __device__ static __forceinline__ float rsqrtNormal(float z) {
     const float y = __builtin_amdgcn_rsqf(z);
     const float e = __builtin_fmaf(-(z * y), y, 1.0f); // 1 - z y^2
     return __builtin_fmaf(y * e, 0.5f, y);
   }
-  // Any z: the same value as rsqrtNormal where that applies, so a lane gets
-  // the same price whichever body its wave runs.
+  // Any z, for options outside the plain body's range: the Newton form for
+  // ordinary magnitudes, the library's two operations for the rest (zero,
+  // denormals, infinities, NaN, negative numbers).
   __device__ static __forceinline__ float rsqrt_(float z) {
     return (__float_as_uint(z) - 0x21800000u) < 0x3C000000u ? rsqrtNormal(z)
                                                             : 1.0f / sqrtf(z);
