@@ -218,16 +218,23 @@ class Yardsticks:
         self.no_deps = (ctypes.c_void_p * 1)(None)
         self.events, self.keep, self.kernels = [], [], []
 
-    def launcher(self, name, blocks, threads, pointers, n):
-        """A callable that enqueues kernel(pointers..., int64 n)."""
+    def launcher(self, name, blocks, threads, pointers, n, distance=None, trips=None):
+        """A callable that enqueues kernel(pointers..., int64 n, int distance,
+        int trips): block b takes ``trips`` pieces of ``threads`` words
+        ``distance`` pieces apart (by default a grid apart, as many as cover
+        the n / 4 words)."""
         kern = self.lib.gpuxKernelGet(self.module, name.encode())
         self.kernels.append(kern)
-        values = [ctypes.c_void_p(p) for p in pointers] + [ctypes.c_int64(n)]
+        if distance is None:
+            distance = blocks
+            trips = -(-(n // 4) // (threads * blocks))
+        values = [ctypes.c_void_p(p) for p in pointers] + [
+            ctypes.c_int64(n), ctypes.c_int32(distance), ctypes.c_int32(trips)]
         descs = (self.rt.GPUParamDesc * (len(values) + 1))()
         for i, v in enumerate(values):
             descs[i].data = ctypes.cast(ctypes.pointer(v), ctypes.c_void_p)
             descs[i].size = ctypes.sizeof(v)
-            descs[i].type = 8 if i < len(pointers) else 5
+            descs[i].type = 8 if i < len(pointers) else (5 if i == len(pointers) else 4)
         self.keep.append((values, descs))
 
         def launch():
@@ -329,6 +336,14 @@ def pairwise_body(X1, X2, D):
     D[i, j] = np.sqrt(d)
 
 
+def BS_WALK(nopt):
+    """(blocks, distance, trips) of the Black-Scholes launch over ``nopt``
+    options, as nmhipBlackScholesF32 chooses them: two trips a lane, 128
+    pieces of 256 words apart."""
+    need = -(-(nopt // 4) // 256)
+    return -(-need // 256) * 128, 128, 2
+
+
 def c_call(fn, *args):
     """A step with no Python-side work: the lowered C entry point with its
     arguments marshalled once (the compiled host code's per-call cost)."""
@@ -392,6 +407,7 @@ def stream_placement_study(b):
     slabs = [da.empty((5 * (nbytes + pad),), np.uint8) for _ in range(b.sets)]
     yard = Yardsticks(b.ctx)
     blocks2 = -(-(nopt // 4) // 256) // 2
+    walk = BS_WALK(nopt)
     rows = []
     for delta in (0, 256, 1024, 4096, 4096 + 256, 8192, 12800, 65536, 65536 + 4096,
                   1 << 19, 1 << 20, (1 << 20) + 4096):
@@ -400,9 +416,12 @@ def stream_placement_study(b):
             for k, host in enumerate((price, strike, t)):
                 b.lib.nmhipMemcpyHtoD(b.ctx.handle, p[k], host.ctypes.data, nbytes)
         row = {"delta_bytes": delta}
-        for key, blocks in (("yardstick_2trips_us", blocks2), ("yardstick_1trip_us", 2 * blocks2)):
-            ty = b.measure([yard.launcher("bench_streams_3r2w_f32", blocks, 256, p, nopt)
-                            for p in ptrs], regions=3)
+        for key, blocks, distance, trips in (
+                ("yardstick_2trips_a_grid_apart_us", blocks2, None, None),
+                ("yardstick_1trip_us", 2 * blocks2, None, None),
+                ("yardstick_kernel_walk_us",) + walk):
+            ty = b.measure([yard.launcher("bench_streams_3r2w_f32", blocks, 256, p, nopt,
+                                          distance, trips) for p in ptrs], regions=3)
             row[key] = round(ty.ev * 1e3, 2)
         tk = b.measure([c_call(b.lib.nmhipBlackScholesF32, b.ctx.handle, p[0], p[1], p[2],
                                float(rate), float(vol), p[3], p[4], nopt, 1)
@@ -473,13 +492,13 @@ def run(args):
                 # rungs below it (fewer streams of the same arrays), which show
                 # what each stream adds.
                 yard = Yardsticks(b.ctx)
-                blocks = -(-(nopt // 4) // 256) // 2
+                blocks, distance, trips = BS_WALK(nopt)
                 ladder = {}
                 for rung, streams in (("1r0w", 1), ("0r1w", 1), ("1r1w", 2), ("2r1w", 3),
                                       ("3r1w", 4), ("3r2w", 5)):
                     ty = b.measure([yard.launcher(
-                        f"bench_streams_{rung}_f32", blocks, 256, [x.ptr for x in d], nopt)
-                        for d in sets], regions=3)
+                        f"bench_streams_{rung}_f32", blocks, 256, [x.ptr for x in d], nopt,
+                        distance, trips) for d in sets], regions=3)
                     moved = 4 * nopt * streams
                     ladder[rung] = {
                         "kernel_ms": round(ty.ev, 5),

@@ -2,28 +2,37 @@
 //
 // bench_streams_3r2w_f32 moves exactly the five streams of the Black-Scholes
 // kernel -- three float32 arrays read, two written, 128-bit non-temporal
-// accesses, four elements a lane per trip, the same grid -- with two
-// instructions of arithmetic per output.  Its duration, measured in the same
-// run on the same arrays, is the time the memory system needs for that
-// pattern: the floor any Black-Scholes kernel over these arrays can reach.
+// accesses, four elements a lane per trip, the same grid and the same walk
+// over the arrays (block b takes `trips` pieces of 256 words `distance`
+// pieces apart, as BsTrips in kernels/maps.hip) -- with two instructions of
+// arithmetic per output.  Its duration, measured in the same run on the same
+// arrays, is the time the memory system needs for that pattern.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
 typedef float float4_y __attribute__((ext_vector_type(4)));
 
+__device__ __forceinline__ int64_t walkWord(int distance, int trips, int trip) {
+  const int64_t b = blockIdx.x;
+  const int64_t piece =
+      (b / distance) * (int64_t(trips) * distance) + b % distance + int64_t(trip) * distance;
+  return piece * blockDim.x + threadIdx.x;
+}
+
 extern "C" __global__ __launch_bounds__(256) void
 bench_streams_3r2w_f32(const float *__restrict__ a, const float *__restrict__ b,
                        const float *__restrict__ c, float *__restrict__ x,
-                       float *__restrict__ y, int64_t n) {
+                       float *__restrict__ y, int64_t n, int distance, int trips) {
   const int64_t nvec = n / 4;
   const float4_y *av = reinterpret_cast<const float4_y *>(a);
   const float4_y *bv = reinterpret_cast<const float4_y *>(b);
   const float4_y *cv = reinterpret_cast<const float4_y *>(c);
   float4_y *xv = reinterpret_cast<float4_y *>(x);
   float4_y *yv = reinterpret_cast<float4_y *>(y);
-  const int64_t stride = int64_t(gridDim.x) * blockDim.x;
-  for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec;
-       i += stride) {
+  for (int trip = 0; trip < trips; ++trip) {
+    const int64_t i = walkWord(distance, trips, trip);
+    if (i >= nvec)
+      break;
     const float4_y A = __builtin_nontemporal_load(av + i);
     const float4_y B = __builtin_nontemporal_load(bv + i);
     const float4_y C = __builtin_nontemporal_load(cv + i);
@@ -44,11 +53,13 @@ struct StreamSet {
 };
 
 template <int R, int W>
-__device__ __forceinline__ void streamsBody(const StreamSet &p, int64_t n) {
+__device__ __forceinline__ void streamsBody(const StreamSet &p, int64_t n, int distance,
+                                            int trips) {
   const int64_t nvec = n / 4;
-  const int64_t stride = int64_t(gridDim.x) * blockDim.x;
-  for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec;
-       i += stride) {
+  for (int trip = 0; trip < trips; ++trip) {
+    const int64_t i = walkWord(distance, trips, trip);
+    if (i >= nvec)
+      break;
     float4_y acc = {1.f, 1.f, 1.f, 1.f};
     float4_y v[R > 0 ? R : 1];
 #pragma unroll
@@ -68,14 +79,14 @@ __device__ __forceinline__ void streamsBody(const StreamSet &p, int64_t n) {
 #define BENCH_STREAMS(NAME, R, W)                                              \
   extern "C" __global__ __launch_bounds__(256) void NAME(                      \
       const float *a, const float *b, const float *c, float *x, float *y,      \
-      int64_t n) {                                                             \
+      int64_t n, int distance, int trips) {                                    \
     StreamSet p;                                                               \
     p.r[0] = reinterpret_cast<const float4_y *>(a);                            \
     p.r[1] = reinterpret_cast<const float4_y *>(b);                            \
     p.r[2] = reinterpret_cast<const float4_y *>(c);                            \
     p.w[0] = reinterpret_cast<float4_y *>(x);                                  \
     p.w[1] = reinterpret_cast<float4_y *>(y);                                  \
-    streamsBody<R, W>(p, n);                                                   \
+    streamsBody<R, W>(p, n, distance, trips);                                  \
   }
 BENCH_STREAMS(bench_streams_1r0w_f32, 1, 0)
 BENCH_STREAMS(bench_streams_0r1w_f32, 0, 1)

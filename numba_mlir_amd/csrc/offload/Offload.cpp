@@ -710,18 +710,31 @@ NMHIP_EXPORT void nmhipBlackScholesF32(void *ctx, const float *price,
     // Four options per lane and trip.  Both kernels stream best from many
     // short blocks, two trips a lane (8192 blocks at 2^24 options: 56.5 us
     // against 59 us for 4096 blocks and for 16384, where staging the erf
-    // table once per block weighs more).
+    // table once per block weighs more), the two trips 128 pieces of 256
+    // words (512 KiB of each array) apart (maps.hip, BsTrips); small inputs
+    // and a block count set by hand walk by whole grids.
     const int64_t need = ceilDiv(ceilDiv(n, 4), 256);
-    int64_t blocks = tuning().bsBlocks ? tuning().bsBlocks : ceilDiv(need, 2);
-    if (blocks > need)
-      blocks = need;
-    if (blocks > 0x7fffffff)
-      blocks = 0x7fffffff;
+    int64_t blocks, distance, trips;
+    if (!tuning().bsBlocks && need >= 4 * 128) {
+      distance = 128;
+      trips = 2;
+      blocks = ceilDiv(need, distance * trips) * distance;
+    } else {
+      blocks = tuning().bsBlocks ? tuning().bsBlocks : ceilDiv(need, 2);
+      if (blocks > need)
+        blocks = need;
+      if (blocks > 0x7fffffff)
+        blocks = 0x7fffffff;
+      distance = blocks;
+      trips = ceilDiv(need, blocks);
+    }
+    if (blocks > 0x7fffffff || trips > 0x7fffffff)
+      fail("nmhipBlackScholesF32: %lld options are more than one launch holds", (long long)n);
     c->launch(wide ? "nmk_black_scholes_f32_w64" : "nmk_black_scholes_f32_w32",
               size_t(blocks), 1, 1, 256, 1, 1,
               {Arg::Ptr(price), Arg::Ptr(strike), Arg::Ptr(t), Arg::F32(rate),
                Arg::F32(volatility), Arg::Ptr(call), Arg::Ptr(put),
-               Arg::I64(n)});
+               Arg::I64(n), Arg::I32(int32_t(distance)), Arg::I32(int32_t(trips))});
   });
 }
 

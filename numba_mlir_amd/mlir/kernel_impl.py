@@ -650,8 +650,9 @@ def plan_compiled(ctx, compiled, func_name, global_size, args, ret=None,
             and not make_partials and grid[0] >= 4096:
         # Every block stages its table before its first element: half the
         # blocks, two trips a lane (the Black-Scholes body over 2^24 options:
-        # 8192 blocks against 16384).
-        grid[0] = -(-grid[0] // 2)
+        # 8192 blocks against 16384), in whole groups of 128 blocks (the
+        # kernel then takes its two trips 128 pieces apart).
+        grid[0] = -(-grid[0] // 256) * 128
     if make_partials and getattr(compiled, "grid_stride", False):
         # a reduction: few, long-running blocks (one partial result each); the
         # more arrays they stream at once, the fewer (two arrays of 512 MiB:
