@@ -428,11 +428,30 @@ def stream_placement_study(b):
                         for p in ptrs], regions=3)
         row["black_scholes_us"] = round(tk.ev * 1e3, 2)
         rows.append(row)
+    del slabs
+    # The same rungs on longer arrays: what a stream costs once the start
+    # and the end of the launch no longer weigh, and whether that depends on
+    # how many streams run side by side.
+    sizes = []
+    ones = np.ones(2 ** 26, np.float32)
+    big = [[da.asarray(ones) for _ in range(5)] for _ in range(2)]
+    for log2n in (22, 23, 24, 25, 26):
+        n = 2 ** log2n
+        row = {"elements_per_array": f"2^{log2n}", "MiB_per_array": 4 * n >> 20}
+        for rung, streams in (("1r0w", 1), ("0r1w", 1), ("0r2w", 2), ("1r1w", 2), ("3r2w", 5)):
+            ty = b.measure([yard.launcher(f"bench_streams_{rung}_f32", *BS_WALK(n)[:1], 256,
+                                          [x.ptr for x in arrays], n, *BS_WALK(n)[1:])
+                            for arrays in big], regions=3)
+            row[rung] = {"us": round(ty.ev * 1e3, 2),
+                         "frac_of_peak": round(4 * n * streams / (ty.ev * 1e-3) / 1e9
+                                               / HBM_PEAK_GBS, 4)}
+        sizes.append(row)
     yard.close()
     return {"name": "streams",
             "workload": "five float32 arrays of 2^24 elements carved from one slab, "
-                        "array k at k * (64 MiB + delta)",
-            "placements": rows}
+                        "array k at k * (64 MiB + delta); then the rungs of the ladder "
+                        "on separately allocated arrays of 2^22 .. 2^26 elements",
+            "placements": rows, "sizes": sizes}
 
 
 def run(args):

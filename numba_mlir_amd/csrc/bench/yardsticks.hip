@@ -42,8 +42,8 @@ bench_streams_3r2w_f32(const float *__restrict__ a, const float *__restrict__ b,
 }
 
 // The ladder: R float32 arrays read and W written with the same accesses and
-// grid as above (1r0w, 0r1w, 1r1w, 2r1w, 3r1w; bench_streams_3r2w_f32 is the
-// top rung).  It shows what each additional stream costs on this memory
+// grid as above (1r0w, 0r1w, 0r2w, 1r1w, 2r1w, 3r1w; bench_streams_3r2w_f32
+// is the top rung).  It shows what each additional stream costs on this memory
 // system, i.e. whether the five-stream mix is slower than fewer streams of
 // the same total size.  A read-only rung consumes what it loads through a
 // store that no input ever triggers.
@@ -90,6 +90,7 @@ __device__ __forceinline__ void streamsBody(const StreamSet &p, int64_t n, int d
   }
 BENCH_STREAMS(bench_streams_1r0w_f32, 1, 0)
 BENCH_STREAMS(bench_streams_0r1w_f32, 0, 1)
+BENCH_STREAMS(bench_streams_0r2w_f32, 0, 2)
 BENCH_STREAMS(bench_streams_1r1w_f32, 1, 1)
 BENCH_STREAMS(bench_streams_2r1w_f32, 2, 1)
 BENCH_STREAMS(bench_streams_3r1w_f32, 3, 1)
