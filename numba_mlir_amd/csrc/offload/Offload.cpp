@@ -700,19 +700,20 @@ NMHIP_EXPORT void nmhipBlackScholesF32(void *ctx, const float *price,
   guarded([&]() {
     Context *c = toCtx(ctx);
     std::lock_guard<std::mutex> lock(c->mutex);
-    if (n <= 0)
+    if (n < 0)
+      fail("nmhipBlackScholesF32: negative extent");
+    if (n == 0)
       return;
     if (!(aligned16(price) && aligned16(strike) && aligned16(t) &&
           aligned16(call) && aligned16(put)))
       fail("nmhipBlackScholesF32: arrays must be 16-byte aligned");
-    if (n < 0)
-      fail("nmhipBlackScholesF32: negative extent");
     // Four options per lane and trip.  Both kernels stream best from many
-    // short blocks, two trips a lane (8192 blocks at 2^24 options: 56.5 us
-    // against 59 us for 4096 blocks and for 16384, where staging the erf
-    // table once per block weighs more), the two trips 128 pieces of 256
-    // words (512 KiB of each array) apart (maps.hip, BsTrips); small inputs
-    // and a block count set by hand walk by whole grids.
+    // short blocks, two trips a lane (8192 blocks at 2^24 options: 2.5 us
+    // faster than 4096 blocks and than 16384, where staging the erf table
+    // once per block weighs more), the two trips 128 pieces of 256 words
+    // (512 KiB of each array) apart (maps.hip, BsTrips: 1 to 1.6 us faster
+    // than a grid apart); small inputs and a block count set by hand walk by
+    // whole grids.
     const int64_t need = ceilDiv(ceilDiv(n, 4), 256);
     int64_t blocks, distance, trips;
     if (!tuning().bsBlocks && need >= 4 * 128) {
