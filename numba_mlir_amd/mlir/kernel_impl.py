@@ -626,12 +626,6 @@ def plan_key(args):
                  for a in args)
 
 
-def _launch_loaded(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret=None,
-                   partials=()):
-    LaunchPlan(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret,
-               partials).run()
-
-
 def plan_compiled(ctx, compiled, func_name, global_size, args, ret=None,
                   make_partials=None):
     """Loads a translated function (once) and prepares its launch over
@@ -663,14 +657,6 @@ def plan_compiled(ctx, compiled, func_name, global_size, args, ret=None,
     partials = make_partials(grid[0] * grid[1] * grid[2]) if make_partials else ()
     return LaunchPlan(ctx, compiled, kern, func_name, grid, block, gsize3, args, ret,
                       partials)
-
-
-def launch_compiled(ctx, compiled, func_name, global_size, args, ret=None,
-                    make_partials=None):
-    """plan_compiled + one launch; returns the launch geometry."""
-    plan = plan_compiled(ctx, compiled, func_name, global_size, args, ret, make_partials)
-    plan.run()
-    return plan.info
 
 
 def kernel(func=None, **kwargs):
