@@ -98,16 +98,21 @@ rowSumF32(const float *__restrict__ x, float *__restrict__ out, int64_t rows,
   }
 }
 
-#define NMK_DEFINE_ROWSUM(NAME, NORM, WPR)                                     \
-  NMK_KERNEL(256)                                                              \
+// The block-per-row kernels run at most three waves a SIMD (three blocks a
+// CU, 12 MiB of loads in flight over the device): with the eight that would
+// fit, the memory system queues more than it can use (measured on MI355X,
+// [16384, 8192]: 8 waves 78.4 us, 5 78.5, 4 77.2, 3 74.1, 2 89.0).
+#define NMK_DEFINE_ROWSUM(NAME, NORM, WPR, WAVES)                              \
+  extern "C" __global__ __launch_bounds__(256)                                 \
+  __attribute__((amdgpu_waves_per_eu(1, WAVES))) void                          \
   NAME(const float *x, float *out, int64_t rows, int64_t cols, int64_t ld,     \
        int32_t vec) {                                                          \
     rowSumF32<NORM, WPR>(x, out, rows, cols, ld, vec);                         \
   }
-NMK_DEFINE_ROWSUM(nmk_sum_axis1_f32, false, 1)
-NMK_DEFINE_ROWSUM(nmk_sum_axis1_wide_f32, false, 4)
-NMK_DEFINE_ROWSUM(nmk_norm2_axis1_f32, true, 1)
-NMK_DEFINE_ROWSUM(nmk_norm2_axis1_wide_f32, true, 4)
+NMK_DEFINE_ROWSUM(nmk_sum_axis1_f32, false, 1, 8)
+NMK_DEFINE_ROWSUM(nmk_sum_axis1_wide_f32, false, 4, 3)
+NMK_DEFINE_ROWSUM(nmk_norm2_axis1_f32, true, 1, 8)
+NMK_DEFINE_ROWSUM(nmk_norm2_axis1_wide_f32, true, 4, 3)
 
 // ---------------------------------------------------------------------------
 // out[c] = sum_r int64(x[r * ld + c]), int32 input.  Requires cols % 4 == 0,
