@@ -47,7 +47,7 @@ MEASURED_TRAFFIC = {
     "bench_streams_3r2w_f32": 335539264,
     "nmk_black_scholes_f32_w32": 335608254,
     "nmk_map2_rowbcast_add_f64": 268482872,
-    "nmk_sum_axis1_wide_f32": 537407528,
+    "nmk_sum_axis1_wide_w3_f32": 537407528,
     "nmk_norm2_f32": 536935334,
     "nmk_sum_axis0_i32_i64": 538046216,
     "nmk_twin_pairwise_f64_rows": 540389308,

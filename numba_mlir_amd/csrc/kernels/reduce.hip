@@ -98,10 +98,14 @@ rowSumF32(const float *__restrict__ x, float *__restrict__ out, int64_t rows,
   }
 }
 
-// The block-per-row kernels run at most three waves a SIMD (three blocks a
-// CU, 12 MiB of loads in flight over the device): with the eight that would
-// fit, the memory system queues more than it can use (measured on MI355X,
-// [16384, 8192]: 8 waves 78.4 us, 5 78.5, 4 77.2, 3 74.1, 2 89.0).
+// The block-per-row kernels also come capped at three and at four waves a
+// SIMD (three or four blocks a CU): with the eight that fit, the memory
+// system queues more loads than it can use.  Which cap wins depends on how
+// many 16 KiB batches a row holds; the host chooses (measured on MI355X,
+// 8 / 4 / 3 waves: [16384, 8192] 78.6 / 76.6 / 74.5 us, [16384, 12288]
+// 117.1 / 115.1 / 112.9, [32768, 4096] 78.5 / 74.2 / 84.4, [65536, 4096]
+// 156 / 146 / 167; rows that do not end on a batch and rows of four batches
+// or more are as fast or faster uncapped).
 #define NMK_DEFINE_ROWSUM(NAME, NORM, WPR, WAVES)                              \
   extern "C" __global__ __launch_bounds__(256)                                 \
   __attribute__((amdgpu_waves_per_eu(1, WAVES))) void                          \
@@ -110,9 +114,13 @@ rowSumF32(const float *__restrict__ x, float *__restrict__ out, int64_t rows,
     rowSumF32<NORM, WPR>(x, out, rows, cols, ld, vec);                         \
   }
 NMK_DEFINE_ROWSUM(nmk_sum_axis1_f32, false, 1, 8)
-NMK_DEFINE_ROWSUM(nmk_sum_axis1_wide_f32, false, 4, 3)
+NMK_DEFINE_ROWSUM(nmk_sum_axis1_wide_f32, false, 4, 8)
+NMK_DEFINE_ROWSUM(nmk_sum_axis1_wide_w4_f32, false, 4, 4)
+NMK_DEFINE_ROWSUM(nmk_sum_axis1_wide_w3_f32, false, 4, 3)
 NMK_DEFINE_ROWSUM(nmk_norm2_axis1_f32, true, 1, 8)
-NMK_DEFINE_ROWSUM(nmk_norm2_axis1_wide_f32, true, 4, 3)
+NMK_DEFINE_ROWSUM(nmk_norm2_axis1_wide_f32, true, 4, 8)
+NMK_DEFINE_ROWSUM(nmk_norm2_axis1_wide_w4_f32, true, 4, 4)
+NMK_DEFINE_ROWSUM(nmk_norm2_axis1_wide_w3_f32, true, 4, 3)
 
 // ---------------------------------------------------------------------------
 // out[c] = sum_r int64(x[r * ld + c]), int32 input.  Requires cols % 4 == 0,

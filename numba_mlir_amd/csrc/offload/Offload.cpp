@@ -113,6 +113,25 @@ Tuning &tuning() {
   return t;
 }
 
+// Which of the block-per-row kernels of float32 rows (`stem`_wide[_w4|_w3]_f32;
+// reduce.hip) suits rows of n1 elements read as 128-bit words: a row is read
+// in batches of 16 KiB (1024 words), the rest word by word a lane.  Rows of
+// exactly one batch run fastest at four waves a SIMD, rows of two or three
+// whole batches at three when there are thousands of them, anything else
+// uncapped.
+std::string wideRowKernel(const char *stem, int64_t n0, int64_t n1, bool words) {
+  const int64_t nvec = n1 / 4;
+  const char *cap = "";
+  if (words && nvec % 1024 == 0) {
+    const int64_t batches = nvec / 1024;
+    if (batches == 1)
+      cap = "_w4";
+    else if (batches <= 3 && n0 >= 4096)
+      cap = "_w3";
+  }
+  return std::string(stem) + "_wide" + cap + "_f32";
+}
+
 // Blocks of the float32 full sums (nmk_sum_all_f32, nmk_norm2_f32), each with
 // 16 KiB of loads in flight: 6 MiB over the device.  Measured on MI355X over
 // 512 MiB: 256 blocks 88.9 us, 320 80.5, 384 76.5, 448 77.1, 512 78.2, 768 79.4.
@@ -766,7 +785,8 @@ NMHIP_EXPORT void nmhipReduce(void *ctx, int op, int dtype, const void *x,
       const int vec = (aligned16(x) && s0 % 4 == 0 && n1 % 4 == 0) ? 1 : 0;
       // a block per row for long rows, a wave per row otherwise
       const bool wide = n1 >= 4096;
-      c->launchBlocksXY(wide ? "nmk_sum_axis1_wide_f32" : "nmk_sum_axis1_f32",
+      c->launchBlocksXY(wide ? wideRowKernel("nmk_sum_axis1", n0, n1, vec != 0)
+                             : std::string("nmk_sum_axis1_f32"),
                         wide ? n0 : ceilDiv(n0, 4),
                         {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(n0), Arg::I64(n1),
                          Arg::I64(s0), Arg::I32(vec)});
@@ -937,7 +957,8 @@ NMHIP_EXPORT void nmhipNorm2RowsF32(void *ctx, const float *x, int64_t n0,
       return;
     const int vec = (aligned16(x) && s0 % 4 == 0 && n1 % 4 == 0) ? 1 : 0;
     const bool wide = n1 >= 4096;
-    c->launchBlocksXY(wide ? "nmk_norm2_axis1_wide_f32" : "nmk_norm2_axis1_f32",
+    c->launchBlocksXY(wide ? wideRowKernel("nmk_norm2_axis1", n0, n1, vec != 0)
+                           : std::string("nmk_norm2_axis1_f32"),
                       wide ? n0 : ceilDiv(n0, 4),
                       {Arg::Ptr(x), Arg::Ptr(out), Arg::I64(n0), Arg::I64(n1),
                        Arg::I64(s0), Arg::I32(vec)});

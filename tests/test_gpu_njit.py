@@ -315,7 +315,7 @@ def test_reductions_and_contractions_go_to_the_library(env):
     xi = workloads.reduce_i32(256, 512)
     f = njit(cases.row_sums)
     got = f(hip.asarray(x))
-    assert f.last_launch == {"path": "library", "kernel": "nmk_sum_axis1_wide_f32"}
+    assert f.last_launch == {"path": "library", "kernel": "nmk_sum_axis1_wide_w4_f32"}
     np.testing.assert_allclose(got.asnumpy(), x.astype(np.float64).sum(axis=1), rtol=1e-4,
                                atol=1e-3)
     f = njit(cases.col_sums)

@@ -125,15 +125,19 @@ def test_sum_axis0_i32_bit_exact(env, shape):
 # The reference states rel 1e-4/1e-5 on positive data; for zero-mean data the
 # sum itself can be arbitrarily close to 0, so the bound is relative to the
 # sum of magnitudes.
-@pytest.mark.parametrize("shape", [(4, 8192), (333, 1000), (16384, 8192),
-                                   (7, 5), (1024, 4100)])
-def test_sum_axis1_f32(env, shape):
+# (rows of one 16 KiB batch run the kernel capped at four waves a SIMD, many
+# rows of two or three whole batches the one capped at three)
+@pytest.mark.parametrize("shape, kernel", [
+    ((4, 8192), "nmk_sum_axis1_wide_f32"), ((333, 1000), "nmk_sum_axis1_f32"),
+    ((16384, 8192), "nmk_sum_axis1_wide_w3_f32"), ((7, 5), "nmk_sum_axis1_f32"),
+    ((1024, 4100), "nmk_sum_axis1_wide_f32"), ((600, 4096), "nmk_sum_axis1_wide_w4_f32"),
+    ((4100, 12288), "nmk_sum_axis1_wide_w3_f32"), ((4100, 16384), "nmk_sum_axis1_wide_f32")])
+def test_sum_axis1_f32(env, shape, kernel):
     hip, ops, orc = env
     rng = np.random.Generator(np.random.PCG64(1003))
     x = rng.standard_normal(shape, dtype=np.float32)
     got = ops.sum(hip.asarray(x), axis=1).asnumpy()
-    assert hip.get_context().last_kernel() == (
-        "nmk_sum_axis1_wide_f32" if shape[1] >= 4096 else "nmk_sum_axis1_f32")
+    assert hip.get_context().last_kernel() == kernel
     x64 = x.astype(np.float64)
     truth, mag = x64.sum(axis=1), np.abs(x64).sum(axis=1)
     assert (np.abs(got - truth) <= 1e-4 * mag).all()
