@@ -43,22 +43,22 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 WAKE_SECONDS = 0.1
 
 MEASURED_TRAFFIC = {
-    "nmk_black_scholes_f32_w64": 335628470,
-    "bench_streams_3r2w_f32": 335539264,
-    "nmk_black_scholes_f32_w32": 335608254,
-    "nmk_map2_rowbcast_add_f64": 268482872,
-    "nmk_sum_axis1_wide_w3_f32": 537407528,
-    "nmk_norm2_f32": 536935334,
-    "nmk_sum_axis0_i32_i64": 538046216,
-    "nmk_twin_pairwise_f64_rows": 540389308,
+    "nmk_black_scholes_f32_w64": 335649485,
+    "bench_streams_3r2w_f32": 335534747,
+    "nmk_black_scholes_f32_w32": 335642360,
+    "nmk_map2_rowbcast_add_f64": 268472994,
+    "nmk_sum_axis1_wide_w3_f32": 537389868,
+    "nmk_norm2_f32": 536908191,
+    "nmk_sum_axis0_i32_i64": 538010333,
+    "nmk_twin_pairwise_f64_rows": 540311645,
     "nmk_copy_b128": 536870912,
-    "sgemm_mfma_256x256": 671610898,
-    "sgemm_thin_rows": 1074402309,
+    "sgemm_mfma_256x256": 671673097,
+    "sgemm_thin_rows": 1074340818,
     # generated kernels, without the hash of the body at the end of their names
-    "nmkjit_black_scholes_body": 335622063,
-    "nmkjit_black_scholes_loop_body": 335634761,
-    "nmkjit_scaled_add_body": 402646767,
-    "nmkjit_pairwise_body": 540463079,
+    "nmkjit_black_scholes_body": 335659027,
+    "nmkjit_black_scholes_loop_body": 335656068,
+    "nmkjit_scaled_add_body": 402630317,
+    "nmkjit_pairwise_body": 540468990,
 }
 
 
