@@ -12,10 +12,13 @@
 
 typedef float float4_y __attribute__((ext_vector_type(4)));
 
+// (distance: a power of two, or at least the number of blocks)
 __device__ __forceinline__ int64_t walkWord(int distance, int trips, int trip) {
-  const int64_t b = blockIdx.x;
-  const int64_t piece =
-      (b / distance) * (int64_t(trips) * distance) + b % distance + int64_t(trip) * distance;
+  const uint32_t b = blockIdx.x, d = uint32_t(distance);
+  const bool shared = (d & (d - 1)) == 0;
+  const uint32_t run = shared ? b >> (31 - __builtin_clz(d)) : 0;
+  const uint32_t place = shared ? b & (d - 1) : b;
+  const int64_t piece = int64_t(run) * (int64_t(trips) * d) + place + int64_t(trip) * d;
   return piece * blockDim.x + threadIdx.x;
 }
 

@@ -499,18 +499,22 @@ bsCareful32(float P, float S, float T, float mr, float sigSigTwo,
 // takes `count` pieces `distance` pieces apart,
 //   piece(b, trip) = (b / distance) * count * distance + b % distance + trip * distance,
 // so every run of count * distance pieces is shared out among `distance`
-// consecutive blocks.  distance = number of blocks is the usual grid-stride
-// walk.  Two trips 128 pieces (512 KiB) apart measured fastest for the five
-// streams of this kernel at 2^24 options: 55.3-55.8 us against 56.4-57.2 for
-// two trips a grid apart, 58-62 for pieces 2 to 64 apart and 57-59 for 256 to
-// 1024 (the memory-only kernel with the same walk: 53.4-54.0 against
-// 55.2-55.8).
+// consecutive blocks.  `distance` is a power of two (quotient and remainder
+// are a shift and a mask: a division of 64-bit integers is some 150 scalar
+// instructions at the head of every wave, 1 us of this kernel) or at least
+// the number of blocks, which is the usual grid-stride walk.  Two trips 128
+// pieces (512 KiB) apart measured fastest for the five streams of this kernel
+// at 2^24 options: 55.3-55.8 us against 56.4-57.2 for two trips a grid
+// apart, 58-62 for pieces 2 to 64 apart and 57-59 for 256 to 1024 (the
+// memory-only kernel with the same walk: 53.4-54.0 against 55.2-55.8).
 struct BsTrips {
   int distance, count;
   __device__ __forceinline__ int64_t word(int trip) const {
-    const int64_t b = blockIdx.x;
-    const int64_t piece =
-        (b / distance) * (int64_t(count) * distance) + b % distance + int64_t(trip) * distance;
+    const uint32_t b = blockIdx.x, d = uint32_t(distance);
+    const bool shared = (d & (d - 1)) == 0; // else d >= gridDim.x > b
+    const uint32_t run = shared ? b >> (31 - __builtin_clz(d)) : 0;
+    const uint32_t place = shared ? b & (d - 1) : b;
+    const int64_t piece = int64_t(run) * (int64_t(count) * d) + place + int64_t(trip) * d;
     return piece * blockDim.x + threadIdx.x;
   }
 };

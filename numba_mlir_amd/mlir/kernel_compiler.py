@@ -776,15 +776,18 @@ class FunctionTranslator:
             # lie 128 pieces (of one word a lane of a block) apart, not a grid
             # apart: the fastest walk measured for such kernels (the
             # Black-Scholes body over 2^24 options: 55.8 against 57.2 us).
+            # Written without divisions: one of 64-bit integers is some 150
+            # scalar instructions at the head of every wave.
             out += [
-                "  const int64_t nmk_pieces = (nmk_nvec + nmk_lsz0 - 1) / nmk_lsz0;",
-                "  const int64_t nmk_trips = (nmk_pieces + gridDim.x - 1) / gridDim.x;",
-                "  const int64_t nmk_apart = (nmk_trips == 2 && gridDim.x % 128 == 0) ? 128 "
-                ": gridDim.x;",
-                "  for (int64_t nmk_trip = 0; nmk_trip < nmk_trips; ++nmk_trip) {",
-                "    const int64_t nmk_i = ((nmk_grp0 / nmk_apart) * (nmk_trips * nmk_apart) + "
-                "nmk_grp0 % nmk_apart + nmk_trip * nmk_apart) * nmk_lsz0 + nmk_lid0;",
-                "    if (nmk_i >= nmk_nvec) break;",
+                "  const int64_t nmk_sweep = nmk_lanes;    // words a trip of the whole grid takes",
+                "  const bool nmk_paired = gridDim.x % 128 == 0 && nmk_nvec > nmk_sweep && "
+                "nmk_nvec <= 2 * nmk_sweep;",
+                "  const int64_t nmk_step = nmk_paired ? 128 * nmk_lsz0 : nmk_sweep;",
+                "  const int64_t nmk_first = nmk_paired ? (((nmk_grp0 >> 7) << 8) + "
+                "(nmk_grp0 & 127)) * nmk_lsz0 + nmk_lid0 : nmk_lane;",
+                "  const int64_t nmk_behind = nmk_paired ? nmk_first + 2 * nmk_step : nmk_nvec;",
+                "  for (int64_t nmk_i = nmk_first; nmk_i < nmk_nvec && nmk_i < nmk_behind; "
+                "nmk_i += nmk_step) {",
             ]
         else:
             out.append("  for (int64_t nmk_i = nmk_lane; nmk_i < nmk_nvec; nmk_i += nmk_lanes) {")
