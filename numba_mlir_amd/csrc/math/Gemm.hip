@@ -218,7 +218,12 @@ struct EvenShares {
 };
 __host__ __device__ inline int64_t evenSharesStart(int64_t g, int64_t units,
                                                    int64_t blocks) {
-  return g * units / blocks; // (units * blocks stays far below 2^63)
+  const int64_t scaled = g * units; // (units * blocks stays far below 2^63)
+  // (32-bit operands wherever they fit: on the device a division of 64-bit
+  // integers is some 150 instructions, and the kernels call this per piece)
+  if ((uint64_t(scaled) | uint64_t(blocks)) >> 32)
+    return scaled / blocks;
+  return int64_t(uint32_t(scaled) / uint32_t(blocks));
 }
 
 // GUARD: 0 whole tiles; 1 loads and stores guarded (operands and C of any
@@ -442,7 +447,7 @@ gemm_even_fold(const T *__restrict__ W, int64_t blocks, int slabs, int tilesN,
   const int64_t tile = blockIdx.x;
   const int64_t u0 = tile * slabs, u1 = u0 + slabs;
   // the block whose share holds the tile's first unit
-  int64_t g = u0 * blocks / units;
+  int64_t g = evenSharesStart(u0, blocks, units); // u0 * blocks / units
   while (g > 0 && evenSharesStart(g, units, blocks) > u0)
     --g;
   while (g + 1 < blocks && evenSharesStart(g + 1, units, blocks) <= u0)
@@ -482,11 +487,6 @@ gemm_even_fold(const T *__restrict__ W, int64_t blocks, int slabs, int tilesN,
 }
 
 // ---------------------------------------------------------------------------
-// C[m][n] = alpha * (W[0][m][n] + W[1][m][n] + ...) + beta * C[m][n]: the
-// slices of a split-K product added in index order (a fixed order, so the
-// result does not depend on which block finished first).  One thread per
-// 128-bit word of a row of W (ldw and the slice stride are multiples of the
-// word); stores to C are per element, C may end inside the last word.
 // word = row * perRow + inRow, for a lane's word of a matrix of perRow words a
 // row: with 32-bit operands wherever they fit (a division of 64-bit integers
 // is a hundred vector instructions a lane, 0.8 us of a fold of 1024 x 1024).
@@ -502,6 +502,12 @@ __device__ __forceinline__ void splitWord(int64_t word, int64_t perRow, int64_t 
   }
 }
 
+// ---------------------------------------------------------------------------
+// C[m][n] = alpha * (W[0][m][n] + W[1][m][n] + ...) + beta * C[m][n]: the
+// slices of a split-K product added in index order (a fixed order, so the
+// result does not depend on which block finished first).  One thread per
+// 128-bit word of a row of W (ldw and the slice stride are multiples of the
+// word); stores to C are per element, C may end inside the last word.
 template <typename T>
 __global__ __launch_bounds__(256) void
 gemm_splitk_fold(const T *__restrict__ W, int slices, int64_t sliceStride,
