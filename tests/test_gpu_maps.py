@@ -303,6 +303,25 @@ def test_black_scholes_float32_typing(env):
     np.testing.assert_allclose(put, wp, atol=GOLD["black_scholes"]["atol"])
 
 
+@pytest.mark.parametrize("wide", [True, False])
+def test_black_scholes_block_counts_set_by_hand(env, wide):
+    """Which block takes which options (two trips 128 pieces apart by default,
+    whole grids apart for a block count set by hand, a power of two or not)
+    does not change a price: on everyday operands every wave runs the same
+    arithmetic."""
+    from numba_mlir_amd.mlir import lowered
+    hip, ops, _ = env
+    n = 700003
+    _, call, put = _run_bs(hip, ops, n, wide)
+    try:
+        for blocks in (1, 3, 100, 128, 1000, 4096):
+            lowered.set_tuning("bs_blocks", blocks)
+            _, c2, p2 = _run_bs(hip, ops, n, wide)
+            assert c2.tobytes() == call.tobytes() and p2.tobytes() == put.tobytes(), blocks
+    finally:
+        lowered.set_tuning("bs_blocks", 0)
+
+
 def test_black_scholes_full_size(env):
     """2^24 options: oracle parity plus put-call parity and the closed form."""
     hip, ops, orc = env
